@@ -1,0 +1,301 @@
+#!/usr/bin/env python3
+"""Benchmark of the CSR SpMV / SpMM / csr2csc path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME]
+
+A step is one pass of the hot path (one mcsparseSpMV / mcsparseSpMM / mcsparseCsr2cscEx2 call
+through the C ABI) over one synthetic operand set that is already resident in HBM.  Several
+independent copies of all operands are rotated so the 256 MB Infinity Cache cannot hold a
+matrix between steps.  The default workload is the configuration the metric is quoted on:
+fp64 CSR SpMV, 1,048,576 rows x 16 nonzeros per row.  Prints one JSON line.
+
+Workloads: c1 (5-pt Laplacian 256^2 fp32), c2 (default), c3 / c3t (power-law fp32, op N / T),
+c4-8 / c4-64 / c4-256 (27-pt stencil 128^3 SpMM), c5 (csr2csc on the c3 matrix),
+c5-coo (csr2coo on it), c5-spmv (A^T x from the converted CSC).
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
+
+
+def parse():
+    p = argparse.ArgumentParser()
+    p.add_argument("--gpus", type=int, default=1)
+    p.add_argument("--steps", type=int, default=None)
+    p.add_argument("--warmup", type=int, default=None)
+    p.add_argument("--workload", default="c2")
+    p.add_argument("--copies", type=int, default=None, help="independent operand sets rotated between steps")
+    p.add_argument("--scale", type=float, default=1.0, help="shrink the workload (for dry runs); 1.0 = as specified")
+    p.add_argument("--no-cpu-baseline", action="store_true")
+    p.add_argument("--family", type=int, default=0, help="force the SpMV kernel family (1 vector, 2 merge)")
+    p.add_argument("--lanes", type=int, default=0, help="force lanes per row of the vector family")
+    return p.parse_args()
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this path has no multi-GPU part (got --gpus %d)" % args.gpus,
+              file=sys.stderr)
+        return 2
+
+    import torch
+    from mcsparse_amd import api
+    from mcsparse_amd import workloads as wl
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        return 2
+    torch.cuda.set_device(0)
+    stream = torch.cuda.current_stream()
+    handle = api.Handle(stream=stream.cuda_stream)
+    name = args.workload
+    s = args.scale
+
+    def dev(a):
+        return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+    t_gen = time.time()
+    kind = "spmv"
+    op = api.OP_N
+    n_cols = 0
+    if name == "c1":
+        a = wl.laplacian_5pt(max(4, int(256 * s)), dtype=np.float32)
+        alpha, beta, desc = 1.0, 0.0, "fp32 CSR SpMV, 5-pt Laplacian 256x256"
+    elif name == "c2":
+        a = wl.uniform_rows(m=max(64, int((1 << 20) * s)), per_row=16, dtype=np.float64)
+        alpha, beta, desc = 1.5, 0.5, "fp64 CSR SpMV, 1048576 rows x 16 nnz/row uniform"
+    elif name in ("c3", "c3t", "c5", "c5-coo", "c5-spmv"):
+        a = wl.power_law(m=max(64, int((1 << 22) * s)), max_len=max(8, int(200000 * min(1.0, s * 4))),
+                         dtype=np.float32)
+        alpha, beta = 1.0, 0.0
+        desc = "fp32 CSR SpMV, 4194304 rows power-law (Zipf 1.8, <=200000 nnz/row)"
+        if name == "c3t":
+            op = api.OP_T
+            desc += ", op T"
+        if name == "c5":
+            kind, desc = "csr2csc", "csr2csc (values + structure) of the fp32 power-law matrix"
+        if name == "c5-coo":
+            kind, desc = "csr2coo", "csr2coo of the power-law matrix"
+        if name == "c5-spmv":
+            kind, desc = "spmv-csc", "fp32 SpMV op T from the CSC produced by csr2csc (power-law matrix)"
+    elif name.startswith("c4-"):
+        n_cols = int(name.split("-")[1])
+        a = wl.stencil_27pt(max(4, int(round(128 * s ** (1 / 3)))), dtype=np.float32)
+        alpha, beta, kind = 1.0, 0.0, "spmm"
+        desc = "fp32 CSR SpMM, 27-pt stencil 128^3, B row-major N=%d" % n_cols
+    else:
+        print("unknown workload %r" % name, file=sys.stderr)
+        return 2
+    gen_s = time.time() - t_gen
+
+    dt = a.val.dtype
+    vb = dt.itemsize
+    ct = api.maca_type(dt)
+    tdt = torch.float32 if vb == 4 else torch.float64
+    if kind in ("spmv", "spmv-csc"):
+        algo_bytes = wl.spmv_bytes(a, vb)
+        flops = 2 * a.nnz
+        extra_read = a.m * vb if beta != 0 else 0
+    elif kind == "spmm":
+        algo_bytes = wl.spmm_bytes(a, n_cols, vb)
+        flops = 2 * a.nnz * n_cols
+        extra_read = 0
+    elif kind == "csr2csc":
+        algo_bytes = (a.m + 1) * 4 + (a.n + 1) * 4 + 2 * a.nnz * (4 + vb)
+        flops, extra_read = 0, 0
+    else:
+        algo_bytes = (a.m + 1) * 4 + 4 * a.nnz
+        flops, extra_read = 0, 0
+
+    # enough copies that the rotated footprint exceeds the 256 MB Infinity Cache several times
+    copies = args.copies or max(2, min(8, int(np.ceil(1.2e9 / max(algo_bytes, 1)))))
+    if algo_bytes > 8e8:
+        copies = args.copies or 2
+    steps = args.steps if args.steps is not None else (200 if algo_bytes < 6e8 else 40)
+    warmup = args.warmup if args.warmup is not None else (20 if algo_bytes < 6e8 else 5)
+
+    rng = np.random.default_rng(12345)
+    sets = []
+    for c in range(copies):
+        st = {"ptr": dev(a.ptr), "col": dev(a.col), "val": dev(a.val)}
+        if kind == "spmv":
+            xs, ys = (a.n, a.m) if op == api.OP_N else (a.m, a.n)
+            st["x"] = dev(rng.uniform(-1, 1, xs).astype(dt))
+            st["y"] = dev(rng.uniform(-1, 1, ys).astype(dt))
+            st["mat"] = api.SpMat(a.m, a.n, a.nnz, st["ptr"], st["col"], st["val"], base=a.base)
+            if args.family or args.lanes:
+                st["mat"].set_plan(args.family, args.lanes)
+            st["vx"], st["vy"] = api.DnVec(st["x"]), api.DnVec(st["y"])
+            rc, size = api.spmv_buffer_size(handle, op, alpha, st["mat"], st["vx"], beta, st["vy"], ct)
+            api.check(rc, "mcsparseSpMV_bufferSize")
+            st["buf"] = torch.empty(size, dtype=torch.uint8, device="cuda")
+        elif kind == "spmm":
+            st["B"] = dev(rng.uniform(-1, 1, (a.n, n_cols)).astype(dt))
+            st["C"] = torch.zeros((a.m, n_cols), dtype=tdt, device="cuda")
+            st["mat"] = api.SpMat(a.m, a.n, a.nnz, st["ptr"], st["col"], st["val"], base=a.base)
+            st["mB"] = api.DnMat(a.n, n_cols, n_cols, st["B"], order=api.ORDER_ROW)
+            st["mC"] = api.DnMat(a.m, n_cols, n_cols, st["C"], order=api.ORDER_ROW)
+            rc, size = api.spmm_buffer_size(handle, api.OP_N, api.OP_N, alpha, st["mat"], st["mB"], beta, st["mC"], ct)
+            api.check(rc, "mcsparseSpMM_bufferSize")
+            st["buf"] = torch.empty(size, dtype=torch.uint8, device="cuda")
+        elif kind in ("csr2csc", "spmv-csc"):
+            st["o_val"] = torch.zeros(a.nnz, dtype=tdt, device="cuda")
+            st["o_ptr"] = torch.zeros(a.n + 1, dtype=torch.int32, device="cuda")
+            st["o_row"] = torch.zeros(a.nnz, dtype=torch.int32, device="cuda")
+            rc, size = api.csr2csc_buffer_size(handle, a.m, a.n, a.nnz, st["val"], st["ptr"], st["col"], st["o_val"],
+                                               st["o_ptr"], st["o_row"], ct, api.ACTION_NUMERIC, a.base)
+            api.check(rc, "mcsparseCsr2cscEx2_bufferSize")
+            st["buf"] = torch.empty(size, dtype=torch.uint8, device="cuda")
+            if kind == "spmv-csc":
+                api.check(api.csr2csc(handle, a.m, a.n, a.nnz, st["val"], st["ptr"], st["col"], st["o_val"],
+                                      st["o_ptr"], st["o_row"], ct, api.ACTION_NUMERIC, a.base, st["buf"]))
+                torch.cuda.synchronize()
+                del st["buf"]
+                st["x"] = dev(rng.uniform(-1, 1, a.m).astype(dt))
+                st["y"] = dev(rng.uniform(-1, 1, a.n).astype(dt))
+                st["mat"] = api.SpMat(a.m, a.n, a.nnz, st["o_ptr"], st["o_row"], st["o_val"], base=a.base,
+                                      fmt=api.FORMAT_CSC)
+                if args.family or args.lanes:
+                    st["mat"].set_plan(args.family, args.lanes)
+                st["vx"], st["vy"] = api.DnVec(st["x"]), api.DnVec(st["y"])
+                rc, size = api.spmv_buffer_size(handle, api.OP_T, alpha, st["mat"], st["vx"], beta, st["vy"], ct)
+                api.check(rc)
+                st["buf"] = torch.empty(size, dtype=torch.uint8, device="cuda")
+        else:
+            st["coo"] = torch.zeros(a.nnz, dtype=torch.int32, device="cuda")
+        sets.append(st)
+
+    def step(i):
+        st = sets[i % copies]
+        if kind == "spmv":
+            rc = api.spmv(handle, op, alpha, st["mat"], st["vx"], beta, st["vy"], ct, st["buf"])
+        elif kind == "spmv-csc":
+            rc = api.spmv(handle, api.OP_T, alpha, st["mat"], st["vx"], beta, st["vy"], ct, st["buf"])
+        elif kind == "spmm":
+            rc = api.spmm(handle, api.OP_N, api.OP_N, alpha, st["mat"], st["mB"], beta, st["mC"], ct, st["buf"])
+        elif kind == "csr2csc":
+            rc = api.csr2csc(handle, a.m, a.n, a.nnz, st["val"], st["ptr"], st["col"], st["o_val"], st["o_ptr"],
+                             st["o_row"], ct, api.ACTION_NUMERIC, a.base, st["buf"])
+        else:
+            rc = api.xcsr2coo(handle, st["ptr"], a.nnz, a.m, st["coo"], a.base)
+        if rc != 0:
+            raise api.McsparseError(rc, "step")
+
+    # one-time preprocessing (row-length analysis per descriptor), timed apart from the steady state
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(copies):
+        step(i)
+    torch.cuda.synchronize()
+    first_pass_ms = (time.perf_counter() - t0) * 1e3 / copies
+
+    for i in range(warmup):
+        step(i)
+    torch.cuda.synchronize()
+
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        ev[i][0].record(stream)
+        step(i)
+        ev[i][1].record(stream)
+    torch.cuda.synchronize()
+    wall_s = time.perf_counter() - t0
+    ms_per_step = wall_s * 1e3 / steps
+    dev_ms = np.array([e0.elapsed_time(e1) for e0, e1 in ev])
+    dev_avg_ms = float(dev_ms.mean())
+
+    value = algo_bytes / (ms_per_step * 1e-3) / 1e9
+    achieved = algo_bytes / (dev_avg_ms * 1e-3) / 1e9
+    plan = sets[0]["mat"].plan() if "mat" in sets[0] and kind != "spmm" else None
+
+    out = {
+        "metric": "CSR SpMV/SpMM achieved HBM GB/s (% of MI355X peak) + GFLOP/s at 1 GPU",
+        "value": round(value, 2),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": steps,
+        "warmup": warmup,
+        "ms_per_step": round(ms_per_step, 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f64" if vb == 8 else "f32",
+        "data": "synthetic",
+        "config": {"workload": "%s: %s" % (name, desc), "rows": a.m, "cols": a.n, "nnz": a.nnz,
+                   "dense_cols": n_cols, "alpha": alpha, "beta": beta, "operand_copies_rotated": copies,
+                   "max_row_nnz": int(a.row_lengths().max()), "scale": s},
+        "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBS, 2),
+        "gflops": round(flops / (ms_per_step * 1e-3) / 1e9, 2),
+        "algorithmic_bytes_per_step": int(algo_bytes),
+        "extra_bytes_not_counted": int(extra_read),
+        "first_call_ms": round(first_pass_ms, 4),
+        "device_ms_per_step": {"mean": round(dev_avg_ms, 5), "median": round(float(np.median(dev_ms)), 5),
+                               "min": round(float(dev_ms.min()), 5)},
+        "spmv_plan": {"family": plan[0], "lanes_per_row": plan[1]} if plan else None,
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None},
+    }
+
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(kind, a, alpha, beta, n_cols, algo_bytes, op)
+    print(json.dumps(out))
+    return 0
+
+
+def cpu_baseline(kind, a, alpha, beta, n_cols, algo_bytes, op):
+    """Times the oracle's OpenMP port of the same semantics on the host cores (reported only)."""
+    import oracle
+    from mcsparse_amd import api
+    oracle.build()
+    threads = oracle.max_threads()
+    rng = np.random.default_rng(1)
+    dt = a.val.dtype
+    if kind == "spmv" and op == api.OP_N:
+        x = rng.uniform(-1, 1, a.n).astype(dt)
+        y = rng.uniform(-1, 1, a.m).astype(dt)
+        dyn = int(a.row_lengths().max()) > 4096
+
+        def run():
+            oracle.spmv_omp(a.m, a.base, a.ptr, a.col, a.val, alpha, beta, x, y, dynamic=dyn)
+        sample = "whole workload per repetition"
+    elif kind == "spmm":
+        rows = min(a.m, max(1024, int(2e9 / max(1, 27 * n_cols * 4 * 10))))
+        sub_ptr = a.ptr[:rows + 1]
+        B = rng.uniform(-1, 1, (a.n, n_cols)).astype(dt)
+        C = np.zeros((rows, n_cols), dtype=dt)
+
+        def run():
+            oracle.spmm_omp_f32(rows, n_cols, a.base, sub_ptr, a.col, a.val, alpha, beta, B, C)
+        frac = rows / a.m
+        algo_bytes = algo_bytes * frac
+        sample = "first %d of %d rows per repetition, rate scaled by bytes" % (rows, a.m)
+    else:
+        return {"value": None, "unit": "GB/s", "cores": threads, "kind": "port",
+                "sample": "no OpenMP port of this workload"}
+    for _ in range(2):
+        run()
+    times = []
+    t_end = time.perf_counter() + 10.0
+    while len(times) < 10 and (time.perf_counter() < t_end or len(times) < 3):
+        t0 = time.perf_counter()
+        run()
+        times.append(time.perf_counter() - t0)
+    med = float(np.median(times))
+    return {"value": round(algo_bytes / med / 1e9, 3), "unit": "GB/s", "cores": threads, "kind": "port",
+            "sample": "%s; median of %d (%.3f ms)" % (sample, len(times), med * 1e3)}
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -1,0 +1,289 @@
+/*
+ * mcsparse.h -- C ABI of the CSR SpMV / SpMM / csr2csc / csr2coo path, MI355X (gfx950) build.
+ *
+ * This is the drop-in boundary: every enum value, opaque handle name and prototype below
+ * is the one a program written against MetaX mcSparse already uses for this path, so that
+ * program relinks against libmcsparse.so from this repository unchanged.  Each block cites
+ * the reference declaration it stands in for (paths relative to the reference checkout,
+ * mcsparse/...).  Functions marked EXTENSION have no counterpart in the reference.
+ *
+ * The stream type of the reference is a build-time substitution
+ * (include/interface/mcsp_helper.h.in:21); here it is HIP's stream handle.
+ */
+#ifndef MCSPARSE_H__
+#define MCSPARSE_H__
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* HIP stream handle.  Re-declaring the typedef is legal when <hip/hip_runtime_api.h>
+ * is also included; mcStream_t is kept as the name the reference's users spell. */
+struct ihipStream_t;
+typedef struct ihipStream_t* hipStream_t;
+typedef hipStream_t mcStream_t;
+
+/* ---- value types: include/common/internal/mcsp_datatype.h:5-41 ------------------- */
+typedef enum libraryPropertyType_t { MAJOR_VERSION, MINOR_VERSION, PATCH_LEVEL } libraryPropertyType;
+
+typedef enum macaDataType_t {
+    MACA_R_32F = 0,
+    MACA_R_64F = 1,
+    MACA_R_16F = 2,
+    MACA_R_8I = 3,
+    MACA_C_32F = 4,
+    MACA_C_64F = 5,
+    MACA_C_16F = 6,
+    MACA_C_8I = 7,
+    MACA_R_8U = 8,
+    MACA_C_8U = 9,
+    MACA_R_32I = 10,
+    MACA_C_32I = 11,
+    MACA_R_32U = 12,
+    MACA_C_32U = 13,
+    MACA_R_16BF = 14,
+    MACA_C_16BF = 15,
+    MACA_R_4I = 16,
+    MACA_C_4I = 17,
+    MACA_R_4U = 18,
+    MACA_C_4U = 19,
+    MACA_R_16I = 20,
+    MACA_C_16I = 21,
+    MACA_R_16U = 22,
+    MACA_C_16U = 23,
+    MACA_R_64I = 24,
+    MACA_C_64I = 25,
+    MACA_R_64U = 26,
+    MACA_C_64U = 27
+} macaDataType;
+
+/* ---- enums: include/common/mcsp_types.h.in --------------------------------------- */
+/* :18-31 */
+typedef enum {
+    MCSPARSE_STATUS_SUCCESS = 0,
+    MCSPARSE_STATUS_NOT_INITIALIZED = 1,
+    MCSPARSE_STATUS_ALLOC_FAILED = 2,
+    MCSPARSE_STATUS_INVALID_VALUE = 3,
+    MCSPARSE_STATUS_ARCH_MISMATCH = 4,
+    MCSPARSE_STATUS_MAPPING_ERROR = 5,
+    MCSPARSE_STATUS_EXECUTION_FAILED = 6,
+    MCSPARSE_STATUS_INTERNAL_ERROR = 7,
+    MCSPARSE_STATUS_MATRIX_TYPE_NOT_SUPPORTED = 8,
+    MCSPARSE_STATUS_ZERO_PIVOT = 9,
+    MCSPARSE_STATUS_NOT_SUPPORTED = 10,
+    MCSPARSE_STATUS_INSUFFICIENT_RESOURCES = 11
+} mcsparseStatus_t;
+
+/* :12-16 */
+typedef enum {
+    MCSPARSE_OPERATION_NON_TRANSPOSE = 0,
+    MCSPARSE_OPERATION_TRANSPOSE = 1,
+    MCSPARSE_OPERATION_CONJUGATE_TRANSPOSE = 2
+} mcsparseOperation_t;
+
+/* :40-44 */
+typedef enum { MCSPARSE_INDEX_BASE_ZERO = 0, MCSPARSE_INDEX_BASE_ONE = 1 } mcsparseIndexBase_t;
+
+/* :76-79 */
+typedef enum { MCSPARSE_POINTER_MODE_HOST = 0, MCSPARSE_POINTER_MODE_DEVICE = 1 } mcsparsePointerMode_t;
+
+/* :81-84 -- SYMBOLIC converts indices only, NUMERIC converts indices and values */
+typedef enum { MCSPARSE_ACTION_SYMBOLIC = 0, MCSPARSE_ACTION_NUMERIC = 1 } mcsparseAction_t;
+
+/* :99-105 */
+typedef enum {
+    MCSPARSE_FORMAT_CSR = 1,
+    MCSPARSE_FORMAT_CSC = 2,
+    MCSPARSE_FORMAT_COO = 3,
+    MCSPARSE_FORMAT_COO_AOS = 4,
+    MCSPARSE_FORMAT_BLOCKED_ELL = 5
+} mcsparseFormat_t;
+
+/* :107-110 */
+typedef enum { MCSPARSE_ORDER_COL = 1, MCSPARSE_ORDER_ROW = 2 } mcsparseOrder_t;
+
+/* :112-116 -- 32I arrays are processed as unsigned 32-bit (src/include/mcsp_internal_types.h:4) */
+typedef enum { MCSPARSE_INDEX_16U = 1, MCSPARSE_INDEX_32I = 2, MCSPARSE_INDEX_64I = 3 } mcsparseIndexType_t;
+
+/* :124-134 -- accepted and ignored on this path, as in the reference */
+typedef enum {
+    MCSPARSE_MV_ALG_DEFAULT = 0,
+    MCSPARSE_COOMV_ALG = 1,
+    MCSPARSE_CSRMV_ALG1 = 2,
+    MCSPARSE_CSRMV_ALG2 = 3,
+    MCSPARSE_SPMV_ALG_DEFAULT = 0,
+    MCSPARSE_SPMV_CSR_ALG1 = 2,
+    MCSPARSE_SPMV_CSR_ALG2 = 3,
+    MCSPARSE_SPMV_COO_ALG1 = 1,
+    MCSPARSE_SPMV_COO_ALG2 = 4
+} mcsparseSpMVAlg_t;
+
+/* :140-155 -- accepted and ignored on this path, as in the reference */
+typedef enum {
+    MCSPARSE_MM_ALG_DEFAULT = 0,
+    MCSPARSE_COOMM_ALG1 = 1,
+    MCSPARSE_COOMM_ALG2 = 2,
+    MCSPARSE_COOMM_ALG3 = 3,
+    MCSPARSE_CSRMM_ALG1 = 4,
+    MCSPARSE_SPMM_ALG_DEFAULT = 0,
+    MCSPARSE_SPMM_COO_ALG1 = 1,
+    MCSPARSE_SPMM_COO_ALG2 = 2,
+    MCSPARSE_SPMM_COO_ALG3 = 3,
+    MCSPARSE_SPMM_COO_ALG4 = 5,
+    MCSPARSE_SPMM_CSR_ALG1 = 4,
+    MCSPARSE_SPMM_CSR_ALG2 = 6,
+    MCSPARSE_SPMM_CSR_ALG3 = 12,
+    MCSPARSE_SPMM_BLOCKED_ELL_ALG1 = 13
+} mcsparseSpMMAlg_t;
+
+/* :167-170 -- accepted and ignored (mcsp_csr2csc.cpp:293-310 never reads alg) */
+typedef enum { MCSPARSE_CSR2CSC_ALG1 = 1, MCSPARSE_CSR2CSC_ALG2 = 2 } mcsparseCsr2CscAlg_t;
+
+/* ---- opaque handles: include/common/mcsp_types.h.in:190-242 ---------------------- */
+struct mcsparseContext;
+typedef struct mcsparseContext* mcsparseHandle_t;
+struct mcsparseSpMatDescr;
+typedef struct mcsparseSpMatDescr* mcsparseSpMatDescr_t;
+struct mcsparseDnVecDescr;
+typedef struct mcsparseDnVecDescr* mcsparseDnVecDescr_t;
+struct mcsparseDnMatDescr;
+typedef struct mcsparseDnMatDescr* mcsparseDnMatDescr_t;
+
+/* ---- library handle: include/interface/mcsp_helper.h.in:12-29 --------------------- */
+/* Unlike src/common/mcsp_handle.cpp:5-22 no device memory pool is reserved: the pool only
+ * serves COO SpMV (mcsp_spmv_gpu.cpp:69-75), which is outside this path.  Creating a handle
+ * therefore touches no device and succeeds on a host without a GPU. */
+mcsparseStatus_t mcsparseCreate(mcsparseHandle_t* handle);                                   /* :12 */
+mcsparseStatus_t mcsparseDestroy(mcsparseHandle_t handle);                                   /* :13 */
+mcsparseStatus_t mcsparseGetVersion(mcsparseHandle_t handle, int* version);                  /* :15 */
+mcsparseStatus_t mcsparseGetProperty(libraryPropertyType type, int* value);                  /* :16 */
+const char* mcsparseGetErrorName(mcsparseStatus_t status);                                   /* :18 */
+const char* mcsparseGetErrorString(mcsparseStatus_t status);                                 /* :19 */
+mcsparseStatus_t mcsparseSetStream(mcsparseHandle_t handle, hipStream_t sid);                /* :21 */
+mcsparseStatus_t mcsparseGetStream(const mcsparseHandle_t handle, hipStream_t* sid);         /* :22 */
+mcsparseStatus_t mcsparseSetPointerMode(mcsparseHandle_t handle, mcsparsePointerMode_t m);   /* :28 */
+mcsparseStatus_t mcsparseGetPointerMode(const mcsparseHandle_t handle, mcsparsePointerMode_t* m); /* :29 */
+
+/* ---- dense vector descriptor: mcsp_helper.h.in:46-50 ------------------------------ */
+mcsparseStatus_t mcsparseCreateDnVec(mcsparseDnVecDescr_t* dnVecDescr, int64_t size, void* values,
+                                     macaDataType valueType);
+mcsparseStatus_t mcsparseDestroyDnVec(mcsparseDnVecDescr_t dnVecDescr);
+mcsparseStatus_t mcsparseDnVecGet(mcsparseDnVecDescr_t dnVecDescr, int64_t* size, void** values,
+                                  macaDataType* valueType);
+mcsparseStatus_t mcsparseDnVecGetValues(mcsparseDnVecDescr_t dnVecDescr, void** values);
+mcsparseStatus_t mcsparseDnVecSetValues(mcsparseDnVecDescr_t dnVecDescr, void* values);
+
+/* ---- sparse matrix descriptor: mcsp_helper.h.in:60-86 ------------------------------ */
+/* Descriptors borrow the device pointers; nothing is copied or owned. */
+mcsparseStatus_t mcsparseCreateCsr(mcsparseSpMatDescr_t* spMatDescr, int64_t rows, int64_t cols, int64_t nnz,
+                                   void* csrRowOffsets, void* csrColInd, void* csrValues,
+                                   mcsparseIndexType_t csrRowOffsetsType, mcsparseIndexType_t csrColIndType,
+                                   mcsparseIndexBase_t idxBase, macaDataType valueType);    /* :60 */
+mcsparseStatus_t mcsparseCsrGet(mcsparseSpMatDescr_t spMatDescr, int64_t* rows, int64_t* cols, int64_t* nnz,
+                                void** csrRowOffsets, void** csrColInd, void** csrValues,
+                                mcsparseIndexType_t* csrRowOffsetsType, mcsparseIndexType_t* csrColIndType,
+                                mcsparseIndexBase_t* idxBase, macaDataType* valueType);     /* :63 */
+mcsparseStatus_t mcsparseCsrSetPointers(mcsparseSpMatDescr_t spMatDescr, void* csrRowOffsets, void* csrColInd,
+                                        void* csrValues);                                   /* :66 */
+mcsparseStatus_t mcsparseCreateCsc(mcsparseSpMatDescr_t* spMatDescr, int64_t rows, int64_t cols, int64_t nnz,
+                                   void* cscColOffsets, void* cscRowInd, void* cscValues,
+                                   mcsparseIndexType_t cscColOffsetsType, mcsparseIndexType_t cscRowIndType,
+                                   mcsparseIndexBase_t idxBase, macaDataType valueType);    /* :69 */
+mcsparseStatus_t mcsparseCscSetPointers(mcsparseSpMatDescr_t spMatDescr, void* cscColOffsets, void* cscRowInd,
+                                        void* cscValues);                                   /* :72 */
+mcsparseStatus_t mcsparseDestroySpMat(mcsparseSpMatDescr_t spMatDescr);                     /* :81 */
+mcsparseStatus_t mcsparseSpMatGetSize(mcsparseSpMatDescr_t spMatDescr, int64_t* rows, int64_t* cols,
+                                      int64_t* nnz);                                        /* :82 */
+mcsparseStatus_t mcsparseSpMatGetFormat(mcsparseSpMatDescr_t spMatDescr, mcsparseFormat_t* format);      /* :83 */
+mcsparseStatus_t mcsparseSpMatGetIndexBase(mcsparseSpMatDescr_t spMatDescr, mcsparseIndexBase_t* idxBase); /* :84 */
+mcsparseStatus_t mcsparseSpMatGetValues(mcsparseSpMatDescr_t spMatDescr, void** values);    /* :85 */
+mcsparseStatus_t mcsparseSpMatSetValues(mcsparseSpMatDescr_t spMatDescr, void* values);     /* :86 */
+
+/* ---- dense matrix descriptor: mcsp_helper.h.in:92-98 ------------------------------- */
+mcsparseStatus_t mcsparseCreateDnMat(mcsparseDnMatDescr_t* dnMatDescr, int64_t rows, int64_t cols, int64_t ld,
+                                     void* values, macaDataType valueType, mcsparseOrder_t order);
+mcsparseStatus_t mcsparseDestroyDnMat(mcsparseDnMatDescr_t dnMatDescr);
+mcsparseStatus_t mcsparseDnMatGet(mcsparseDnMatDescr_t dnMatDescr, int64_t* rows, int64_t* cols, int64_t* ld,
+                                  void** values, macaDataType* type, mcsparseOrder_t* order);
+mcsparseStatus_t mcsparseDnMatGetValues(mcsparseDnMatDescr_t dnMatDescr, void** values);
+mcsparseStatus_t mcsparseDnMatSetValues(mcsparseDnMatDescr_t dnMatDescr, void* values);
+
+/* ---- y = alpha*op(A)*x + beta*y : include/interface/mcsp_generic.h:43-51 ---------- */
+/* externalBuffer is caller-allocated device scratch of at least *bufferSize bytes and must be
+ * non-NULL even for op N (src/kernels/level2/spmv/mcsp_spmv_gpu.cpp:703-705).  Work is
+ * enqueued on the handle's stream.  With MCSPARSE_POINTER_MODE_DEVICE the scalars are read
+ * with a blocking copy, as the reference does (src/include/mcsp_internal_host_utils.hpp:34-63). */
+mcsparseStatus_t mcsparseSpMV(mcsparseHandle_t handle, mcsparseOperation_t opA, const void* alpha,
+                              mcsparseSpMatDescr_t matA, mcsparseDnVecDescr_t vecX, const void* beta,
+                              mcsparseDnVecDescr_t vecY, macaDataType computeType, mcsparseSpMVAlg_t alg,
+                              void* externalBuffer);
+mcsparseStatus_t mcsparseSpMV_bufferSize(mcsparseHandle_t handle, mcsparseOperation_t opA, const void* alpha,
+                                         mcsparseSpMatDescr_t matA, mcsparseDnVecDescr_t vecX, const void* beta,
+                                         mcsparseDnVecDescr_t vecY, macaDataType computeType,
+                                         mcsparseSpMVAlg_t alg, size_t* bufferSize);
+
+/* ---- C = alpha*A*op(B) + beta*C : include/interface/mcsp_generic.h:54-67 ---------- */
+/* opA must be NON_TRANSPOSE for CSR (src/kernels/level3/spmm/mcsp_spmm_gpu.cpp:105-108). */
+mcsparseStatus_t mcsparseSpMM_bufferSize(mcsparseHandle_t handle, mcsparseOperation_t opA, mcsparseOperation_t opB,
+                                         const void* alpha, mcsparseSpMatDescr_t matA, mcsparseDnMatDescr_t matB,
+                                         const void* beta, mcsparseDnMatDescr_t matC, macaDataType computeType,
+                                         mcsparseSpMMAlg_t alg, size_t* bufferSize);
+mcsparseStatus_t mcsparseSpMM_preprocess(mcsparseHandle_t handle, mcsparseOperation_t opA, mcsparseOperation_t opB,
+                                         const void* alpha, mcsparseSpMatDescr_t matA, mcsparseDnMatDescr_t matB,
+                                         const void* beta, mcsparseDnMatDescr_t matC, macaDataType computeType,
+                                         mcsparseSpMMAlg_t alg, void* externalBuffer);
+mcsparseStatus_t mcsparseSpMM(mcsparseHandle_t handle, mcsparseOperation_t opA, mcsparseOperation_t opB,
+                              const void* alpha, mcsparseSpMatDescr_t matA, mcsparseDnMatDescr_t matB,
+                              const void* beta, mcsparseDnMatDescr_t matC, macaDataType computeType,
+                              mcsparseSpMMAlg_t alg, void* externalBuffer);
+
+/* ---- index conversions: include/interface/mcsp_conversion.h:11-28 ------------------ */
+/* coo_rows must be sorted; csr_rows receives m+1 offsets.                       :11 */
+mcsparseStatus_t mcsparseXcoo2csr(mcsparseHandle_t handle, const int* coo_rows, int nnz, int m, int* csr_rows,
+                                  mcsparseIndexBase_t idx_base);
+/* coo_rows[j] = row of nonzero j (+ idx_base).                                  :15 */
+mcsparseStatus_t mcsparseXcsr2coo(mcsparseHandle_t handle, const int* csr_rows, int nnz, int m, int* coo_rows,
+                                  mcsparseIndexBase_t idx_base);
+/* Note the output order: csc_val, csc_cols (= n+1 column offsets), csc_rows (= nnz row indices).
+ * Entries of one column keep their CSR order (a stable sort by column).         :19 */
+mcsparseStatus_t mcsparseCsr2cscEx2(mcsparseHandle_t handle, int m, int n, int nnz, const void* csr_val,
+                                    const int* csr_rows, const int* csr_cols, void* csc_val, int* csc_cols,
+                                    int* csc_rows, macaDataType val_type, mcsparseAction_t csc_action,
+                                    mcsparseIndexBase_t idx_base, mcsparseCsr2CscAlg_t alg, void* temp_buffer);
+/*                                                                               :24 */
+mcsparseStatus_t mcsparseCsr2cscEx2_bufferSize(mcsparseHandle_t handle, int m, int n, int nnz, const void* csr_val,
+                                               const int* csr_rows, const int* csr_cols, void* csc_val,
+                                               int* csc_cols, int* csc_rows, macaDataType val_type,
+                                               mcsparseAction_t csc_action, mcsparseIndexBase_t idx_base,
+                                               mcsparseCsr2CscAlg_t alg, size_t* buffer_size);
+
+/* ---- EXTENSIONS (no counterpart in the reference) ---------------------------------- */
+
+/* Number of row-length classes: class 0 holds empty rows, class b >= 1 holds rows whose
+ * length lies in [2^(b-1), 2^b). */
+#define MCSPARSE_ROW_BIN_COUNT 33
+
+/* Row-length binning that steers the SpMV kernel choice.  All arrays are device memory.
+ *   row_bins  : m bytes, class of every row (may be NULL)
+ *   bin_hist  : MCSPARSE_ROW_BIN_COUNT uint32 counters + 1 trailing uint32 = longest row
+ *               (34 uint32 in all; must not be NULL)
+ * The result is a pure function of csr_rows, so it can be checked bit for bit on the host. */
+mcsparseStatus_t mcsparseXcsrRowBins(mcsparseHandle_t handle, int m, const int* csr_rows,
+                                     mcsparseIndexBase_t idx_base, uint8_t* row_bins, uint32_t* bin_hist);
+
+/* Which SpMV kernel family a CSR op-N call on this descriptor runs:
+ * 0 = not analysed yet, 1 = sub-wavefront vector kernel, 2 = merge-path kernel.
+ * lanes_per_row is the sub-wavefront width for family 1 (0 otherwise). */
+mcsparseStatus_t mcsparseSpMatGetSpMVPlan(mcsparseSpMatDescr_t spMatDescr, int* family, int* lanes_per_row);
+
+/* Forces the SpMV kernel family for a descriptor (0 = automatic).  For tests and benchmarks. */
+mcsparseStatus_t mcsparseSpMatSetSpMVPlan(mcsparseSpMatDescr_t spMatDescr, int family, int lanes_per_row);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* MCSPARSE_H__ */

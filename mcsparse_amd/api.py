@@ -1,0 +1,260 @@
+"""Thin Python view of the C ABI in include/mcsparse.h.
+
+Names and argument order are those of the C functions; every call goes through
+libmcsparse.so.  Device memory is passed as raw pointers (torch tensors' data_ptr()); torch is
+only the allocator here.
+"""
+import ctypes
+
+import numpy as np
+
+from . import _lib
+
+# ---- enum values (include/mcsparse.h) ----
+STATUS_SUCCESS = 0
+STATUS_NOT_INITIALIZED = 1
+STATUS_ALLOC_FAILED = 2
+STATUS_INVALID_VALUE = 3
+STATUS_INTERNAL_ERROR = 7
+STATUS_NOT_SUPPORTED = 10
+
+OP_N, OP_T, OP_C = 0, 1, 2
+BASE_ZERO, BASE_ONE = 0, 1
+PTR_HOST, PTR_DEVICE = 0, 1
+ACTION_SYMBOLIC, ACTION_NUMERIC = 0, 1
+FORMAT_CSR, FORMAT_CSC, FORMAT_COO, FORMAT_COO_AOS, FORMAT_BLOCKED_ELL = 1, 2, 3, 4, 5
+ORDER_COL, ORDER_ROW = 1, 2
+INDEX_16U, INDEX_32I, INDEX_64I = 1, 2, 3
+R_32F, R_64F, R_16F, C_32F, C_64F, R_32I = 0, 1, 2, 4, 5, 10
+SPMV_ALG_DEFAULT = 0
+SPMM_ALG_DEFAULT = 0
+CSR2CSC_ALG1 = 1
+ROW_BIN_COUNT = 33
+FAMILY_AUTO, FAMILY_VECTOR, FAMILY_MERGE = 0, 1, 2
+
+_DTYPE_OF = {np.dtype(np.float32): R_32F, np.dtype(np.float64): R_64F}
+
+
+class McsparseError(RuntimeError):
+    def __init__(self, status, where):
+        self.status = status
+        name = _lib.load().mcsparseGetErrorName(status).decode()
+        super().__init__("%s returned %s" % (where, name))
+
+
+def check(status, where="mcsparse call"):
+    if status != STATUS_SUCCESS:
+        raise McsparseError(status, where)
+
+
+def maca_type(dtype):
+    """macaDataType of a numpy/torch real dtype."""
+    try:
+        return _DTYPE_OF[np.dtype(dtype)]
+    except TypeError:
+        import torch  # torch dtypes
+        return {torch.float32: R_32F, torch.float64: R_64F}[dtype]
+
+
+def _ptr(t):
+    """Raw address of a torch tensor / numpy array / int / None."""
+    if t is None:
+        return None
+    if isinstance(t, int):
+        return t
+    if hasattr(t, "data_ptr"):
+        return t.data_ptr()
+    return t.ctypes.data
+
+
+def _scalar(value, dtype_code):
+    """Host scalar of the compute type, as a ctypes object whose address can be passed."""
+    return (ctypes.c_float if dtype_code == R_32F else ctypes.c_double)(value)
+
+
+class Handle:
+    """mcsparseHandle_t with its stream bound to torch's current stream by default."""
+
+    def __init__(self, stream=None):
+        self.lib = _lib.load()
+        self._h = ctypes.c_void_p()
+        check(self.lib.mcsparseCreate(ctypes.byref(self._h)), "mcsparseCreate")
+        if stream is not None:
+            self.set_stream(stream)
+
+    @property
+    def ptr(self):
+        return self._h
+
+    def set_stream(self, raw_stream):
+        check(self.lib.mcsparseSetStream(self._h, ctypes.c_void_p(raw_stream)), "mcsparseSetStream")
+
+    def set_pointer_mode(self, mode):
+        check(self.lib.mcsparseSetPointerMode(self._h, mode), "mcsparseSetPointerMode")
+
+    def destroy(self):
+        if self._h:
+            self.lib.mcsparseDestroy(self._h)
+            self._h = ctypes.c_void_p()
+
+    def __del__(self):
+        try:
+            self.destroy()
+        except Exception:
+            pass
+
+
+class SpMat:
+    """mcsparseSpMatDescr_t for CSR or CSC device arrays (borrowed, kept alive by this object)."""
+
+    def __init__(self, rows, cols, nnz, offsets, indices, values, base=BASE_ZERO, fmt=FORMAT_CSR,
+                 index_type=INDEX_32I, value_type=None):
+        self.lib = _lib.load()
+        self._keep = (offsets, indices, values)
+        self._d = ctypes.c_void_p()
+        vt = value_type if value_type is not None else maca_type(values.dtype)
+        create = self.lib.mcsparseCreateCsr if fmt == FORMAT_CSR else self.lib.mcsparseCreateCsc
+        check(create(ctypes.byref(self._d), rows, cols, nnz, _ptr(offsets), _ptr(indices), _ptr(values), index_type,
+                     index_type, base, vt), "mcsparseCreateCsr/Csc")
+
+    @property
+    def ptr(self):
+        return self._d
+
+    def set_plan(self, family, lanes=0):
+        check(self.lib.mcsparseSpMatSetSpMVPlan(self._d, family, lanes), "mcsparseSpMatSetSpMVPlan")
+
+    def plan(self):
+        fam, lanes = ctypes.c_int(), ctypes.c_int()
+        check(self.lib.mcsparseSpMatGetSpMVPlan(self._d, ctypes.byref(fam), ctypes.byref(lanes)))
+        return fam.value, lanes.value
+
+    def destroy(self):
+        if self._d:
+            self.lib.mcsparseDestroySpMat(self._d)
+            self._d = ctypes.c_void_p()
+
+    def __del__(self):
+        try:
+            self.destroy()
+        except Exception:
+            pass
+
+
+class DnVec:
+    def __init__(self, values, size=None, value_type=None):
+        self.lib = _lib.load()
+        self._keep = values
+        self._d = ctypes.c_void_p()
+        n = size if size is not None else values.numel()
+        vt = value_type if value_type is not None else maca_type(values.dtype)
+        check(self.lib.mcsparseCreateDnVec(ctypes.byref(self._d), n, _ptr(values), vt), "mcsparseCreateDnVec")
+
+    @property
+    def ptr(self):
+        return self._d
+
+    def destroy(self):
+        if self._d:
+            self.lib.mcsparseDestroyDnVec(self._d)
+            self._d = ctypes.c_void_p()
+
+    def __del__(self):
+        try:
+            self.destroy()
+        except Exception:
+            pass
+
+
+class DnMat:
+    def __init__(self, rows, cols, ld, values, order=ORDER_ROW, value_type=None):
+        self.lib = _lib.load()
+        self._keep = values
+        self._d = ctypes.c_void_p()
+        vt = value_type if value_type is not None else maca_type(values.dtype)
+        check(self.lib.mcsparseCreateDnMat(ctypes.byref(self._d), rows, cols, ld, _ptr(values), vt, order),
+              "mcsparseCreateDnMat")
+
+    @property
+    def ptr(self):
+        return self._d
+
+    def destroy(self):
+        if self._d:
+            self.lib.mcsparseDestroyDnMat(self._d)
+            self._d = ctypes.c_void_p()
+
+    def __del__(self):
+        try:
+            self.destroy()
+        except Exception:
+            pass
+
+
+# ---- compute calls: return the status code (tests of error paths need it) -------------------
+
+def spmv_buffer_size(handle, op, alpha, mat, x, beta, y, compute_type):
+    size = ctypes.c_size_t(0)
+    a, b = _scalar(alpha, compute_type), _scalar(beta, compute_type)
+    st = handle.lib.mcsparseSpMV_bufferSize(handle.ptr, op, ctypes.addressof(a), mat.ptr, x.ptr, ctypes.addressof(b),
+                                            y.ptr, compute_type, SPMV_ALG_DEFAULT, ctypes.byref(size))
+    return st, size.value
+
+
+def spmv(handle, op, alpha, mat, x, beta, y, compute_type, buffer):
+    """alpha/beta are Python floats (host pointer mode) or device tensors (device pointer mode)."""
+    if hasattr(alpha, "data_ptr"):
+        pa, pb = alpha.data_ptr(), beta.data_ptr()
+        keep = None
+    else:
+        a, b = _scalar(alpha, compute_type), _scalar(beta, compute_type)
+        pa, pb = ctypes.addressof(a), ctypes.addressof(b)
+        keep = (a, b)
+    st = handle.lib.mcsparseSpMV(handle.ptr, op, pa, mat.ptr, x.ptr, pb, y.ptr, compute_type, SPMV_ALG_DEFAULT,
+                                 _ptr(buffer))
+    del keep
+    return st
+
+
+def spmm_buffer_size(handle, op_a, op_b, alpha, mat, B, beta, C, compute_type):
+    size = ctypes.c_size_t(0)
+    a, b = _scalar(alpha, compute_type), _scalar(beta, compute_type)
+    st = handle.lib.mcsparseSpMM_bufferSize(handle.ptr, op_a, op_b, ctypes.addressof(a), mat.ptr, B.ptr,
+                                            ctypes.addressof(b), C.ptr, compute_type, SPMM_ALG_DEFAULT,
+                                            ctypes.byref(size))
+    return st, size.value
+
+
+def spmm(handle, op_a, op_b, alpha, mat, B, beta, C, compute_type, buffer):
+    a, b = _scalar(alpha, compute_type), _scalar(beta, compute_type)
+    return handle.lib.mcsparseSpMM(handle.ptr, op_a, op_b, ctypes.addressof(a), mat.ptr, B.ptr, ctypes.addressof(b),
+                                   C.ptr, compute_type, SPMM_ALG_DEFAULT, _ptr(buffer))
+
+
+def xcsr2coo(handle, csr_rows, nnz, m, coo_rows, base):
+    return handle.lib.mcsparseXcsr2coo(handle.ptr, _ptr(csr_rows), nnz, m, _ptr(coo_rows), base)
+
+
+def xcoo2csr(handle, coo_rows, nnz, m, csr_rows, base):
+    return handle.lib.mcsparseXcoo2csr(handle.ptr, _ptr(coo_rows), nnz, m, _ptr(csr_rows), base)
+
+
+def csr2csc_buffer_size(handle, m, n, nnz, csr_val, csr_rows, csr_cols, csc_val, csc_cols, csc_rows, val_type,
+                        action, base):
+    size = ctypes.c_size_t(0)
+    st = handle.lib.mcsparseCsr2cscEx2_bufferSize(handle.ptr, m, n, nnz, _ptr(csr_val), _ptr(csr_rows),
+                                                  _ptr(csr_cols), _ptr(csc_val), _ptr(csc_cols), _ptr(csc_rows),
+                                                  val_type, action, base, CSR2CSC_ALG1, ctypes.byref(size))
+    return st, size.value
+
+
+def csr2csc(handle, m, n, nnz, csr_val, csr_rows, csr_cols, csc_val, csc_cols, csc_rows, val_type, action, base,
+            buffer):
+    """csc_cols = n+1 column offsets, csc_rows = nnz row indices (the reference's naming)."""
+    return handle.lib.mcsparseCsr2cscEx2(handle.ptr, m, n, nnz, _ptr(csr_val), _ptr(csr_rows), _ptr(csr_cols),
+                                         _ptr(csc_val), _ptr(csc_cols), _ptr(csc_rows), val_type, action, base,
+                                         CSR2CSC_ALG1, _ptr(buffer))
+
+
+def csr_row_bins(handle, m, csr_rows, base, row_bins, bin_hist):
+    return handle.lib.mcsparseXcsrRowBins(handle.ptr, m, _ptr(csr_rows), base, _ptr(row_bins), _ptr(bin_hist))

@@ -1,0 +1,62 @@
+// Row-length binning of a CSR structure.  Class 0 = empty row, class b >= 1 = length in
+// [2^(b-1), 2^b).  The histogram (and the longest row) steer the SpMV kernel choice; the
+// per-row classes are exported for inspection.  Integer work only, so the result does not
+// depend on the order in which workgroups finish.
+#include "device_util.h"
+#include "internal.h"
+
+namespace mcsp {
+
+namespace {
+
+constexpr int kBinsBlock = 256;
+constexpr int kBinsMaxGrid = 1024;
+
+__global__ __launch_bounds__(kBinsBlock) void row_bins_kernel(idx_t m, const idx_t* __restrict__ row_ptr,
+                                                              uint8_t* __restrict__ row_bins,
+                                                              uint32_t* __restrict__ hist_out) {
+    __shared__ uint32_t s_hist[MCSPARSE_ROW_BIN_COUNT + 1];
+    if (threadIdx.x <= MCSPARSE_ROW_BIN_COUNT) s_hist[threadIdx.x] = 0;
+    __syncthreads();
+
+    uint32_t local_max = 0;
+    // row_ptr differences do not depend on the index base
+    for (uint64_t r = static_cast<uint64_t>(blockIdx.x) * kBinsBlock + threadIdx.x; r < m;
+         r += static_cast<uint64_t>(gridDim.x) * kBinsBlock) {
+        const uint32_t len = row_ptr[r + 1] - row_ptr[r];
+        const uint32_t bin = len == 0 ? 0u : 32u - static_cast<uint32_t>(__clz(static_cast<int>(len)));
+        if (row_bins != nullptr) row_bins[r] = static_cast<uint8_t>(bin);
+        atomicAdd(&s_hist[bin], 1u);
+        local_max = max(local_max, len);
+    }
+    atomicMax(&s_hist[MCSPARSE_ROW_BIN_COUNT], local_max);
+    __syncthreads();
+
+    if (threadIdx.x < MCSPARSE_ROW_BIN_COUNT) {
+        const uint32_t c = s_hist[threadIdx.x];
+        if (c != 0) atomicAdd(&hist_out[threadIdx.x], c);
+    } else if (threadIdx.x == MCSPARSE_ROW_BIN_COUNT) {
+        const uint32_t c = s_hist[threadIdx.x];
+        if (c != 0) atomicMax(&hist_out[MCSPARSE_ROW_BIN_COUNT], c);
+    }
+}
+
+__global__ void zero_u32_kernel(uint32_t* p, uint32_t n) {
+    const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = 0;
+}
+
+}  // namespace
+
+void launch_row_bins(hipStream_t stream, idx_t m, const idx_t* row_ptr, idx_t /*base*/, uint8_t* row_bins,
+                     uint32_t* hist_out) {
+    // a fill kernel rather than a memset node, so that the sequence can be captured in a HIP graph
+    hipLaunchKernelGGL(zero_u32_kernel, dim3(1), dim3(64), 0, stream, hist_out,
+                       static_cast<uint32_t>(MCSPARSE_ROW_BIN_COUNT + 1));
+    if (m == 0) return;
+    const uint64_t blocks = (static_cast<uint64_t>(m) + kBinsBlock - 1) / kBinsBlock;
+    const uint32_t grid = static_cast<uint32_t>(blocks < kBinsMaxGrid ? blocks : kBinsMaxGrid);
+    hipLaunchKernelGGL(row_bins_kernel, dim3(grid), dim3(kBinsBlock), 0, stream, m, row_ptr, row_bins, hist_out);
+}
+
+}  // namespace mcsp

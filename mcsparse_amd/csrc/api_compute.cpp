@@ -1,0 +1,476 @@
+// mcsparseSpMV / mcsparseSpMM / conversion entry points: argument validation in the order of the
+// reference's host drivers, scratch-buffer carving, kernel-family choice and launches.
+#include <cstring>
+
+#include "internal.h"
+
+using mcsp::idx_t;
+
+namespace {
+
+// Leading part of every SpMV scratch buffer: the 34 counters of the row-length analysis.
+constexpr size_t kAnalysisBytes = align_up((MCSPARSE_ROW_BIN_COUNT + 1) * sizeof(uint32_t));
+
+bool fits_32(int64_t v) { return (v >> 32) == 0; }
+
+// Reads a scalar of the compute type.  Device pointer mode costs one blocking copy, like the
+// reference (src/include/mcsp_internal_host_utils.hpp:34-63).
+template <typename T>
+bool scalar_to_host(mcsparseHandle_t h, const void* p, T* out) {
+    if (h->ptr_mode == MCSPARSE_POINTER_MODE_HOST) {
+        std::memcpy(out, p, sizeof(T));
+        return true;
+    }
+    if (hipMemcpyAsync(out, p, sizeof(T), hipMemcpyDeviceToHost, h->stream) != hipSuccess) return false;
+    return hipStreamSynchronize(h->stream) == hipSuccess;
+}
+
+// The CSR-shaped view an SpMV call works on after CSC inputs have been re-read as the CSR of
+// the transpose (src/kernels/level2/spmv/mcsp_spmv_gpu.cpp:734-739).
+struct CsrView {
+    int64_t m, n;        // shape of the matrix whose CSR arrays these are
+    const idx_t* ptr;    // m+1 offsets
+    const idx_t* ind;    // nnz indices
+    const void* val;
+    bool transpose;      // the call needs view^T * x
+};
+
+CsrView make_view(const mcsparseSpMatDescr* A, mcsparseOperation_t op) {
+    CsrView v;
+    const bool op_t = op != MCSPARSE_OPERATION_NON_TRANSPOSE;
+    if (A->format == MCSPARSE_FORMAT_CSC) {
+        v.m = A->col_num;
+        v.n = A->row_num;
+        v.ptr = static_cast<const idx_t*>(A->cols);  // column offsets
+        v.ind = static_cast<const idx_t*>(A->rows);  // row indices
+        v.transpose = !op_t;
+    } else {
+        v.m = A->row_num;
+        v.n = A->col_num;
+        v.ptr = static_cast<const idx_t*>(A->rows);
+        v.ind = static_cast<const idx_t*>(A->cols);
+        v.transpose = op_t;
+    }
+    v.val = A->vals;
+    return v;
+}
+
+// Scratch layout of a transposing SpMV:
+//   [analysis][merge workspace of the transposed matrix][col_ptr n+1 | row_ind nnz][values][csr2csc workspace]
+// (the reference's layout, src/kernels/level2/spmv/mcsp_spmv_gpu.cpp:308 and :813-831, plus the
+// merge-path workspace in front).
+struct TransposeLayout {
+    size_t merge_ws, col_ptr, row_ind, vals, csr2csc_ws, total;
+};
+
+TransposeLayout transpose_layout(int64_t m, int64_t n, int64_t nnz, size_t value_bytes) {
+    TransposeLayout l;
+    size_t off = kAnalysisBytes;
+    l.merge_ws = off;
+    off += align_up(mcsp::spmv_merge_workspace_bytes(static_cast<idx_t>(n), static_cast<idx_t>(nnz), value_bytes));
+    l.col_ptr = off;
+    l.row_ind = off + static_cast<size_t>(n + 1) * sizeof(idx_t);
+    off += align_up(static_cast<size_t>(n + 1 + nnz) * sizeof(idx_t));
+    l.vals = off;
+    off += align_up(static_cast<size_t>(nnz) * value_bytes);
+    l.csr2csc_ws = off;
+    off += align_up(mcsp::csr2csc_workspace_bytes(static_cast<idx_t>(m), static_cast<idx_t>(n),
+                                                  static_cast<idx_t>(nnz), value_bytes));
+    l.total = off;
+    return l;
+}
+
+size_t direct_spmv_bytes(int64_t m, int64_t nnz, size_t value_bytes) {
+    return kAnalysisBytes +
+           align_up(mcsp::spmv_merge_workspace_bytes(static_cast<idx_t>(m), static_cast<idx_t>(nnz), value_bytes));
+}
+
+// Checks shared by SpMV and SpMV_bufferSize, in the reference's order
+// (mcsp_spmv_gpu.cpp:686-714 and :309-334).  `need_buffer` is the SpMV-only externalBuffer check,
+// which sits between the size-range and the format checks; `other_pointers_ok` carries the
+// bufferSize pointer of SpMV_bufferSize, which the reference tests with the other pointers.
+mcspStatus_t check_spmv_args(mcsparseHandle_t handle, mcsparseOperation_t opA, const void* alpha,
+                             const mcsparseSpMatDescr* A, const mcsparseDnVecDescr* x, const void* beta,
+                             const mcsparseDnVecDescr* y, bool other_pointers_ok, bool need_buffer,
+                             const void* buffer) {
+    if (handle == nullptr) return MCSP_STATUS_INVALID_HANDLE;
+    if (alpha == nullptr || beta == nullptr || A == nullptr || x == nullptr || y == nullptr || !other_pointers_ok)
+        return MCSP_STATUS_INVALID_POINTER;
+    if (!fits_32(A->row_num) || !fits_32(A->col_num) || !fits_32(A->nnz) || !fits_32(x->size) || !fits_32(y->size))
+        return MCSP_STATUS_NOT_IMPLEMENTED;
+    if (need_buffer && buffer == nullptr) return MCSP_STATUS_INVALID_POINTER;
+    if (!(A->format == MCSPARSE_FORMAT_CSR || A->format == MCSPARSE_FORMAT_COO ||
+          A->format == MCSPARSE_FORMAT_COO_AOS || A->format == MCSPARSE_FORMAT_CSC))
+        return MCSP_STATUS_NOT_IMPLEMENTED;
+    const bool op_n = opA == MCSPARSE_OPERATION_NON_TRANSPOSE;
+    if (!((op_n && x->size == A->col_num && y->size == A->row_num) ||
+          (!op_n && x->size == A->row_num && y->size == A->col_num)))
+        return MCSP_STATUS_INVALID_SIZE;
+    return MCSP_STATUS_SUCCESS;
+}
+
+// Row and column index types must agree; 32I and 64I are the two the reference dispatches on
+// (mcsp_spmv_gpu.cpp:1123-1133).  Only 32I is built here.
+mcspStatus_t check_index_types(const mcsparseSpMatDescr* A) {
+    if (A->rowIdxType == MCSPARSE_INDEX_32I && A->colIdxType == MCSPARSE_INDEX_32I) return MCSP_STATUS_SUCCESS;
+    return MCSP_STATUS_NOT_IMPLEMENTED;
+}
+
+// Chooses the kernel family for a structure; runs the row-length analysis (one kernel, one
+// blocking 136-byte read-back) the first time a structure is seen.
+mcspStatus_t ensure_plan(mcsparseHandle_t h, mcsparseSpMatDescr* A, const idx_t* ptr, int64_t m, int64_t nnz,
+                         void* buffer) {
+    SpmvPlan& p = A->plan;
+    if (p.valid && p.rows == ptr && p.m == m && p.nnz == nnz && p.base == static_cast<int>(A->idxBase))
+        return MCSP_STATUS_SUCCESS;
+    p.rows = ptr;
+    p.m = m;
+    p.nnz = nnz;
+    p.base = static_cast<int>(A->idxBase);
+    const int mean_lanes = mcsp::spmv_pick_lanes(static_cast<idx_t>(m), static_cast<idx_t>(nnz));
+    if (p.forced_family != kFamilyAuto) {
+        p.family = p.forced_family;
+        p.lanes = p.family == kFamilyVector ? (p.forced_lanes ? p.forced_lanes : mean_lanes) : 0;
+        p.max_row_len = 0;
+        p.valid = true;
+        return MCSP_STATUS_SUCCESS;
+    }
+    uint32_t* dev_hist = static_cast<uint32_t*>(buffer);
+    mcsp::launch_row_bins(h->stream, static_cast<idx_t>(m), ptr, static_cast<idx_t>(A->idxBase), nullptr, dev_hist);
+    uint32_t host_hist[MCSPARSE_ROW_BIN_COUNT + 1];
+    if (hipMemcpyAsync(host_hist, dev_hist, sizeof(host_hist), hipMemcpyDeviceToHost, h->stream) != hipSuccess ||
+        hipStreamSynchronize(h->stream) != hipSuccess)
+        return MCSP_STATUS_INTERNAL_ERROR;
+    std::memcpy(p.hist, host_hist, sizeof(p.hist));
+    p.max_row_len = host_hist[MCSPARSE_ROW_BIN_COUNT];
+    // A row much longer than its lane group serialises one wave while the rest of the chip
+    // idles; past that point the merge-path split wins.
+    const uint32_t limit = static_cast<uint32_t>(32 * mean_lanes > 512 ? 32 * mean_lanes : 512);
+    if (p.max_row_len > limit) {
+        p.family = kFamilyMerge;
+        p.lanes = 0;
+    } else {
+        p.family = kFamilyVector;
+        p.lanes = p.forced_lanes ? p.forced_lanes : mean_lanes;
+    }
+    p.valid = true;
+    return MCSP_STATUS_SUCCESS;
+}
+
+template <typename T>
+mcspStatus_t spmv_typed(mcsparseHandle_t h, mcsparseSpMatDescr* A, const CsrView& v, const void* alpha,
+                        const void* beta, const mcsparseDnVecDescr* x, mcsparseDnVecDescr* y, void* buffer) {
+    T h_alpha, h_beta;
+    if (!scalar_to_host(h, beta, &h_beta) || !scalar_to_host(h, alpha, &h_alpha)) return MCSP_STATUS_INTERNAL_ERROR;
+    // reference: mcsp_spmv_gpu.cpp:235-237 -- y is left untouched in both cases
+    if (A->nnz == 0 || (h_alpha == T(0) && h_beta == T(0))) return MCSP_STATUS_SUCCESS;
+
+    const idx_t nnz = static_cast<idx_t>(A->nnz);
+    const idx_t base = static_cast<idx_t>(A->idxBase);
+    char* buf = static_cast<char*>(buffer);
+    mcsp::SpmvArgs a;
+    a.nnz = nnz;
+    a.base = base;
+    a.x = x->values;
+    a.y = y->values;
+
+    if (!v.transpose) {
+        a.m = static_cast<idx_t>(v.m);
+        a.n = static_cast<idx_t>(v.n);
+        a.row_ptr = v.ptr;
+        a.col = v.ind;
+        a.val = v.val;
+        const mcspStatus_t st = ensure_plan(h, A, v.ptr, v.m, A->nnz, buffer);
+        if (st != MCSP_STATUS_SUCCESS) return st;
+        if (A->plan.family == kFamilyMerge) {
+            mcsp::launch_spmv_merge<T>(h->stream, a, h_alpha, h_beta, buf + kAnalysisBytes);
+        } else {
+            mcsp::launch_spmv_vector<T>(h->stream, a, h_alpha, h_beta, A->plan.lanes);
+        }
+        return MCSP_STATUS_SUCCESS;
+    }
+
+    // Transposing call: materialise the transpose in the scratch buffer on every call, as the
+    // reference does (mcsp_spmv_gpu.cpp:797-845) -- the caller may have changed the values.
+    const TransposeLayout l = transpose_layout(v.m, v.n, A->nnz, sizeof(T));
+    idx_t* t_ptr = reinterpret_cast<idx_t*>(buf + l.col_ptr);
+    idx_t* t_ind = reinterpret_cast<idx_t*>(buf + l.row_ind);
+    void* t_val = buf + l.vals;
+    mcsp::launch_csr2csc(h->stream, static_cast<idx_t>(v.m), static_cast<idx_t>(v.n), nnz, v.val, v.ptr, v.ind, t_val,
+                         t_ind, t_ptr, sizeof(T), base, buf + l.csr2csc_ws);
+    a.m = static_cast<idx_t>(v.n);
+    a.n = static_cast<idx_t>(v.m);
+    a.row_ptr = t_ptr;
+    a.col = t_ind;
+    a.val = t_val;
+    // no analysis of the freshly built structure (it would need a read-back): merge-path is
+    // insensitive to the row-length distribution
+    mcsp::launch_spmv_merge<T>(h->stream, a, h_alpha, h_beta, buf + l.merge_ws);
+    return MCSP_STATUS_SUCCESS;
+}
+
+template <typename T>
+mcspStatus_t spmm_typed(mcsparseHandle_t h, const mcsparseSpMatDescr* A, mcsparseOperation_t opB, const void* alpha,
+                        const void* beta, const mcsparseDnMatDescr* B, mcsparseDnMatDescr* C) {
+    T h_alpha, h_beta;
+    if (!scalar_to_host(h, beta, &h_beta) || !scalar_to_host(h, alpha, &h_alpha)) return MCSP_STATUS_INTERNAL_ERROR;
+    // reference: mcsp_spmm_gpu.cpp:110-114
+    if (A->nnz == 0 && h_beta == T(1)) return MCSP_STATUS_SUCCESS;
+
+    mcsp::SpmmArgs a;
+    a.m = static_cast<idx_t>(A->row_num);
+    a.n = static_cast<idx_t>(C->col_num);
+    a.k = static_cast<idx_t>(A->col_num);
+    a.nnz = static_cast<idx_t>(A->nnz);
+    a.base = static_cast<idx_t>(A->idxBase);
+    a.row_ptr = static_cast<const idx_t*>(A->rows);
+    a.col = static_cast<const idx_t*>(A->cols);
+    a.val = A->vals;
+    a.B = B->values;
+    a.ldb = B->ld;
+    // op(B)(kk, j) sits at kk*ldb + j for (N, row-major) and (T, column-major), else at j*ldb + kk;
+    // the reference copies the first kind into the second (mcsp_spmm_gpu.cpp:119-133).
+    const bool op_n = opB == MCSPARSE_OPERATION_NON_TRANSPOSE;
+    a.b_row_major = (op_n && B->order == MCSPARSE_ORDER_ROW) || (!op_n && B->order == MCSPARSE_ORDER_COL);
+    a.C = C->values;
+    a.ldc = C->ld;
+    a.c_row_major = C->order == MCSPARSE_ORDER_ROW;
+    mcsp::launch_spmm<T>(h->stream, a, h_alpha, h_beta);
+    return MCSP_STATUS_SUCCESS;
+}
+
+mcspStatus_t check_spmm_args(mcsparseHandle_t handle, const void* alpha, const mcsparseSpMatDescr* A,
+                             const mcsparseDnMatDescr* B, const void* beta, const mcsparseDnMatDescr* C) {
+    // reference: mcsp_spmm_gpu.cpp:313-332 / :789-807
+    if (handle == nullptr) return MCSP_STATUS_INVALID_HANDLE;
+    if (A == nullptr || B == nullptr || C == nullptr || alpha == nullptr || beta == nullptr)
+        return MCSP_STATUS_INVALID_POINTER;
+    if (!fits_32(A->row_num) || !fits_32(A->col_num) || !fits_32(A->nnz) || !fits_32(B->row_num) ||
+        !fits_32(B->col_num) || !fits_32(B->ld) || !fits_32(C->row_num) || !fits_32(C->col_num) || !fits_32(C->ld))
+        return MCSP_STATUS_NOT_IMPLEMENTED;
+    if (A->format != MCSPARSE_FORMAT_CSR && A->format != MCSPARSE_FORMAT_COO &&
+        A->format != MCSPARSE_FORMAT_BLOCKED_ELL && A->format != MCSPARSE_FORMAT_CSC)
+        return MCSP_STATUS_NOT_IMPLEMENTED;
+    return MCSP_STATUS_SUCCESS;
+}
+
+}  // namespace
+
+extern "C" {
+
+// reference: src/kernels/level2/spmv/mcsp_spmv_gpu.cpp:309-352, :1108-1121
+mcsparseStatus_t mcsparseSpMV_bufferSize(mcsparseHandle_t handle, mcsparseOperation_t opA, const void* alpha,
+                                         mcsparseSpMatDescr_t matA, mcsparseDnVecDescr_t vecX, const void* beta,
+                                         mcsparseDnVecDescr_t vecY, macaDataType /*computeType*/,
+                                         mcsparseSpMVAlg_t /*alg*/, size_t* bufferSize) {
+    if (matA != nullptr) {
+        const mcspStatus_t it = check_index_types(matA);
+        if (it != MCSP_STATUS_SUCCESS) return to_public_status(it);
+    }
+    const mcspStatus_t st =
+        check_spmv_args(handle, opA, alpha, matA, vecX, beta, vecY, bufferSize != nullptr, false, nullptr);
+    if (st != MCSP_STATUS_SUCCESS) return to_public_status(st);
+    if (matA->format != MCSPARSE_FORMAT_CSR && matA->format != MCSPARSE_FORMAT_CSC)
+        return to_public_status(MCSP_STATUS_NOT_IMPLEMENTED);  // COO inputs are not built here
+
+    const size_t vb = value_size(matA->valueType);
+    const CsrView v = make_view(matA, opA);
+    if (!v.transpose) {
+        *bufferSize = direct_spmv_bytes(v.m, matA->nnz, vb);
+    } else {
+        const TransposeLayout l = transpose_layout(v.m, v.n, matA->nnz, vb);
+        matA->assist_index_buffer_size = l.vals - l.col_ptr;
+        matA->fixed_length_buffer_size = l.csr2csc_ws;
+        matA->is_buffersize_called = 1;
+        *bufferSize = l.total;
+    }
+    if (*bufferSize < kMinBuffer) *bufferSize = kMinBuffer;
+    return MCSPARSE_STATUS_SUCCESS;
+}
+
+// reference: src/kernels/level2/spmv/mcsp_spmv_gpu.cpp:686-903, :1123-1147
+mcsparseStatus_t mcsparseSpMV(mcsparseHandle_t handle, mcsparseOperation_t opA, const void* alpha,
+                              mcsparseSpMatDescr_t matA, mcsparseDnVecDescr_t vecX, const void* beta,
+                              mcsparseDnVecDescr_t vecY, macaDataType computeType, mcsparseSpMVAlg_t /*alg*/,
+                              void* externalBuffer) {
+    if (matA != nullptr) {
+        const mcspStatus_t it = check_index_types(matA);
+        if (it != MCSP_STATUS_SUCCESS) return to_public_status(it);
+    }
+    mcspStatus_t st = check_spmv_args(handle, opA, alpha, matA, vecX, beta, vecY, true, true, externalBuffer);
+    if (st != MCSP_STATUS_SUCCESS) return to_public_status(st);
+    const bool real_type = computeType == MACA_R_32F || computeType == MACA_R_64F || computeType == MACA_R_16F ||
+                           computeType == MACA_R_16BF;
+    if (real_type && opA == MCSPARSE_OPERATION_CONJUGATE_TRANSPOSE) return to_public_status(MCSP_STATUS_INVALID_VALUE);
+    if (matA->format != MCSPARSE_FORMAT_CSR && matA->format != MCSPARSE_FORMAT_CSC)
+        return to_public_status(MCSP_STATUS_NOT_IMPLEMENTED);  // COO inputs are not built here
+    // Same-type real fp32/fp64 only; the reference's mixed-precision and complex routes
+    // (:848-860) are outside this path.  x is checked too, which the reference omits.
+    if (!(computeType == matA->valueType && computeType == vecY->valueType && computeType == vecX->valueType))
+        return to_public_status(MCSP_STATUS_NOT_IMPLEMENTED);
+
+    const CsrView v = make_view(matA, opA);
+    switch (computeType) {
+        case MACA_R_32F:
+            st = spmv_typed<float>(handle, matA, v, alpha, beta, vecX, vecY, externalBuffer);
+            break;
+        case MACA_R_64F:
+            st = spmv_typed<double>(handle, matA, v, alpha, beta, vecX, vecY, externalBuffer);
+            break;
+        default:
+            st = MCSP_STATUS_NOT_IMPLEMENTED;
+    }
+    return to_public_status(st);
+}
+
+// reference: src/kernels/level3/spmm/mcsp_spmm_gpu.cpp:309-342, :950-963
+mcsparseStatus_t mcsparseSpMM_bufferSize(mcsparseHandle_t handle, mcsparseOperation_t /*opA*/,
+                                         mcsparseOperation_t /*opB*/, const void* alpha, mcsparseSpMatDescr_t matA,
+                                         mcsparseDnMatDescr_t matB, const void* beta, mcsparseDnMatDescr_t matC,
+                                         macaDataType /*computeType*/, mcsparseSpMMAlg_t /*alg*/,
+                                         size_t* bufferSize) {
+    if (matA != nullptr) {
+        const mcspStatus_t it = check_index_types(matA);
+        if (it != MCSP_STATUS_SUCCESS) return to_public_status(it);
+    }
+    const mcspStatus_t st = check_spmm_args(handle, alpha, matA, matB, beta, matC);
+    if (st != MCSP_STATUS_SUCCESS) return to_public_status(st);
+    if (bufferSize == nullptr) return to_public_status(MCSP_STATUS_INVALID_POINTER);
+    if (matA->format != MCSPARSE_FORMAT_CSR) return to_public_status(MCSP_STATUS_NOT_IMPLEMENTED);
+    *bufferSize = kMinBuffer;
+    return MCSPARSE_STATUS_SUCCESS;
+}
+
+// reference: src/kernels/level3/spmm/mcsp_spmm_gpu.cpp:965-970 -- a no-op there as well
+mcsparseStatus_t mcsparseSpMM_preprocess(mcsparseHandle_t, mcsparseOperation_t, mcsparseOperation_t, const void*,
+                                         mcsparseSpMatDescr_t, mcsparseDnMatDescr_t, const void*,
+                                         mcsparseDnMatDescr_t, macaDataType, mcsparseSpMMAlg_t, void*) {
+    return MCSPARSE_STATUS_SUCCESS;
+}
+
+// reference: src/kernels/level3/spmm/mcsp_spmm_gpu.cpp:785-867, :972-982, :82-162
+mcsparseStatus_t mcsparseSpMM(mcsparseHandle_t handle, mcsparseOperation_t opA, mcsparseOperation_t opB,
+                              const void* alpha, mcsparseSpMatDescr_t matA, mcsparseDnMatDescr_t matB,
+                              const void* beta, mcsparseDnMatDescr_t matC, macaDataType computeType,
+                              mcsparseSpMMAlg_t /*alg*/, void* externalBuffer) {
+    if (matA != nullptr) {
+        const mcspStatus_t it = check_index_types(matA);
+        if (it != MCSP_STATUS_SUCCESS) return to_public_status(it);
+    }
+    if (handle == nullptr) return to_public_status(MCSP_STATUS_INVALID_HANDLE);
+    if (externalBuffer == nullptr) return to_public_status(MCSP_STATUS_INVALID_POINTER);
+    mcspStatus_t st = check_spmm_args(handle, alpha, matA, matB, beta, matC);
+    if (st != MCSP_STATUS_SUCCESS) return to_public_status(st);
+    if (matA->format != MCSPARSE_FORMAT_CSR) return to_public_status(MCSP_STATUS_NOT_IMPLEMENTED);
+    if (!(computeType == matA->valueType && computeType == matC->valueType && computeType == matB->valueType))
+        return to_public_status(MCSP_STATUS_NOT_IMPLEMENTED);
+    // CSR with op(A) != N is not implemented by the reference either (:105-108)
+    if (opA != MCSPARSE_OPERATION_NON_TRANSPOSE) return to_public_status(MCSP_STATUS_NOT_IMPLEMENTED);
+    // Shapes the reference never checks and then reads out of bounds on: C is m x n, op(B) is k x n.
+    const bool op_n = opB == MCSPARSE_OPERATION_NON_TRANSPOSE;
+    const int64_t b_rows = op_n ? matB->row_num : matB->col_num;
+    const int64_t b_cols = op_n ? matB->col_num : matB->row_num;
+    if (matC->row_num != matA->row_num || b_rows != matA->col_num || b_cols != matC->col_num)
+        return to_public_status(MCSP_STATUS_INVALID_SIZE);
+    const int64_t b_lead = matB->order == MCSPARSE_ORDER_ROW ? matB->col_num : matB->row_num;
+    const int64_t c_lead = matC->order == MCSPARSE_ORDER_ROW ? matC->col_num : matC->row_num;
+    if (matB->ld < b_lead || matC->ld < c_lead) return to_public_status(MCSP_STATUS_INVALID_SIZE);
+
+    switch (computeType) {
+        case MACA_R_32F: st = spmm_typed<float>(handle, matA, opB, alpha, beta, matB, matC); break;
+        case MACA_R_64F: st = spmm_typed<double>(handle, matA, opB, alpha, beta, matB, matC); break;
+        default: st = MCSP_STATUS_NOT_IMPLEMENTED;
+    }
+    return to_public_status(st);
+}
+
+// reference: src/kernels/conversion/mcsp_coo2csr.cpp:7-32, :85-88
+mcsparseStatus_t mcsparseXcoo2csr(mcsparseHandle_t handle, const int* coo_rows, int nnz, int m, int* csr_rows,
+                                  mcsparseIndexBase_t idx_base) {
+    if (handle == nullptr) return to_public_status(MCSP_STATUS_INVALID_HANDLE);
+    if (nnz == 0) return MCSPARSE_STATUS_SUCCESS;  // csr_rows is left untouched, as in the reference
+    // negative sizes arrive as huge unsigned values in the reference (uint32 casts); refuse them
+    if (m < 0 || nnz < 0) return to_public_status(MCSP_STATUS_INVALID_SIZE);
+    if (coo_rows == nullptr || csr_rows == nullptr) return to_public_status(MCSP_STATUS_INVALID_POINTER);
+    mcsp::launch_coo2csr(handle->stream, static_cast<idx_t>(nnz), static_cast<idx_t>(m),
+                         reinterpret_cast<const idx_t*>(coo_rows), static_cast<idx_t>(idx_base),
+                         reinterpret_cast<idx_t*>(csr_rows));
+    return MCSPARSE_STATUS_SUCCESS;
+}
+
+// reference: src/kernels/conversion/mcsp_coo2csr.cpp:34-59, :90-93
+mcsparseStatus_t mcsparseXcsr2coo(mcsparseHandle_t handle, const int* csr_rows, int nnz, int m, int* coo_rows,
+                                  mcsparseIndexBase_t idx_base) {
+    if (handle == nullptr) return to_public_status(MCSP_STATUS_INVALID_HANDLE);
+    if (nnz == 0) return MCSPARSE_STATUS_SUCCESS;
+    if (m < 0 || nnz < 0) return to_public_status(MCSP_STATUS_INVALID_SIZE);
+    if (coo_rows == nullptr || csr_rows == nullptr) return to_public_status(MCSP_STATUS_INVALID_POINTER);
+    mcsp::launch_csr2coo(handle->stream, static_cast<idx_t>(m), static_cast<idx_t>(nnz),
+                         reinterpret_cast<const idx_t*>(csr_rows), static_cast<idx_t>(idx_base),
+                         reinterpret_cast<idx_t*>(coo_rows));
+    return MCSPARSE_STATUS_SUCCESS;
+}
+
+// reference: src/kernels/conversion/mcsp_csr2csc.cpp:9-41, :312-320
+mcsparseStatus_t mcsparseCsr2cscEx2_bufferSize(mcsparseHandle_t handle, int m, int n, int nnz, const void* /*csr_val*/,
+                                               const int* /*csr_rows*/, const int* /*csr_cols*/, void* /*csc_val*/,
+                                               int* /*csc_cols*/, int* /*csc_rows*/, macaDataType val_type,
+                                               mcsparseAction_t csc_action, mcsparseIndexBase_t /*idx_base*/,
+                                               mcsparseCsr2CscAlg_t /*alg*/, size_t* buffer_size) {
+    if (handle == nullptr) return to_public_status(MCSP_STATUS_INVALID_HANDLE);
+    if (n < 0 || m < 0 || nnz < 0) return to_public_status(MCSP_STATUS_INVALID_SIZE);
+    if (buffer_size == nullptr) return to_public_status(MCSP_STATUS_INVALID_POINTER);
+    if (n == 0 || m == 0 || nnz == 0) {
+        *buffer_size = kMinBuffer;
+        return MCSPARSE_STATUS_SUCCESS;
+    }
+    // The reference sizes for the numeric case whatever the action; so does this.
+    size_t vb = value_size(val_type);
+    if (vb != 4 && vb != 8) vb = 8;
+    (void)csc_action;
+    *buffer_size = mcsp::csr2csc_workspace_bytes(static_cast<idx_t>(m), static_cast<idx_t>(n),
+                                                 static_cast<idx_t>(nnz), vb);
+    if (*buffer_size < kMinBuffer) *buffer_size = kMinBuffer;
+    return MCSPARSE_STATUS_SUCCESS;
+}
+
+// reference: src/kernels/conversion/mcsp_csr2csc.cpp:43-132, :293-310
+mcsparseStatus_t mcsparseCsr2cscEx2(mcsparseHandle_t handle, int m, int n, int nnz, const void* csr_val,
+                                    const int* csr_rows, const int* csr_cols, void* csc_val, int* csc_cols,
+                                    int* csc_rows, macaDataType val_type, mcsparseAction_t csc_action,
+                                    mcsparseIndexBase_t idx_base, mcsparseCsr2CscAlg_t /*alg*/, void* temp_buffer) {
+    // value types the reference's switch accepts (:297-309); complex ones are not built here
+    size_t vb;
+    switch (val_type) {
+        case MACA_R_32F: vb = 4; break;
+        case MACA_R_64F: vb = 8; break;
+        case MACA_C_32F: case MACA_C_64F: return to_public_status(MCSP_STATUS_NOT_IMPLEMENTED);
+        default: return to_public_status(MCSP_STATUS_TYPE_MISMATCH);
+    }
+    if (handle == nullptr) return to_public_status(MCSP_STATUS_INVALID_HANDLE);
+    if (n < 0 || m < 0 || nnz < 0) return to_public_status(MCSP_STATUS_INVALID_SIZE);
+    if (n == 0 || m == 0 || nnz == 0) return MCSPARSE_STATUS_SUCCESS;  // outputs untouched (:56-58)
+    // value pointers are required even for SYMBOLIC (:60-63)
+    if (csr_val == nullptr || csr_rows == nullptr || csr_cols == nullptr || csc_val == nullptr ||
+        csc_rows == nullptr || csc_cols == nullptr || temp_buffer == nullptr)
+        return to_public_status(MCSP_STATUS_INVALID_POINTER);
+    if (csc_action == MCSPARSE_ACTION_SYMBOLIC) vb = 0;
+    mcsp::launch_csr2csc(handle->stream, static_cast<idx_t>(m), static_cast<idx_t>(n), static_cast<idx_t>(nnz), csr_val,
+                         reinterpret_cast<const idx_t*>(csr_rows), reinterpret_cast<const idx_t*>(csr_cols), csc_val,
+                         reinterpret_cast<idx_t*>(csc_rows), reinterpret_cast<idx_t*>(csc_cols), vb,
+                         static_cast<idx_t>(idx_base), temp_buffer);
+    return MCSPARSE_STATUS_SUCCESS;
+}
+
+// EXTENSION
+mcsparseStatus_t mcsparseXcsrRowBins(mcsparseHandle_t handle, int m, const int* csr_rows, mcsparseIndexBase_t idx_base,
+                                     uint8_t* row_bins, uint32_t* bin_hist) {
+    if (handle == nullptr) return to_public_status(MCSP_STATUS_INVALID_HANDLE);
+    if (m < 0) return to_public_status(MCSP_STATUS_INVALID_SIZE);
+    if (csr_rows == nullptr || bin_hist == nullptr) return to_public_status(MCSP_STATUS_INVALID_POINTER);
+    mcsp::launch_row_bins(handle->stream, static_cast<idx_t>(m), reinterpret_cast<const idx_t*>(csr_rows),
+                          static_cast<idx_t>(idx_base), row_bins, bin_hist);
+    return MCSPARSE_STATUS_SUCCESS;
+}
+
+}  // extern "C"

@@ -1,0 +1,470 @@
+// Index conversions for gfx950: csr2coo, coo2csr and csr2csc.
+//
+// csr2csc must reproduce the reference's order exactly: a stable sort of the nonzeros by
+// column (src/kernels/conversion/mcsp_csr2csc.cpp:97-98, LSD radix sort with 2-bit digits,
+// src/mcprim/device_radix_sort.hpp:283-306), so entries of one column keep their CSR order.
+// A stable sort has exactly one result, which leaves the digit width free: here the (column,
+// row, value) triples are carried through ceil(bits/8) LSD passes of up to 8 bits instead of
+// sorting a permutation in bits/2 passes and gathering through it afterwards, which on HBM
+// trades ~24 sweeps plus two random gathers for 3 sweeps.
+#include "device_util.h"
+#include "internal.h"
+
+namespace mcsp {
+
+namespace {
+
+constexpr int kBlock = 256;
+
+// ------------------------------------------------------------------------------------------
+// merge-path tiles over (row ends, nonzero indices), shared by csr2coo
+// ------------------------------------------------------------------------------------------
+constexpr int kExpandIpt = 8;
+constexpr int kExpandTile = kBlock * kExpandIpt;
+
+// Wavefront-cooperative merge-path search: number of row ends that precede diagonal d.
+// 64 probes per round shrink the interval 64-fold, so 4M rows need 4 dependent loads instead
+// of 22.  Every lane of the wave must call this; all lanes return the same value.
+__device__ __forceinline__ idx_t wave_merge_search(uint64_t d, idx_t m, idx_t nnz, idx_t base,
+                                                   const idx_t* __restrict__ row_ptr) {
+    uint64_t lo = d > nnz ? d - nnz : 0;
+    uint64_t hi = d < m ? d : m;
+    const unsigned lane = lane_id();
+    while (lo < hi) {
+        const uint64_t span = hi - lo;
+        const uint64_t step = (span + kWave - 1) / kWave;
+        const uint64_t probe = lo + lane * step;
+        bool pred = false;
+        if (probe < hi) {
+            const uint64_t row_end = row_ptr[probe + 1] - base;
+            pred = row_end <= d - probe - 1;
+        }
+        const unsigned count = __popcll(__ballot(pred));
+        if (count == 0) {
+            hi = lo;
+        } else {
+            const uint64_t new_hi = lo + static_cast<uint64_t>(count) * step;
+            lo = lo + static_cast<uint64_t>(count - 1) * step + 1;
+            hi = new_hi < hi ? new_hi : hi;
+        }
+    }
+    return static_cast<idx_t>(lo);
+}
+
+// coo_rows[j] = row of nonzero j (+ base).  One tile of the merged path per workgroup, so empty
+// rows, 1-nonzero rows and 200k-nonzero rows all cost one item each.
+// Reference semantics: src/kernels/conversion/coo2csr_device.hpp:26-41.
+__global__ __launch_bounds__(kBlock) void csr2coo_kernel(idx_t m, idx_t nnz, idx_t base,
+                                                         const idx_t* __restrict__ row_ptr,
+                                                         idx_t* __restrict__ coo_rows) {
+    __shared__ idx_t s_row_end[kExpandTile + 1];
+    __shared__ idx_t s_ids[kExpandTile];
+    __shared__ idx_t s_x[2];
+
+    const uint32_t tid = threadIdx.x;
+    const uint64_t total = static_cast<uint64_t>(m) + nnz;
+    const uint64_t d0 = static_cast<uint64_t>(blockIdx.x) * kExpandTile;
+    const uint64_t d1 = d0 + kExpandTile < total ? d0 + kExpandTile : total;
+    const unsigned wave = tid / kWave;
+    if (wave < 2) {
+        const idx_t x = wave_merge_search(wave == 0 ? d0 : d1, m, nnz, base, row_ptr);
+        if (tid % kWave == 0) s_x[wave] = x;
+    }
+    __syncthreads();
+    const idx_t x0 = s_x[0];
+    const idx_t x1 = s_x[1];
+    const idx_t y0 = static_cast<idx_t>(d0 - x0);
+    const idx_t y1 = static_cast<idx_t>(d1 - x1);
+    const idx_t tile_rows = x1 - x0;
+    const idx_t tile_nnz = y1 - y0;
+    const idx_t tile_items = tile_rows + tile_nnz;
+
+    for (idx_t i = tid; i <= tile_rows; i += kBlock) {
+        const idx_t r = x0 + i;
+        s_row_end[i] = r < m ? row_ptr[r + 1] - base : 0xFFFFFFFFu;
+    }
+    __syncthreads();
+
+    const idx_t dt = min(static_cast<idx_t>(tid * kExpandIpt), tile_items);
+    idx_t lo = dt > tile_nnz ? dt - tile_nnz : 0;
+    idx_t hi = dt < tile_rows ? dt : tile_rows;
+    while (lo < hi) {
+        const idx_t mid = (lo + hi) >> 1;
+        if (s_row_end[mid] <= y0 + (dt - mid - 1)) {
+            lo = mid + 1;
+        } else {
+            hi = mid;
+        }
+    }
+    idx_t row_l = lo;
+    idx_t nz = y0 + (dt - lo);
+#pragma unroll
+    for (int i = 0; i < kExpandIpt; ++i) {
+        if (dt + i < tile_items) {
+            if (nz < s_row_end[row_l]) {
+                s_ids[nz - y0] = x0 + row_l + base;
+                ++nz;
+            } else {
+                ++row_l;
+            }
+        }
+    }
+    __syncthreads();
+    for (idx_t k = tid; k < tile_nnz; k += kBlock) coo_rows[y0 + k] = s_ids[k];
+}
+
+// Offsets from sorted row indices: thread t fills the offsets of the rows that lie between
+// entry t-1 and entry t, so empty rows are covered.
+// Reference semantics: src/kernels/conversion/coo2csr_device.hpp:8-24.
+__global__ __launch_bounds__(kBlock) void coo2csr_kernel(idx_t nnz, idx_t m, idx_t base,
+                                                         const idx_t* __restrict__ coo_rows,
+                                                         idx_t* __restrict__ row_ptr) {
+    const uint64_t t = static_cast<uint64_t>(blockIdx.x) * kBlock + threadIdx.x;
+    if (t > nnz) return;
+    const uint64_t first = t == 0 ? 0 : static_cast<uint64_t>(coo_rows[t - 1] - base) + 1;
+    const uint64_t last = t == nnz ? static_cast<uint64_t>(m) + 1 : static_cast<uint64_t>(coo_rows[t] - base) + 1;
+    for (uint64_t i = first; i < last; ++i) row_ptr[i] = static_cast<idx_t>(t) + base;
+}
+
+// ------------------------------------------------------------------------------------------
+// device-wide exclusive scan of uint32 (in place), chunks of 2048
+// ------------------------------------------------------------------------------------------
+constexpr int kScanIpt = 8;
+constexpr int kScanChunk = kBlock * kScanIpt;
+
+__device__ __forceinline__ uint32_t block_exclusive_scan(uint32_t v, uint32_t* s_wave, uint32_t* total) {
+    const unsigned lane = threadIdx.x % kWave;
+    const unsigned wave = threadIdx.x / kWave;
+    uint32_t inc = v;
+#pragma unroll
+    for (int off = 1; off < kWave; off <<= 1) {
+        const uint32_t up = __shfl_up(inc, off, kWave);
+        if (lane >= static_cast<unsigned>(off)) inc += up;
+    }
+    if (lane == kWave - 1) s_wave[wave] = inc;
+    __syncthreads();
+    uint32_t wave_off = 0, all = 0;
+#pragma unroll
+    for (unsigned w = 0; w < kBlock / kWave; ++w) {
+        const uint32_t s = s_wave[w];
+        if (w < wave) wave_off += s;
+        all += s;
+    }
+    __syncthreads();  // s_wave may be reused by the caller
+    *total = all;
+    return wave_off + inc - v;
+}
+
+__global__ __launch_bounds__(kBlock) void scan_reduce_kernel(const uint32_t* __restrict__ data, uint64_t n,
+                                                             uint32_t* __restrict__ chunk_sums) {
+    __shared__ uint32_t s_wave[kBlock / kWave];
+    const uint64_t start = static_cast<uint64_t>(blockIdx.x) * kScanChunk;
+    uint32_t v = 0;
+#pragma unroll
+    for (int i = 0; i < kScanIpt; ++i) {
+        const uint64_t p = start + static_cast<uint64_t>(i) * kBlock + threadIdx.x;
+        if (p < n) v += data[p];
+    }
+    uint32_t total;
+    block_exclusive_scan(v, s_wave, &total);
+    if (threadIdx.x == 0) chunk_sums[blockIdx.x] = total;
+}
+
+// chunk_offsets == nullptr: single chunk starting at 0.
+__global__ __launch_bounds__(kBlock) void scan_chunks_kernel(uint32_t* __restrict__ data, uint64_t n,
+                                                             const uint32_t* __restrict__ chunk_offsets) {
+    __shared__ uint32_t s_wave[kBlock / kWave];
+    // thread owns kScanIpt consecutive elements so that its local prefix is sequential
+    const uint64_t start = static_cast<uint64_t>(blockIdx.x) * kScanChunk + static_cast<uint64_t>(threadIdx.x) * kScanIpt;
+    uint32_t v[kScanIpt];
+    uint32_t sum = 0;
+#pragma unroll
+    for (int i = 0; i < kScanIpt; ++i) {
+        v[i] = start + i < n ? data[start + i] : 0;
+        sum += v[i];
+    }
+    uint32_t total;
+    uint32_t off = block_exclusive_scan(sum, s_wave, &total);
+    if (chunk_offsets != nullptr) off += chunk_offsets[blockIdx.x];
+#pragma unroll
+    for (int i = 0; i < kScanIpt; ++i) {
+        if (start + i < n) data[start + i] = off;
+        off += v[i];
+    }
+}
+
+size_t scan_workspace_elems(uint64_t n) {
+    size_t elems = 0;
+    while (n > kScanChunk) {
+        n = (n + kScanChunk - 1) / kScanChunk;
+        elems += align_up(n * sizeof(uint32_t)) / sizeof(uint32_t);
+    }
+    return elems;
+}
+
+void launch_exclusive_scan(hipStream_t stream, uint32_t* data, uint64_t n, uint32_t* workspace) {
+    if (n == 0) return;
+    if (n <= kScanChunk) {
+        hipLaunchKernelGGL(scan_chunks_kernel, dim3(1), dim3(kBlock), 0, stream, data, n,
+                           static_cast<const uint32_t*>(nullptr));
+        return;
+    }
+    const uint64_t chunks = (n + kScanChunk - 1) / kScanChunk;
+    uint32_t* sums = workspace;
+    uint32_t* next_ws = workspace + align_up(chunks * sizeof(uint32_t)) / sizeof(uint32_t);
+    hipLaunchKernelGGL(scan_reduce_kernel, dim3(static_cast<uint32_t>(chunks)), dim3(kBlock), 0, stream, data, n, sums);
+    launch_exclusive_scan(stream, sums, chunks, next_ws);
+    hipLaunchKernelGGL(scan_chunks_kernel, dim3(static_cast<uint32_t>(chunks)), dim3(kBlock), 0, stream, data, n,
+                       static_cast<const uint32_t*>(sums));
+}
+
+// ------------------------------------------------------------------------------------------
+// one stable LSD radix pass over (key, row, value) triples
+// ------------------------------------------------------------------------------------------
+constexpr int kSortIpt = 16;
+constexpr int kSortTile = kBlock * kSortIpt;          // 4096 triples per workgroup
+constexpr int kSortWaves = kBlock / kWave;            // 4
+constexpr int kSortWaveItems = kWave * kSortIpt;      // each wave owns 1024 consecutive triples
+constexpr int kMaxRadix = 256;
+
+// counters[digit * tiles + tile] = how many keys of `tile` carry `digit`.
+__global__ __launch_bounds__(kBlock) void radix_hist_kernel(const idx_t* __restrict__ keys, idx_t count,
+                                                            uint32_t shift, uint32_t bits, uint32_t tiles,
+                                                            uint32_t* __restrict__ counters) {
+    __shared__ uint32_t s_cnt[kMaxRadix];
+    const uint32_t radix = 1u << bits;
+    const uint32_t mask = radix - 1;
+    s_cnt[threadIdx.x] = 0;
+    __syncthreads();
+    const uint64_t start = static_cast<uint64_t>(blockIdx.x) * kSortTile;
+#pragma unroll
+    for (int i = 0; i < kSortIpt; ++i) {
+        const uint64_t p = start + static_cast<uint64_t>(i) * kBlock + threadIdx.x;
+        if (p < count) atomicAdd(&s_cnt[(keys[p] >> shift) & mask], 1u);
+    }
+    __syncthreads();
+    if (threadIdx.x < radix) counters[static_cast<uint64_t>(threadIdx.x) * tiles + blockIdx.x] = s_cnt[threadIdx.x];
+}
+
+// VB = bytes per value (0 = no values).  counters hold, after the exclusive scan, the output
+// position of the first key of each (digit, tile).
+template <int VB>
+struct ValueOf { typedef uint32_t type; };
+template <>
+struct ValueOf<8> { typedef uint64_t type; };
+
+template <int VB>
+__global__ __launch_bounds__(kBlock) void radix_scatter_kernel(
+    const idx_t* __restrict__ keys_in, const idx_t* __restrict__ rows_in, const void* __restrict__ vals_in_v,
+    idx_t* __restrict__ keys_out, idx_t* __restrict__ rows_out, void* __restrict__ vals_out_v, idx_t count,
+    uint32_t shift, uint32_t bits, uint32_t tiles, const uint32_t* __restrict__ counters) {
+    typedef typename ValueOf<VB>::type val_t;
+    const val_t* vals_in = static_cast<const val_t*>(vals_in_v);
+    val_t* vals_out = static_cast<val_t*>(vals_out_v);
+
+    __shared__ uint32_t s_cnt[kSortWaves][kMaxRadix];  // per-wave digit counts, then wave offsets
+    __shared__ uint32_t s_start[kMaxRadix];            // first sorted slot of each digit in the tile
+    __shared__ uint32_t s_dest[kMaxRadix];             // global position of that slot
+    __shared__ uint32_t s_wave[kSortWaves];
+    __shared__ idx_t s_keys[kSortTile];
+    __shared__ idx_t s_rows[kSortTile];
+    __shared__ val_t s_vals[VB ? kSortTile : 1];
+
+    const uint32_t tid = threadIdx.x;
+    const unsigned lane = tid % kWave;
+    const unsigned wave = tid / kWave;
+    const uint32_t radix = 1u << bits;
+    const uint32_t mask = radix - 1;
+    const uint64_t tile_start = static_cast<uint64_t>(blockIdx.x) * kSortTile;
+    const uint32_t tile_count =
+        static_cast<uint32_t>(count - tile_start < kSortTile ? count - tile_start : kSortTile);
+
+#pragma unroll
+    for (int w = 0; w < kSortWaves; ++w) s_cnt[w][tid] = 0;
+    __syncthreads();
+
+    // Position inside the tile of this thread's i-th triple: waves own consecutive 1024-triple
+    // slabs, lanes are interleaved inside a slab, so (wave, i, lane) order is input order.
+    idx_t key[kSortIpt], row[kSortIpt];
+    val_t val[kSortIpt];
+    uint32_t rank[kSortIpt];
+    const uint64_t lanemask_lt = (1ull << lane) - 1ull;
+#pragma unroll
+    for (int i = 0; i < kSortIpt; ++i) {
+        const uint32_t p = wave * kSortWaveItems + i * kWave + lane;
+        const bool live = p < tile_count;
+        key[i] = live ? load_stream(keys_in + tile_start + p) : 0;
+        row[i] = live ? load_stream(rows_in + tile_start + p) : 0;
+        if constexpr (VB != 0) val[i] = live ? load_stream(vals_in + tile_start + p) : val_t(0);
+    }
+#pragma unroll
+    for (int i = 0; i < kSortIpt; ++i) {
+        const uint32_t p = wave * kSortWaveItems + i * kWave + lane;
+        const bool live = p < tile_count;
+        const uint32_t d = (key[i] >> shift) & mask;
+        // lanes of this wave holding the same digit in this round
+        uint64_t peers = __ballot(live);
+        for (uint32_t b = 0; b < bits; ++b) {
+            const bool bit = (d >> b) & 1u;
+            const uint64_t vote = __ballot(bit);
+            peers &= bit ? vote : ~vote;
+        }
+        rank[i] = 0;
+        if (live) {
+            // The counter is shared by the lanes of this wave across rounds, so it is accessed
+            // as volatile: every peer reads it, then the lowest peer alone adds the round's
+            // count.  LDS operations of one wave complete in program order.
+            volatile uint32_t* counter = &s_cnt[wave][d];
+            const uint32_t before = *counter;
+            rank[i] = before + __popcll(peers & lanemask_lt);
+            if ((peers & lanemask_lt) == 0) *counter = before + __popcll(peers);
+        }
+    }
+    __syncthreads();
+
+    // per digit: turn the wave counts into wave offsets, then lay the digits out in order
+    uint32_t digit_total = 0;
+    if (tid < radix) {
+#pragma unroll
+        for (int w = 0; w < kSortWaves; ++w) {
+            const uint32_t c = s_cnt[w][tid];
+            s_cnt[w][tid] = digit_total;
+            digit_total += c;
+        }
+    }
+    uint32_t unused_total;
+    const uint32_t digit_start = block_exclusive_scan(digit_total, s_wave, &unused_total);
+    if (tid < radix) {
+        s_start[tid] = digit_start;
+        s_dest[tid] = counters[static_cast<uint64_t>(tid) * tiles + blockIdx.x];
+    }
+    __syncthreads();
+
+#pragma unroll
+    for (int i = 0; i < kSortIpt; ++i) {
+        const uint32_t p = wave * kSortWaveItems + i * kWave + lane;
+        if (p < tile_count) {
+            const uint32_t d = (key[i] >> shift) & mask;
+            const uint32_t slot = s_start[d] + s_cnt[wave][d] + rank[i];
+            s_keys[slot] = key[i];
+            s_rows[slot] = row[i];
+            if constexpr (VB != 0) s_vals[slot] = val[i];
+        }
+    }
+    __syncthreads();
+
+    // sorted tile -> global: neighbouring threads write neighbouring addresses inside a digit run
+#pragma unroll
+    for (int i = 0; i < kSortIpt; ++i) {
+        const uint32_t slot = i * kBlock + tid;
+        if (slot < tile_count) {
+            const idx_t k = s_keys[slot];
+            const uint32_t d = (k >> shift) & mask;
+            const uint64_t out = static_cast<uint64_t>(s_dest[d]) + (slot - s_start[d]);
+            keys_out[out] = k;
+            rows_out[out] = s_rows[slot];
+            if constexpr (VB != 0) vals_out[out] = s_vals[slot];
+        }
+    }
+}
+
+uint32_t sort_tiles(idx_t nnz) { return static_cast<uint32_t>((static_cast<uint64_t>(nnz) + kSortTile - 1) / kSortTile); }
+
+struct Csr2CscLayout {
+    size_t coo_rows, sorted_keys, keys_a, rows_a, vals_a, keys_b, rows_b, vals_b, counters, scan_ws, total;
+};
+
+Csr2CscLayout csr2csc_layout(idx_t nnz, size_t value_bytes) {
+    Csr2CscLayout l;
+    const size_t idx_bytes = align_up(static_cast<size_t>(nnz) * sizeof(idx_t));
+    const size_t val_bytes = align_up(static_cast<size_t>(nnz) * value_bytes);
+    const size_t counter_elems = static_cast<size_t>(kMaxRadix) * sort_tiles(nnz);
+    size_t off = 0;
+    l.coo_rows = off; off += idx_bytes;
+    l.sorted_keys = off; off += idx_bytes;
+    l.keys_a = off; off += idx_bytes;
+    l.rows_a = off; off += idx_bytes;
+    l.vals_a = off; off += val_bytes;
+    l.keys_b = off; off += idx_bytes;
+    l.rows_b = off; off += idx_bytes;
+    l.vals_b = off; off += val_bytes;
+    l.counters = off; off += align_up(counter_elems * sizeof(uint32_t));
+    l.scan_ws = off; off += align_up(scan_workspace_elems(counter_elems) * sizeof(uint32_t)) + kAlign;
+    l.total = off;
+    return l;
+}
+
+}  // namespace
+
+void launch_csr2coo(hipStream_t stream, idx_t m, idx_t nnz, const idx_t* row_ptr, idx_t base, idx_t* coo_rows) {
+    if (nnz == 0) return;
+    const uint64_t total = static_cast<uint64_t>(m) + nnz;
+    const uint32_t tiles = static_cast<uint32_t>((total + kExpandTile - 1) / kExpandTile);
+    hipLaunchKernelGGL(csr2coo_kernel, dim3(tiles), dim3(kBlock), 0, stream, m, nnz, base, row_ptr, coo_rows);
+}
+
+void launch_coo2csr(hipStream_t stream, idx_t nnz, idx_t m, const idx_t* coo_rows, idx_t base, idx_t* row_ptr) {
+    const uint64_t threads = static_cast<uint64_t>(nnz) + 1;
+    hipLaunchKernelGGL(coo2csr_kernel, dim3(static_cast<uint32_t>((threads + kBlock - 1) / kBlock)), dim3(kBlock), 0,
+                       stream, nnz, m, base, coo_rows, row_ptr);
+}
+
+size_t csr2csc_workspace_bytes(idx_t /*m*/, idx_t /*n*/, idx_t nnz, size_t value_bytes) {
+    return csr2csc_layout(nnz, value_bytes).total;
+}
+
+void launch_csr2csc(hipStream_t stream, idx_t m, idx_t n, idx_t nnz, const void* csr_val, const idx_t* row_ptr,
+                    const idx_t* col, void* csc_val, idx_t* row_ind, idx_t* col_ptr, size_t value_bytes, idx_t base,
+                    void* workspace) {
+    if (m == 0 || n == 0 || nnz == 0) return;
+    const Csr2CscLayout l = csr2csc_layout(nnz, value_bytes);
+    char* w = static_cast<char*>(workspace);
+    idx_t* coo_rows = reinterpret_cast<idx_t*>(w + l.coo_rows);
+    idx_t* sorted_keys = reinterpret_cast<idx_t*>(w + l.sorted_keys);
+    idx_t* keys_t[2] = {reinterpret_cast<idx_t*>(w + l.keys_a), reinterpret_cast<idx_t*>(w + l.keys_b)};
+    idx_t* rows_t[2] = {reinterpret_cast<idx_t*>(w + l.rows_a), reinterpret_cast<idx_t*>(w + l.rows_b)};
+    void* vals_t[2] = {w + l.vals_a, w + l.vals_b};
+    uint32_t* counters = reinterpret_cast<uint32_t*>(w + l.counters);
+    uint32_t* scan_ws = reinterpret_cast<uint32_t*>(w + l.scan_ws);
+
+    launch_csr2coo(stream, m, nnz, row_ptr, base, coo_rows);
+
+    // keys are the raw column indices (index base included), so the largest key is n - 1 + base
+    const uint32_t key_bits = bit_length(n - 1 + base);
+    const uint32_t passes = key_bits == 0 ? 1 : (key_bits + 7) / 8;
+    const uint32_t bits_per_pass = key_bits == 0 ? 1 : (key_bits + passes - 1) / passes;
+    const uint32_t tiles = sort_tiles(nnz);
+
+    const idx_t* keys_in = col;
+    const idx_t* rows_in = coo_rows;
+    const void* vals_in = csr_val;
+    uint32_t shift = 0;
+    for (uint32_t p = 0; p < passes; ++p) {
+        const bool last = p + 1 == passes;
+        idx_t* keys_out = last ? sorted_keys : keys_t[p & 1];
+        idx_t* rows_out = last ? row_ind : rows_t[p & 1];
+        void* vals_out = last ? csc_val : vals_t[p & 1];
+        const uint32_t bits = bits_per_pass;
+        const uint32_t radix = 1u << bits;
+        hipLaunchKernelGGL(radix_hist_kernel, dim3(tiles), dim3(kBlock), 0, stream, keys_in, nnz, shift, bits, tiles,
+                           counters);
+        launch_exclusive_scan(stream, counters, static_cast<uint64_t>(radix) * tiles, scan_ws);
+        if (value_bytes == 0) {
+            hipLaunchKernelGGL((radix_scatter_kernel<0>), dim3(tiles), dim3(kBlock), 0, stream, keys_in, rows_in,
+                               vals_in, keys_out, rows_out, vals_out, nnz, shift, bits, tiles, counters);
+        } else if (value_bytes == 4) {
+            hipLaunchKernelGGL((radix_scatter_kernel<4>), dim3(tiles), dim3(kBlock), 0, stream, keys_in, rows_in,
+                               vals_in, keys_out, rows_out, vals_out, nnz, shift, bits, tiles, counters);
+        } else {
+            hipLaunchKernelGGL((radix_scatter_kernel<8>), dim3(tiles), dim3(kBlock), 0, stream, keys_in, rows_in,
+                               vals_in, keys_out, rows_out, vals_out, nnz, shift, bits, tiles, counters);
+        }
+        keys_in = keys_out;
+        rows_in = rows_out;
+        vals_in = vals_out;
+        shift += bits;
+    }
+    launch_coo2csr(stream, nnz, n, sorted_keys, base, col_ptr);
+}
+
+}  // namespace mcsp

@@ -1,0 +1,191 @@
+// Host-side objects behind the opaque handles of mcsparse.h, and the launch entry points
+// the host layer calls.  Not installed; the ABI is include/mcsparse.h only.
+#ifndef MCSPARSE_AMD_INTERNAL_H_
+#define MCSPARSE_AMD_INTERNAL_H_
+
+#include <hip/hip_runtime_api.h>
+
+#include <cstddef>
+#include <cstdint>
+
+#include "mcsparse.h"
+
+// Sub-buffer alignment and the smallest size any *_bufferSize reports
+// (reference: src/include/mcsp_config.h:13-15).
+constexpr size_t kAlign = 128;
+constexpr size_t kMinBuffer = 128;
+
+static constexpr inline size_t align_up(size_t n, size_t a = kAlign) { return (n + a - 1) / a * a; }
+
+// reference: src/include/mcsp_handle.h:11-27 (device pool dropped, see mcsparse.h)
+struct mcsparseContext {
+    hipStream_t stream = nullptr;
+    mcsparsePointerMode_t ptr_mode = MCSPARSE_POINTER_MODE_HOST;
+};
+
+// reference: src/include/mcsp_internal_types.h:127-133
+struct mcsparseDnVecDescr {
+    macaDataType valueType = MACA_R_32F;
+    int64_t size = 0;
+    void* values = nullptr;
+};
+
+// reference: src/include/mcsp_internal_types.h:135-147 (batch fields are not on this path)
+struct mcsparseDnMatDescr {
+    macaDataType valueType = MACA_R_32F;
+    mcsparseOrder_t order = MCSPARSE_ORDER_COL;
+    int64_t row_num = 0;
+    int64_t col_num = 0;
+    int64_t ld = 0;
+    void* values = nullptr;
+};
+
+// Kernel family of an SpMV call.
+enum SpmvFamily : int { kFamilyAuto = 0, kFamilyVector = 1, kFamilyMerge = 2 };
+
+// Result of the row-length analysis of one CSR structure.  It only steers which kernel
+// runs; both kernel families are correct for any structure, so a stale plan costs time,
+// never correctness.
+struct SpmvPlan {
+    bool valid = false;
+    // signature of the structure the plan was computed for
+    const void* rows = nullptr;
+    int64_t m = 0, nnz = 0;
+    int base = 0;
+    // outcome
+    int family = kFamilyAuto;
+    int lanes = 0;
+    uint32_t max_row_len = 0;
+    uint32_t hist[MCSPARSE_ROW_BIN_COUNT] = {0};
+    // user override (mcsparseSpMatSetSpMVPlan); kFamilyAuto = none
+    int forced_family = kFamilyAuto;
+    int forced_lanes = 0;
+};
+
+// reference: src/include/mcsp_internal_types.h:184-225.  rows/cols follow the reference's
+// convention: for CSR rows = row offsets, cols = column indices; for CSC rows = row indices,
+// cols = column offsets (src/common/mcsp_helper.cpp:447-452).
+struct mcsparseSpMatDescr {
+    mcsparseFormat_t format = MCSPARSE_FORMAT_CSR;
+    mcsparseIndexType_t rowIdxType = MCSPARSE_INDEX_32I;
+    mcsparseIndexType_t colIdxType = MCSPARSE_INDEX_32I;
+    mcsparseIndexBase_t idxBase = MCSPARSE_INDEX_BASE_ZERO;
+    macaDataType valueType = MACA_R_32F;
+    int64_t row_num = 0;
+    int64_t col_num = 0;
+    int64_t nnz = 0;
+    void* rows = nullptr;
+    void* cols = nullptr;
+    void* vals = nullptr;
+    // sizes of the transpose scratch layout, filled by *_bufferSize
+    // (reference: src/common/mcsp_internal_transpose_sparse.hpp:517-549)
+    int is_buffersize_called = 0;
+    size_t assist_index_buffer_size = 0;
+    size_t fixed_length_buffer_size = 0;
+    SpmvPlan plan;
+};
+
+// Internal status, mapped to the public one exactly as the reference's wrapper does
+// (src/include/mcsp_internal_types.h:13-30, src/wrapper/mcsp_interface_wrapper.cpp:5-42).
+enum mcspStatus_t {
+    MCSP_STATUS_SUCCESS = 0,
+    MCSP_STATUS_INVALID_HANDLE = 1,
+    MCSP_STATUS_NOT_IMPLEMENTED = 2,
+    MCSP_STATUS_INVALID_POINTER = 3,
+    MCSP_STATUS_INVALID_SIZE = 4,
+    MCSP_STATUS_MEMORY_ERROR = 5,
+    MCSP_STATUS_INTERNAL_ERROR = 6,
+    MCSP_STATUS_INVALID_VALUE = 7,
+    MCSP_STATUS_ARCH_MISMATCH = 8,
+    MCSP_STATUS_ZERO_PIVOT = 9,
+    MCSP_STATUS_NOT_INITIALIZED = 10,
+    MCSP_STATUS_TYPE_MISMATCH = 11,
+    MCSP_STATUS_MAPPING_ERROR = 12,
+    MCSP_STATUS_EXECUTION_FAILED = 13,
+    MCSP_STATUS_MATRIX_TYPE_NOT_SUPPORTED = 14,
+    MCSP_STATUS_INSUFFICIENT_RESOURCES = 15
+};
+mcsparseStatus_t to_public_status(mcspStatus_t s);
+
+static inline size_t value_size(macaDataType t) {
+    switch (t) {
+        case MACA_R_32F: return 4;
+        case MACA_R_64F: return 8;
+        case MACA_C_32F: return 8;
+        case MACA_C_64F: return 16;
+        case MACA_R_16F: case MACA_R_16BF: return 2;
+        case MACA_C_16F: case MACA_C_16BF: return 4;
+        case MACA_R_8I: return 1;
+        case MACA_R_32I: return 4;
+        default: return 0;
+    }
+}
+
+// Bits needed to write n: 0 -> 0, 1 -> 1, 2..3 -> 2 ...
+// (reference: src/include/mcsp_internal_host_utils.hpp:25-32)
+static inline uint32_t bit_length(uint32_t n) {
+    uint32_t b = 0;
+    while (n) { ++b; n >>= 1; }
+    return b;
+}
+
+// ---------------------------------------------------------------------------------------
+// Device work.  Every function enqueues on `stream` and returns without synchronising
+// unless stated.  Index arrays are unsigned 32-bit.  "base" is 0 or 1.
+// ---------------------------------------------------------------------------------------
+namespace mcsp {
+
+typedef uint32_t idx_t;
+
+// ---- row-length analysis (analysis.hip) ----
+// hist_out: MCSPARSE_ROW_BIN_COUNT counters followed by the longest row length (34 x u32),
+// zeroed by this call.  row_bins may be null.
+void launch_row_bins(hipStream_t stream, idx_t m, const idx_t* row_ptr, idx_t base, uint8_t* row_bins,
+                     uint32_t* hist_out);
+
+// ---- SpMV (spmv.hip) ----
+struct SpmvArgs {
+    idx_t m, n, nnz, base;
+    const idx_t* row_ptr;
+    const idx_t* col;
+    const void* val;
+    const void* x;
+    void* y;
+};
+// y = alpha*A*x + beta*y; beta == 0 never reads y.
+template <typename T>
+void launch_spmv_vector(hipStream_t stream, const SpmvArgs& a, T alpha, T beta, int lanes);
+// workspace: spmv_merge_workspace_bytes(m, nnz, sizeof(T)) bytes of device scratch.
+size_t spmv_merge_workspace_bytes(idx_t m, idx_t nnz, size_t value_bytes);
+template <typename T>
+void launch_spmv_merge(hipStream_t stream, const SpmvArgs& a, T alpha, T beta, void* workspace);
+int spmv_pick_lanes(idx_t m, idx_t nnz);
+
+// ---- SpMM (spmm.hip) ----
+struct SpmmArgs {
+    idx_t m, n, k, nnz, base;   // C is m x n, A is m x k
+    const idx_t* row_ptr;
+    const idx_t* col;
+    const void* val;
+    const void* B;
+    int64_t ldb;
+    bool b_row_major;           // element (kk, j) of op(B) at kk*ldb + j, else at j*ldb + kk
+    void* C;
+    int64_t ldc;
+    bool c_row_major;
+};
+template <typename T>
+void launch_spmm(hipStream_t stream, const SpmmArgs& a, T alpha, T beta);
+
+// ---- conversions (convert.hip) ----
+void launch_csr2coo(hipStream_t stream, idx_t m, idx_t nnz, const idx_t* row_ptr, idx_t base, idx_t* coo_rows);
+void launch_coo2csr(hipStream_t stream, idx_t nnz, idx_t m, const idx_t* coo_rows, idx_t base, idx_t* row_ptr);
+size_t csr2csc_workspace_bytes(idx_t m, idx_t n, idx_t nnz, size_t value_bytes);
+// value_bytes 0 = structure only.  Writes col_ptr[n+1], row_ind[nnz] (both + base) and csc_val.
+void launch_csr2csc(hipStream_t stream, idx_t m, idx_t n, idx_t nnz, const void* csr_val, const idx_t* row_ptr,
+                    const idx_t* col, void* csc_val, idx_t* row_ind, idx_t* col_ptr, size_t value_bytes,
+                    idx_t base, void* workspace);
+
+}  // namespace mcsp
+
+#endif  // MCSPARSE_AMD_INTERNAL_H_

@@ -1,0 +1,378 @@
+// CSR SpMV for gfx950: y = alpha*A*x + beta*y.
+//
+// Two kernel families, picked from the row-length analysis of the structure:
+//  * vector : L consecutive lanes of a wavefront own one row (L = 1..64, chosen from the mean
+//             row length); U rows per lane group are kept in flight at once so that a wave has
+//             enough bytes outstanding to cover HBM latency.  Best for regular matrices.
+//  * merge  : the rows' end offsets and the nonzero indices are merged into one path of m+nnz
+//             items that is cut into equal tiles, one per workgroup, so a 200k-nonzero row and
+//             a million 1-nonzero rows cost the same per item.  Rows that straddle tiles leave a
+//             (row, partial sum) carry that a second kernel adds in a fixed order, so results do
+//             not depend on scheduling.
+// Both families are correct for any CSR structure.  With beta == 0, y is never read.
+//
+// Stands in for mcspSpmvCsrVectorKernel of the reference
+// (src/kernels/level2/spmv/csr_vector_device.hpp:22-79), which runs one wavefront per row.
+#include "device_util.h"
+#include "internal.h"
+
+namespace mcsp {
+
+namespace {
+
+constexpr int kBlock = 256;
+
+// ------------------------------------------------------------------------------------------
+// vector family
+// ------------------------------------------------------------------------------------------
+template <typename T, int L, int U, bool BETA0>
+__global__ __launch_bounds__(kBlock) void spmv_vector_kernel(idx_t m, idx_t base, const idx_t* __restrict__ row_ptr,
+                                                             const idx_t* __restrict__ col,
+                                                             const T* __restrict__ val, const T* __restrict__ x,
+                                                             T* __restrict__ y, T alpha, T beta) {
+    constexpr int kGroups = kBlock / L;  // lane groups (= rows per pass) in a workgroup
+    const idx_t lane = threadIdx.x % L;
+    const idx_t group = threadIdx.x / L;
+    const uint64_t row0 = static_cast<uint64_t>(blockIdx.x) * (kGroups * U) + group;
+
+    idx_t j[U], e[U];
+    T s[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        const uint64_t row = row0 + static_cast<uint64_t>(u) * kGroups;
+        if (row < m) {
+            j[u] = row_ptr[row] - base + lane;
+            e[u] = row_ptr[row + 1] - base;
+        } else {
+            j[u] = 0;
+            e[u] = 0;
+        }
+        s[u] = T(0);
+    }
+
+    // All lanes stay in the loop until every row of the wave is done, so that the loads of the
+    // U rows are issued back to back and the DPP reduction below sees 64 active lanes.
+    bool more;
+    do {
+        idx_t c[U];
+        T v[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const bool act = j[u] < e[u];
+            c[u] = act ? load_stream(col + j[u]) : base;
+            v[u] = act ? load_stream(val + j[u]) : T(0);
+        }
+        more = false;
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            s[u] += v[u] * x[c[u] - base];
+            j[u] += L;
+            more |= j[u] < e[u];
+        }
+    } while (__any(more));
+
+#pragma unroll
+    for (int u = 0; u < U; ++u) s[u] = group_sum<L>(s[u]);
+
+    if (lane == 0) {
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const uint64_t row = row0 + static_cast<uint64_t>(u) * kGroups;
+            if (row < m) {
+                if constexpr (BETA0) {
+                    y[row] = alpha * s[u];
+                } else {
+                    y[row] = beta * y[row] + alpha * s[u];
+                }
+            }
+        }
+    }
+}
+
+template <typename T, int L, int U>
+void launch_vector_lu(hipStream_t stream, const SpmvArgs& a, T alpha, T beta) {
+    constexpr int rows_per_block = (kBlock / L) * U;
+    const uint64_t blocks = (static_cast<uint64_t>(a.m) + rows_per_block - 1) / rows_per_block;
+    const dim3 grid(static_cast<uint32_t>(blocks));
+    const T* val = static_cast<const T*>(a.val);
+    const T* x = static_cast<const T*>(a.x);
+    T* y = static_cast<T*>(a.y);
+    if (beta == T(0)) {
+        hipLaunchKernelGGL((spmv_vector_kernel<T, L, U, true>), grid, dim3(kBlock), 0, stream, a.m, a.base, a.row_ptr,
+                           a.col, val, x, y, alpha, beta);
+    } else {
+        hipLaunchKernelGGL((spmv_vector_kernel<T, L, U, false>), grid, dim3(kBlock), 0, stream, a.m, a.base,
+                           a.row_ptr, a.col, val, x, y, alpha, beta);
+    }
+}
+
+// ------------------------------------------------------------------------------------------
+// merge family
+// ------------------------------------------------------------------------------------------
+constexpr int kItemsPerThread = 8;
+constexpr int kTile = kBlock * kItemsPerThread;  // path items per workgroup
+
+// Path coordinate of diagonal d: how many row ends (x) precede it; nonzeros consumed = d - x.
+// A row end is consumed before a nonzero whenever row_end <= nonzero index.
+__device__ __forceinline__ idx_t merge_search_global(uint64_t d, idx_t m, idx_t nnz, idx_t base,
+                                                     const idx_t* __restrict__ row_ptr) {
+    uint64_t lo = d > nnz ? d - nnz : 0;
+    uint64_t hi = d < m ? d : m;
+    while (lo < hi) {
+        const uint64_t mid = (lo + hi) >> 1;
+        const uint64_t row_end = row_ptr[mid + 1] - base;
+        if (row_end <= d - mid - 1) {
+            lo = mid + 1;
+        } else {
+            hi = mid;
+        }
+    }
+    return static_cast<idx_t>(lo);
+}
+
+__global__ __launch_bounds__(kBlock) void merge_partition_kernel(idx_t m, idx_t nnz, idx_t base,
+                                                                 const idx_t* __restrict__ row_ptr, uint32_t tiles,
+                                                                 idx_t* __restrict__ tile_row) {
+    const uint32_t t = blockIdx.x * kBlock + threadIdx.x;
+    if (t > tiles) return;
+    const uint64_t total = static_cast<uint64_t>(m) + nnz;
+    uint64_t d = static_cast<uint64_t>(t) * kTile;
+    if (d > total) d = total;
+    tile_row[t] = merge_search_global(d, m, nnz, base, row_ptr);
+}
+
+template <typename T, bool BETA0>
+__global__ __launch_bounds__(kBlock) void spmv_merge_kernel(idx_t m, idx_t nnz, idx_t base,
+                                                            const idx_t* __restrict__ row_ptr,
+                                                            const idx_t* __restrict__ col, const T* __restrict__ val,
+                                                            const T* __restrict__ x, T* __restrict__ y, T alpha,
+                                                            T beta, const idx_t* __restrict__ tile_row,
+                                                            idx_t* __restrict__ carry_row, T* __restrict__ carry_val) {
+    // s_row_end[i] = end offset of row x0+i; one extra slot closes the tile.
+    __shared__ idx_t s_row_end[kTile + 1];
+    // [0, tile_nnz) holds the products, [tile_nnz, tile_nnz + tile_rows) the finished row sums.
+    __shared__ T s_data[kTile];
+    __shared__ idx_t s_wave_key[kBlock / kWave];
+    __shared__ T s_wave_val[kBlock / kWave];
+
+    const uint32_t tile = blockIdx.x;
+    const uint32_t tid = threadIdx.x;
+    const uint64_t total = static_cast<uint64_t>(m) + nnz;
+    const uint64_t d0 = static_cast<uint64_t>(tile) * kTile;
+    const uint64_t d1 = d0 + kTile < total ? d0 + kTile : total;
+    const idx_t x0 = tile_row[tile];
+    const idx_t x1 = tile_row[tile + 1];
+    const idx_t y0 = static_cast<idx_t>(d0 - x0);
+    const idx_t y1 = static_cast<idx_t>(d1 - x1);
+    const idx_t tile_rows = x1 - x0;
+    const idx_t tile_nnz = y1 - y0;
+    const idx_t tile_items = tile_rows + tile_nnz;
+
+    for (idx_t i = tid; i <= tile_rows; i += kBlock) {
+        const idx_t r = x0 + i;
+        s_row_end[i] = r < m ? row_ptr[r + 1] - base : 0xFFFFFFFFu;
+    }
+#pragma unroll
+    for (int i = 0; i < kItemsPerThread; ++i) {
+        const idx_t k = tid + i * kBlock;
+        if (k < tile_nnz) {
+            const idx_t c = load_stream(col + y0 + k) - base;
+            const T v = load_stream(val + y0 + k);
+            s_data[k] = v * x[c];
+        }
+    }
+    __syncthreads();
+
+    // this thread's start on the tile's path
+    const idx_t dt = min(static_cast<idx_t>(tid * kItemsPerThread), tile_items);
+    idx_t lo = dt > tile_nnz ? dt - tile_nnz : 0;
+    idx_t hi = dt < tile_rows ? dt : tile_rows;
+    while (lo < hi) {
+        const idx_t mid = (lo + hi) >> 1;
+        if (s_row_end[mid] <= y0 + (dt - mid - 1)) {
+            lo = mid + 1;
+        } else {
+            hi = mid;
+        }
+    }
+    idx_t row_l = lo;
+    idx_t nz = y0 + (dt - lo);
+    const idx_t first_row_l = row_l;
+    bool emitted = false;
+    T first_val = T(0);
+    T running = T(0);
+    T* s_out = s_data + tile_nnz;
+#pragma unroll
+    for (int i = 0; i < kItemsPerThread; ++i) {
+        if (dt + i < tile_items) {
+            if (nz < s_row_end[row_l]) {
+                running += s_data[nz - y0];
+                ++nz;
+            } else {
+                if (!emitted) {
+                    first_val = running;  // completed below, once the carry-in is known
+                    emitted = true;
+                } else {
+                    s_out[row_l] = running;
+                }
+                running = T(0);
+                ++row_l;
+            }
+        }
+    }
+
+    // Exclusive reduce-by-row scan of (open row, partial sum) over the threads.  Keys never
+    // decrease along the path, so "same key: add, else keep the later value" is associative.
+    idx_t key = row_l;
+    T value = running;
+    const unsigned lane = tid % kWave;
+    const unsigned wave = tid / kWave;
+#pragma unroll
+    for (int off = 1; off < kWave; off <<= 1) {
+        const idx_t k_up = __shfl_up(key, off, kWave);
+        const T v_up = __shfl_up(value, off, kWave);
+        if (lane >= static_cast<unsigned>(off) && k_up == key) value += v_up;
+    }
+    if (lane == kWave - 1) {
+        s_wave_key[wave] = key;
+        s_wave_val[wave] = value;
+    }
+    // exclusive within the wave
+    idx_t ex_key = __shfl_up(key, 1, kWave);
+    T ex_val = __shfl_up(value, 1, kWave);
+    bool has_prefix = lane != 0;
+    __syncthreads();
+    {
+        // fold the totals of the earlier waves
+        bool w_has = false;
+        idx_t w_key = 0;
+        T w_val = T(0);
+        for (unsigned w = 0; w < wave; ++w) {
+            const idx_t k = s_wave_key[w];
+            const T v = s_wave_val[w];
+            w_val = (w_has && w_key == k) ? w_val + v : v;
+            w_key = k;
+            w_has = true;
+        }
+        if (w_has) {
+            if (has_prefix) {
+                if (w_key == ex_key) ex_val += w_val;
+            } else {
+                ex_key = w_key;
+                ex_val = w_val;
+                has_prefix = true;
+            }
+        }
+    }
+    const T carry_in = (has_prefix && ex_key == first_row_l) ? ex_val : T(0);
+    if (emitted) s_out[first_row_l] = first_val + carry_in;
+
+    if (tid == kBlock - 1) {
+        // inclusive total of the whole tile = partial sum of the row left open at its end
+        const T tile_total = (has_prefix && ex_key == key) ? ex_val + running : running;
+        // `running` only covers this thread; if it emitted, earlier partials do not belong
+        const T open_sum = emitted ? running : tile_total;
+        carry_row[tile] = x1;
+        carry_val[tile] = open_sum;
+    }
+    __syncthreads();
+
+    for (idx_t i = tid; i < tile_rows; i += kBlock) {
+        const idx_t r = x0 + i;
+        if constexpr (BETA0) {
+            y[r] = alpha * s_out[i];
+        } else {
+            y[r] = beta * y[r] + alpha * s_out[i];
+        }
+    }
+}
+
+// Adds the carries of rows that straddle tiles.  carry_row is non-decreasing; the first tile of
+// each run of equal rows sums the run and updates y once.
+template <typename T>
+__global__ __launch_bounds__(kBlock) void spmv_merge_fixup_kernel(idx_t m, uint32_t tiles,
+                                                                  const idx_t* __restrict__ carry_row,
+                                                                  const T* __restrict__ carry_val, T* __restrict__ y,
+                                                                  T alpha) {
+    const uint32_t t = blockIdx.x * kBlock + threadIdx.x;
+    if (t >= tiles) return;
+    const idx_t r = carry_row[t];
+    if (r >= m) return;
+    if (t > 0 && carry_row[t - 1] == r) return;
+    T sum = carry_val[t];
+    for (uint32_t u = t + 1; u < tiles && carry_row[u] == r; ++u) sum += carry_val[u];
+    if (sum != T(0)) y[r] += alpha * sum;
+}
+
+inline uint32_t merge_tiles(idx_t m, idx_t nnz) {
+    const uint64_t total = static_cast<uint64_t>(m) + nnz;
+    return static_cast<uint32_t>((total + kTile - 1) / kTile);
+}
+
+}  // namespace
+
+// Lanes per row for the vector family: the power of two nearest the mean row length from
+// above, so that a typical row is read in one pass of its lane group.
+int spmv_pick_lanes(idx_t m, idx_t nnz) {
+    if (m == 0) return 1;
+    const double mean = static_cast<double>(nnz) / static_cast<double>(m);
+    int lanes = 1;
+    while (lanes < 64 && static_cast<double>(lanes) < mean) lanes <<= 1;
+    return lanes;
+}
+
+template <typename T>
+void launch_spmv_vector(hipStream_t stream, const SpmvArgs& a, T alpha, T beta, int lanes) {
+    if (a.m == 0) return;
+    switch (lanes) {
+        case 1: launch_vector_lu<T, 1, 2>(stream, a, alpha, beta); break;
+        case 2: launch_vector_lu<T, 2, 4>(stream, a, alpha, beta); break;
+        case 4: launch_vector_lu<T, 4, 4>(stream, a, alpha, beta); break;
+        case 8: launch_vector_lu<T, 8, 4>(stream, a, alpha, beta); break;
+        case 16: launch_vector_lu<T, 16, 4>(stream, a, alpha, beta); break;
+        case 32: launch_vector_lu<T, 32, 4>(stream, a, alpha, beta); break;
+        default: launch_vector_lu<T, 64, 4>(stream, a, alpha, beta); break;
+    }
+}
+
+// Workspace layout: [tile_row: tiles+1 idx][carry_row: tiles idx][carry_val: tiles T], each
+// sub-array aligned to 128 bytes.
+size_t spmv_merge_workspace_bytes(idx_t m, idx_t nnz, size_t value_bytes) {
+    const size_t tiles = merge_tiles(m, nnz);
+    return align_up((tiles + 1) * sizeof(idx_t)) + align_up(tiles * sizeof(idx_t)) + align_up(tiles * value_bytes);
+}
+
+template <typename T>
+void launch_spmv_merge(hipStream_t stream, const SpmvArgs& a, T alpha, T beta, void* workspace) {
+    if (a.m == 0) return;
+    const uint32_t tiles = merge_tiles(a.m, a.nnz);
+    char* w = static_cast<char*>(workspace);
+    idx_t* tile_row = reinterpret_cast<idx_t*>(w);
+    w += align_up((static_cast<size_t>(tiles) + 1) * sizeof(idx_t));
+    idx_t* carry_row = reinterpret_cast<idx_t*>(w);
+    w += align_up(static_cast<size_t>(tiles) * sizeof(idx_t));
+    T* carry_val = reinterpret_cast<T*>(w);
+
+    const T* val = static_cast<const T*>(a.val);
+    const T* x = static_cast<const T*>(a.x);
+    T* y = static_cast<T*>(a.y);
+
+    hipLaunchKernelGGL(merge_partition_kernel, dim3((tiles + 1 + kBlock - 1) / kBlock), dim3(kBlock), 0, stream, a.m,
+                       a.nnz, a.base, a.row_ptr, tiles, tile_row);
+    if (beta == T(0)) {
+        hipLaunchKernelGGL((spmv_merge_kernel<T, true>), dim3(tiles), dim3(kBlock), 0, stream, a.m, a.nnz, a.base,
+                           a.row_ptr, a.col, val, x, y, alpha, beta, tile_row, carry_row, carry_val);
+    } else {
+        hipLaunchKernelGGL((spmv_merge_kernel<T, false>), dim3(tiles), dim3(kBlock), 0, stream, a.m, a.nnz, a.base,
+                           a.row_ptr, a.col, val, x, y, alpha, beta, tile_row, carry_row, carry_val);
+    }
+    hipLaunchKernelGGL((spmv_merge_fixup_kernel<T>), dim3((tiles + kBlock - 1) / kBlock), dim3(kBlock), 0, stream, a.m,
+                       tiles, carry_row, carry_val, y, alpha);
+}
+
+template void launch_spmv_vector<float>(hipStream_t, const SpmvArgs&, float, float, int);
+template void launch_spmv_vector<double>(hipStream_t, const SpmvArgs&, double, double, int);
+template void launch_spmv_merge<float>(hipStream_t, const SpmvArgs&, float, float, void*);
+template void launch_spmv_merge<double>(hipStream_t, const SpmvArgs&, double, double, void*);
+
+}  // namespace mcsp

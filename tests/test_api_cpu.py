@@ -1,0 +1,281 @@
+"""Host-side behaviour of the C ABI that needs no GPU: exported symbols, handle and descriptor
+objects, and the argument checks, which all return before any device work.  Expected codes
+follow the reference's host drivers (cited per test, paths relative to mcsparse/src)."""
+import ctypes
+import re
+import os
+
+import pytest
+
+from mcsparse_amd import api, _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+FAKE = 0x1000  # a non-NULL "device pointer"; never dereferenced on these paths
+
+
+def test_library_exports_every_declared_symbol(lib):
+    header = open(os.path.join(ROOT, "include", "mcsparse.h")).read()
+    declared = set(re.findall(r"\b(mcsparse[A-Za-z0-9_]+)\s*\(", header))
+    assert declared, "no prototypes found in include/mcsparse.h"
+    assert declared == set(_lib.PROTOTYPES), declared ^ set(_lib.PROTOTYPES)
+    for name in declared:
+        assert hasattr(lib, name), name
+
+
+def test_status_strings(lib):
+    # wrapper/mcsp_interface_wrapper.cpp:48-108
+    assert lib.mcsparseGetErrorName(0) == b"MCSPARSE_STATUS_SUCCESS"
+    assert lib.mcsparseGetErrorName(10) == b"MCSPARSE_STATUS_NOT_SUPPORTED"
+    assert lib.mcsparseGetErrorString(3) == b"invalid value"
+    assert lib.mcsparseGetErrorString(6) == b"kernel launch failure"
+    assert lib.mcsparseGetErrorName(99) == b"unrecognized error code"
+    assert lib.mcsparseGetErrorString(-1) == b"unrecognized error code"
+
+
+def test_handle_lifecycle(lib):
+    # common/mcsp_helper.cpp:69-88, :154-198, :294-322
+    assert lib.mcsparseCreate(None) == api.STATUS_INVALID_VALUE
+    h = ctypes.c_void_p()
+    assert lib.mcsparseCreate(ctypes.byref(h)) == 0 and h.value
+    v = ctypes.c_int(-1)
+    assert lib.mcsparseGetVersion(h, ctypes.byref(v)) == 0 and v.value == 1000000
+    assert lib.mcsparseGetVersion(None, ctypes.byref(v)) == api.STATUS_NOT_INITIALIZED
+    assert lib.mcsparseGetVersion(h, None) == api.STATUS_INVALID_VALUE
+    assert lib.mcsparseGetVersion(None, None) == api.STATUS_INVALID_VALUE  # pointer is tested first
+    for prop, want in ((0, 1), (1, 0), (2, 0)):
+        assert lib.mcsparseGetProperty(prop, ctypes.byref(v)) == 0 and v.value == want
+    assert lib.mcsparseGetProperty(7, ctypes.byref(v)) == api.STATUS_INVALID_VALUE
+    s = ctypes.c_void_p(123)
+    assert lib.mcsparseGetStream(h, ctypes.byref(s)) == 0 and not s.value  # default: NULL stream
+    assert lib.mcsparseSetStream(h, ctypes.c_void_p(0xABC0)) == 0
+    assert lib.mcsparseGetStream(h, ctypes.byref(s)) == 0 and s.value == 0xABC0
+    assert lib.mcsparseSetStream(None, None) == api.STATUS_NOT_INITIALIZED
+    assert lib.mcsparseGetStream(h, None) == api.STATUS_INVALID_VALUE
+    pm = ctypes.c_int(-1)
+    assert lib.mcsparseGetPointerMode(h, ctypes.byref(pm)) == 0 and pm.value == api.PTR_HOST
+    assert lib.mcsparseSetPointerMode(h, api.PTR_DEVICE) == 0
+    assert lib.mcsparseGetPointerMode(h, ctypes.byref(pm)) == 0 and pm.value == api.PTR_DEVICE
+    assert lib.mcsparseSetPointerMode(None, 0) == api.STATUS_NOT_INITIALIZED
+    assert lib.mcsparseDestroy(h) == 0
+    assert lib.mcsparseDestroy(None) == 0  # NULL accepted
+
+
+def test_dense_descriptors(lib):
+    # common/mcsp_helper.cpp:325-387, :715-800
+    d = ctypes.c_void_p()
+    assert lib.mcsparseCreateDnVec(ctypes.byref(d), -1, FAKE, api.R_32F) == api.STATUS_INVALID_VALUE
+    assert lib.mcsparseCreateDnVec(ctypes.byref(d), 4, None, api.R_32F) == api.STATUS_INVALID_VALUE
+    assert lib.mcsparseCreateDnVec(None, 4, FAKE, api.R_32F) == api.STATUS_INVALID_VALUE
+    assert lib.mcsparseCreateDnVec(ctypes.byref(d), 4, FAKE, 24) == api.STATUS_NOT_SUPPORTED  # R_64I
+    assert lib.mcsparseCreateDnVec(ctypes.byref(d), 4, FAKE, api.R_64F) == 0
+    size, vals, vt = ctypes.c_int64(), ctypes.c_void_p(), ctypes.c_int()
+    assert lib.mcsparseDnVecGet(d, ctypes.byref(size), ctypes.byref(vals), ctypes.byref(vt)) == 0
+    assert (size.value, vals.value, vt.value) == (4, FAKE, api.R_64F)
+    assert lib.mcsparseDnVecGet(d, None, ctypes.byref(vals), ctypes.byref(vt)) == api.STATUS_INVALID_VALUE
+    assert lib.mcsparseDnVecSetValues(d, 0x2000) == 0
+    assert lib.mcsparseDnVecGetValues(d, ctypes.byref(vals)) == 0 and vals.value == 0x2000
+    assert lib.mcsparseDnVecSetValues(None, 0x2000) == api.STATUS_INVALID_VALUE
+    assert lib.mcsparseDestroyDnVec(d) == 0 and lib.mcsparseDestroyDnVec(None) == 0
+
+    m = ctypes.c_void_p()
+    assert lib.mcsparseCreateDnMat(ctypes.byref(m), 3, -2, 3, FAKE, api.R_32F, api.ORDER_ROW) == api.STATUS_INVALID_VALUE
+    assert lib.mcsparseCreateDnMat(ctypes.byref(m), 3, 2, 3, FAKE, 24, api.ORDER_ROW) == api.STATUS_NOT_SUPPORTED
+    assert lib.mcsparseCreateDnMat(ctypes.byref(m), 3, 2, 3, None, api.R_32F, api.ORDER_ROW) == api.STATUS_INVALID_VALUE
+    assert lib.mcsparseCreateDnMat(ctypes.byref(m), 3, 2, 5, FAKE, api.R_32F, api.ORDER_COL) == 0
+    r, c, ld, order = ctypes.c_int64(), ctypes.c_int64(), ctypes.c_int64(), ctypes.c_int()
+    assert lib.mcsparseDnMatGet(m, ctypes.byref(r), ctypes.byref(c), ctypes.byref(ld), ctypes.byref(vals),
+                                ctypes.byref(vt), ctypes.byref(order)) == 0
+    assert (r.value, c.value, ld.value, vals.value, vt.value, order.value) == (3, 2, 5, FAKE, api.R_32F, api.ORDER_COL)
+    assert lib.mcsparseDnMatSetValues(m, 0x3000) == 0
+    assert lib.mcsparseDnMatGetValues(m, ctypes.byref(vals)) == 0 and vals.value == 0x3000
+    assert lib.mcsparseDestroyDnMat(m) == 0 and lib.mcsparseDestroyDnMat(None) == 0
+
+
+def test_sparse_descriptors(lib):
+    # common/mcsp_helper.cpp:389-452, :503-524, :587-683
+    d = ctypes.c_void_p()
+    mk = lib.mcsparseCreateCsr
+    assert mk(ctypes.byref(d), -1, 4, 5, 0x10, 0x20, 0x30, 2, 2, 0, api.R_32F) == api.STATUS_INVALID_VALUE
+    assert mk(ctypes.byref(d), 3, 4, 5, 0x10, 0x20, 0x30, 2, 2, 0, api.R_32I) == api.STATUS_NOT_SUPPORTED
+    assert mk(None, 3, 4, 5, 0x10, 0x20, 0x30, 2, 2, 0, api.R_32F) == api.STATUS_INVALID_VALUE
+    assert mk(ctypes.byref(d), 3, 4, 5, 0x10, 0x20, 0x30, 2, 2, 7, api.R_32F) == api.STATUS_INVALID_VALUE  # bad base
+    assert mk(ctypes.byref(d), 3, 4, 5, None, None, None, 2, 2, 1, api.R_64F) == 0  # pointers are not checked
+    i64 = [ctypes.c_int64() for _ in range(3)]
+    ptrs = [ctypes.c_void_p() for _ in range(3)]
+    ints = [ctypes.c_int() for _ in range(4)]
+    assert lib.mcsparseCsrSetPointers(d, 0x10, 0x20, 0x30) == 0
+    assert lib.mcsparseCsrGet(d, *[ctypes.byref(x) for x in i64 + ptrs + ints]) == 0
+    assert [x.value for x in i64] == [3, 4, 5]
+    assert [x.value for x in ptrs] == [0x10, 0x20, 0x30]
+    assert [x.value for x in ints] == [2, 2, 1, api.R_64F]
+    assert lib.mcsparseCsrGet(d, None, *[ctypes.byref(x) for x in i64[1:] + ptrs + ints]) == api.STATUS_INVALID_VALUE
+    fmt, base = ctypes.c_int(), ctypes.c_int()
+    assert lib.mcsparseSpMatGetFormat(d, ctypes.byref(fmt)) == 0 and fmt.value == api.FORMAT_CSR
+    assert lib.mcsparseSpMatGetIndexBase(d, ctypes.byref(base)) == 0 and base.value == 1
+    assert lib.mcsparseSpMatGetSize(d, *[ctypes.byref(x) for x in i64]) == 0
+    assert lib.mcsparseSpMatSetValues(d, 0x44) == 0
+    v = ctypes.c_void_p()
+    assert lib.mcsparseSpMatGetValues(d, ctypes.byref(v)) == 0 and v.value == 0x44
+    assert lib.mcsparseSpMatGetValues(None, ctypes.byref(v)) == api.STATUS_INVALID_VALUE
+    assert lib.mcsparseDestroySpMat(d) == 0 and lib.mcsparseDestroySpMat(None) == 0
+    # CSC: offsets are the columns' (mcsp_helper.cpp:447-452)
+    assert lib.mcsparseCreateCsc(ctypes.byref(d), 3, 4, 5, 0x50, 0x60, 0x70, 2, 2, 0, api.R_32F) == 0
+    assert lib.mcsparseSpMatGetFormat(d, ctypes.byref(fmt)) == 0 and fmt.value == api.FORMAT_CSC
+    assert lib.mcsparseCscSetPointers(d, 0x51, 0x61, 0x71) == 0
+    assert lib.mcsparseCscSetPointers(None, 0x51, 0x61, 0x71) == api.STATUS_INVALID_VALUE
+    assert lib.mcsparseDestroySpMat(d) == 0
+
+
+class Objs:
+    """A handle and descriptors over fake pointers for the argument-check tests."""
+
+    def __init__(self, lib, m=8, n=6, nnz=20, vt=api.R_32F, fmt=api.FORMAT_CSR, idx=(2, 2)):
+        self.lib = lib
+        self.h = ctypes.c_void_p()
+        lib.mcsparseCreate(ctypes.byref(self.h))
+        self.A = ctypes.c_void_p()
+        mk = lib.mcsparseCreateCsr if fmt == api.FORMAT_CSR else lib.mcsparseCreateCsc
+        assert mk(ctypes.byref(self.A), m, n, nnz, FAKE, FAKE, FAKE, idx[0], idx[1], 0, vt) == 0
+        self.x, self.y, self.xm = ctypes.c_void_p(), ctypes.c_void_p(), ctypes.c_void_p()
+        lib.mcsparseCreateDnVec(ctypes.byref(self.x), n, FAKE, vt)
+        lib.mcsparseCreateDnVec(ctypes.byref(self.y), m, FAKE, vt)
+        self.one = ctypes.c_float(1.0)
+        self.pa = ctypes.addressof(self.one)
+
+    def spmv(self, h="h", op=api.OP_N, alpha="a", A="A", x="x", beta="a", y="y", ct=api.R_32F, buf=FAKE):
+        g = lambda k: {"h": self.h, "a": self.pa, "A": self.A, "x": self.x, "y": self.y, None: None}[k]
+        return self.lib.mcsparseSpMV(g(h), op, g(alpha), g(A), g(x), g(beta), g(y), ct, 0, buf)
+
+    def spmv_size(self, h="h", op=api.OP_N, alpha="a", A="A", x="x", beta="a", y="y", out=True):
+        g = lambda k: {"h": self.h, "a": self.pa, "A": self.A, "x": self.x, "y": self.y, None: None}[k]
+        size = ctypes.c_size_t(0)
+        st = self.lib.mcsparseSpMV_bufferSize(g(h), op, g(alpha), g(A), g(x), g(beta), g(y), api.R_32F, 0,
+                                              ctypes.byref(size) if out else None)
+        return st, size.value
+
+
+def test_spmv_argument_checks(lib):
+    # level2/spmv/mcsp_spmv_gpu.cpp:686-720 in order
+    o = Objs(lib)
+    assert o.spmv(h=None) == api.STATUS_NOT_INITIALIZED
+    for k in ("alpha", "A", "x", "beta", "y"):
+        assert o.spmv(**{k: None}) == api.STATUS_INVALID_VALUE, k
+    assert o.spmv(buf=None) == api.STATUS_INVALID_VALUE  # required even for op N (:703-705)
+    assert o.spmv(op=api.OP_T) == api.STATUS_INVALID_VALUE  # x, y sizes do not fit the transpose (:711)
+    assert o.spmv(x="y", y="x") == api.STATUS_INVALID_VALUE
+    assert o.spmv(op=api.OP_T, x="y", y="x", ct=api.R_64F) == api.STATUS_NOT_SUPPORTED  # mixed types
+    assert o.spmv(ct=api.R_64F) == api.STATUS_NOT_SUPPORTED
+    sq = Objs(lib, m=6, n=6)
+    assert sq.spmv(op=api.OP_C) == api.STATUS_INVALID_VALUE  # conjugate on a real type (:716-720)
+    big = Objs(lib, m=1 << 32, n=6)
+    assert big.spmv() == api.STATUS_NOT_SUPPORTED  # sizes must fit 32 bits (:698-701)
+    mixed = Objs(lib, idx=(2, 3))
+    assert mixed.spmv() == api.STATUS_NOT_SUPPORTED  # row/col index types differ (:1126-1132)
+    assert mixed.spmv(h=None) == api.STATUS_NOT_SUPPORTED  # the index-type dispatch comes first
+    i64 = Objs(lib, idx=(3, 3))
+    assert i64.spmv() == api.STATUS_NOT_SUPPORTED  # 64-bit indices are not built
+    cplx = Objs(lib, vt=api.C_32F)
+    assert cplx.spmv(ct=api.C_32F) == api.STATUS_NOT_SUPPORTED
+
+
+def test_spmv_early_outs_touch_nothing(lib):
+    # mcsp_spmv_gpu.cpp:235-237: nnz == 0, or alpha == beta == 0, returns before any launch.
+    # The pointers here are fake, so reaching a kernel would fault rather than pass.
+    empty = Objs(lib, nnz=0)
+    assert empty.spmv() == api.STATUS_SUCCESS
+    o = Objs(lib)
+    zero = ctypes.c_float(0.0)
+    pz = ctypes.addressof(zero)
+    assert lib.mcsparseSpMV(o.h, api.OP_N, pz, o.A, o.x, pz, o.y, api.R_32F, 0, FAKE) == api.STATUS_SUCCESS
+
+
+def test_spmv_buffer_size(lib):
+    # level2/spmv/mcsp_spmv_gpu.cpp:309-352
+    o = Objs(lib, m=1000, n=800, nnz=16000)
+    st, n_size = o.spmv_size()
+    assert st == 0 and n_size >= 128 and n_size % 128 == 0
+    assert o.spmv_size(h=None)[0] == api.STATUS_NOT_INITIALIZED
+    assert o.spmv_size(out=False)[0] == api.STATUS_INVALID_VALUE
+    assert o.spmv_size(A=None)[0] == api.STATUS_INVALID_VALUE
+    assert o.spmv_size(op=api.OP_T)[0] == api.STATUS_INVALID_VALUE
+    st, t_size = o.spmv_size(op=api.OP_T, x="y", y="x")
+    assert st == 0 and t_size % 128 == 0
+    # the transpose needs room for A^T (n+1+nnz indices, nnz values) on top of the sort scratch
+    assert t_size >= (800 + 1 + 16000) * 4 + 16000 * 4
+    bigger = Objs(lib, m=1000, n=800, nnz=32000)
+    assert bigger.spmv_size(op=api.OP_T, x="y", y="x")[1] > t_size  # monotone in nnz
+    csc = Objs(lib, m=1000, n=800, nnz=16000, fmt=api.FORMAT_CSC)
+    assert csc.spmv_size()[1] > csc.spmv_size(op=api.OP_T, x="y", y="x")[1]  # CSC op N is the transposing case
+
+
+def test_spmm_argument_checks(lib):
+    # level3/spmm/mcsp_spmm_gpu.cpp:785-807, :105-108, :309-342
+    o = Objs(lib, m=8, n=6, nnz=20)
+    B, C, Bt, Cbad = (ctypes.c_void_p() for _ in range(4))
+    lib.mcsparseCreateDnMat(ctypes.byref(B), 6, 4, 4, FAKE, api.R_32F, api.ORDER_ROW)
+    lib.mcsparseCreateDnMat(ctypes.byref(C), 8, 4, 4, FAKE, api.R_32F, api.ORDER_ROW)
+    lib.mcsparseCreateDnMat(ctypes.byref(Bt), 4, 6, 6, FAKE, api.R_32F, api.ORDER_ROW)
+    lib.mcsparseCreateDnMat(ctypes.byref(Cbad), 7, 4, 4, FAKE, api.R_32F, api.ORDER_ROW)
+    call = lambda h=o.h, opA=0, opB=0, a=o.pa, A=o.A, b=B, be=o.pa, c=C, ct=api.R_32F, buf=FAKE: lib.mcsparseSpMM(
+        h, opA, opB, a, A, b, be, c, ct, 0, buf)
+    assert call(h=None) == api.STATUS_NOT_INITIALIZED
+    for kw in ({"a": None}, {"A": None}, {"b": None}, {"be": None}, {"c": None}, {"buf": None}):
+        assert call(**kw) == api.STATUS_INVALID_VALUE, kw
+    assert call(opA=api.OP_T) == api.STATUS_NOT_SUPPORTED  # CSR op(A) != N (:105-108)
+    assert call(ct=api.R_64F) == api.STATUS_NOT_SUPPORTED
+    assert call(c=Cbad) == api.STATUS_INVALID_VALUE  # C rows != A rows
+    assert call(b=Bt) == api.STATUS_INVALID_VALUE  # B is 4 x 6 but op(B) must be 6 x 4
+    size = ctypes.c_size_t()
+    assert lib.mcsparseSpMM_bufferSize(o.h, 0, 0, o.pa, o.A, B, o.pa, C, api.R_32F, 0, ctypes.byref(size)) == 0
+    assert size.value == 128
+    assert lib.mcsparseSpMM_bufferSize(None, 0, 0, o.pa, o.A, B, o.pa, C, api.R_32F, 0, ctypes.byref(size)) == 1
+    assert lib.mcsparseSpMM_bufferSize(o.h, 0, 0, o.pa, o.A, None, o.pa, C, api.R_32F, 0, ctypes.byref(size)) == 3
+    assert lib.mcsparseSpMM_preprocess(o.h, 0, 0, o.pa, o.A, B, o.pa, C, api.R_32F, 0, FAKE) == 0  # no-op (:965-970)
+    # nnz == 0 with beta == 1 returns before any launch (:110-114)
+    e = Objs(lib, m=8, n=6, nnz=0)
+    assert lib.mcsparseSpMM(e.h, 0, 0, e.pa, e.A, B, e.pa, C, api.R_32F, 0, FAKE) == 0
+
+
+def test_conversion_argument_checks(lib):
+    # conversion/mcsp_coo2csr.cpp:7-59, mcsp_csr2csc.cpp:9-63, :293-310
+    h = ctypes.c_void_p()
+    lib.mcsparseCreate(ctypes.byref(h))
+    assert lib.mcsparseXcsr2coo(None, FAKE, 5, 3, FAKE, 0) == api.STATUS_NOT_INITIALIZED
+    assert lib.mcsparseXcsr2coo(h, FAKE, 0, 3, FAKE, 0) == 0  # nnz == 0: nothing to do
+    assert lib.mcsparseXcsr2coo(h, None, 0, 3, None, 0) == 0  # ... tested before the pointers
+    assert lib.mcsparseXcsr2coo(h, None, 5, 3, FAKE, 0) == api.STATUS_INVALID_VALUE
+    assert lib.mcsparseXcsr2coo(h, FAKE, 5, 3, None, 0) == api.STATUS_INVALID_VALUE
+    assert lib.mcsparseXcoo2csr(None, FAKE, 5, 3, FAKE, 0) == api.STATUS_NOT_INITIALIZED
+    assert lib.mcsparseXcoo2csr(h, FAKE, 0, 3, FAKE, 0) == 0
+    assert lib.mcsparseXcoo2csr(h, None, 5, 3, FAKE, 0) == api.STATUS_INVALID_VALUE
+    size = ctypes.c_size_t()
+    bs = lambda hh=h, m=4, n=5, nnz=9, out=ctypes.byref(size): lib.mcsparseCsr2cscEx2_bufferSize(
+        hh, m, n, nnz, FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, api.R_32F, 1, 0, 1, out)
+    assert bs(hh=None) == api.STATUS_NOT_INITIALIZED
+    assert bs(out=None) == api.STATUS_INVALID_VALUE
+    assert bs(nnz=0) == 0 and size.value == 128
+    assert bs() == 0 and size.value >= 128
+    small = size.value
+    assert bs(nnz=9000) == 0 and size.value > small
+    cv = lambda hh=h, m=4, n=5, nnz=9, vt=api.R_32F, val=FAKE, buf=FAKE, act=1: lib.mcsparseCsr2cscEx2(
+        hh, m, n, nnz, val, FAKE, FAKE, FAKE, FAKE, FAKE, vt, act, 0, 1, buf)
+    assert cv(vt=api.R_16F) == api.STATUS_INVALID_VALUE  # type switch comes first (:297-309)
+    assert cv(hh=None) == api.STATUS_NOT_INITIALIZED
+    assert cv(nnz=0) == 0 and cv(m=0) == 0 and cv(n=0) == 0  # early success, outputs untouched (:56-58)
+    assert cv(val=None) == api.STATUS_INVALID_VALUE
+    assert cv(val=None, act=0) == api.STATUS_INVALID_VALUE  # values required even for SYMBOLIC (:60-63)
+    assert cv(buf=None) == api.STATUS_INVALID_VALUE
+    assert lib.mcsparseXcsrRowBins(None, 3, FAKE, 0, None, FAKE) == api.STATUS_NOT_INITIALIZED
+    assert lib.mcsparseXcsrRowBins(h, 3, None, 0, None, FAKE) == api.STATUS_INVALID_VALUE
+    assert lib.mcsparseXcsrRowBins(h, 3, FAKE, 0, None, None) == api.STATUS_INVALID_VALUE
+
+
+def test_plan_override_api(lib):
+    o = Objs(lib)
+    fam, lanes = ctypes.c_int(-1), ctypes.c_int(-1)
+    assert lib.mcsparseSpMatGetSpMVPlan(o.A, ctypes.byref(fam), ctypes.byref(lanes)) == 0
+    assert (fam.value, lanes.value) == (0, 0)  # nothing analysed yet
+    assert lib.mcsparseSpMatSetSpMVPlan(o.A, 3, 0) == api.STATUS_INVALID_VALUE
+    assert lib.mcsparseSpMatSetSpMVPlan(o.A, 1, 3) == api.STATUS_INVALID_VALUE  # lanes must be a power of two
+    assert lib.mcsparseSpMatSetSpMVPlan(o.A, 1, 16) == 0
+    assert lib.mcsparseSpMatSetSpMVPlan(None, 1, 16) == api.STATUS_INVALID_VALUE

@@ -1,0 +1,148 @@
+"""GPU parity of the index conversions (through the C ABI): bit-exact against the CPU oracle."""
+import glob
+import os
+
+import numpy as np
+import pytest
+
+from mcsparse_amd import api
+from mcsparse_amd import workloads as wl
+
+from gpu_util import dev
+
+pytestmark = pytest.mark.gpu
+
+GOLDEN = sorted(glob.glob(os.path.join(os.path.dirname(__file__), "golden", "csr_*.npz")))
+
+
+def gpu_csr2coo(torch, handle, a):
+    d_ptr = dev(torch, a.ptr)
+    d_out = torch.full((max(a.nnz, 1),), -7, dtype=torch.int32, device="cuda")
+    st = api.xcsr2coo(handle, d_ptr, a.nnz, a.m, d_out, a.base)
+    torch.cuda.synchronize()
+    return st, d_out.cpu().numpy()[:a.nnz]
+
+
+def gpu_coo2csr(torch, handle, coo, nnz, m, base):
+    d_coo = dev(torch, coo)
+    d_out = torch.full((m + 1,), -7, dtype=torch.int32, device="cuda")
+    st = api.xcoo2csr(handle, d_coo, nnz, m, d_out, base)
+    torch.cuda.synchronize()
+    return st, d_out.cpu().numpy()
+
+
+def gpu_csr2csc(torch, handle, a, action=api.ACTION_NUMERIC):
+    d_ptr, d_col, d_val = dev(torch, a.ptr), dev(torch, a.col), dev(torch, a.val)
+    vt = api.maca_type(a.val.dtype)
+    o_val = torch.zeros_like(d_val)
+    o_ptr = torch.full((a.n + 1,), -7, dtype=torch.int32, device="cuda")
+    o_row = torch.full((max(a.nnz, 1),), -7, dtype=torch.int32, device="cuda")
+    st, size = api.csr2csc_buffer_size(handle, a.m, a.n, a.nnz, d_val, d_ptr, d_col, o_val, o_ptr, o_row, vt, action,
+                                       a.base)
+    assert st == 0 and size >= 128
+    buf = torch.empty(size, dtype=torch.uint8, device="cuda")
+    st = api.csr2csc(handle, a.m, a.n, a.nnz, d_val, d_ptr, d_col, o_val, o_ptr, o_row, vt, action, a.base, buf)
+    torch.cuda.synchronize()
+    return st, o_ptr.cpu().numpy(), o_row.cpu().numpy()[:a.nnz], o_val.cpu().numpy()
+
+
+def check_csr2csc(torch, handle, oracle, a, what):
+    st, cp, ri, cv = gpu_csr2csc(torch, handle, a)
+    assert st == 0
+    w_cp, w_ri, w_cv = oracle.csr2csc(a.m, a.n, a.base, a.ptr, a.col, a.val, method="counting")
+    assert np.array_equal(cp.view(np.uint32), w_cp), what + ": col_ptr"
+    assert np.array_equal(ri.view(np.uint32), w_ri), what + ": row_ind"
+    assert np.array_equal(cv.view(np.uint8), w_cv.view(np.uint8)), what + ": values"
+    return cp, ri, cv
+
+
+CASES = {
+    "ragged_f32": lambda: wl.random_ragged(5003, 4099, 23, dtype=np.float32, seed=1),
+    "ragged_f64_base1": lambda: wl.random_ragged(5003, 4099, 23, dtype=np.float64, seed=2).with_base(1),
+    "wide": lambda: wl.random_ragged(300, 100000, 3, dtype=np.float32, seed=3),
+    "tall_sparse": lambda: wl.random_ragged(100000, 300, 0.4, dtype=np.float32, seed=4),
+    "one_by_one": lambda: wl.random_ragged(1, 1, 1, dtype=np.float64, seed=5, empty_fraction=0.0),
+    "power_law": lambda: wl.power_law(m=1 << 16, max_len=30000, dtype=np.float32),
+    "power_law_base1_f64": lambda: wl.power_law(m=1 << 14, max_len=9000, dtype=np.float64).with_base(1),
+    "n_pow2": lambda: wl.random_ragged(4096, 65536, 20, dtype=np.float32, seed=6),
+    "n_pow2_minus1_base1": lambda: wl.random_ragged(4096, 65535, 20, dtype=np.float32, seed=7).with_base(1),
+    "n_small": lambda: wl.random_ragged(70000, 3, 2, dtype=np.float32, seed=8),
+    "stencil": lambda: wl.stencil_27pt(20, dtype=np.float32),
+}
+
+
+@pytest.mark.parametrize("name", list(CASES))
+def test_conversions_bit_exact(torch_gpu, handle, oracle, name):
+    a = CASES[name]()
+    if a.nnz == 0:
+        pytest.skip("empty draw")
+    st, coo = gpu_csr2coo(torch_gpu, handle, a)
+    assert st == 0
+    want = oracle.csr2coo(a.m, a.base, a.ptr, a.nnz)
+    assert np.array_equal(coo.view(np.uint32), want), name + ": csr2coo"
+    st, back = gpu_coo2csr(torch_gpu, handle, coo, a.nnz, a.m, a.base)
+    assert st == 0 and np.array_equal(back, a.ptr), name + ": coo2csr"
+    assert np.array_equal(back.view(np.uint32), oracle.coo2csr(a.nnz, a.m, a.base, want))
+    cp, ri, cv = check_csr2csc(torch_gpu, handle, oracle, a, name)
+    assert int(cp[0]) == a.base and int(cp[-1]) - a.base == a.nnz
+    # transposing the result gives the matrix back (sorted, duplicate-free input)
+    t = wl.Csr(a.n, a.m, cp, ri, cv, a.base)
+    st, cp2, ri2, cv2 = gpu_csr2csc(torch_gpu, handle, t)
+    assert st == 0 and np.array_equal(cp2, a.ptr) and np.array_equal(ri2, a.col)
+    assert np.array_equal(cv2.view(np.uint8), a.val.view(np.uint8))
+
+
+def test_csr2csc_symbolic_and_literal_oracle(torch_gpu, handle, oracle):
+    a = wl.random_ragged(3000, 5000, 11, dtype=np.float32, seed=5)
+    st, cp, ri, cv = gpu_csr2csc(torch_gpu, handle, a, action=api.ACTION_SYMBOLIC)
+    w_cp, w_ri, _ = oracle.csr2csc(a.m, a.n, 0, a.ptr, a.col, a.val, method="radix2")
+    assert st == 0 and np.array_equal(cp.view(np.uint32), w_cp) and np.array_equal(ri.view(np.uint32), w_ri)
+    assert not cv.any()  # values are not written for SYMBOLIC
+
+
+def test_csr2csc_keeps_input_order_of_duplicates(torch_gpu, handle, oracle):
+    # unsorted columns with repeated (row, col) pairs: a stable sort keeps them in input order
+    rng = np.random.default_rng(9)
+    m, n, nnz = 500, 37, 20000
+    lens = rng.multinomial(nnz, np.ones(m) / m)
+    ptr = np.concatenate([[0], np.cumsum(lens)])
+    col = rng.integers(0, n, nnz)
+    val = np.arange(nnz, dtype=np.float64)
+    a = wl.Csr(m, n, ptr, col, val)
+    cp, ri, cv = check_csr2csc(torch_gpu, handle, oracle, a, "duplicates")
+    assert np.array_equal(cv, val[np.argsort(col, kind="stable")])
+
+
+@pytest.mark.parametrize("path", GOLDEN, ids=[os.path.basename(p) for p in GOLDEN])
+def test_golden_conversions(torch_gpu, handle, path):
+    with np.load(path) as z:
+        g = {k: z[k] for k in z.files}
+    for base in (0, 1):
+        a = wl.Csr(int(g["m"]), int(g["n"]), g["ptr"] + base, g["col"] + base, g["val"], base)
+        st, cp, ri, cv = gpu_csr2csc(torch_gpu, handle, a)
+        assert st == 0 and np.array_equal(cp, g["csc_ptr"] + base) and np.array_equal(ri, g["csc_row"] + base)
+        assert np.array_equal(cv, g["csc_val"])
+        st, coo = gpu_csr2coo(torch_gpu, handle, a)
+        assert st == 0 and np.array_equal(coo, g["coo_row"] + base)
+
+
+def test_empty_inputs_leave_outputs_untouched(torch_gpu, handle):
+    # nnz == 0 returns before any work in the reference (mcsp_coo2csr.cpp:14-16, mcsp_csr2csc.cpp:56-58)
+    a = wl.Csr(5, 4, np.zeros(6, np.int32), np.zeros(0, np.int32), np.zeros(0, np.float32))
+    st, cp, ri, cv = gpu_csr2csc(torch_gpu, handle, a)
+    assert st == 0 and (cp == -7).all()
+    st, back = gpu_coo2csr(torch_gpu, handle, np.zeros(1, np.int32), 0, 5, 0)
+    assert st == 0 and (back == -7).all()
+
+
+@pytest.mark.parametrize("name", ["ragged_f32", "power_law", "tall_sparse", "one_by_one"])
+def test_row_bins_bit_exact(torch_gpu, handle, oracle, name):
+    a = CASES[name]()
+    d_ptr = dev(torch_gpu, a.ptr)
+    d_bins = torch_gpu.full((a.m,), 255, dtype=torch_gpu.uint8, device="cuda")
+    d_hist = torch_gpu.full((34,), 12345, dtype=torch_gpu.int32, device="cuda")
+    assert api.csr_row_bins(handle, a.m, d_ptr, a.base, d_bins, d_hist) == 0
+    torch_gpu.cuda.synchronize()
+    bins, hist = oracle.row_bins(a.m, a.ptr)
+    assert np.array_equal(d_bins.cpu().numpy(), bins)
+    assert np.array_equal(d_hist.cpu().numpy().view(np.uint32), hist)

@@ -1,0 +1,182 @@
+"""Pins the CPU oracle (oracle/oracle.c) without the reference, which ships no vectors:
+golden fixtures from scipy (tests/golden), dense brute force, closed forms and round trips,
+chosen so that a dropped term, wrong sign, shifted index or transposed operand fails."""
+import glob
+import os
+
+import numpy as np
+import pytest
+import scipy.sparse as sp
+
+from mcsparse_amd import workloads as wl
+
+GOLDEN = sorted(glob.glob(os.path.join(os.path.dirname(__file__), "golden", "csr_*.npz")))
+
+
+def load(path):
+    with np.load(path) as z:
+        return {k: z[k] for k in z.files}
+
+
+@pytest.mark.parametrize("path", GOLDEN, ids=[os.path.basename(p) for p in GOLDEN])
+@pytest.mark.parametrize("base", [0, 1])
+def test_golden_spmv_spmm(oracle, path, base):
+    g = load(path)
+    m, n = int(g["m"]), int(g["n"])
+    ptr, col = g["ptr"] + base, g["col"] + base
+    alpha, beta = float(g["alpha"]), float(g["beta"])
+    for dtype in (np.float64, np.float32):  # integer data: exact in both
+        val = g["val"].astype(dtype)
+        y, bound = oracle.spmv(False, m, n, base, ptr, col, val, alpha, beta, g["x"].astype(dtype),
+                               g["y0"].astype(dtype))
+        assert np.array_equal(y.astype(np.float64), g["y_n"])
+        assert (bound >= np.abs(y)).all()
+        yt, _ = oracle.spmv(True, m, n, base, ptr, col, val, alpha, 0.0, g["xt"].astype(dtype), None)
+        assert np.array_equal(yt.astype(np.float64), g["y_t"])
+        B, C0 = g["B"].astype(dtype), g["C0"].astype(dtype)
+        for b_row in (True, False):
+            for c_row in (True, False):
+                Bm = B if b_row else np.asfortranarray(B)
+                Cm = C0 if c_row else np.asfortranarray(C0)
+                ldb = B.shape[1] if b_row else B.shape[0]
+                ldc = C0.shape[1] if c_row else C0.shape[0]
+                Bflat = Bm.ravel(order="C" if b_row else "F")
+                Cflat = Cm.ravel(order="C" if c_row else "F")
+                c, _ = oracle.spmm(m, B.shape[1], base, ptr, col, val, alpha, beta, Bflat, ldb, b_row, Cflat, ldc,
+                                   c_row)
+                assert np.array_equal(c.astype(np.float64), g["C"])
+
+
+@pytest.mark.parametrize("path", GOLDEN, ids=[os.path.basename(p) for p in GOLDEN])
+@pytest.mark.parametrize("base", [0, 1])
+@pytest.mark.parametrize("method", ["radix2", "counting"])
+def test_golden_conversions(oracle, path, base, method):
+    g = load(path)
+    m, n = int(g["m"]), int(g["n"])
+    ptr, col = g["ptr"] + base, g["col"] + base
+    nnz = col.shape[0]
+    cp, ri, cv = oracle.csr2csc(m, n, base, ptr, col, g["val"], method=method)
+    assert np.array_equal(cp.astype(np.int64), g["csc_ptr"].astype(np.int64) + base)
+    assert np.array_equal(ri.astype(np.int64), g["csc_row"].astype(np.int64) + base)
+    assert np.array_equal(cv, g["csc_val"])
+    cp2, ri2, none = oracle.csr2csc(m, n, base, ptr, col, None, method=method)
+    assert none is None and np.array_equal(cp2, cp) and np.array_equal(ri2, ri)
+    coo = oracle.csr2coo(m, base, ptr, nnz)
+    assert np.array_equal(coo.astype(np.int64), g["coo_row"].astype(np.int64) + base)
+    back = oracle.coo2csr(nnz, m, base, coo)
+    assert np.array_equal(back.astype(np.int64), ptr.astype(np.int64))
+
+
+def test_spmv_dense_bruteforce_and_float_bound(oracle):
+    rng = np.random.default_rng(7)
+    for dtype in (np.float32, np.float64):
+        a = wl.random_ragged(48, 61, 9, dtype=dtype, seed=3)
+        A = a.to_scipy().toarray().astype(np.longdouble)
+        x = rng.uniform(-1, 1, a.n).astype(dtype)
+        y0 = rng.uniform(-1, 1, a.m).astype(dtype)
+        y, bound = oracle.spmv(False, a.m, a.n, 0, a.ptr, a.col, a.val, 1.5, 0.5, x, y0)
+        want = np.longdouble(0.5) * y0.astype(np.longdouble) + np.longdouble(1.5) * (A @ x.astype(np.longdouble))
+        assert np.max(np.abs(y - want)) <= 1e-17 * max(1.0, float(np.max(np.abs(want))))
+        wb = 1.5 * (np.abs(A) @ np.abs(x.astype(np.longdouble))) + np.abs(0.5 * y0.astype(np.longdouble))
+        assert np.allclose(bound.astype(np.float64), wb.astype(np.float64), rtol=1e-15)
+        # transposed operand would fail here: non-square, and A^T y pairing
+        xt = rng.uniform(-1, 1, a.m).astype(dtype)
+        yt, _ = oracle.spmv(True, a.m, a.n, 0, a.ptr, a.col, a.val, 1.0, 0.0, xt, None)
+        assert np.max(np.abs(yt - A.T @ xt.astype(np.longdouble))) <= 1e-17
+        # y^T (A x) == (A^T y)^T x
+        ax, _ = oracle.spmv(False, a.m, a.n, 0, a.ptr, a.col, a.val, 1.0, 0.0, x, None)
+        lhs = np.dot(xt.astype(np.longdouble), ax)
+        rhs = np.dot(yt, x.astype(np.longdouble))
+        assert abs(lhs - rhs) <= 1e-16 * max(1.0, abs(float(lhs)))
+
+
+def test_spmv_closed_forms(oracle):
+    # identity and diagonal
+    n = 33
+    ptr = np.arange(n + 1, dtype=np.int32)
+    col = np.arange(n, dtype=np.int32)
+    x = np.linspace(-2, 2, n)
+    d = np.arange(1, n + 1, dtype=np.float64)
+    y, _ = oracle.spmv(False, n, n, 0, ptr, col, np.ones(n), 1.0, 0.0, x, None)
+    assert np.array_equal(y.astype(np.float64), x)
+    y, _ = oracle.spmv(False, n, n, 0, ptr, col, d, 1.0, 0.0, x, None)
+    assert np.array_equal(y.astype(np.float64), d * x)
+    # alpha = 0 leaves beta*y; beta = 1, alpha = 0 leaves y
+    y0 = np.cos(np.arange(n))
+    y, _ = oracle.spmv(False, n, n, 0, ptr, col, d, 0.0, 2.0, x, y0)
+    assert np.array_equal(y.astype(np.float64), 2.0 * y0)
+    y, _ = oracle.spmv(False, n, n, 0, ptr, col, d, 0.0, 1.0, x, y0)
+    assert np.array_equal(y.astype(np.float64), y0)
+    # 5-point Laplacian times the constant vector: 0 inside, 1 on edges, 2 in corners
+    g = 16
+    lap = wl.laplacian_5pt(g, dtype=np.float32)
+    assert lap.nnz == 5 * g * g - 4 * g
+    y, _ = oracle.spmv(False, lap.m, lap.n, 0, lap.ptr, lap.col, lap.val, 1.0, 0.0, np.ones(lap.n, np.float32), None)
+    yy = y.astype(np.float64).reshape(g, g)
+    assert (yy[1:-1, 1:-1] == 0).all()
+    assert (yy[0, 1:-1] == 1).all() and (yy[-1, 1:-1] == 1).all() and (yy[1:-1, 0] == 1).all()
+    assert yy[0, 0] == 2 and yy[0, -1] == 2 and yy[-1, 0] == 2 and yy[-1, -1] == 2
+    # rows of ones times small integers: exact row sums
+    a = wl.random_ragged(40, 40, 6, dtype=np.float32, seed=1)
+    xi = np.arange(a.n, dtype=np.float32) % 7
+    y, _ = oracle.spmv(False, a.m, a.n, 0, a.ptr, a.col, np.ones(a.nnz, np.float32), 1.0, 0.0, xi, None)
+    want = np.array([xi[a.col[a.ptr[r]:a.ptr[r + 1]]].sum() for r in range(a.m)], dtype=np.float64)
+    assert np.array_equal(y.astype(np.float64), want)
+    # index base does not change the result
+    b1 = a.with_base(1)
+    y1, _ = oracle.spmv(False, a.m, a.n, 1, b1.ptr, b1.col, b1.val, 1.0, 0.0, xi, None)
+    y0_, _ = oracle.spmv(False, a.m, a.n, 0, a.ptr, a.col, a.val, 1.0, 0.0, xi, None)
+    assert np.array_equal(y1, y0_)
+
+
+def test_csr2csc_is_the_stable_sort(oracle):
+    # duplicates of one (row, col) pair must keep their input order: values tell them apart
+    ptr = np.array([0, 4, 4, 7], dtype=np.int32)
+    col = np.array([2, 0, 2, 2, 1, 2, 0], dtype=np.int32)  # unsorted, with repeats
+    val = np.arange(10, 17, dtype=np.float64)
+    for method in ("radix2", "counting"):
+        cp, ri, cv = oracle.csr2csc(3, 3, 0, ptr, col, val, method=method)
+        order = np.argsort(col, kind="stable")
+        assert np.array_equal(cv, val[order])
+        rows = np.array([0, 0, 0, 0, 2, 2, 2])
+        assert np.array_equal(ri, rows[order])
+        assert np.array_equal(cp, [0, 2, 3, 7])
+    # the two oracle variants agree on a larger ragged case with empty rows and columns
+    a = wl.random_ragged(3000, 5000, 11, dtype=np.float32, seed=5)
+    for base in (0, 1):
+        b = a.with_base(base)
+        r1 = oracle.csr2csc(b.m, b.n, base, b.ptr, b.col, b.val, method="radix2")
+        r2 = oracle.csr2csc(b.m, b.n, base, b.ptr, b.col, b.val, method="counting")
+        for u, v in zip(r1, r2):
+            assert np.array_equal(u, v)
+        cp, ri, cv = r1
+        assert int(cp[-1]) - base == b.nnz and int(cp[0]) == base
+        assert np.array_equal(np.sort(cv.view(np.uint32)), np.sort(b.val.view(np.uint32)))  # a permutation
+        s = a.to_scipy().tocsc()
+        assert np.array_equal(cp.astype(np.int64) - base, s.indptr) and np.array_equal(ri.astype(np.int64) - base,
+                                                                                         s.indices)
+        # transposing twice gives the matrix back (sorted, duplicate-free CSR)
+        cp2, ri2, cv2 = oracle.csr2csc(b.n, b.m, base, cp, ri, cv, method="counting")
+        assert np.array_equal(cp2.view(np.int32), b.ptr) and np.array_equal(ri2.view(np.int32), b.col)
+        assert np.array_equal(cv2, b.val)
+
+
+def test_coo_round_trip_with_empty_rows(oracle):
+    for base in (0, 1):
+        ptr = np.array([0, 0, 3, 3, 3, 5, 6, 6], dtype=np.int32) + base
+        coo = oracle.csr2coo(7, base, ptr, 6)
+        assert np.array_equal(coo, np.array([1, 1, 1, 4, 4, 5]) + base)
+        assert np.array_equal(oracle.coo2csr(6, 7, base, coo).view(np.int32), ptr)
+
+
+def test_row_bins_definition(oracle):
+    a = wl.power_law(m=5000, max_len=700, dtype=np.float32)
+    bins, hist = oracle.row_bins(a.m, a.ptr)
+    lens = a.row_lengths()
+    want = np.where(lens == 0, 0, np.floor(np.log2(np.maximum(lens, 1))).astype(np.int64) + 1)
+    assert np.array_equal(bins, want)
+    assert np.array_equal(hist[:33], np.bincount(want, minlength=33))
+    assert hist[33] == lens.max()
+    ptr = np.array([0, 0, 1, 3, 7, 15, 16], dtype=np.int32)  # lengths 0 1 2 4 8 1
+    bins, hist = oracle.row_bins(6, ptr)
+    assert list(bins) == [0, 1, 2, 3, 4, 1] and hist[33] == 8
