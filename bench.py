@@ -38,6 +38,7 @@ def parse():
     p.add_argument("--no-cpu-baseline", action="store_true")
     p.add_argument("--family", type=int, default=0, help="force the SpMV kernel family (1 vector, 2 merge)")
     p.add_argument("--lanes", type=int, default=0, help="force lanes per row of the vector family")
+    p.add_argument("--cache", default=None, help="directory to keep generated matrices in between runs")
     return p.parse_args()
 
 
@@ -75,8 +76,8 @@ def main():
         a = wl.uniform_rows(m=max(64, int((1 << 20) * s)), per_row=16, dtype=np.float64)
         alpha, beta, desc = 1.5, 0.5, "fp64 CSR SpMV, 1048576 rows x 16 nnz/row uniform"
     elif name in ("c3", "c3t", "c5", "c5-coo", "c5-spmv"):
-        a = wl.power_law(m=max(64, int((1 << 22) * s)), max_len=max(8, int(200000 * min(1.0, s * 4))),
-                         dtype=np.float32)
+        a = cached(args.cache, "power_law_%g" % s, lambda: wl.power_law(
+            m=max(64, int((1 << 22) * s)), max_len=max(8, int(200000 * min(1.0, s * 4))), dtype=np.float32))
         alpha, beta = 1.0, 0.0
         desc = "fp32 CSR SpMV, 4194304 rows power-law (Zipf 1.8, <=200000 nnz/row)"
         if name == "c3t":
@@ -252,6 +253,21 @@ def main():
         out["cpu_baseline"] = cpu_baseline(kind, a, alpha, beta, n_cols, algo_bytes, op)
     print(json.dumps(out))
     return 0
+
+
+def cached(directory, key, make):
+    """Generated matrices are deterministic; keeping them on disk only saves generation time."""
+    from mcsparse_amd import workloads as wl
+    if not directory:
+        return make()
+    path = os.path.join(directory, key + ".npz")
+    if os.path.exists(path):
+        with np.load(path) as z:
+            return wl.Csr(int(z["m"]), int(z["n"]), z["ptr"], z["col"], z["val"], int(z["base"]))
+    a = make()
+    os.makedirs(directory, exist_ok=True)
+    np.savez(path, m=a.m, n=a.n, ptr=a.ptr, col=a.col, val=a.val, base=a.base)
+    return a
 
 
 def cpu_baseline(kind, a, alpha, beta, n_cols, algo_bytes, op):
