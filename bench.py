@@ -26,6 +26,13 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 
+# HBM/fabric bytes per launch of the dominant kernel, from rocprofv3 FETCH_SIZE and WRITE_SIZE
+# (each scaled by what the same counter reads on a 1 GiB copy: 2 KiB and 1 KiB per count).
+# The counter summaries are kept under profiles/.
+MEASURED_TRAFFIC_BYTES = {
+    "c2": int((654222.0 * 2 + 10263.5 * 1) * 1024),
+}
+
 
 def parse():
     p = argparse.ArgumentParser()
@@ -94,6 +101,10 @@ def main():
         a = wl.stencil_27pt(max(4, int(round(128 * s ** (1 / 3)))), dtype=np.float32)
         alpha, beta, kind = 1.0, 0.0, "spmm"
         desc = "fp32 CSR SpMM, 27-pt stencil 128^3, B row-major N=%d" % n_cols
+    elif name == "copy":
+        # plain device copy of known size: the yardstick the rocprofv3 FETCH_SIZE / WRITE_SIZE
+        # counters are scaled by
+        return copy_probe(torch, args)
     else:
         print("unknown workload %r" % name, file=sys.stderr)
         return 2
@@ -246,12 +257,29 @@ def main():
                                "min": round(float(dev_ms.min()), 5)},
         "spmv_plan": {"family": plan[0], "lanes_per_row": plan[1]} if plan else None,
         "roofline": {"bound": "hbm", "achieved": round(achieved, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None},
+                     "frac": round(achieved / HBM_PEAK_GBS, 4),
+                     "traffic": MEASURED_TRAFFIC_BYTES.get(name) if s == 1.0 else None},
     }
 
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(kind, a, alpha, beta, n_cols, algo_bytes, op)
     print(json.dumps(out))
+    return 0
+
+
+def copy_probe(torch, args):
+    n = 1 << 28  # 1 GiB of fp32 read, 1 GiB written per step
+    src = torch.ones(n, dtype=torch.float32, device="cuda")
+    dst = torch.zeros(n, dtype=torch.float32, device="cuda")
+    steps = args.steps or 10
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        dst.copy_(src)
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / steps
+    print(json.dumps({"workload": "copy", "bytes_read_per_step": 4 * n, "bytes_written_per_step": 4 * n,
+                      "steps": steps, "ms_per_step": round(ms, 4), "GBps": round(8 * n / ms / 1e6, 1)}))
     return 0
 
 
