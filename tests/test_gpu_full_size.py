@@ -1,0 +1,84 @@
+"""Parity at the full sizes of the benchmark configurations (config 2 is in test_gpu_spmv.py).
+
+The CPU oracle is plain C and finishes these sizes in seconds, so SpMV and the conversions are
+compared with it directly; SpMM is compared on a sample of rows (the oracle's long-double triple
+loop over 2 M rows x 64 columns would take minutes) plus a linearity property over all rows."""
+import numpy as np
+import pytest
+
+from mcsparse_amd import api
+from mcsparse_amd import workloads as wl
+
+from gpu_util import assert_within, dev, run_spmv
+from test_gpu_convert import gpu_csr2coo, gpu_csr2csc
+from test_gpu_spmm import run_spmm
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def power_law_full():
+    a = wl.power_law(m=1 << 22, max_len=200000, dtype=np.float32)
+    assert a.m == 4194304 and a.nnz > 100_000_000 and a.row_lengths().max() > 100_000
+    return a
+
+
+def test_config3_power_law_full_size(torch_gpu, handle, oracle, power_law_full):
+    a = power_law_full
+    rng = np.random.default_rng(3)
+    x = rng.uniform(-1, 1, a.n).astype(np.float32)
+    st, y, plan = run_spmv(torch_gpu, handle, a, x, np.zeros(a.m, np.float32), 1.0, 0.0)
+    assert st == 0 and plan[0] == api.FAMILY_MERGE
+    y_ref, bound = oracle.spmv(False, a.m, a.n, 0, a.ptr, a.col, a.val, 1.0, 0.0, x, None)
+    worst = assert_within(y, y_ref, bound, np.float32, what="C3 op N")
+    # op T through the library's own transposition
+    xt = rng.uniform(-1, 1, a.m).astype(np.float32)
+    st, yt, _ = run_spmv(torch_gpu, handle, a, xt, np.zeros(a.n, np.float32), 1.0, 0.0, op=api.OP_T)
+    assert st == 0
+    yt_ref, bound_t = oracle.spmv(True, a.m, a.n, 0, a.ptr, a.col, a.val, 1.0, 0.0, xt, None)
+    assert_within(yt, yt_ref, bound_t, np.float32, what="C3 op T")
+
+
+def test_config5_conversions_full_size(torch_gpu, handle, oracle, power_law_full):
+    a = power_law_full
+    st, coo = gpu_csr2coo(torch_gpu, handle, a)
+    assert st == 0 and np.array_equal(coo.view(np.uint32), oracle.csr2coo(a.m, 0, a.ptr, a.nnz))
+    del coo
+    st, cp, ri, cv = gpu_csr2csc(torch_gpu, handle, a)
+    assert st == 0
+    w_cp, w_ri, w_cv = oracle.csr2csc(a.m, a.n, 0, a.ptr, a.col, a.val, method="counting")
+    assert np.array_equal(cp.view(np.uint32), w_cp)
+    assert np.array_equal(ri.view(np.uint32), w_ri)
+    assert np.array_equal(cv.view(np.uint32), w_cv.view(np.uint32))
+    # transposed SpMV from the produced CSC (descriptor of A in CSC format, op T -> direct kernel)
+    rng = np.random.default_rng(5)
+    xt = rng.uniform(-1, 1, a.m).astype(np.float32)
+    csc_as_csr = wl.Csr(a.n, a.m, cp, ri, cv)  # arrays of A^T in CSR form
+    st, yt, plan = run_spmv(torch_gpu, handle, csc_as_csr, xt, np.zeros(a.n, np.float32), 1.0, 0.0, op=api.OP_T,
+                            fmt=api.FORMAT_CSC)
+    assert st == 0 and plan[0] == api.FAMILY_VECTOR
+    yt_ref, bound_t = oracle.spmv(True, a.m, a.n, 0, a.ptr, a.col, a.val, 1.0, 0.0, xt, None)
+    assert_within(yt, yt_ref, bound_t, np.float32, what="C5 A^T x from CSC")
+
+
+@pytest.mark.parametrize("n", [8, 64, 256])
+def test_config4_stencil_full_size(torch_gpu, handle, oracle, n):
+    a = wl.stencil_27pt(128, dtype=np.float32)
+    assert (a.m, a.nnz) == (2097152, 55742968)
+    rng = np.random.default_rng(n)
+    B = rng.uniform(-1, 1, (a.n, n)).astype(np.float32)
+    st, got, _ = run_spmm(torch_gpu, handle, a, B, np.zeros((a.m, n), np.float32), 1.0, 0.0)
+    assert st == 0
+    # oracle on a sample of rows: first/last planes, and random interior rows
+    rows = np.unique(np.concatenate([np.arange(0, 300), np.arange(a.m - 300, a.m),
+                                     rng.integers(0, a.m, 1500)]))
+    lens = a.row_lengths()[rows]
+    sub_ptr = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    take = np.concatenate([np.arange(a.ptr[r], a.ptr[r + 1]) for r in rows])
+    c_ref, bound = oracle.spmm(len(rows), n, 0, sub_ptr, a.col[take], a.val[take], 1.0, 0.0, B.ravel(), n, True, None,
+                               n, True)
+    assert_within(np.ascontiguousarray(got[rows]), c_ref, bound, np.float32, what="C4 N=%d sample" % n)
+    # all rows: column j of C equals the SpMV of A with column j of B (checked for two columns)
+    for j in (0, n - 1):
+        y_ref, bnd = oracle.spmv(False, a.m, a.n, 0, a.ptr, a.col, a.val, 1.0, 0.0, np.ascontiguousarray(B[:, j]), None)
+        assert_within(np.ascontiguousarray(got[:, j]), y_ref, bnd, np.float32, what="C4 N=%d column %d" % (n, j))
