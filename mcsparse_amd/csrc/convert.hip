@@ -113,17 +113,26 @@ __global__ __launch_bounds__(kBlock) void csr2coo_kernel(idx_t m, idx_t nnz, idx
     for (idx_t k = tid; k < tile_nnz; k += kBlock) coo_rows[y0 + k] = s_ids[k];
 }
 
-// Offsets from sorted row indices: thread t fills the offsets of the rows that lie between
-// entry t-1 and entry t, so empty rows are covered.
+// Offsets from sorted row indices: boundary t (between entry t-1 and entry t, 0 <= t <= nnz) fills
+// the offsets of the rows that lie in between, so empty rows are covered.  Each thread takes four
+// consecutive boundaries and reads its entries once.
 // Reference semantics: src/kernels/conversion/coo2csr_device.hpp:8-24.
+constexpr int kCooPerThread = 4;
 __global__ __launch_bounds__(kBlock) void coo2csr_kernel(idx_t nnz, idx_t m, idx_t base,
                                                          const idx_t* __restrict__ coo_rows,
                                                          idx_t* __restrict__ row_ptr) {
-    const uint64_t t = static_cast<uint64_t>(blockIdx.x) * kBlock + threadIdx.x;
-    if (t > nnz) return;
-    const uint64_t first = t == 0 ? 0 : static_cast<uint64_t>(coo_rows[t - 1] - base) + 1;
-    const uint64_t last = t == nnz ? static_cast<uint64_t>(m) + 1 : static_cast<uint64_t>(coo_rows[t] - base) + 1;
-    for (uint64_t i = first; i < last; ++i) row_ptr[i] = static_cast<idx_t>(t) + base;
+    const uint64_t t0 = (static_cast<uint64_t>(blockIdx.x) * kBlock + threadIdx.x) * kCooPerThread;
+    if (t0 > nnz) return;
+    // row (0-based, +1) of the entry before boundary t0; 0 in front of the first entry
+    uint64_t prev = t0 == 0 ? 0 : static_cast<uint64_t>(coo_rows[t0 - 1] - base) + 1;
+#pragma unroll
+    for (int e = 0; e < kCooPerThread; ++e) {
+        const uint64_t t = t0 + e;
+        if (t > nnz) break;
+        const uint64_t cur = t == nnz ? static_cast<uint64_t>(m) + 1 : static_cast<uint64_t>(coo_rows[t] - base) + 1;
+        for (uint64_t i = prev; i < cur; ++i) row_ptr[i] = static_cast<idx_t>(t) + base;
+        prev = cur;
+    }
 }
 
 // ------------------------------------------------------------------------------------------
@@ -221,16 +230,22 @@ void launch_exclusive_scan(hipStream_t stream, uint32_t* data, uint64_t n, uint3
 // ------------------------------------------------------------------------------------------
 // one stable LSD radix pass over (key, row, value) triples
 // ------------------------------------------------------------------------------------------
-constexpr int kSortIpt = 16;
-constexpr int kSortTile = kBlock * kSortIpt;          // 4096 triples per workgroup
-constexpr int kSortWaves = kBlock / kWave;            // 4
-constexpr int kSortWaveItems = kWave * kSortIpt;      // each wave owns 1024 consecutive triples
+constexpr int kSortBlock = 1024;                       // threads per tile: many waves hide the barriers
+constexpr int kSortIpt = 4;
+constexpr int kSortTile = kSortBlock * kSortIpt;       // 4096 triples per workgroup
+constexpr int kSortWaves = kSortBlock / kWave;         // 16
+constexpr int kSortWaveItems = kWave * kSortIpt;       // each wave owns 256 consecutive triples
 constexpr int kMaxRadix = 256;
+constexpr uint32_t kXcds = 8;                          // accelerator complex dies of an MI355X
+static_assert(kSortBlock >= kMaxRadix, "one thread per digit");
 
-// counters[digit * tiles + tile] = how many keys of `tile` carry `digit`.
-__global__ __launch_bounds__(kBlock) void radix_hist_kernel(const idx_t* __restrict__ keys, idx_t count,
-                                                            uint32_t shift, uint32_t bits, uint32_t tiles,
-                                                            uint32_t* __restrict__ counters) {
+// counters[digit * tiles + tile] = how many keys of `tile` carry `digit`.  256 threads, 16 keys
+// each, read as four 128-bit loads (tiles start at multiples of 4096 keys, so they are aligned).
+constexpr int kHistBlock = 256;
+__global__ __launch_bounds__(kHistBlock) void radix_hist_kernel(const idx_t* __restrict__ keys, idx_t count,
+                                                                uint32_t shift, uint32_t bits, uint32_t tiles,
+                                                                uint32_t* __restrict__ counters) {
+    typedef idx_t idx4 __attribute__((ext_vector_type(4)));
     __shared__ uint32_t s_cnt[kMaxRadix];
     const uint32_t radix = 1u << bits;
     const uint32_t mask = radix - 1;
@@ -238,12 +253,38 @@ __global__ __launch_bounds__(kBlock) void radix_hist_kernel(const idx_t* __restr
     __syncthreads();
     const uint64_t start = static_cast<uint64_t>(blockIdx.x) * kSortTile;
 #pragma unroll
-    for (int i = 0; i < kSortIpt; ++i) {
-        const uint64_t p = start + static_cast<uint64_t>(i) * kBlock + threadIdx.x;
-        if (p < count) atomicAdd(&s_cnt[(keys[p] >> shift) & mask], 1u);
+    for (int i = 0; i < kSortTile / (kHistBlock * 4); ++i) {
+        const uint64_t p = start + (static_cast<uint64_t>(i) * kHistBlock + threadIdx.x) * 4;
+        if (p + 4 <= count) {
+            const idx4 k = __builtin_nontemporal_load(reinterpret_cast<const idx4*>(keys + p));
+#pragma unroll
+            for (int e = 0; e < 4; ++e) atomicAdd(&s_cnt[(k[e] >> shift) & mask], 1u);
+        } else {
+            for (uint64_t q = p; q < count; ++q) atomicAdd(&s_cnt[(keys[q] >> shift) & mask], 1u);
+        }
     }
     __syncthreads();
     if (threadIdx.x < radix) counters[static_cast<uint64_t>(threadIdx.x) * tiles + blockIdx.x] = s_cnt[threadIdx.x];
+}
+
+// Exclusive scan over the kSortBlock threads of the scatter kernel.
+__device__ __forceinline__ uint32_t sort_block_exclusive_scan(uint32_t v, uint32_t* s_wave) {
+    const unsigned lane = threadIdx.x % kWave;
+    const unsigned wave = threadIdx.x / kWave;
+    uint32_t inc = v;
+#pragma unroll
+    for (int off = 1; off < kWave; off <<= 1) {
+        const uint32_t up = __shfl_up(inc, off, kWave);
+        if (lane >= static_cast<unsigned>(off)) inc += up;
+    }
+    if (lane == kWave - 1) s_wave[wave] = inc;
+    __syncthreads();
+    uint32_t wave_off = 0;
+#pragma unroll
+    for (unsigned w = 0; w < kSortWaves; ++w) {
+        if (w < wave) wave_off += s_wave[w];
+    }
+    return wave_off + inc - v;
 }
 
 // VB = bytes per value (0 = no values).  counters hold, after the exclusive scan, the output
@@ -254,7 +295,7 @@ template <>
 struct ValueOf<8> { typedef uint64_t type; };
 
 template <int VB>
-__global__ __launch_bounds__(kBlock) void radix_scatter_kernel(
+__global__ __launch_bounds__(kSortBlock) void radix_scatter_kernel(
     const idx_t* __restrict__ keys_in, const idx_t* __restrict__ rows_in, const void* __restrict__ vals_in_v,
     idx_t* __restrict__ keys_out, idx_t* __restrict__ rows_out, void* __restrict__ vals_out_v, idx_t count,
     uint32_t shift, uint32_t bits, uint32_t tiles, const uint32_t* __restrict__ counters) {
@@ -275,16 +316,21 @@ __global__ __launch_bounds__(kBlock) void radix_scatter_kernel(
     const unsigned wave = tid / kWave;
     const uint32_t radix = 1u << bits;
     const uint32_t mask = radix - 1;
-    const uint64_t tile_start = static_cast<uint64_t>(blockIdx.x) * kSortTile;
+    // Workgroups are handed to the 8 XCDs round-robin.  Tile t+1 appends to the digit runs tile t
+    // started, so each XCD walks a contiguous range of tiles: the partial cache lines at the run
+    // ends then meet in one L2 and leave as full lines.
+    const uint32_t tiles_per_xcd = (tiles + kXcds - 1) / kXcds;
+    const uint32_t tile = (blockIdx.x % kXcds) * tiles_per_xcd + blockIdx.x / kXcds;
+    if (tile >= tiles) return;  // whole workgroup
+    const uint64_t tile_start = static_cast<uint64_t>(tile) * kSortTile;
     const uint32_t tile_count =
         static_cast<uint32_t>(count - tile_start < kSortTile ? count - tile_start : kSortTile);
 
-#pragma unroll
-    for (int w = 0; w < kSortWaves; ++w) s_cnt[w][tid] = 0;
+    for (uint32_t i = tid; i < kSortWaves * kMaxRadix; i += kSortBlock) (&s_cnt[0][0])[i] = 0;
     __syncthreads();
 
-    // Position inside the tile of this thread's i-th triple: waves own consecutive 1024-triple
-    // slabs, lanes are interleaved inside a slab, so (wave, i, lane) order is input order.
+    // Position inside the tile of this thread's i-th triple: waves own consecutive slabs, lanes
+    // are interleaved inside a slab, so (wave, i, lane) order is input order.
     idx_t key[kSortIpt], row[kSortIpt];
     val_t val[kSortIpt];
     uint32_t rank[kSortIpt];
@@ -332,11 +378,10 @@ __global__ __launch_bounds__(kBlock) void radix_scatter_kernel(
             digit_total += c;
         }
     }
-    uint32_t unused_total;
-    const uint32_t digit_start = block_exclusive_scan(digit_total, s_wave, &unused_total);
+    const uint32_t digit_start = sort_block_exclusive_scan(digit_total, s_wave);
     if (tid < radix) {
         s_start[tid] = digit_start;
-        s_dest[tid] = counters[static_cast<uint64_t>(tid) * tiles + blockIdx.x];
+        s_dest[tid] = counters[static_cast<uint64_t>(tid) * tiles + tile];
     }
     __syncthreads();
 
@@ -356,7 +401,7 @@ __global__ __launch_bounds__(kBlock) void radix_scatter_kernel(
     // sorted tile -> global: neighbouring threads write neighbouring addresses inside a digit run
 #pragma unroll
     for (int i = 0; i < kSortIpt; ++i) {
-        const uint32_t slot = i * kBlock + tid;
+        const uint32_t slot = i * kSortBlock + tid;
         if (slot < tile_count) {
             const idx_t k = s_keys[slot];
             const uint32_t d = (k >> shift) & mask;
@@ -404,7 +449,7 @@ void launch_csr2coo(hipStream_t stream, idx_t m, idx_t nnz, const idx_t* row_ptr
 }
 
 void launch_coo2csr(hipStream_t stream, idx_t nnz, idx_t m, const idx_t* coo_rows, idx_t base, idx_t* row_ptr) {
-    const uint64_t threads = static_cast<uint64_t>(nnz) + 1;
+    const uint64_t threads = (static_cast<uint64_t>(nnz) + kCooPerThread) / kCooPerThread;
     hipLaunchKernelGGL(coo2csr_kernel, dim3(static_cast<uint32_t>((threads + kBlock - 1) / kBlock)), dim3(kBlock), 0,
                        stream, nnz, m, base, coo_rows, row_ptr);
 }
@@ -446,17 +491,18 @@ void launch_csr2csc(hipStream_t stream, idx_t m, idx_t n, idx_t nnz, const void*
         void* vals_out = last ? csc_val : vals_t[p & 1];
         const uint32_t bits = bits_per_pass;
         const uint32_t radix = 1u << bits;
-        hipLaunchKernelGGL(radix_hist_kernel, dim3(tiles), dim3(kBlock), 0, stream, keys_in, nnz, shift, bits, tiles,
+        const uint32_t scatter_grid = (tiles + kXcds - 1) / kXcds * kXcds;
+        hipLaunchKernelGGL(radix_hist_kernel, dim3(tiles), dim3(kHistBlock), 0, stream, keys_in, nnz, shift, bits, tiles,
                            counters);
         launch_exclusive_scan(stream, counters, static_cast<uint64_t>(radix) * tiles, scan_ws);
         if (value_bytes == 0) {
-            hipLaunchKernelGGL((radix_scatter_kernel<0>), dim3(tiles), dim3(kBlock), 0, stream, keys_in, rows_in,
+            hipLaunchKernelGGL((radix_scatter_kernel<0>), dim3(scatter_grid), dim3(kSortBlock), 0, stream, keys_in, rows_in,
                                vals_in, keys_out, rows_out, vals_out, nnz, shift, bits, tiles, counters);
         } else if (value_bytes == 4) {
-            hipLaunchKernelGGL((radix_scatter_kernel<4>), dim3(tiles), dim3(kBlock), 0, stream, keys_in, rows_in,
+            hipLaunchKernelGGL((radix_scatter_kernel<4>), dim3(scatter_grid), dim3(kSortBlock), 0, stream, keys_in, rows_in,
                                vals_in, keys_out, rows_out, vals_out, nnz, shift, bits, tiles, counters);
         } else {
-            hipLaunchKernelGGL((radix_scatter_kernel<8>), dim3(tiles), dim3(kBlock), 0, stream, keys_in, rows_in,
+            hipLaunchKernelGGL((radix_scatter_kernel<8>), dim3(scatter_grid), dim3(kSortBlock), 0, stream, keys_in, rows_in,
                                vals_in, keys_out, rows_out, vals_out, nnz, shift, bits, tiles, counters);
         }
         keys_in = keys_out;
