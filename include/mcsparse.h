@@ -84,6 +84,24 @@ typedef enum {
     MCSPARSE_OPERATION_CONJUGATE_TRANSPOSE = 2
 } mcsparseOperation_t;
 
+/* :33-38, :52-62 -- matrix descriptor attributes of the legacy typed entry points */
+typedef enum {
+    MCSPARSE_MATRIX_TYPE_GENERAL = 0,
+    MCSPARSE_MATRIX_TYPE_SYMMETRIC = 1,
+    MCSPARSE_MATRIX_TYPE_HERMITIAN = 2,
+    MCSPARSE_MATRIX_TYPE_TRIANGULAR = 3
+} mcsparseMatrixType_t;
+typedef enum { MCSPARSE_DIAG_TYPE_NON_UNIT = 0, MCSPARSE_DIAG_TYPE_UNIT = 1 } mcsparseDiagType_t;
+typedef enum {
+    MCSPARSE_FILL_MODE_LOWER = 0,
+    MCSPARSE_FILL_MODE_UPPER = 1,
+    MCSPARSE_FILL_MODE_FULL = 2
+} mcsparseFillMode_t;
+/* :46-49 */
+typedef enum { MCSPARSE_STORAGE_MODE_SORTED = 0, MCSPARSE_STORAGE_MODE_UNSORTED = 1 } mcsparseStorageMode_t;
+/* :91-93 -- accepted and ignored by mcsparseCsrmvEx, as in the reference */
+typedef enum { MCSPARSE_ALG_MERGE_PATH } mcsparseAlgMode_t;
+
 /* :40-44 */
 typedef enum { MCSPARSE_INDEX_BASE_ZERO = 0, MCSPARSE_INDEX_BASE_ONE = 1 } mcsparseIndexBase_t;
 
@@ -145,6 +163,8 @@ typedef enum { MCSPARSE_CSR2CSC_ALG1 = 1, MCSPARSE_CSR2CSC_ALG2 = 2 } mcsparseCs
 /* ---- opaque handles: include/common/mcsp_types.h.in:190-242 ---------------------- */
 struct mcsparseContext;
 typedef struct mcsparseContext* mcsparseHandle_t;
+struct mcsparseMatDescr;
+typedef struct mcsparseMatDescr* mcsparseMatDescr_t;
 struct mcsparseSpMatDescr;
 typedef struct mcsparseSpMatDescr* mcsparseSpMatDescr_t;
 struct mcsparseDnVecDescr;
@@ -166,6 +186,23 @@ mcsparseStatus_t mcsparseSetStream(mcsparseHandle_t handle, hipStream_t sid);   
 mcsparseStatus_t mcsparseGetStream(const mcsparseHandle_t handle, hipStream_t* sid);         /* :22 */
 mcsparseStatus_t mcsparseSetPointerMode(mcsparseHandle_t handle, mcsparsePointerMode_t m);   /* :28 */
 mcsparseStatus_t mcsparseGetPointerMode(const mcsparseHandle_t handle, mcsparsePointerMode_t* m); /* :29 */
+
+/* ---- legacy matrix descriptor: mcsp_helper.h.in:24-44 ------------------------------ */
+/* Defaults: GENERAL, FULL, NON_UNIT, SORTED, base 0 (src/include/mcsp_internal_types.h:86-94).
+ * The getters return (enum)-1 for a NULL descriptor, as the reference does. */
+mcsparseStatus_t mcsparseCreateMatDescr(mcsparseMatDescr_t* descr);
+mcsparseStatus_t mcsparseDestroyMatDescr(mcsparseMatDescr_t descr);
+mcsparseStatus_t mcsparseCopyMatDescr(mcsparseMatDescr_t dest, const mcsparseMatDescr_t src); /* NOT_SUPPORTED there too */
+mcsparseStatus_t mcsparseSetMatIndexBase(mcsparseMatDescr_t descr, mcsparseIndexBase_t index_base);
+mcsparseIndexBase_t mcsparseGetMatIndexBase(const mcsparseMatDescr_t descr);
+mcsparseStatus_t mcsparseSetMatType(mcsparseMatDescr_t descr, mcsparseMatrixType_t matrix_type);
+mcsparseMatrixType_t mcsparseGetMatType(const mcsparseMatDescr_t descr);
+mcsparseStatus_t mcsparseSetMatFillMode(mcsparseMatDescr_t descr, mcsparseFillMode_t mode);
+mcsparseFillMode_t mcsparseGetMatFillMode(const mcsparseMatDescr_t descr);
+mcsparseStatus_t mcsparseSetMatDiagType(mcsparseMatDescr_t descr, mcsparseDiagType_t diag_type);
+mcsparseDiagType_t mcsparseGetMatDiagType(const mcsparseMatDescr_t descr);
+mcsparseStatus_t mcsparseSetStorageMode(mcsparseMatDescr_t descr, mcsparseStorageMode_t storage_mode);
+mcsparseStatus_t mcsparseGetStorageMode(const mcsparseMatDescr_t descr, mcsparseStorageMode_t* storage_mode);
 
 /* ---- dense vector descriptor: mcsp_helper.h.in:46-50 ------------------------------ */
 mcsparseStatus_t mcsparseCreateDnVec(mcsparseDnVecDescr_t* dnVecDescr, int64_t size, void* values,
@@ -239,6 +276,53 @@ mcsparseStatus_t mcsparseSpMM(mcsparseHandle_t handle, mcsparseOperation_t opA, 
                               const void* alpha, mcsparseSpMatDescr_t matA, mcsparseDnMatDescr_t matB,
                               const void* beta, mcsparseDnMatDescr_t matC, macaDataType computeType,
                               mcsparseSpMMAlg_t alg, void* externalBuffer);
+
+/* ---- legacy typed entry points onto the same kernels ------------------------------- */
+/* y = alpha*A*x + beta*y: include/interface/mcsp_level2.h:11-36.  transA is accepted and
+ * ignored, exactly as in the reference (src/kernels/level2/spmv/mcsp_spmv_gpu.cpp:946-953 hands it
+ * to a template that never reads it), so these always apply A itself.  The index base comes from
+ * descrA.  csrmv has no scratch buffer and runs the sub-wavefront vector kernel; CsrmvEx gets a
+ * buffer of *bufferSizeInBytes and runs the merge-path kernel. */
+mcsparseStatus_t mcsparseScsrmv(mcsparseHandle_t handle, mcsparseOperation_t transA, int m, int n, int nnz,
+                                const float* alpha, const mcsparseMatDescr_t descrA, const float* csrValA,
+                                const int* csrRowPtrA, const int* csrColIndA, const float* x, const float* beta,
+                                float* y);
+mcsparseStatus_t mcsparseDcsrmv(mcsparseHandle_t handle, mcsparseOperation_t transA, int m, int n, int nnz,
+                                const double* alpha, const mcsparseMatDescr_t descrA, const double* csrValA,
+                                const int* csrRowPtrA, const int* csrColIndA, const double* x, const double* beta,
+                                double* y);
+mcsparseStatus_t mcsparseCsrmvEx_bufferSize(mcsparseHandle_t handle, mcsparseAlgMode_t alg, mcsparseOperation_t transA,
+                                            int m, int n, int nnz, const void* alpha, macaDataType alphatype,
+                                            const mcsparseMatDescr_t descrA, const void* csrValA,
+                                            macaDataType csrValAtype, const int* csrRowPtrA, const int* csrColIndA,
+                                            const void* x, macaDataType xtype, const void* beta, macaDataType betatype,
+                                            void* y, macaDataType ytype, macaDataType executiontype,
+                                            size_t* bufferSizeInBytes);
+mcsparseStatus_t mcsparseCsrmvEx(mcsparseHandle_t handle, mcsparseAlgMode_t alg, mcsparseOperation_t transA, int m,
+                                 int n, int nnz, const void* alpha, macaDataType alphatype,
+                                 const mcsparseMatDescr_t descrA, const void* csrValA, macaDataType csrValAtype,
+                                 const int* csrRowPtrA, const int* csrColIndA, const void* x, macaDataType xtype,
+                                 const void* beta, macaDataType betatype, void* y, macaDataType ytype,
+                                 macaDataType executiontype, void* buffer);
+/* C = alpha*A*op(B) + beta*C with column-major B and C: include/interface/mcsp_level3.h:139-169.
+ * A is m x k, C is m x n; B is k x n (transB = N) or n x k (transB = T).  transA must be N
+ * (src/kernels/level3/spmm/mcsp_spmm_gpu.cpp:39-42).  csrmm is csrmm2 with transB = N. */
+mcsparseStatus_t mcsparseScsrmm2(mcsparseHandle_t handle, mcsparseOperation_t transA, mcsparseOperation_t transB, int m,
+                                 int n, int k, int nnz, const float* alpha, const mcsparseMatDescr_t descrA,
+                                 const float* csrValA, const int* csrRowPtrA, const int* csrColIndA, const float* B,
+                                 int ldb, const float* beta, float* C, int ldc);
+mcsparseStatus_t mcsparseDcsrmm2(mcsparseHandle_t handle, mcsparseOperation_t transA, mcsparseOperation_t transB, int m,
+                                 int n, int k, int nnz, const double* alpha, const mcsparseMatDescr_t descrA,
+                                 const double* csrValA, const int* csrRowPtrA, const int* csrColIndA, const double* B,
+                                 int ldb, const double* beta, double* C, int ldc);
+mcsparseStatus_t mcsparseScsrmm(mcsparseHandle_t handle, mcsparseOperation_t transA, int m, int n, int k, int nnz,
+                                const float* alpha, const mcsparseMatDescr_t descrA, const float* csrValA,
+                                const int* csrRowPtrA, const int* csrColIndA, const float* B, int ldb,
+                                const float* beta, float* C, int ldc);
+mcsparseStatus_t mcsparseDcsrmm(mcsparseHandle_t handle, mcsparseOperation_t transA, int m, int n, int k, int nnz,
+                                const double* alpha, const mcsparseMatDescr_t descrA, const double* csrValA,
+                                const int* csrRowPtrA, const int* csrColIndA, const double* B, int ldb,
+                                const double* beta, double* C, int ldc);
 
 /* ---- index conversions: include/interface/mcsp_conversion.h:11-28 ------------------ */
 /* coo_rows must be sorted; csr_rows receives m+1 offsets.                       :11 */

@@ -58,6 +58,31 @@ PROTOTYPES = {
     "mcsparseCsr2cscEx2": (c_int, [vp, c_int, c_int, c_int, vp, vp, vp, vp, vp, vp, c_int, c_int, c_int, c_int, vp]),
     "mcsparseCsr2cscEx2_bufferSize": (c_int, [vp, c_int, c_int, c_int, vp, vp, vp, vp, vp, vp, c_int, c_int, c_int,
                                               c_int, P(c_size)]),
+    "mcsparseCreateMatDescr": (c_int, [P(vp)]),
+    "mcsparseDestroyMatDescr": (c_int, [vp]),
+    "mcsparseCopyMatDescr": (c_int, [vp, vp]),
+    "mcsparseSetMatIndexBase": (c_int, [vp, c_int]),
+    "mcsparseGetMatIndexBase": (c_int, [vp]),
+    "mcsparseSetMatType": (c_int, [vp, c_int]),
+    "mcsparseGetMatType": (c_int, [vp]),
+    "mcsparseSetMatFillMode": (c_int, [vp, c_int]),
+    "mcsparseGetMatFillMode": (c_int, [vp]),
+    "mcsparseSetMatDiagType": (c_int, [vp, c_int]),
+    "mcsparseGetMatDiagType": (c_int, [vp]),
+    "mcsparseSetStorageMode": (c_int, [vp, c_int]),
+    "mcsparseGetStorageMode": (c_int, [vp, P(c_int)]),
+    "mcsparseScsrmv": (c_int, [vp, c_int, c_int, c_int, c_int, vp, vp, vp, vp, vp, vp, vp, vp]),
+    "mcsparseDcsrmv": (c_int, [vp, c_int, c_int, c_int, c_int, vp, vp, vp, vp, vp, vp, vp, vp]),
+    "mcsparseCsrmvEx_bufferSize": (c_int, [vp, c_int, c_int, c_int, c_int, c_int, vp, c_int, vp, vp, c_int, vp, vp,
+                                           vp, c_int, vp, c_int, vp, c_int, c_int, P(c_size)]),
+    "mcsparseCsrmvEx": (c_int, [vp, c_int, c_int, c_int, c_int, c_int, vp, c_int, vp, vp, c_int, vp, vp, vp, c_int,
+                                vp, c_int, vp, c_int, c_int, vp]),
+    "mcsparseScsrmm2": (c_int, [vp, c_int, c_int, c_int, c_int, c_int, c_int, vp, vp, vp, vp, vp, vp, c_int, vp, vp,
+                                c_int]),
+    "mcsparseDcsrmm2": (c_int, [vp, c_int, c_int, c_int, c_int, c_int, c_int, vp, vp, vp, vp, vp, vp, c_int, vp, vp,
+                                c_int]),
+    "mcsparseScsrmm": (c_int, [vp, c_int, c_int, c_int, c_int, c_int, vp, vp, vp, vp, vp, vp, c_int, vp, vp, c_int]),
+    "mcsparseDcsrmm": (c_int, [vp, c_int, c_int, c_int, c_int, c_int, vp, vp, vp, vp, vp, vp, c_int, vp, vp, c_int]),
     "mcsparseXcsrRowBins": (c_int, [vp, c_int, vp, c_int, vp, vp]),
     "mcsparseSpMatGetSpMVPlan": (c_int, [vp, P(c_int), P(c_int)]),
     "mcsparseSpMatSetSpMVPlan": (c_int, [vp, c_int, c_int]),

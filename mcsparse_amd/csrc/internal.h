@@ -23,6 +23,15 @@ struct mcsparseContext {
     mcsparsePointerMode_t ptr_mode = MCSPARSE_POINTER_MODE_HOST;
 };
 
+// reference: src/include/mcsp_internal_types.h:86-94
+struct mcsparseMatDescr {
+    mcsparseMatrixType_t type = MCSPARSE_MATRIX_TYPE_GENERAL;
+    mcsparseFillMode_t fill_mode = MCSPARSE_FILL_MODE_FULL;
+    mcsparseDiagType_t diag_type = MCSPARSE_DIAG_TYPE_NON_UNIT;
+    mcsparseStorageMode_t storage_mode = MCSPARSE_STORAGE_MODE_SORTED;
+    mcsparseIndexBase_t base = MCSPARSE_INDEX_BASE_ZERO;
+};
+
 // reference: src/include/mcsp_internal_types.h:127-133
 struct mcsparseDnVecDescr {
     macaDataType valueType = MACA_R_32F;
