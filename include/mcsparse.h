@@ -231,6 +231,19 @@ mcsparseStatus_t mcsparseCreateCsc(mcsparseSpMatDescr_t* spMatDescr, int64_t row
                                    mcsparseIndexBase_t idxBase, macaDataType valueType);    /* :69 */
 mcsparseStatus_t mcsparseCscSetPointers(mcsparseSpMatDescr_t spMatDescr, void* cscColOffsets, void* cscRowInd,
                                         void* cscValues);                                   /* :72 */
+/* COO (structure of arrays) with entries sorted by row, the order the reference's COO kernels
+ * assume as well (src/kernels/level2/spmv/coo_flat_device.hpp:65-171 adds partial sums of
+ * adjacent equal rows without atomics).  SpMV and SpMM build the row offsets in the scratch
+ * buffer and run the CSR kernels.                                                :52-58 */
+mcsparseStatus_t mcsparseCreateCoo(mcsparseSpMatDescr_t* spMatDescr, int64_t rows, int64_t cols, int64_t nnz,
+                                   void* cooRowInd, void* cooColInd, void* cooValues,
+                                   mcsparseIndexType_t cooIdxType, mcsparseIndexBase_t idxBase,
+                                   macaDataType valueType);
+mcsparseStatus_t mcsparseCooGet(mcsparseSpMatDescr_t spMatDescr, int64_t* rows, int64_t* cols, int64_t* nnz,
+                                void** cooRowInd, void** cooColInd, void** cooValues, mcsparseIndexType_t* idxType,
+                                mcsparseIndexBase_t* idxBase, macaDataType* valueType);
+mcsparseStatus_t mcsparseCooSetPointers(mcsparseSpMatDescr_t spMatDescr, void* cooRows, void* cooColumns,
+                                        void* cooValues);
 mcsparseStatus_t mcsparseDestroySpMat(mcsparseSpMatDescr_t spMatDescr);                     /* :81 */
 mcsparseStatus_t mcsparseSpMatGetSize(mcsparseSpMatDescr_t spMatDescr, int64_t* rows, int64_t* cols,
                                       int64_t* nnz);                                        /* :82 */

@@ -37,6 +37,9 @@ PROTOTYPES = {
     "mcsparseCsrSetPointers": (c_int, [vp, vp, vp, vp]),
     "mcsparseCreateCsc": (c_int, [P(vp), c_i64, c_i64, c_i64, vp, vp, vp, c_int, c_int, c_int, c_int]),
     "mcsparseCscSetPointers": (c_int, [vp, vp, vp, vp]),
+    "mcsparseCreateCoo": (c_int, [P(vp), c_i64, c_i64, c_i64, vp, vp, vp, c_int, c_int, c_int]),
+    "mcsparseCooGet": (c_int, [vp, P(c_i64), P(c_i64), P(c_i64), P(vp), P(vp), P(vp), P(c_int), P(c_int), P(c_int)]),
+    "mcsparseCooSetPointers": (c_int, [vp, vp, vp, vp]),
     "mcsparseDestroySpMat": (c_int, [vp]),
     "mcsparseSpMatGetSize": (c_int, [vp, P(c_i64), P(c_i64), P(c_i64)]),
     "mcsparseSpMatGetFormat": (c_int, [vp, P(c_int)]),

@@ -113,6 +113,10 @@ class SpMat:
         self._keep = (offsets, indices, values)
         self._d = ctypes.c_void_p()
         vt = value_type if value_type is not None else maca_type(values.dtype)
+        if fmt == FORMAT_COO:  # offsets = row indices, indices = column indices
+            check(self.lib.mcsparseCreateCoo(ctypes.byref(self._d), rows, cols, nnz, _ptr(offsets), _ptr(indices),
+                                             _ptr(values), index_type, base, vt), "mcsparseCreateCoo")
+            return
         create = self.lib.mcsparseCreateCsr if fmt == FORMAT_CSR else self.lib.mcsparseCreateCsc
         check(create(ctypes.byref(self._d), rows, cols, nnz, _ptr(offsets), _ptr(indices), _ptr(values), index_type,
                      index_type, base, vt), "mcsparseCreateCsr/Csc")

@@ -25,19 +25,22 @@ bool scalar_to_host(mcsparseHandle_t h, const void* p, T* out) {
     return hipStreamSynchronize(h->stream) == hipSuccess;
 }
 
-// The CSR-shaped view an SpMV call works on after CSC inputs have been re-read as the CSR of
-// the transpose (src/kernels/level2/spmv/mcsp_spmv_gpu.cpp:734-739).
+// The CSR-shaped view a call works on.  CSC inputs are re-read as the CSR of the transpose
+// (src/kernels/level2/spmv/mcsp_spmv_gpu.cpp:734-739); row-sorted COO inputs get their row
+// offsets built in the scratch buffer by coo2csr (:817-825), so `ptr` is null until then.
 struct CsrView {
     int64_t m, n;        // shape of the matrix whose CSR arrays these are
-    const idx_t* ptr;    // m+1 offsets
+    const idx_t* ptr;    // m+1 offsets (null for COO: built into the scratch buffer)
     const idx_t* ind;    // nnz indices
     const void* val;
-    bool transpose;      // the call needs view^T * x
+    const idx_t* coo_rows;  // COO only: the nnz row indices the offsets are built from
+    bool transpose;      // the call needs view^T
 };
 
 CsrView make_view(const mcsparseSpMatDescr* A, mcsparseOperation_t op) {
     CsrView v;
     const bool op_t = op != MCSPARSE_OPERATION_NON_TRANSPOSE;
+    v.coo_rows = nullptr;
     if (A->format == MCSPARSE_FORMAT_CSC) {
         v.m = A->col_num;
         v.n = A->row_num;
@@ -50,39 +53,48 @@ CsrView make_view(const mcsparseSpMatDescr* A, mcsparseOperation_t op) {
         v.ptr = static_cast<const idx_t*>(A->rows);
         v.ind = static_cast<const idx_t*>(A->cols);
         v.transpose = op_t;
+        if (A->format == MCSPARSE_FORMAT_COO) {
+            v.coo_rows = v.ptr;
+            v.ptr = nullptr;
+        }
     }
     v.val = A->vals;
     return v;
 }
 
-// Scratch layout of a transposing SpMV:
-//   [analysis][merge workspace of the transposed matrix][col_ptr n+1 | row_ind nnz][values][csr2csc workspace]
-// (the reference's layout, src/kernels/level2/spmv/mcsp_spmv_gpu.cpp:308 and :813-831, plus the
-// merge-path workspace in front).
-struct TransposeLayout {
-    size_t merge_ws, col_ptr, row_ind, vals, csr2csc_ws, total;
-};
-
-TransposeLayout transpose_layout(int64_t m, int64_t n, int64_t nnz, size_t value_bytes) {
-    TransposeLayout l;
-    size_t off = kAnalysisBytes;
-    l.merge_ws = off;
-    off += align_up(mcsp::spmv_merge_workspace_bytes(static_cast<idx_t>(n), static_cast<idx_t>(nnz), value_bytes));
-    l.col_ptr = off;
-    l.row_ind = off + static_cast<size_t>(n + 1) * sizeof(idx_t);
-    off += align_up(static_cast<size_t>(n + 1 + nnz) * sizeof(idx_t));
-    l.vals = off;
-    off += align_up(static_cast<size_t>(nnz) * value_bytes);
-    l.csr2csc_ws = off;
-    off += align_up(mcsp::csr2csc_workspace_bytes(static_cast<idx_t>(m), static_cast<idx_t>(n),
-                                                  static_cast<idx_t>(nnz), value_bytes));
-    l.total = off;
-    return l;
+bool format_is_built(mcsparseFormat_t f) {
+    return f == MCSPARSE_FORMAT_CSR || f == MCSPARSE_FORMAT_CSC || f == MCSPARSE_FORMAT_COO;
 }
 
-size_t direct_spmv_bytes(int64_t m, int64_t nnz, size_t value_bytes) {
-    return kAnalysisBytes +
-           align_up(mcsp::spmv_merge_workspace_bytes(static_cast<idx_t>(m), static_cast<idx_t>(nnz), value_bytes));
+// Scratch layout of an SpMV call, all parts aligned to 128 bytes:
+//   [analysis][merge workspace][COO only: row offsets m+1]
+//   transposing calls add [col_ptr n+1 | row_ind nnz][values][csr2csc workspace]
+// (the transposed part is the reference's layout, mcsp_spmv_gpu.cpp:308 and :813-831).
+struct SpmvLayout {
+    size_t merge_ws, coo_ptr, col_ptr, row_ind, vals, csr2csc_ws, total;
+};
+
+SpmvLayout spmv_layout(const CsrView& v, int64_t nnz, size_t value_bytes) {
+    SpmvLayout l = {};
+    const int64_t out_rows = v.transpose ? v.n : v.m;  // rows of the matrix the SpMV kernel sees
+    size_t off = kAnalysisBytes;
+    l.merge_ws = off;
+    off += align_up(mcsp::spmv_merge_workspace_bytes(static_cast<idx_t>(out_rows), static_cast<idx_t>(nnz),
+                                                     value_bytes));
+    l.coo_ptr = off;
+    if (v.coo_rows != nullptr) off += align_up(static_cast<size_t>(v.m + 1) * sizeof(idx_t));
+    if (v.transpose) {
+        l.col_ptr = off;
+        l.row_ind = off + static_cast<size_t>(v.n + 1) * sizeof(idx_t);
+        off += align_up(static_cast<size_t>(v.n + 1 + nnz) * sizeof(idx_t));
+        l.vals = off;
+        off += align_up(static_cast<size_t>(nnz) * value_bytes);
+        l.csr2csc_ws = off;
+        off += align_up(mcsp::csr2csc_workspace_bytes(static_cast<idx_t>(v.m), static_cast<idx_t>(v.n),
+                                                      static_cast<idx_t>(nnz), value_bytes));
+    }
+    l.total = off < kMinBuffer ? kMinBuffer : off;
+    return l;
 }
 
 // Checks shared by SpMV and SpMV_bufferSize, in the reference's order
@@ -117,13 +129,14 @@ mcspStatus_t check_index_types(const mcsparseSpMatDescr* A) {
 }
 
 // Chooses the kernel family for a structure; runs the row-length analysis (one kernel, one
-// blocking 136-byte read-back) the first time a structure is seen.
-mcspStatus_t ensure_plan(mcsparseHandle_t h, mcsparseSpMatDescr* A, const idx_t* ptr, int64_t m, int64_t nnz,
-                         void* buffer) {
+// blocking 136-byte read-back) the first time a structure is seen.  `ptr` are the offsets to
+// analyse, `signature` the caller's array that identifies the structure.
+mcspStatus_t ensure_plan(mcsparseHandle_t h, mcsparseSpMatDescr* A, const idx_t* ptr, const void* signature,
+                         int64_t m, int64_t nnz, void* buffer) {
     SpmvPlan& p = A->plan;
-    if (p.valid && p.rows == ptr && p.m == m && p.nnz == nnz && p.base == static_cast<int>(A->idxBase))
+    if (p.valid && p.rows == signature && p.m == m && p.nnz == nnz && p.base == static_cast<int>(A->idxBase))
         return MCSP_STATUS_SUCCESS;
-    p.rows = ptr;
+    p.rows = signature;
     p.m = m;
     p.nnz = nnz;
     p.base = static_cast<int>(A->idxBase);
@@ -158,8 +171,8 @@ mcspStatus_t ensure_plan(mcsparseHandle_t h, mcsparseSpMatDescr* A, const idx_t*
 }
 
 template <typename T>
-mcspStatus_t spmv_typed(mcsparseHandle_t h, mcsparseSpMatDescr* A, const CsrView& v, const void* alpha,
-                        const void* beta, const mcsparseDnVecDescr* x, mcsparseDnVecDescr* y, void* buffer) {
+mcspStatus_t spmv_typed(mcsparseHandle_t h, mcsparseSpMatDescr* A, CsrView v, const void* alpha, const void* beta,
+                        const mcsparseDnVecDescr* x, mcsparseDnVecDescr* y, void* buffer) {
     T h_alpha, h_beta;
     if (!scalar_to_host(h, beta, &h_beta) || !scalar_to_host(h, alpha, &h_alpha)) return MCSP_STATUS_INTERNAL_ERROR;
     // reference: mcsp_spmv_gpu.cpp:235-237 -- y is left untouched in both cases
@@ -168,6 +181,13 @@ mcspStatus_t spmv_typed(mcsparseHandle_t h, mcsparseSpMatDescr* A, const CsrView
     const idx_t nnz = static_cast<idx_t>(A->nnz);
     const idx_t base = static_cast<idx_t>(A->idxBase);
     char* buf = static_cast<char*>(buffer);
+    const SpmvLayout l = spmv_layout(v, A->nnz, sizeof(T));
+    const void* signature = v.coo_rows != nullptr ? static_cast<const void*>(v.coo_rows) : v.ptr;
+    if (v.coo_rows != nullptr) {
+        idx_t* built = reinterpret_cast<idx_t*>(buf + l.coo_ptr);
+        mcsp::launch_coo2csr(h->stream, nnz, static_cast<idx_t>(v.m), v.coo_rows, base, built);
+        v.ptr = built;
+    }
     mcsp::SpmvArgs a;
     a.nnz = nnz;
     a.base = base;
@@ -180,10 +200,10 @@ mcspStatus_t spmv_typed(mcsparseHandle_t h, mcsparseSpMatDescr* A, const CsrView
         a.row_ptr = v.ptr;
         a.col = v.ind;
         a.val = v.val;
-        const mcspStatus_t st = ensure_plan(h, A, v.ptr, v.m, A->nnz, buffer);
+        const mcspStatus_t st = ensure_plan(h, A, v.ptr, signature, v.m, A->nnz, buffer);
         if (st != MCSP_STATUS_SUCCESS) return st;
         if (A->plan.family == kFamilyMerge) {
-            mcsp::launch_spmv_merge<T>(h->stream, a, h_alpha, h_beta, buf + kAnalysisBytes);
+            mcsp::launch_spmv_merge<T>(h->stream, a, h_alpha, h_beta, buf + l.merge_ws);
         } else {
             mcsp::launch_spmv_vector<T>(h->stream, a, h_alpha, h_beta, A->plan.lanes);
         }
@@ -192,7 +212,6 @@ mcspStatus_t spmv_typed(mcsparseHandle_t h, mcsparseSpMatDescr* A, const CsrView
 
     // Transposing call: materialise the transpose in the scratch buffer on every call, as the
     // reference does (mcsp_spmv_gpu.cpp:797-845) -- the caller may have changed the values.
-    const TransposeLayout l = transpose_layout(v.m, v.n, A->nnz, sizeof(T));
     idx_t* t_ptr = reinterpret_cast<idx_t*>(buf + l.col_ptr);
     idx_t* t_ind = reinterpret_cast<idx_t*>(buf + l.row_ind);
     void* t_val = buf + l.vals;
@@ -209,9 +228,34 @@ mcspStatus_t spmv_typed(mcsparseHandle_t h, mcsparseSpMatDescr* A, const CsrView
     return MCSP_STATUS_SUCCESS;
 }
 
+// Scratch layout of an SpMM call: CSR needs none; COO gets [row offsets m+1]; CSC gets the
+// transposed copy [row_ptr m+1 | col_ind nnz][values][csr2csc workspace]
+// (mcsp_spmm_gpu.cpp:818-849).
+struct SpmmLayout {
+    size_t ptr, ind, vals, csr2csc_ws, total;
+};
+
+SpmmLayout spmm_layout(const mcsparseSpMatDescr* A, size_t value_bytes) {
+    SpmmLayout l = {};
+    size_t off = 0;
+    if (A->format == MCSPARSE_FORMAT_COO) {
+        off += align_up(static_cast<size_t>(A->row_num + 1) * sizeof(idx_t));
+    } else if (A->format == MCSPARSE_FORMAT_CSC) {
+        l.ind = static_cast<size_t>(A->row_num + 1) * sizeof(idx_t);
+        off += align_up(static_cast<size_t>(A->row_num + 1 + A->nnz) * sizeof(idx_t));
+        l.vals = off;
+        off += align_up(static_cast<size_t>(A->nnz) * value_bytes);
+        l.csr2csc_ws = off;
+        off += align_up(mcsp::csr2csc_workspace_bytes(static_cast<idx_t>(A->col_num), static_cast<idx_t>(A->row_num),
+                                                      static_cast<idx_t>(A->nnz), value_bytes));
+    }
+    l.total = off < kMinBuffer ? kMinBuffer : off;
+    return l;
+}
+
 template <typename T>
 mcspStatus_t spmm_typed(mcsparseHandle_t h, const mcsparseSpMatDescr* A, mcsparseOperation_t opB, const void* alpha,
-                        const void* beta, const mcsparseDnMatDescr* B, mcsparseDnMatDescr* C) {
+                        const void* beta, const mcsparseDnMatDescr* B, mcsparseDnMatDescr* C, void* buffer) {
     T h_alpha, h_beta;
     if (!scalar_to_host(h, beta, &h_beta) || !scalar_to_host(h, alpha, &h_alpha)) return MCSP_STATUS_INTERNAL_ERROR;
     // reference: mcsp_spmm_gpu.cpp:110-114
@@ -226,6 +270,29 @@ mcspStatus_t spmm_typed(mcsparseHandle_t h, const mcsparseSpMatDescr* A, mcspars
     a.row_ptr = static_cast<const idx_t*>(A->rows);
     a.col = static_cast<const idx_t*>(A->cols);
     a.val = A->vals;
+    char* buf = static_cast<char*>(buffer);
+    const SpmmLayout l = spmm_layout(A, sizeof(T));
+    if (A->format == MCSPARSE_FORMAT_COO && A->nnz != 0) {
+        idx_t* built = reinterpret_cast<idx_t*>(buf + l.ptr);
+        mcsp::launch_coo2csr(h->stream, a.nnz, a.m, static_cast<const idx_t*>(A->rows), a.base, built);
+        a.row_ptr = built;
+    } else if (A->format == MCSPARSE_FORMAT_CSC && A->nnz != 0) {
+        // the CSC arrays are the CSR of A^T (col_num x row_num); transposing them gives the CSR of A
+        idx_t* t_ptr = reinterpret_cast<idx_t*>(buf + l.ptr);
+        idx_t* t_ind = reinterpret_cast<idx_t*>(buf + l.ind);
+        void* t_val = buf + l.vals;
+        mcsp::launch_csr2csc(h->stream, static_cast<idx_t>(A->col_num), static_cast<idx_t>(A->row_num), a.nnz, A->vals,
+                             static_cast<const idx_t*>(A->cols), static_cast<const idx_t*>(A->rows), t_val, t_ind,
+                             t_ptr, sizeof(T), a.base, buf + l.csr2csc_ws);
+        a.row_ptr = t_ptr;
+        a.col = t_ind;
+        a.val = t_val;
+    } else if (A->format != MCSPARSE_FORMAT_CSR) {
+        // no nonzeros: C = beta*C over m empty rows; coo2csr with nnz = 0 writes the m+1 offsets
+        idx_t* built = reinterpret_cast<idx_t*>(buf + l.ptr);
+        mcsp::launch_coo2csr(h->stream, 0, a.m, built, a.base, built);
+        a.row_ptr = built;
+    }
     a.B = B->values;
     a.ldb = B->ld;
     // op(B)(kk, j) sits at kk*ldb + j for (N, row-major) and (T, column-major), else at j*ldb + kk;
@@ -270,21 +337,17 @@ mcsparseStatus_t mcsparseSpMV_bufferSize(mcsparseHandle_t handle, mcsparseOperat
     const mcspStatus_t st =
         check_spmv_args(handle, opA, alpha, matA, vecX, beta, vecY, bufferSize != nullptr, false, nullptr);
     if (st != MCSP_STATUS_SUCCESS) return to_public_status(st);
-    if (matA->format != MCSPARSE_FORMAT_CSR && matA->format != MCSPARSE_FORMAT_CSC)
-        return to_public_status(MCSP_STATUS_NOT_IMPLEMENTED);  // COO inputs are not built here
+    if (!format_is_built(matA->format)) return to_public_status(MCSP_STATUS_NOT_IMPLEMENTED);  // COO_AOS
 
     const size_t vb = value_size(matA->valueType);
     const CsrView v = make_view(matA, opA);
-    if (!v.transpose) {
-        *bufferSize = direct_spmv_bytes(v.m, matA->nnz, vb);
-    } else {
-        const TransposeLayout l = transpose_layout(v.m, v.n, matA->nnz, vb);
+    const SpmvLayout l = spmv_layout(v, matA->nnz, vb);
+    if (v.transpose) {
         matA->assist_index_buffer_size = l.vals - l.col_ptr;
         matA->fixed_length_buffer_size = l.csr2csc_ws;
         matA->is_buffersize_called = 1;
-        *bufferSize = l.total;
     }
-    if (*bufferSize < kMinBuffer) *bufferSize = kMinBuffer;
+    *bufferSize = l.total;
     return MCSPARSE_STATUS_SUCCESS;
 }
 
@@ -302,8 +365,7 @@ mcsparseStatus_t mcsparseSpMV(mcsparseHandle_t handle, mcsparseOperation_t opA, 
     const bool real_type = computeType == MACA_R_32F || computeType == MACA_R_64F || computeType == MACA_R_16F ||
                            computeType == MACA_R_16BF;
     if (real_type && opA == MCSPARSE_OPERATION_CONJUGATE_TRANSPOSE) return to_public_status(MCSP_STATUS_INVALID_VALUE);
-    if (matA->format != MCSPARSE_FORMAT_CSR && matA->format != MCSPARSE_FORMAT_CSC)
-        return to_public_status(MCSP_STATUS_NOT_IMPLEMENTED);  // COO inputs are not built here
+    if (!format_is_built(matA->format)) return to_public_status(MCSP_STATUS_NOT_IMPLEMENTED);  // COO_AOS
     // Same-type real fp32/fp64 only; the reference's mixed-precision and complex routes
     // (:848-860) are outside this path.  x is checked too, which the reference omits.
     if (!(computeType == matA->valueType && computeType == vecY->valueType && computeType == vecX->valueType))
@@ -336,8 +398,9 @@ mcsparseStatus_t mcsparseSpMM_bufferSize(mcsparseHandle_t handle, mcsparseOperat
     const mcspStatus_t st = check_spmm_args(handle, alpha, matA, matB, beta, matC);
     if (st != MCSP_STATUS_SUCCESS) return to_public_status(st);
     if (bufferSize == nullptr) return to_public_status(MCSP_STATUS_INVALID_POINTER);
-    if (matA->format != MCSPARSE_FORMAT_CSR) return to_public_status(MCSP_STATUS_NOT_IMPLEMENTED);
-    *bufferSize = kMinBuffer;
+    if (!format_is_built(matA->format)) return to_public_status(MCSP_STATUS_NOT_IMPLEMENTED);  // Blocked-ELL
+    *bufferSize = spmm_layout(matA, value_size(matA->valueType)).total;
+    if (matA->format == MCSPARSE_FORMAT_CSC) matA->is_buffersize_called = 1;
     return MCSPARSE_STATUS_SUCCESS;
 }
 
@@ -361,10 +424,10 @@ mcsparseStatus_t mcsparseSpMM(mcsparseHandle_t handle, mcsparseOperation_t opA, 
     if (externalBuffer == nullptr) return to_public_status(MCSP_STATUS_INVALID_POINTER);
     mcspStatus_t st = check_spmm_args(handle, alpha, matA, matB, beta, matC);
     if (st != MCSP_STATUS_SUCCESS) return to_public_status(st);
-    if (matA->format != MCSPARSE_FORMAT_CSR) return to_public_status(MCSP_STATUS_NOT_IMPLEMENTED);
+    if (!format_is_built(matA->format)) return to_public_status(MCSP_STATUS_NOT_IMPLEMENTED);  // Blocked-ELL
     if (!(computeType == matA->valueType && computeType == matC->valueType && computeType == matB->valueType))
         return to_public_status(MCSP_STATUS_NOT_IMPLEMENTED);
-    // CSR with op(A) != N is not implemented by the reference either (:105-108)
+    // op(A) != N is not implemented by the reference for CSR, COO or transposed CSC (:105-108)
     if (opA != MCSPARSE_OPERATION_NON_TRANSPOSE) return to_public_status(MCSP_STATUS_NOT_IMPLEMENTED);
     // Shapes the reference never checks and then reads out of bounds on: C is m x n, op(B) is k x n.
     const bool op_n = opB == MCSPARSE_OPERATION_NON_TRANSPOSE;
@@ -377,8 +440,8 @@ mcsparseStatus_t mcsparseSpMM(mcsparseHandle_t handle, mcsparseOperation_t opA, 
     if (matB->ld < b_lead || matC->ld < c_lead) return to_public_status(MCSP_STATUS_INVALID_SIZE);
 
     switch (computeType) {
-        case MACA_R_32F: st = spmm_typed<float>(handle, matA, opB, alpha, beta, matB, matC); break;
-        case MACA_R_64F: st = spmm_typed<double>(handle, matA, opB, alpha, beta, matB, matC); break;
+        case MACA_R_32F: st = spmm_typed<float>(handle, matA, opB, alpha, beta, matB, matC, externalBuffer); break;
+        case MACA_R_64F: st = spmm_typed<double>(handle, matA, opB, alpha, beta, matB, matC, externalBuffer); break;
         default: st = MCSP_STATUS_NOT_IMPLEMENTED;
     }
     return to_public_status(st);

@@ -233,6 +233,42 @@ mcsparseStatus_t mcsparseCreateCsc(mcsparseSpMatDescr_t* spMatDescr, int64_t row
                                          MCSPARSE_FORMAT_CSC));
 }
 
+mcsparseStatus_t mcsparseCreateCoo(mcsparseSpMatDescr_t* spMatDescr, int64_t rows, int64_t cols, int64_t nnz,
+                                   void* cooRowInd, void* cooColInd, void* cooValues,
+                                   mcsparseIndexType_t cooIdxType, mcsparseIndexBase_t idxBase,
+                                   macaDataType valueType) {
+    return to_public_status(create_spmat(spMatDescr, rows, cols, nnz, cooRowInd, cooColInd, cooValues, cooIdxType,
+                                         cooIdxType, idxBase, valueType, MCSPARSE_FORMAT_COO));
+}
+
+mcsparseStatus_t mcsparseCooGet(mcsparseSpMatDescr_t d, int64_t* rows, int64_t* cols, int64_t* nnz, void** cooRowInd,
+                                void** cooColInd, void** cooValues, mcsparseIndexType_t* idxType,
+                                mcsparseIndexBase_t* idxBase, macaDataType* valueType) {
+    if (d == nullptr || rows == nullptr || cols == nullptr || nnz == nullptr || cooRowInd == nullptr ||
+        cooColInd == nullptr || cooValues == nullptr || idxType == nullptr || idxBase == nullptr ||
+        valueType == nullptr)
+        return to_public_status(MCSP_STATUS_INVALID_POINTER);
+    *rows = d->row_num;
+    *cols = d->col_num;
+    *nnz = d->nnz;
+    *cooRowInd = d->rows;
+    *cooColInd = d->cols;
+    *cooValues = d->vals;
+    *idxType = d->rowIdxType;
+    *idxBase = d->idxBase;
+    *valueType = d->valueType;
+    return MCSPARSE_STATUS_SUCCESS;
+}
+
+mcsparseStatus_t mcsparseCooSetPointers(mcsparseSpMatDescr_t d, void* cooRows, void* cooColumns, void* cooValues) {
+    if (d == nullptr) return to_public_status(MCSP_STATUS_INVALID_POINTER);
+    d->rows = cooRows;
+    d->cols = cooColumns;
+    d->vals = cooValues;
+    d->plan.valid = false;
+    return MCSPARSE_STATUS_SUCCESS;
+}
+
 mcsparseStatus_t mcsparseCsrGet(mcsparseSpMatDescr_t d, int64_t* rows, int64_t* cols, int64_t* nnz,
                                 void** csrRowOffsets, void** csrColInd, void** csrValues,
                                 mcsparseIndexType_t* csrRowOffsetsType, mcsparseIndexType_t* csrColIndType,

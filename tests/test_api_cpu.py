@@ -124,6 +124,21 @@ def test_sparse_descriptors(lib):
     assert lib.mcsparseCscSetPointers(d, 0x51, 0x61, 0x71) == 0
     assert lib.mcsparseCscSetPointers(None, 0x51, 0x61, 0x71) == api.STATUS_INVALID_VALUE
     assert lib.mcsparseDestroySpMat(d) == 0
+    # COO: one index type for both arrays (mcsp_helper.cpp:526-585)
+    mkc = lib.mcsparseCreateCoo
+    assert mkc(ctypes.byref(d), 3, -4, 5, 0x10, 0x20, 0x30, 2, 0, api.R_32F) == api.STATUS_INVALID_VALUE
+    assert mkc(None, 3, 4, 5, 0x10, 0x20, 0x30, 2, 0, api.R_32F) == api.STATUS_INVALID_VALUE
+    assert mkc(ctypes.byref(d), 3, 4, 5, 0x10, 0x20, 0x30, 2, 1, api.R_32F) == 0
+    assert lib.mcsparseSpMatGetFormat(d, ctypes.byref(fmt)) == 0 and fmt.value == api.FORMAT_COO
+    assert lib.mcsparseCooSetPointers(d, 0x11, 0x21, 0x31) == 0
+    ints3 = [ctypes.c_int() for _ in range(3)]
+    assert lib.mcsparseCooGet(d, *[ctypes.byref(x) for x in i64 + ptrs + ints3]) == 0
+    assert [x.value for x in i64] == [3, 4, 5]
+    assert [x.value for x in ptrs] == [0x11, 0x21, 0x31]
+    assert [x.value for x in ints3] == [2, 1, api.R_32F]
+    assert lib.mcsparseCooGet(d, *[ctypes.byref(x) for x in i64 + ptrs + ints3[:2]], None) == api.STATUS_INVALID_VALUE
+    assert lib.mcsparseCooSetPointers(None, 0x11, 0x21, 0x31) == api.STATUS_INVALID_VALUE
+    assert lib.mcsparseDestroySpMat(d) == 0
 
 
 class Objs:
@@ -134,8 +149,11 @@ class Objs:
         self.h = ctypes.c_void_p()
         lib.mcsparseCreate(ctypes.byref(self.h))
         self.A = ctypes.c_void_p()
-        mk = lib.mcsparseCreateCsr if fmt == api.FORMAT_CSR else lib.mcsparseCreateCsc
-        assert mk(ctypes.byref(self.A), m, n, nnz, FAKE, FAKE, FAKE, idx[0], idx[1], 0, vt) == 0
+        if fmt == api.FORMAT_COO:
+            assert lib.mcsparseCreateCoo(ctypes.byref(self.A), m, n, nnz, FAKE, FAKE, FAKE, idx[0], 0, vt) == 0
+        else:
+            mk = lib.mcsparseCreateCsr if fmt == api.FORMAT_CSR else lib.mcsparseCreateCsc
+            assert mk(ctypes.byref(self.A), m, n, nnz, FAKE, FAKE, FAKE, idx[0], idx[1], 0, vt) == 0
         self.x, self.y, self.xm = ctypes.c_void_p(), ctypes.c_void_p(), ctypes.c_void_p()
         lib.mcsparseCreateDnVec(ctypes.byref(self.x), n, FAKE, vt)
         lib.mcsparseCreateDnVec(ctypes.byref(self.y), m, FAKE, vt)
@@ -206,6 +224,9 @@ def test_spmv_buffer_size(lib):
     assert bigger.spmv_size(op=api.OP_T, x="y", y="x")[1] > t_size  # monotone in nnz
     csc = Objs(lib, m=1000, n=800, nnz=16000, fmt=api.FORMAT_CSC)
     assert csc.spmv_size()[1] > csc.spmv_size(op=api.OP_T, x="y", y="x")[1]  # CSC op N is the transposing case
+    coo = Objs(lib, m=1000, n=800, nnz=16000, fmt=api.FORMAT_COO)
+    assert coo.spmv_size()[1] >= n_size + 1001 * 4  # row offsets are rebuilt in the buffer
+    assert coo.spmv_size(op=api.OP_T, x="y", y="x")[1] >= t_size + 1001 * 4
 
 
 def test_spmm_argument_checks(lib):
@@ -231,6 +252,12 @@ def test_spmm_argument_checks(lib):
     assert lib.mcsparseSpMM_bufferSize(None, 0, 0, o.pa, o.A, B, o.pa, C, api.R_32F, 0, ctypes.byref(size)) == 1
     assert lib.mcsparseSpMM_bufferSize(o.h, 0, 0, o.pa, o.A, None, o.pa, C, api.R_32F, 0, ctypes.byref(size)) == 3
     assert lib.mcsparseSpMM_preprocess(o.h, 0, 0, o.pa, o.A, B, o.pa, C, api.R_32F, 0, FAKE) == 0  # no-op (:965-970)
+    for f, need in ((api.FORMAT_COO, 9 * 4), (api.FORMAT_CSC, (9 + 20) * 4 + 20 * 4)):
+        o2 = Objs(lib, m=8, n=6, nnz=20, fmt=f)
+        assert lib.mcsparseSpMM_bufferSize(o2.h, 0, 0, o2.pa, o2.A, B, o2.pa, C, api.R_32F, 0, ctypes.byref(size)) == 0
+        assert size.value >= need and size.value % 128 == 0
+        assert lib.mcsparseSpMM(o2.h, api.OP_T, 0, o2.pa, o2.A, B, o2.pa, C, api.R_32F, 0, FAKE) == 10
+        assert lib.mcsparseSpMM(o2.h, 0, 0, o2.pa, o2.A, B, o2.pa, C, api.R_32F, 0, None) == 3
     # nnz == 0 with beta == 1 returns before any launch (:110-114)
     e = Objs(lib, m=8, n=6, nnz=0)
     assert lib.mcsparseSpMM(e.h, 0, 0, e.pa, e.A, B, e.pa, C, api.R_32F, 0, FAKE) == 0
