@@ -357,6 +357,37 @@ mcsparseStatus_t mcsparseCsr2cscEx2_bufferSize(mcsparseHandle_t handle, int m, i
                                                mcsparseAction_t csc_action, mcsparseIndexBase_t idx_base,
                                                mcsparseCsr2CscAlg_t alg, size_t* buffer_size);
 
+/* ---- index sorts: include/interface/mcsp_conversion.h:65-107 ------------------------ *
+ * All sorts are stable and in place.  perm may be NULL; otherwise it holds nnz entries that
+ * move with their nonzeros, so after `mcsparseCreateIdentityPermutation` followed by a sort
+ * perm[i] is the old position of the entry now at i, and `mcsparse{S,D}gthr` through it puts
+ * the values in the new order.  The scratch size depends on nnz only. */
+/* Sorts the column indices inside every row.                                     :66, :69 */
+mcsparseStatus_t mcsparseXcsrsort_bufferSizeExt(mcsparseHandle_t handle, int m, int n, int nnz, const int* csr_rows,
+                                                const int* csr_cols, size_t* buffer_size);
+mcsparseStatus_t mcsparseXcsrsort(mcsparseHandle_t handle, int m, int n, int nnz, mcsparseMatDescr_t mcsp_descr_A,
+                                  const int* csr_rows, int* csr_cols, int* perm, void* temp_buffer);
+/* Sorts the row indices inside every column.                                     :90, :93 */
+mcsparseStatus_t mcsparseXcscsort_bufferSizeExt(mcsparseHandle_t handle, int m, int n, int nnz, const int* csc_cols,
+                                                const int* csc_rows, size_t* buffer_size);
+mcsparseStatus_t mcsparseXcscsort(mcsparseHandle_t handle, int m, int n, int nnz, mcsparseMatDescr_t mcsp_descr_A,
+                                  const int* csc_cols, int* csc_rows, int* perm, void* temp_buffer);
+/* Sort COO entries by (row, column) or by (column, row); indices may be zero- or one-based.
+ *                                                                           :97, :100, :103 */
+mcsparseStatus_t mcsparseXcoosort_bufferSizeExt(mcsparseHandle_t handle, int m, int n, int nnz, const int* coo_rows,
+                                                const int* coo_cols, size_t* buffer_size);
+mcsparseStatus_t mcsparseXcoosortByRow(mcsparseHandle_t handle, int m, int n, int nnz, int* coo_rows, int* coo_cols,
+                                       int* perm, void* temp_buffer);
+mcsparseStatus_t mcsparseXcoosortByColumn(mcsparseHandle_t handle, int m, int n, int nnz, int* coo_rows,
+                                          int* coo_cols, int* perm, void* temp_buffer);
+/* p[i] = i for i < n.                                                            :107 */
+mcsparseStatus_t mcsparseCreateIdentityPermutation(mcsparseHandle_t handle, int n, int* p);
+/* x_val[i] = y[x_ind[i] - idx_base]: include/interface/mcsp_level1.h:25-29 */
+mcsparseStatus_t mcsparseSgthr(mcsparseHandle_t handle, int nnz, const float* y, float* x_val, const int* x_ind,
+                               mcsparseIndexBase_t idx_base);
+mcsparseStatus_t mcsparseDgthr(mcsparseHandle_t handle, int nnz, const double* y, double* x_val, const int* x_ind,
+                               mcsparseIndexBase_t idx_base);
+
 /* ---- EXTENSIONS (no counterpart in the reference) ---------------------------------- */
 
 /* Number of row-length classes: class 0 holds empty rows, class b >= 1 holds rows whose

@@ -61,6 +61,16 @@ PROTOTYPES = {
     "mcsparseCsr2cscEx2": (c_int, [vp, c_int, c_int, c_int, vp, vp, vp, vp, vp, vp, c_int, c_int, c_int, c_int, vp]),
     "mcsparseCsr2cscEx2_bufferSize": (c_int, [vp, c_int, c_int, c_int, vp, vp, vp, vp, vp, vp, c_int, c_int, c_int,
                                               c_int, P(c_size)]),
+    "mcsparseXcsrsort_bufferSizeExt": (c_int, [vp, c_int, c_int, c_int, vp, vp, P(c_size)]),
+    "mcsparseXcsrsort": (c_int, [vp, c_int, c_int, c_int, vp, vp, vp, vp, vp]),
+    "mcsparseXcscsort_bufferSizeExt": (c_int, [vp, c_int, c_int, c_int, vp, vp, P(c_size)]),
+    "mcsparseXcscsort": (c_int, [vp, c_int, c_int, c_int, vp, vp, vp, vp, vp]),
+    "mcsparseXcoosort_bufferSizeExt": (c_int, [vp, c_int, c_int, c_int, vp, vp, P(c_size)]),
+    "mcsparseXcoosortByRow": (c_int, [vp, c_int, c_int, c_int, vp, vp, vp, vp]),
+    "mcsparseXcoosortByColumn": (c_int, [vp, c_int, c_int, c_int, vp, vp, vp, vp]),
+    "mcsparseCreateIdentityPermutation": (c_int, [vp, c_int, vp]),
+    "mcsparseSgthr": (c_int, [vp, c_int, vp, vp, vp, c_int]),
+    "mcsparseDgthr": (c_int, [vp, c_int, vp, vp, vp, c_int]),
     "mcsparseCreateMatDescr": (c_int, [P(vp)]),
     "mcsparseDestroyMatDescr": (c_int, [vp]),
     "mcsparseCopyMatDescr": (c_int, [vp, vp]),

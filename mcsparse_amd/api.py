@@ -262,3 +262,41 @@ def csr2csc(handle, m, n, nnz, csr_val, csr_rows, csr_cols, csc_val, csc_cols, c
 
 def csr_row_bins(handle, m, csr_rows, base, row_bins, bin_hist):
     return handle.lib.mcsparseXcsrRowBins(handle.ptr, m, _ptr(csr_rows), base, _ptr(row_bins), _ptr(bin_hist))
+
+
+def sort_buffer_size(handle, kind, m, n, nnz, a, b):
+    """kind is "csr", "csc" or "coo"; a, b are the two index arrays of that structure."""
+    fn = {"csr": handle.lib.mcsparseXcsrsort_bufferSizeExt, "csc": handle.lib.mcsparseXcscsort_bufferSizeExt,
+          "coo": handle.lib.mcsparseXcoosort_bufferSizeExt}[kind]
+    size = ctypes.c_size_t(0)
+    st = fn(handle.ptr, m, n, nnz, _ptr(a), _ptr(b), ctypes.byref(size))
+    return st, size.value
+
+
+def xcsrsort(handle, m, n, nnz, descr, csr_rows, csr_cols, perm, buffer):
+    return handle.lib.mcsparseXcsrsort(handle.ptr, m, n, nnz, descr, _ptr(csr_rows), _ptr(csr_cols), _ptr(perm),
+                                       _ptr(buffer))
+
+
+def xcscsort(handle, m, n, nnz, descr, csc_cols, csc_rows, perm, buffer):
+    return handle.lib.mcsparseXcscsort(handle.ptr, m, n, nnz, descr, _ptr(csc_cols), _ptr(csc_rows), _ptr(perm),
+                                       _ptr(buffer))
+
+
+def xcoosort_by_row(handle, m, n, nnz, coo_rows, coo_cols, perm, buffer):
+    return handle.lib.mcsparseXcoosortByRow(handle.ptr, m, n, nnz, _ptr(coo_rows), _ptr(coo_cols), _ptr(perm),
+                                            _ptr(buffer))
+
+
+def xcoosort_by_column(handle, m, n, nnz, coo_rows, coo_cols, perm, buffer):
+    return handle.lib.mcsparseXcoosortByColumn(handle.ptr, m, n, nnz, _ptr(coo_rows), _ptr(coo_cols), _ptr(perm),
+                                               _ptr(buffer))
+
+
+def create_identity_permutation(handle, n, p):
+    return handle.lib.mcsparseCreateIdentityPermutation(handle.ptr, n, _ptr(p))
+
+
+def gthr(handle, nnz, y, x_val, x_ind, base):
+    fn = handle.lib.mcsparseSgthr if maca_type(x_val.dtype) == R_32F else handle.lib.mcsparseDgthr
+    return fn(handle.ptr, nnz, _ptr(y), _ptr(x_val), _ptr(x_ind), base)

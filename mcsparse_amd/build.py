@@ -8,7 +8,7 @@ INCLUDE = os.path.join(os.path.dirname(HERE), "include")
 LIB_DIR = os.path.join(HERE, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libmcsparse.so")
 
-SOURCES = ["api_helper.cpp", "api_compute.cpp", "api_legacy.cpp", "analysis.hip", "spmv.hip", "spmm.hip", "convert.hip"]
+SOURCES = ["api_helper.cpp", "api_compute.cpp", "api_legacy.cpp", "api_sort.cpp", "analysis.hip", "spmv.hip", "spmm.hip", "convert.hip"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950",

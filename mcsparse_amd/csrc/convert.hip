@@ -415,6 +415,55 @@ __global__ __launch_bounds__(kSortBlock) void radix_scatter_kernel(
 
 uint32_t sort_tiles(idx_t nnz) { return static_cast<uint32_t>((static_cast<uint64_t>(nnz) + kSortTile - 1) / kSortTile); }
 
+size_t sort_counter_elems(idx_t count) { return static_cast<size_t>(kMaxRadix) * sort_tiles(count); }
+
+// Temporaries of one sort: two sets of (keys, aux, values) that the passes alternate between,
+// the per-(digit, tile) counters and the scratch of their scan.
+struct SortScratch {
+    idx_t* keys[2];
+    idx_t* aux[2];
+    void* vals[2];
+    uint32_t* counters;
+    uint32_t* scan_ws;
+};
+
+// Stable LSD radix sort of (key, aux, value) triples on the low key_bits of the keys, in
+// ceil(key_bits / 8) passes of equal width.  The last pass writes keys_out / aux_out / vals_out,
+// which must not overlap the inputs.  value_bytes is 0 (no values), 4 or 8.
+void radix_sort_triples(hipStream_t stream, idx_t count, uint32_t key_bits, const idx_t* keys_in, const idx_t* aux_in,
+                        const void* vals_in, idx_t* keys_out, idx_t* aux_out, void* vals_out, size_t value_bytes,
+                        const SortScratch& t) {
+    const uint32_t passes = key_bits == 0 ? 1 : (key_bits + 7) / 8;
+    const uint32_t bits = key_bits == 0 ? 1 : (key_bits + passes - 1) / passes;
+    const uint32_t radix = 1u << bits;
+    const uint32_t tiles = sort_tiles(count);
+    const uint32_t scatter_grid = (tiles + kXcds - 1) / kXcds * kXcds;
+    uint32_t shift = 0;
+    for (uint32_t p = 0; p < passes; ++p) {
+        const bool last = p + 1 == passes;
+        idx_t* k_out = last ? keys_out : t.keys[p & 1];
+        idx_t* a_out = last ? aux_out : t.aux[p & 1];
+        void* v_out = last ? vals_out : t.vals[p & 1];
+        hipLaunchKernelGGL(radix_hist_kernel, dim3(tiles), dim3(kHistBlock), 0, stream, keys_in, count, shift, bits,
+                           tiles, t.counters);
+        launch_exclusive_scan(stream, t.counters, static_cast<uint64_t>(radix) * tiles, t.scan_ws);
+        if (value_bytes == 0) {
+            hipLaunchKernelGGL((radix_scatter_kernel<0>), dim3(scatter_grid), dim3(kSortBlock), 0, stream, keys_in, aux_in,
+                               vals_in, k_out, a_out, v_out, count, shift, bits, tiles, t.counters);
+        } else if (value_bytes == 4) {
+            hipLaunchKernelGGL((radix_scatter_kernel<4>), dim3(scatter_grid), dim3(kSortBlock), 0, stream, keys_in, aux_in,
+                               vals_in, k_out, a_out, v_out, count, shift, bits, tiles, t.counters);
+        } else {
+            hipLaunchKernelGGL((radix_scatter_kernel<8>), dim3(scatter_grid), dim3(kSortBlock), 0, stream, keys_in, aux_in,
+                               vals_in, k_out, a_out, v_out, count, shift, bits, tiles, t.counters);
+        }
+        keys_in = k_out;
+        aux_in = a_out;
+        vals_in = v_out;
+        shift += bits;
+    }
+}
+
 struct Csr2CscLayout {
     size_t coo_rows, sorted_keys, keys_a, rows_a, vals_a, keys_b, rows_b, vals_b, counters, scan_ws, total;
 };
@@ -423,7 +472,7 @@ Csr2CscLayout csr2csc_layout(idx_t nnz, size_t value_bytes) {
     Csr2CscLayout l;
     const size_t idx_bytes = align_up(static_cast<size_t>(nnz) * sizeof(idx_t));
     const size_t val_bytes = align_up(static_cast<size_t>(nnz) * value_bytes);
-    const size_t counter_elems = static_cast<size_t>(kMaxRadix) * sort_tiles(nnz);
+    const size_t counter_elems = sort_counter_elems(nnz);
     size_t off = 0;
     l.coo_rows = off; off += idx_bytes;
     l.sorted_keys = off; off += idx_bytes;
@@ -437,6 +486,65 @@ Csr2CscLayout csr2csc_layout(idx_t nnz, size_t value_bytes) {
     l.scan_ws = off; off += align_up(scan_workspace_elems(counter_elems) * sizeof(uint32_t)) + kAlign;
     l.total = off;
     return l;
+}
+
+// Scratch of the index sorts: three sets of (keys, aux, permutation) -- the two the passes
+// alternate between and the result of the minor-key sort -- plus one spare index array.
+struct IndexSortLayout {
+    size_t set[3][3];
+    size_t spare, counters, scan_ws, total;
+};
+
+IndexSortLayout index_sort_layout(idx_t nnz) {
+    IndexSortLayout l;
+    const size_t idx_bytes = align_up(static_cast<size_t>(nnz) * sizeof(idx_t));
+    const size_t counter_elems = sort_counter_elems(nnz);
+    size_t off = 0;
+    for (int s = 0; s < 3; ++s) {
+        for (int a = 0; a < 3; ++a) {
+            l.set[s][a] = off;
+            off += idx_bytes;
+        }
+    }
+    l.spare = off; off += idx_bytes;
+    l.counters = off; off += align_up(counter_elems * sizeof(uint32_t));
+    l.scan_ws = off; off += align_up(scan_workspace_elems(counter_elems) * sizeof(uint32_t)) + kAlign;
+    l.total = off;
+    return l;
+}
+
+// Sorts (major, minor, perm) triples by (major, minor): a stable sort on the minor key followed
+// by a stable sort on the major key.  Outputs may be the input arrays themselves: both sorts
+// write to arrays their own inputs do not overlap.  perm_in == nullptr sorts without a payload.
+void sort_by_two_keys(hipStream_t stream, idx_t nnz, uint32_t major_bits, uint32_t minor_bits, const idx_t* major_in,
+                      const idx_t* minor_in, const idx_t* perm_in, idx_t* major_out, idx_t* minor_out, idx_t* perm_out,
+                      char* w, const IndexSortLayout& l) {
+    SortScratch t;
+    for (int s = 0; s < 2; ++s) {
+        t.keys[s] = reinterpret_cast<idx_t*>(w + l.set[s][0]);
+        t.aux[s] = reinterpret_cast<idx_t*>(w + l.set[s][1]);
+        t.vals[s] = w + l.set[s][2];
+    }
+    t.counters = reinterpret_cast<uint32_t*>(w + l.counters);
+    t.scan_ws = reinterpret_cast<uint32_t*>(w + l.scan_ws);
+    idx_t* mid_minor = reinterpret_cast<idx_t*>(w + l.set[2][0]);
+    idx_t* mid_major = reinterpret_cast<idx_t*>(w + l.set[2][1]);
+    idx_t* mid_perm = reinterpret_cast<idx_t*>(w + l.set[2][2]);
+    const size_t vb = perm_in != nullptr ? sizeof(idx_t) : 0;
+    radix_sort_triples(stream, nnz, minor_bits, minor_in, major_in, perm_in, mid_minor, mid_major, mid_perm, vb, t);
+    radix_sort_triples(stream, nnz, major_bits, mid_major, mid_minor, mid_perm, major_out, minor_out, perm_out, vb, t);
+}
+
+__global__ __launch_bounds__(kBlock) void identity_kernel(idx_t n, idx_t* __restrict__ p) {
+    const uint64_t i = static_cast<uint64_t>(blockIdx.x) * kBlock + threadIdx.x;
+    if (i < static_cast<uint64_t>(n)) p[i] = static_cast<idx_t>(i);
+}
+
+template <typename T>
+__global__ __launch_bounds__(kBlock) void gather_kernel(idx_t nnz, const T* __restrict__ y, T* __restrict__ x_val,
+                                                        const idx_t* __restrict__ x_ind, idx_t base) {
+    const uint64_t i = static_cast<uint64_t>(blockIdx.x) * kBlock + threadIdx.x;
+    if (i < static_cast<uint64_t>(nnz)) x_val[i] = y[load_stream(x_ind + i) - base];
 }
 
 }  // namespace
@@ -475,42 +583,54 @@ void launch_csr2csc(hipStream_t stream, idx_t m, idx_t n, idx_t nnz, const void*
     launch_csr2coo(stream, m, nnz, row_ptr, base, coo_rows);
 
     // keys are the raw column indices (index base included), so the largest key is n - 1 + base
-    const uint32_t key_bits = bit_length(n - 1 + base);
-    const uint32_t passes = key_bits == 0 ? 1 : (key_bits + 7) / 8;
-    const uint32_t bits_per_pass = key_bits == 0 ? 1 : (key_bits + passes - 1) / passes;
-    const uint32_t tiles = sort_tiles(nnz);
-
-    const idx_t* keys_in = col;
-    const idx_t* rows_in = coo_rows;
-    const void* vals_in = csr_val;
-    uint32_t shift = 0;
-    for (uint32_t p = 0; p < passes; ++p) {
-        const bool last = p + 1 == passes;
-        idx_t* keys_out = last ? sorted_keys : keys_t[p & 1];
-        idx_t* rows_out = last ? row_ind : rows_t[p & 1];
-        void* vals_out = last ? csc_val : vals_t[p & 1];
-        const uint32_t bits = bits_per_pass;
-        const uint32_t radix = 1u << bits;
-        const uint32_t scatter_grid = (tiles + kXcds - 1) / kXcds * kXcds;
-        hipLaunchKernelGGL(radix_hist_kernel, dim3(tiles), dim3(kHistBlock), 0, stream, keys_in, nnz, shift, bits, tiles,
-                           counters);
-        launch_exclusive_scan(stream, counters, static_cast<uint64_t>(radix) * tiles, scan_ws);
-        if (value_bytes == 0) {
-            hipLaunchKernelGGL((radix_scatter_kernel<0>), dim3(scatter_grid), dim3(kSortBlock), 0, stream, keys_in, rows_in,
-                               vals_in, keys_out, rows_out, vals_out, nnz, shift, bits, tiles, counters);
-        } else if (value_bytes == 4) {
-            hipLaunchKernelGGL((radix_scatter_kernel<4>), dim3(scatter_grid), dim3(kSortBlock), 0, stream, keys_in, rows_in,
-                               vals_in, keys_out, rows_out, vals_out, nnz, shift, bits, tiles, counters);
-        } else {
-            hipLaunchKernelGGL((radix_scatter_kernel<8>), dim3(scatter_grid), dim3(kSortBlock), 0, stream, keys_in, rows_in,
-                               vals_in, keys_out, rows_out, vals_out, nnz, shift, bits, tiles, counters);
-        }
-        keys_in = keys_out;
-        rows_in = rows_out;
-        vals_in = vals_out;
-        shift += bits;
+    SortScratch t;
+    for (int i = 0; i < 2; ++i) {
+        t.keys[i] = keys_t[i];
+        t.aux[i] = rows_t[i];
+        t.vals[i] = vals_t[i];
     }
+    t.counters = counters;
+    t.scan_ws = scan_ws;
+    radix_sort_triples(stream, nnz, bit_length(n - 1 + base), col, coo_rows, csr_val, sorted_keys, row_ind, csc_val,
+                       value_bytes, t);
     launch_coo2csr(stream, nnz, n, sorted_keys, base, col_ptr);
 }
+
+size_t index_sort_workspace_bytes(idx_t nnz) { return index_sort_layout(nnz).total; }
+
+void launch_coosort(hipStream_t stream, idx_t major_extent, idx_t minor_extent, idx_t nnz, idx_t* major, idx_t* minor,
+                    idx_t* perm, void* workspace) {
+    if (nnz == 0) return;
+    // indices may be zero- or one-based: keys reach the extent itself in the second case
+    sort_by_two_keys(stream, nnz, bit_length(major_extent), bit_length(minor_extent), major, minor, perm, major, minor,
+                     perm, static_cast<char*>(workspace), index_sort_layout(nnz));
+}
+
+void launch_csrsort(hipStream_t stream, idx_t m, idx_t n, idx_t nnz, idx_t base, const idx_t* row_ptr, idx_t* col,
+                    idx_t* perm, void* workspace) {
+    if (m == 0 || n == 0 || nnz == 0) return;
+    const IndexSortLayout l = index_sort_layout(nnz);
+    char* w = static_cast<char*>(workspace);
+    idx_t* rows = reinterpret_cast<idx_t*>(w + l.spare);  // row of every entry, then the sorted rows
+    launch_csr2coo(stream, m, nnz, row_ptr, base, rows);
+    sort_by_two_keys(stream, nnz, bit_length(m - 1 + base), bit_length(n - 1 + base), rows, col, perm, rows, col, perm,
+                     w, l);
+}
+
+void launch_identity(hipStream_t stream, idx_t n, idx_t* p) {
+    if (n == 0) return;
+    hipLaunchKernelGGL(identity_kernel, dim3((static_cast<uint32_t>(n) + kBlock - 1) / kBlock), dim3(kBlock), 0, stream,
+                       n, p);
+}
+
+template <typename T>
+void launch_gather(hipStream_t stream, idx_t nnz, const T* y, T* x_val, const idx_t* x_ind, idx_t base) {
+    if (nnz == 0) return;
+    hipLaunchKernelGGL((gather_kernel<T>), dim3((static_cast<uint32_t>(nnz) + kBlock - 1) / kBlock), dim3(kBlock), 0,
+                       stream, nnz, y, x_val, x_ind, base);
+}
+
+template void launch_gather<float>(hipStream_t, idx_t, const float*, float*, const idx_t*, idx_t);
+template void launch_gather<double>(hipStream_t, idx_t, const double*, double*, const idx_t*, idx_t);
 
 }  // namespace mcsp

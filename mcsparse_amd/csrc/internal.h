@@ -195,6 +195,20 @@ void launch_csr2csc(hipStream_t stream, idx_t m, idx_t n, idx_t nnz, const void*
                     const idx_t* col, void* csc_val, idx_t* row_ind, idx_t* col_ptr, size_t value_bytes,
                     idx_t base, void* workspace);
 
+// ---- index sorts (convert.hip) --------------------------------------------------------------
+size_t index_sort_workspace_bytes(idx_t nnz);
+// In-place stable sort of COO entries by (major, minor); perm (may be null) moves with them.
+// The extents bound the index values (inclusive, so one-based indices are covered).
+void launch_coosort(hipStream_t stream, idx_t major_extent, idx_t minor_extent, idx_t nnz, idx_t* major, idx_t* minor,
+                    idx_t* perm, void* workspace);
+// Sorts the column indices inside every row of a CSR structure; perm (may be null) moves along.
+void launch_csrsort(hipStream_t stream, idx_t m, idx_t n, idx_t nnz, idx_t base, const idx_t* row_ptr, idx_t* col,
+                    idx_t* perm, void* workspace);
+void launch_identity(hipStream_t stream, idx_t n, idx_t* p);
+// x_val[i] = y[x_ind[i] - base]
+template <typename T>
+void launch_gather(hipStream_t stream, idx_t nnz, const T* y, T* x_val, const idx_t* x_ind, idx_t base);
+
 }  // namespace mcsp
 
 #endif  // MCSPARSE_AMD_INTERNAL_H_

@@ -121,6 +121,28 @@ def csr2csc(m, n, base, ptr, col, val=None, method="radix2"):
     return col_ptr, row_ind, csc_val
 
 
+def coosort(major_extent, minor_extent, major, minor, perm=None):
+    """Stable sort by (major, minor); returns new (major, minor, perm) arrays, perm None if not given."""
+    major, minor = _idx(major).copy(), _idx(minor).copy()
+    perm = None if perm is None else _idx(perm).copy()
+    fn = lib().orc_coosort
+    fn.restype = _c_int
+    if fn(_c_i64(major_extent), _c_i64(minor_extent), _c_i64(major.shape[0]), _p(major), _p(minor), _p(perm)) != 0:
+        raise MemoryError("oracle coosort")
+    return major, minor, perm
+
+
+def csrsort(m, n, base, ptr, col, perm=None):
+    """Sorts the columns inside every row; returns new (col, perm) arrays."""
+    ptr, col = _idx(ptr), _idx(col).copy()
+    perm = None if perm is None else _idx(perm).copy()
+    fn = lib().orc_csrsort
+    fn.restype = _c_int
+    if fn(_c_i64(m), _c_i64(n), _c_i64(col.shape[0]), _c_int(base), _p(ptr), _p(col), _p(perm)) != 0:
+        raise MemoryError("oracle csrsort")
+    return col, perm
+
+
 def row_bins(m, ptr):
     """Returns (row_bins uint8[m], hist uint32[34])."""
     ptr = _idx(ptr)

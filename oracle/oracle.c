@@ -205,6 +205,59 @@ int orc_csr2csc_counting(int64_t m, int64_t n, int64_t nnz, int base, const idx_
 }
 
 /* ------------------------------------------------------------------------------------------
+ * Index sorts.  The reference sorts (minor key, permutation) pairs, gathers the major keys
+ * through the result, sorts (major key, permutation) pairs and gathers again
+ * (src/kernels/conversion/mcsp_coosort.cpp:63-106, mcsp_csrsort.cpp:66-115): two stable sorts,
+ * minor key first.  Restated with stable counting sorts.  perm may be NULL.
+ * keys are compared as stored (an index base is simply part of the key).
+ * ------------------------------------------------------------------------------------------ */
+static int stable_counting_pass(int64_t nnz, int64_t extent, const idx_t* key, const int64_t* order_in,
+                                int64_t* order_out) {
+    int64_t* next = (int64_t*)calloc((size_t)extent + 2, sizeof(int64_t));
+    if (!next) return -1;
+    for (int64_t j = 0; j < nnz; ++j) ++next[(int64_t)key[j] + 1];
+    for (int64_t k = 0; k <= extent; ++k) next[k + 1] += next[k];
+    for (int64_t j = 0; j < nnz; ++j) {
+        const int64_t src = order_in[j];
+        order_out[next[key[src]]++] = src;
+    }
+    free(next);
+    return 0;
+}
+
+int orc_coosort(int64_t major_extent, int64_t minor_extent, int64_t nnz, idx_t* major, idx_t* minor, idx_t* perm) {
+    if (nnz == 0) return 0;
+    int64_t* o0 = (int64_t*)malloc((size_t)nnz * sizeof(int64_t));
+    int64_t* o1 = (int64_t*)malloc((size_t)nnz * sizeof(int64_t));
+    idx_t* tmp = (idx_t*)malloc((size_t)nnz * sizeof(idx_t));
+    if (!o0 || !o1 || !tmp) return -1;
+    for (int64_t j = 0; j < nnz; ++j) o0[j] = j;
+    if (stable_counting_pass(nnz, minor_extent, minor, o0, o1)) return -1;
+    if (stable_counting_pass(nnz, major_extent, major, o1, o0)) return -1;
+    idx_t* arrays[3] = {major, minor, perm};
+    for (int a = 0; a < 3; ++a) {
+        if (!arrays[a]) continue;
+        for (int64_t j = 0; j < nnz; ++j) tmp[j] = arrays[a][o0[j]];
+        memcpy(arrays[a], tmp, (size_t)nnz * sizeof(idx_t));
+    }
+    free(o0);
+    free(o1);
+    free(tmp);
+    return 0;
+}
+
+/* mcsp_csrsort.cpp:43-121: csr2coo, then the two-key sort; the sorted row indices are dropped. */
+int orc_csrsort(int64_t m, int64_t n, int64_t nnz, int base, const idx_t* ptr, idx_t* col, idx_t* perm) {
+    if (m == 0 || n == 0 || nnz == 0) return 0;
+    idx_t* rows = (idx_t*)malloc((size_t)nnz * sizeof(idx_t));
+    if (!rows) return -1;
+    orc_csr2coo(m, base, ptr, rows);
+    const int rc = orc_coosort(m + base, n + base, nnz, rows, col, perm);
+    free(rows);
+    return rc;
+}
+
+/* ------------------------------------------------------------------------------------------
  * Row-length classes used by the GPU library's SpMV dispatch (no counterpart in the
  * reference): class 0 = empty row, class b >= 1 = length in [2^(b-1), 2^b).
  * hist: 33 class counters followed by the longest row length.

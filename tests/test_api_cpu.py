@@ -124,7 +124,7 @@ def test_sparse_descriptors(lib):
     assert lib.mcsparseCscSetPointers(d, 0x51, 0x61, 0x71) == 0
     assert lib.mcsparseCscSetPointers(None, 0x51, 0x61, 0x71) == api.STATUS_INVALID_VALUE
     assert lib.mcsparseDestroySpMat(d) == 0
-    # COO: one index type for both arrays (mcsp_helper.cpp:526-585)
+    # COO: one index type for both arrays (mcsp_helper.cpp:433-445, :526-549, :597-607)
     mkc = lib.mcsparseCreateCoo
     assert mkc(ctypes.byref(d), 3, -4, 5, 0x10, 0x20, 0x30, 2, 0, api.R_32F) == api.STATUS_INVALID_VALUE
     assert mkc(None, 3, 4, 5, 0x10, 0x20, 0x30, 2, 0, api.R_32F) == api.STATUS_INVALID_VALUE
@@ -306,3 +306,43 @@ def test_plan_override_api(lib):
     assert lib.mcsparseSpMatSetSpMVPlan(o.A, 1, 3) == api.STATUS_INVALID_VALUE  # lanes must be a power of two
     assert lib.mcsparseSpMatSetSpMVPlan(o.A, 1, 16) == 0
     assert lib.mcsparseSpMatSetSpMVPlan(None, 1, 16) == api.STATUS_INVALID_VALUE
+
+
+def test_sort_argument_checks(lib):
+    # conversion/mcsp_csrsort.cpp:13-64, mcsp_coosort.cpp:12-61, mcsp_create_identity.cpp:6-20, level1/mcsp_gthr.cpp:7-23
+    o = Objs(lib)
+    d = ctypes.c_void_p()
+    assert lib.mcsparseCreateMatDescr(ctypes.byref(d)) == 0
+    size = ctypes.c_size_t()
+    for fn in (lib.mcsparseXcsrsort_bufferSizeExt, lib.mcsparseXcscsort_bufferSizeExt, lib.mcsparseXcoosort_bufferSizeExt):
+        assert fn(None, 4, 4, 8, FAKE, FAKE, ctypes.byref(size)) == api.STATUS_NOT_INITIALIZED
+        assert fn(o.h, -1, 4, 8, FAKE, FAKE, ctypes.byref(size)) == api.STATUS_INVALID_VALUE
+        assert fn(o.h, 4, 4, 8, None, FAKE, ctypes.byref(size)) == api.STATUS_INVALID_VALUE
+        assert fn(o.h, 4, 4, 8, FAKE, FAKE, None) == api.STATUS_INVALID_VALUE
+        assert fn(o.h, 4, 4, 0, FAKE, FAKE, ctypes.byref(size)) == 0 and size.value == 128
+        assert fn(o.h, 4, 4, 5000, FAKE, FAKE, ctypes.byref(size)) == 0
+        assert size.value % 128 == 0 and size.value >= 10 * 5000 * 4
+    for fn in (lib.mcsparseXcsrsort, lib.mcsparseXcscsort):
+        assert fn(None, 4, 4, 8, d, FAKE, FAKE, FAKE, FAKE) == api.STATUS_NOT_INITIALIZED
+        assert fn(o.h, 4, -4, 8, d, FAKE, FAKE, FAKE, FAKE) == api.STATUS_INVALID_VALUE
+        assert fn(o.h, 4, 4, 0, d, None, None, None, None) == 0  # empty: nothing is checked or touched
+        assert fn(o.h, 4, 4, 8, d, None, FAKE, FAKE, FAKE) == api.STATUS_INVALID_VALUE
+        assert fn(o.h, 4, 4, 8, d, FAKE, None, FAKE, FAKE) == api.STATUS_INVALID_VALUE
+        assert fn(o.h, 4, 4, 8, d, FAKE, FAKE, FAKE, None) == api.STATUS_INVALID_VALUE
+        assert fn(o.h, 4, 4, 8, None, FAKE, FAKE, FAKE, FAKE) == api.STATUS_INVALID_VALUE
+    for fn in (lib.mcsparseXcoosortByRow, lib.mcsparseXcoosortByColumn):
+        assert fn(None, 4, 4, 8, FAKE, FAKE, FAKE, FAKE) == api.STATUS_NOT_INITIALIZED
+        assert fn(o.h, 4, 4, -8, FAKE, FAKE, FAKE, FAKE) == api.STATUS_INVALID_VALUE
+        assert fn(o.h, 0, 4, 8, None, None, None, None) == 0
+        assert fn(o.h, 4, 4, 8, None, FAKE, FAKE, FAKE) == api.STATUS_INVALID_VALUE
+        assert fn(o.h, 4, 4, 8, FAKE, FAKE, FAKE, None) == api.STATUS_INVALID_VALUE
+    assert lib.mcsparseCreateIdentityPermutation(None, 4, FAKE) == api.STATUS_NOT_INITIALIZED
+    assert lib.mcsparseCreateIdentityPermutation(o.h, -4, FAKE) == api.STATUS_INVALID_VALUE
+    assert lib.mcsparseCreateIdentityPermutation(o.h, 4, None) == api.STATUS_INVALID_VALUE
+    assert lib.mcsparseCreateIdentityPermutation(o.h, 0, FAKE) == 0
+    for fn in (lib.mcsparseSgthr, lib.mcsparseDgthr):
+        assert fn(None, 4, FAKE, FAKE, FAKE, 0) == api.STATUS_NOT_INITIALIZED
+        assert fn(o.h, -4, FAKE, FAKE, FAKE, 0) == api.STATUS_INVALID_VALUE
+        assert fn(o.h, 0, None, None, None, 0) == 0
+        assert fn(o.h, 4, FAKE, None, FAKE, 0) == api.STATUS_INVALID_VALUE
+    lib.mcsparseDestroyMatDescr(d)

@@ -180,3 +180,45 @@ def test_row_bins_definition(oracle):
     ptr = np.array([0, 0, 1, 3, 7, 15, 16], dtype=np.int32)  # lengths 0 1 2 4 8 1
     bins, hist = oracle.row_bins(6, ptr)
     assert list(bins) == [0, 1, 2, 3, 4, 1] and hist[33] == 8
+
+
+def _shuffled_coo(rng, m, n, nnz, base, duplicates):
+    rows = rng.integers(0, m, nnz).astype(np.int32)
+    cols = rng.integers(0, n if not duplicates else max(1, n // 8), nnz).astype(np.int32)
+    return rows + base, cols + base
+
+
+@pytest.mark.parametrize("base", [0, 1])
+@pytest.mark.parametrize("duplicates", [False, True])
+def test_coosort_is_the_stable_lexicographic_sort(oracle, base, duplicates):
+    # numpy's lexsort is an independent stable sort; duplicate (row, col) pairs make stability visible in perm
+    rng = np.random.default_rng(11 + base)
+    m, n, nnz = 37, 53, 4000
+    rows, cols = _shuffled_coo(rng, m, n, nnz, base, duplicates)
+    perm0 = rng.permutation(nnz).astype(np.int32)  # not the identity: the sort must carry it, not recreate it
+    order = np.lexsort((cols, rows))
+    r, c, p = oracle.coosort(m + base, n + base, rows, cols, perm0)
+    assert np.array_equal(r.view(np.int32), rows[order]) and np.array_equal(c.view(np.int32), cols[order])
+    assert np.array_equal(p.view(np.int32), perm0[order])
+    r2, c2, p2 = oracle.coosort(m + base, n + base, rows, cols)
+    assert p2 is None and np.array_equal(r2, r) and np.array_equal(c2, c)
+    # by column: the same routine with the roles exchanged
+    order_c = np.lexsort((rows, cols))
+    c3, r3, p3 = oracle.coosort(n + base, m + base, cols, rows, perm0)
+    assert np.array_equal(r3.view(np.int32), rows[order_c]) and np.array_equal(p3.view(np.int32), perm0[order_c])
+
+
+@pytest.mark.parametrize("base", [0, 1])
+def test_csrsort_sorts_inside_rows_only(oracle, base):
+    rng = np.random.default_rng(5)
+    a = wl.random_ragged(300, 200, 7, dtype=np.float32, seed=3, empty_fraction=0.3).with_base(base)
+    col = a.col.copy()
+    for r in range(a.m):  # shuffle inside every row
+        s, e = a.ptr[r] - base, a.ptr[r + 1] - base
+        col[s:e] = rng.permutation(col[s:e])
+    ident = np.arange(a.nnz, dtype=np.int32)
+    sorted_col, perm = oracle.csrsort(a.m, a.n, base, a.ptr, col, ident)
+    assert np.array_equal(sorted_col.view(np.int32), a.col)  # the generator's columns are sorted and distinct
+    assert np.array_equal(col[perm.view(np.int32)], a.col)   # perm[i] = old position of the entry now at i
+    rows = np.repeat(np.arange(a.m), a.row_lengths())
+    assert np.array_equal(rows[perm.view(np.int32)], rows)   # nothing left its row
