@@ -43,6 +43,7 @@ def parse():
     p.add_argument("--copies", type=int, default=None, help="independent operand sets rotated between steps")
     p.add_argument("--scale", type=float, default=1.0, help="shrink the workload (for dry runs); 1.0 = as specified")
     p.add_argument("--no-cpu-baseline", action="store_true")
+    p.add_argument("--no-preprocess", action="store_true", help="SpMM workloads: skip mcsparseSpMM_preprocess")
     p.add_argument("--family", type=int, default=0, help="force the SpMV kernel family (1 vector, 2 merge)")
     p.add_argument("--lanes", type=int, default=0, help="force lanes per row of the vector family")
     p.add_argument("--cache", default=None, help="directory to keep generated matrices in between runs")
@@ -138,6 +139,7 @@ def main():
 
     rng = np.random.default_rng(12345)
     sets = []
+    preprocess_ms = []
     for c in range(copies):
         st = {"ptr": dev(a.ptr), "col": dev(a.col), "val": dev(a.val)}
         if kind == "spmv":
@@ -160,6 +162,13 @@ def main():
             rc, size = api.spmm_buffer_size(handle, api.OP_N, api.OP_N, alpha, st["mat"], st["mB"], beta, st["mC"], ct)
             api.check(rc, "mcsparseSpMM_bufferSize")
             st["buf"] = torch.empty(size, dtype=torch.uint8, device="cuda")
+            if not args.no_preprocess:
+                torch.cuda.synchronize()
+                t_pre = time.perf_counter()
+                api.check(api.spmm_preprocess(handle, api.OP_N, api.OP_N, alpha, st["mat"], st["mB"], beta, st["mC"],
+                                              ct, st["buf"]), "mcsparseSpMM_preprocess")
+                torch.cuda.synchronize()
+                preprocess_ms.append((time.perf_counter() - t_pre) * 1e3)
         elif kind in ("csr2csc", "spmv-csc"):
             st["o_val"] = torch.zeros(a.nnz, dtype=tdt, device="cuda")
             st["o_ptr"] = torch.zeros(a.n + 1, dtype=torch.int32, device="cuda")
@@ -253,6 +262,7 @@ def main():
         "algorithmic_bytes_per_step": int(algo_bytes),
         "extra_bytes_not_counted": int(extra_read),
         "first_call_ms": round(first_pass_ms, 4),
+        "spmm_preprocess_ms": round(min(preprocess_ms), 4) if preprocess_ms else None,
         "device_ms_per_step": {"mean": round(dev_avg_ms, 5), "median": round(float(np.median(dev_ms)), 5),
                                "min": round(float(dev_ms.min()), 5)},
         "spmv_plan": {"family": plan[0], "lanes_per_row": plan[1]} if plan else None,

@@ -410,6 +410,12 @@ mcsparseStatus_t mcsparseSpMatGetSpMVPlan(mcsparseSpMatDescr_t spMatDescr, int* 
 /* Forces the SpMV kernel family for a descriptor (0 = automatic).  For tests and benchmarks. */
 mcsparseStatus_t mcsparseSpMatSetSpMVPlan(mcsparseSpMatDescr_t spMatDescr, int family, int lanes_per_row);
 
+/* What mcsparseSpMM_preprocess left on a CSR descriptor:
+ * state 0 = no schedule, 1 = built but the rows share too few columns for it to pay off
+ * (SpMM ignores it), 2 = SpMM uses it when called with the same buffer and CSR arrays.
+ * merged_entries = total length of the merged column lists of all row pairs (compare with nnz). */
+mcsparseStatus_t mcsparseSpMatGetSpMMSchedule(mcsparseSpMatDescr_t spMatDescr, int* state, int64_t* merged_entries);
+
 #ifdef __cplusplus
 }
 #endif

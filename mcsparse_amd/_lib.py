@@ -99,6 +99,7 @@ PROTOTYPES = {
     "mcsparseXcsrRowBins": (c_int, [vp, c_int, vp, c_int, vp, vp]),
     "mcsparseSpMatGetSpMVPlan": (c_int, [vp, P(c_int), P(c_int)]),
     "mcsparseSpMatSetSpMVPlan": (c_int, [vp, c_int, c_int]),
+    "mcsparseSpMatGetSpMMSchedule": (c_int, [vp, P(c_int), P(c_i64)]),
 }
 
 _lib = None

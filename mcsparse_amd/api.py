@@ -133,6 +133,12 @@ class SpMat:
         check(self.lib.mcsparseSpMatGetSpMVPlan(self._d, ctypes.byref(fam), ctypes.byref(lanes)))
         return fam.value, lanes.value
 
+    def spmm_schedule(self):
+        """(state, merged_entries) left by mcsparseSpMM_preprocess; state 2 = in use."""
+        state, entries = ctypes.c_int(), ctypes.c_int64()
+        check(self.lib.mcsparseSpMatGetSpMMSchedule(self._d, ctypes.byref(state), ctypes.byref(entries)))
+        return state.value, entries.value
+
     def destroy(self):
         if self._d:
             self.lib.mcsparseDestroySpMat(self._d)
@@ -227,6 +233,12 @@ def spmm_buffer_size(handle, op_a, op_b, alpha, mat, B, beta, C, compute_type):
                                             ctypes.addressof(b), C.ptr, compute_type, SPMM_ALG_DEFAULT,
                                             ctypes.byref(size))
     return st, size.value
+
+
+def spmm_preprocess(handle, op_a, op_b, alpha, mat, B, beta, C, compute_type, buffer):
+    a, b = _scalar(alpha, compute_type), _scalar(beta, compute_type)
+    return handle.lib.mcsparseSpMM_preprocess(handle.ptr, op_a, op_b, ctypes.addressof(a), mat.ptr, B.ptr,
+                                              ctypes.addressof(b), C.ptr, compute_type, SPMM_ALG_DEFAULT, _ptr(buffer))
 
 
 def spmm(handle, op_a, op_b, alpha, mat, B, beta, C, compute_type, buffer):

@@ -228,17 +228,32 @@ mcspStatus_t spmv_typed(mcsparseHandle_t h, mcsparseSpMatDescr* A, CsrView v, co
     return MCSP_STATUS_SUCCESS;
 }
 
-// Scratch layout of an SpMM call: CSR needs none; COO gets [row offsets m+1]; CSC gets the
-// transposed copy [row_ptr m+1 | col_ind nnz][values][csr2csc workspace]
+// Scratch layout of an SpMM call: CSR gets room for the row-pair schedule that
+// mcsparseSpMM_preprocess builds (SpMM itself writes nothing there); COO gets [row offsets m+1];
+// CSC gets the transposed copy [row_ptr m+1 | col_ind nnz][values][csr2csc workspace]
 // (mcsp_spmm_gpu.cpp:818-849).
 struct SpmmLayout {
     size_t ptr, ind, vals, csr2csc_ws, total;
 };
 
+bool schedulable(const mcsparseSpMatDescr* A) {
+    return A->format == MCSPARSE_FORMAT_CSR && A->row_num > 0 && A->nnz > 0 &&
+           A->col_num <= mcsp::kSpmmMaxScheduledColumns;
+}
+
+// The schedule of the descriptor belongs to this call: same buffer, same arrays, same extents.
+bool schedule_matches(const mcsparseSpMatDescr* A, const void* buffer) {
+    const SpmmSchedule& s = A->schedule;
+    return s.valid && s.useful && s.buffer == buffer && s.rows == A->rows && s.cols == A->cols && s.m == A->row_num &&
+           s.nnz == A->nnz && s.base == static_cast<int>(A->idxBase);
+}
+
 SpmmLayout spmm_layout(const mcsparseSpMatDescr* A, size_t value_bytes) {
     SpmmLayout l = {};
     size_t off = 0;
-    if (A->format == MCSPARSE_FORMAT_COO) {
+    if (A->format == MCSPARSE_FORMAT_CSR) {
+        if (schedulable(A)) off += mcsp::spmm_schedule_layout(static_cast<idx_t>(A->row_num), static_cast<idx_t>(A->nnz)).total;
+    } else if (A->format == MCSPARSE_FORMAT_COO) {
         off += align_up(static_cast<size_t>(A->row_num + 1) * sizeof(idx_t));
     } else if (A->format == MCSPARSE_FORMAT_CSC) {
         l.ind = static_cast<size_t>(A->row_num + 1) * sizeof(idx_t);
@@ -302,7 +317,11 @@ mcspStatus_t spmm_typed(mcsparseHandle_t h, const mcsparseSpMatDescr* A, mcspars
     a.C = C->values;
     a.ldc = C->ld;
     a.c_row_major = C->order == MCSPARSE_ORDER_ROW;
-    mcsp::launch_spmm<T>(h->stream, a, h_alpha, h_beta);
+    if (schedule_matches(A, buffer) && mcsp::spmm_schedule_usable(a, sizeof(T))) {
+        mcsp::launch_spmm_scheduled<T>(h->stream, a, buffer, h_alpha, h_beta);
+    } else {
+        mcsp::launch_spmm<T>(h->stream, a, h_alpha, h_beta);
+    }
     return MCSP_STATUS_SUCCESS;
 }
 
@@ -404,10 +423,51 @@ mcsparseStatus_t mcsparseSpMM_bufferSize(mcsparseHandle_t handle, mcsparseOperat
     return MCSPARSE_STATUS_SUCCESS;
 }
 
-// reference: src/kernels/level3/spmm/mcsp_spmm_gpu.cpp:965-970 -- a no-op there as well
-mcsparseStatus_t mcsparseSpMM_preprocess(mcsparseHandle_t, mcsparseOperation_t, mcsparseOperation_t, const void*,
-                                         mcsparseSpMatDescr_t, mcsparseDnMatDescr_t, const void*,
-                                         mcsparseDnMatDescr_t, macaDataType, mcsparseSpMMAlg_t, void*) {
+// reference: src/kernels/level3/spmm/mcsp_spmm_gpu.cpp:965-970 -- a no-op there.  Here a CSR
+// matrix gets its row-pair schedule built into externalBuffer (sized by mcsparseSpMM_bufferSize);
+// mcsparseSpMM uses it when it is handed the same buffer and the same CSR arrays, and falls back
+// to the schedule-free kernel otherwise.  Until then the caller must leave the buffer and the
+// structure of A alone; the values of A may change freely.
+mcsparseStatus_t mcsparseSpMM_preprocess(mcsparseHandle_t handle, mcsparseOperation_t opA, mcsparseOperation_t /*opB*/,
+                                         const void* alpha, mcsparseSpMatDescr_t matA, mcsparseDnMatDescr_t matB,
+                                         const void* beta, mcsparseDnMatDescr_t matC, macaDataType /*computeType*/,
+                                         mcsparseSpMMAlg_t /*alg*/, void* externalBuffer) {
+    if (matA != nullptr) {
+        const mcspStatus_t it = check_index_types(matA);
+        if (it != MCSP_STATUS_SUCCESS) return to_public_status(it);
+    }
+    if (handle == nullptr) return to_public_status(MCSP_STATUS_INVALID_HANDLE);
+    if (externalBuffer == nullptr) return to_public_status(MCSP_STATUS_INVALID_POINTER);
+    const mcspStatus_t st = check_spmm_args(handle, alpha, matA, matB, beta, matC);
+    if (st != MCSP_STATUS_SUCCESS) return to_public_status(st);
+    matA->schedule.valid = false;
+    if (opA != MCSPARSE_OPERATION_NON_TRANSPOSE || !schedulable(matA) || matA->rows == nullptr || matA->cols == nullptr)
+        return MCSPARSE_STATUS_SUCCESS;  // nothing to prepare for this call
+
+    const idx_t m = static_cast<idx_t>(matA->row_num);
+    const idx_t nnz = static_cast<idx_t>(matA->nnz);
+    mcsp::launch_spmm_schedule(handle->stream, m, nnz, static_cast<idx_t>(matA->idxBase),
+                               static_cast<const idx_t*>(matA->rows), static_cast<const idx_t*>(matA->cols),
+                               externalBuffer);
+    const mcsp::SpmmScheduleLayout l = mcsp::spmm_schedule_layout(m, nnz);
+    const uint64_t pairs = (static_cast<uint64_t>(m) + 1) / 2;
+    uint32_t entries = 0;
+    const char* total_slot = static_cast<const char*>(externalBuffer) + l.pair_ptr + pairs * sizeof(uint32_t);
+    if (hipMemcpyAsync(&entries, total_slot, sizeof(entries), hipMemcpyDeviceToHost, handle->stream) != hipSuccess ||
+        hipStreamSynchronize(handle->stream) != hipSuccess)
+        return to_public_status(MCSP_STATUS_INTERNAL_ERROR);
+    SpmmSchedule& s = matA->schedule;
+    s.buffer = externalBuffer;
+    s.rows = matA->rows;
+    s.cols = matA->cols;
+    s.m = matA->row_num;
+    s.nnz = matA->nnz;
+    s.base = static_cast<int>(matA->idxBase);
+    s.entries = entries;
+    // Worth it when the merged lists are clearly shorter than the rows they replace; pairs too
+    // long to merge contribute no entries and are not evidence either way.
+    s.useful = entries != 0 && static_cast<uint64_t>(entries) * 100 <= static_cast<uint64_t>(matA->nnz) * 85;
+    s.valid = true;
     return MCSPARSE_STATUS_SUCCESS;
 }
 

@@ -297,6 +297,7 @@ mcsparseStatus_t mcsparseCsrSetPointers(mcsparseSpMatDescr_t d, void* csrRowOffs
     d->cols = csrColInd;
     d->vals = csrValues;
     d->plan.valid = false;  // new structure, new analysis
+    d->schedule.valid = false;
     return MCSPARSE_STATUS_SUCCESS;
 }
 
@@ -353,6 +354,14 @@ mcsparseStatus_t mcsparseSpMatGetSpMVPlan(mcsparseSpMatDescr_t d, int* family, i
         return to_public_status(MCSP_STATUS_INVALID_POINTER);
     *family = d->plan.valid ? d->plan.family : kFamilyAuto;
     *lanes_per_row = d->plan.valid ? d->plan.lanes : 0;
+    return MCSPARSE_STATUS_SUCCESS;
+}
+
+mcsparseStatus_t mcsparseSpMatGetSpMMSchedule(mcsparseSpMatDescr_t d, int* state, int64_t* merged_entries) {
+    if (d == nullptr || state == nullptr || merged_entries == nullptr)
+        return to_public_status(MCSP_STATUS_INVALID_POINTER);
+    *state = !d->schedule.valid ? 0 : (d->schedule.useful ? 2 : 1);
+    *merged_entries = d->schedule.valid ? static_cast<int64_t>(d->schedule.entries) : 0;
     return MCSPARSE_STATUS_SUCCESS;
 }
 

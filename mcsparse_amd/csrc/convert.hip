@@ -630,6 +630,14 @@ void launch_gather(hipStream_t stream, idx_t nnz, const T* y, T* x_val, const id
                        stream, nnz, y, x_val, x_ind, base);
 }
 
+size_t exclusive_scan_workspace_bytes(uint64_t n) {
+    return align_up(scan_workspace_elems(n) * sizeof(uint32_t)) + kAlign;
+}
+
+void launch_exclusive_scan_u32(hipStream_t stream, uint32_t* data, uint64_t n, void* workspace) {
+    launch_exclusive_scan(stream, data, n, static_cast<uint32_t*>(workspace));
+}
+
 template void launch_gather<float>(hipStream_t, idx_t, const float*, float*, const idx_t*, idx_t);
 template void launch_gather<double>(hipStream_t, idx_t, const double*, double*, const idx_t*, idx_t);
 

@@ -71,6 +71,21 @@ struct SpmvPlan {
     int forced_lanes = 0;
 };
 
+// Row-pair schedule built by mcsparseSpMM_preprocess inside the caller's buffer.  Unlike the
+// SpMV plan it is part of the computation: SpMM uses it only while the buffer and the CSR
+// arrays it was built from are the ones of the call, and the caller must not change the
+// structure or the buffer's contents in between (the contract of a preprocess step).
+struct SpmmSchedule {
+    bool valid = false;
+    bool useful = false;   // the merged lists are short enough to pay off
+    const void* buffer = nullptr;
+    const void* rows = nullptr;
+    const void* cols = nullptr;
+    int64_t m = 0, nnz = 0;
+    int base = 0;
+    uint32_t entries = 0;  // length of all merged lists together
+};
+
 // reference: src/include/mcsp_internal_types.h:184-225.  rows/cols follow the reference's
 // convention: for CSR rows = row offsets, cols = column indices; for CSC rows = row indices,
 // cols = column offsets (src/common/mcsp_helper.cpp:447-452).
@@ -92,6 +107,7 @@ struct mcsparseSpMatDescr {
     size_t assist_index_buffer_size = 0;
     size_t fixed_length_buffer_size = 0;
     SpmvPlan plan;
+    SpmmSchedule schedule;
 };
 
 // Internal status, mapped to the public one exactly as the reference's wrapper does
@@ -186,6 +202,25 @@ struct SpmmArgs {
 template <typename T>
 void launch_spmm(hipStream_t stream, const SpmmArgs& a, T alpha, T beta);
 
+// Row-pair schedule of a CSR structure (spmm.hip): for rows 2p and 2p+1 the merged list of
+// their column indices, each entry = (zero-based column << 2) | bit 0: row 2p has it |
+// bit 1: row 2p+1 has it.  pair_ptr has pairs+1 offsets into entries.  Pairs holding more than
+// kSpmmMaxMergedPair nonzeros get no entries and are processed row by row.
+constexpr idx_t kSpmmMaxMergedPair = 1024;
+constexpr int64_t kSpmmMaxScheduledColumns = int64_t(1) << 30;
+struct SpmmScheduleLayout {
+    size_t pair_ptr, entries, scan_ws, total;
+};
+SpmmScheduleLayout spmm_schedule_layout(idx_t m, idx_t nnz);
+// Fills pair_ptr and entries inside `schedule` (laid out as spmm_schedule_layout says).
+void launch_spmm_schedule(hipStream_t stream, idx_t m, idx_t nnz, idx_t base, const idx_t* row_ptr, const idx_t* col,
+                          void* schedule);
+// Same result as launch_spmm for a row-major op(B) whose rows allow 128-bit accesses
+// (spmm_schedule_usable says so), reading every B row once per row pair.
+bool spmm_schedule_usable(const SpmmArgs& a, size_t value_bytes);
+template <typename T>
+void launch_spmm_scheduled(hipStream_t stream, const SpmmArgs& a, const void* schedule, T alpha, T beta);
+
 // ---- conversions (convert.hip) ----
 void launch_csr2coo(hipStream_t stream, idx_t m, idx_t nnz, const idx_t* row_ptr, idx_t base, idx_t* coo_rows);
 void launch_coo2csr(hipStream_t stream, idx_t nnz, idx_t m, const idx_t* coo_rows, idx_t base, idx_t* row_ptr);
@@ -205,6 +240,9 @@ void launch_coosort(hipStream_t stream, idx_t major_extent, idx_t minor_extent, 
 void launch_csrsort(hipStream_t stream, idx_t m, idx_t n, idx_t nnz, idx_t base, const idx_t* row_ptr, idx_t* col,
                     idx_t* perm, void* workspace);
 void launch_identity(hipStream_t stream, idx_t n, idx_t* p);
+// In-place exclusive prefix sum of n 32-bit counters.
+size_t exclusive_scan_workspace_bytes(uint64_t n);
+void launch_exclusive_scan_u32(hipStream_t stream, uint32_t* data, uint64_t n, void* workspace);
 // x_val[i] = y[x_ind[i] - base]
 template <typename T>
 void launch_gather(hipStream_t stream, idx_t nnz, const T* y, T* x_val, const idx_t* x_ind, idx_t base);

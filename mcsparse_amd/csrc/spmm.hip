@@ -54,59 +54,74 @@ __device__ __forceinline__ void store_vec(T* p, const Vec<T, V>& r) {
     }
 }
 
-// op(B) row-major.  LR lanes per row of A, V adjacent columns per lane; blockIdx.y walks the
-// column panels of LR*V columns.  V > 1 requires n, ldb (and ldc when C is row-major) to be
-// multiples of V and 16-byte aligned base pointers, which the launcher checks.
-template <typename T, int LR, int V, bool BETA0, bool C_ROW>
-__global__ __launch_bounds__(kBlock) void spmm_rowb_kernel(idx_t m, idx_t n, idx_t base,
-                                                           const idx_t* __restrict__ row_ptr,
-                                                           const idx_t* __restrict__ col, const T* __restrict__ val,
-                                                           const T* __restrict__ B, int64_t ldb, T* __restrict__ C,
-                                                           int64_t ldc, T alpha, T beta) {
-    constexpr int kRowsPerBlock = kBlock / LR;
-    const idx_t lane = threadIdx.x % LR;
-    const uint64_t row = static_cast<uint64_t>(blockIdx.x) * kRowsPerBlock + threadIdx.x / LR;
-    const uint64_t c0 = (static_cast<uint64_t>(blockIdx.y) * LR + lane) * V;
-    if (row >= m || c0 >= n) return;
+// Byte offsets into op(B) are 32-bit when the whole operand lies within 4 GiB of its first
+// element (WIDE = false): a row's offset then travels between lanes in one register and the
+// load takes it next to the scalar base address, which leaves one vector instruction of address
+// arithmetic per row of op(B).
+template <bool WIDE>
+struct ByteOffset { typedef uint32_t type; };
+template <>
+struct ByteOffset<true> { typedef uint64_t type; };
 
-    const idx_t start = row_ptr[row] - base;
-    const idx_t end = row_ptr[row + 1] - base;
-    T acc[V];
+// acc += sum over the nonzeros [begin, end) of one row of A of value * (V columns of the row of
+// op(B) the nonzero names), for a group of LR >= 4 lanes that all pass the same range.
+// B_bytes is the operand's first element, lane_off the byte offset of this lane's columns.
+//
+// What bounds these kernels is the return path of the vector memory unit, and a load in which
+// all lanes of a group ask for the same word still returns a word per lane.  So the lanes fetch
+// LR nonzeros of the row at once, one each, turn them into row offsets, and pass offsets and
+// values round in registers; the loop then loads rows of op(B) and nothing else.
+template <typename T, int LR, int V, bool WIDE>
+__device__ __forceinline__ void row_times_b(idx_t begin, idx_t end, idx_t lane, idx_t base,
+                                            const idx_t* __restrict__ col, const T* __restrict__ val,
+                                            const char* __restrict__ B_bytes,
+                                            typename ByteOffset<WIDE>::type lane_off,
+                                            typename ByteOffset<WIDE>::type ldb_bytes, T (&acc)[V]) {
+    typedef typename ByteOffset<WIDE>::type off_t;
+    constexpr int kBatch = LR < 8 ? LR : 8;  // rows of op(B) in flight per lane
+    for (idx_t j = begin; j < end; j += LR) {
+        const bool has = j + lane < end;
+        const off_t roff = has ? static_cast<off_t>(col[j + lane] - base) * ldb_bytes : off_t(0);
+        const T aa = has ? val[j + lane] : T(0);
+        const idx_t left = end - j;
+        auto chunk = [&](auto checked) {
+            constexpr bool kChecked = decltype(checked)::value;
+            static_for<LR / kBatch>([&](auto g) {
+                constexpr int u0 = decltype(g)::value * kBatch;
+                if (!kChecked || u0 < left) {
+                    Vec<T, V> b[kBatch];
+                    static_for<kBatch>([&](auto u) {
+                        constexpr int k = u0 + decltype(u)::value;
+                        if (!kChecked || k < left) {  // the same for all lanes of the group
+                            const off_t off = group_bcast<LR, k>(roff) + lane_off;
+                            b[decltype(u)::value] = load_vec<T, V>(reinterpret_cast<const T*>(B_bytes + off));
+                        }
+                    });
+                    static_for<kBatch>([&](auto u) {
+                        constexpr int k = u0 + decltype(u)::value;
+                        if (!kChecked || k < left) {
+                            const T a = group_bcast<LR, k>(aa);
 #pragma unroll
-    for (int i = 0; i < V; ++i) acc[i] = T(0);
-
-    constexpr int kUnroll = 8;
-    const T* Bc = B + c0;
-    idx_t j = start;
-    for (; j + kUnroll <= end; j += kUnroll) {
-        idx_t c[kUnroll];
-        T a[kUnroll];
-        Vec<T, V> b[kUnroll];
-#pragma unroll
-        for (int u = 0; u < kUnroll; ++u) {
-            c[u] = col[j + u] - base;
-            a[u] = val[j + u];
-        }
-#pragma unroll
-        for (int u = 0; u < kUnroll; ++u) b[u] = load_vec<T, V>(Bc + static_cast<int64_t>(c[u]) * ldb);
-#pragma unroll
-        for (int u = 0; u < kUnroll; ++u) {
-#pragma unroll
-            for (int i = 0; i < V; ++i) acc[i] += a[u] * b[u].v[i];
-        }
+                            for (int i = 0; i < V; ++i) acc[i] += a * b[decltype(u)::value].v[i];
+                        }
+                    });
+                }
+            });
+        };
+        if (left >= LR) chunk(std::false_type{});
+        else chunk(std::true_type{});
     }
-    for (; j < end; ++j) {
-        const idx_t c = col[j] - base;
-        const T a = val[j];
-        const Vec<T, V> b = load_vec<T, V>(Bc + static_cast<int64_t>(c) * ldb);
-#pragma unroll
-        for (int i = 0; i < V; ++i) acc[i] += a * b.v[i];
-    }
+}
 
-    if constexpr (C_ROW) {
+// Writes V adjacent columns of one row of C: beta*C + alpha*acc, C untouched by reads if beta == 0.
+template <typename T, int V>
+__device__ __forceinline__ void store_c(T* __restrict__ C, int64_t ldc, bool c_row_major, uint64_t row, uint64_t c0,
+                                        const T (&acc)[V], T alpha, T beta) {
+    const bool beta0 = beta == T(0);
+    if (c_row_major) {
         T* Cp = C + static_cast<int64_t>(row) * ldc + c0;
         Vec<T, V> out;
-        if constexpr (BETA0) {
+        if (beta0) {
 #pragma unroll
             for (int i = 0; i < V; ++i) out.v[i] = alpha * acc[i];
         } else {
@@ -119,13 +134,71 @@ __global__ __launch_bounds__(kBlock) void spmm_rowb_kernel(idx_t m, idx_t n, idx
 #pragma unroll
         for (int i = 0; i < V; ++i) {
             T* Cp = C + static_cast<int64_t>(c0 + i) * ldc + row;
-            if constexpr (BETA0) {
-                *Cp = alpha * acc[i];
-            } else {
-                *Cp = beta * *Cp + alpha * acc[i];
-            }
+            *Cp = beta0 ? alpha * acc[i] : beta * *Cp + alpha * acc[i];
         }
     }
+}
+
+// op(B) row-major.  LR lanes per row of A, V adjacent columns per lane; blockIdx.y walks the
+// column panels of LR*V columns.  V > 1 requires n, ldb (and ldc when C is row-major) to be
+// multiples of V and 16-byte aligned base pointers, which the launcher checks.
+template <typename T, int LR, int V, bool WIDE>
+__global__ __launch_bounds__(kBlock) void spmm_rowb_kernel(idx_t m, idx_t n, idx_t base,
+                                                           const idx_t* __restrict__ row_ptr,
+                                                           const idx_t* __restrict__ col, const T* __restrict__ val,
+                                                           const T* __restrict__ B, int64_t ldb, T* __restrict__ C,
+                                                           int64_t ldc, bool c_row_major, T alpha, T beta) {
+    typedef typename ByteOffset<WIDE>::type off_t;
+    constexpr int kRowsPerBlock = kBlock / LR;
+    const idx_t lane = threadIdx.x % LR;
+    const uint64_t row = static_cast<uint64_t>(blockIdx.x) * kRowsPerBlock + threadIdx.x / LR;
+    const uint64_t c_own = (static_cast<uint64_t>(blockIdx.y) * LR + lane) * V;
+    if (row >= m) return;  // whole lane groups
+    // Lanes past the last column still fetch their share of the row's nonzeros for the group;
+    // they compute on column 0 and store nothing.
+    const bool stores = c_own < n;
+    const uint64_t c0 = stores ? c_own : 0;
+
+    const idx_t start = row_ptr[row] - base;
+    const idx_t end = row_ptr[row + 1] - base;
+    T acc[V];
+#pragma unroll
+    for (int i = 0; i < V; ++i) acc[i] = T(0);
+
+    if constexpr (LR >= 4) {
+        row_times_b<T, LR, V, WIDE>(start, end, lane, base, col, val, reinterpret_cast<const char*>(B),
+                                    static_cast<off_t>(c0 * sizeof(T)), static_cast<off_t>(ldb * sizeof(T)), acc);
+    } else {
+        constexpr int kUnroll = 8;
+        const T* Bc = B + c0;
+        idx_t j = start;
+        for (; j + kUnroll <= end; j += kUnroll) {
+            idx_t c[kUnroll];
+            T a[kUnroll];
+            Vec<T, V> b[kUnroll];
+#pragma unroll
+            for (int u = 0; u < kUnroll; ++u) {
+                c[u] = col[j + u] - base;
+                a[u] = val[j + u];
+            }
+#pragma unroll
+            for (int u = 0; u < kUnroll; ++u) b[u] = load_vec<T, V>(Bc + static_cast<int64_t>(c[u]) * ldb);
+#pragma unroll
+            for (int u = 0; u < kUnroll; ++u) {
+#pragma unroll
+                for (int i = 0; i < V; ++i) acc[i] += a[u] * b[u].v[i];
+            }
+        }
+        for (; j < end; ++j) {
+            const idx_t c = col[j] - base;
+            const T a = val[j];
+            const Vec<T, V> b = load_vec<T, V>(Bc + static_cast<int64_t>(c) * ldb);
+#pragma unroll
+            for (int i = 0; i < V; ++i) acc[i] += a * b.v[i];
+        }
+    }
+
+    if (stores) store_c<T, V>(C, ldc, c_row_major, row, c0, acc, alpha, beta);
 }
 
 // op(B) column-major: element (kk, j) at j*ldb + kk.  One wavefront per row of A, lanes strided
@@ -174,6 +247,179 @@ __global__ __launch_bounds__(kBlock) void spmm_colb_kernel(idx_t m, idx_t n, idx
     }
 }
 
+// ---- row pairs --------------------------------------------------------------------------
+// Neighbouring rows of a matrix from a mesh or a stencil share most of their columns.  A lane
+// group that owns rows 2p and 2p+1 together walks the merged column list of the pair (built
+// once per structure by launch_spmm_schedule) and feeds every row of op(B) it loads to both
+// accumulators, so the bytes pulled through the vector memory path -- what bounds this
+// kernel -- shrink by the overlap of the two rows.  Values are read from the CSR array on
+// every call: entry k of a row is its k-th nonzero in storage order, whatever the order is,
+// so unsorted rows only lose sharing, never correctness.
+constexpr uint32_t kNoColumn = 0xffffffffu;
+
+template <bool FILL>
+__global__ __launch_bounds__(kBlock) void pair_merge_kernel(idx_t m, idx_t base, const idx_t* __restrict__ row_ptr,
+                                                            const idx_t* __restrict__ col,
+                                                            uint32_t* __restrict__ pair_ptr,
+                                                            uint32_t* __restrict__ entries) {
+    const uint64_t pairs = (static_cast<uint64_t>(m) + 1) / 2;
+    const uint64_t pair = static_cast<uint64_t>(blockIdx.x) * kBlock + threadIdx.x;
+    if (pair > pairs) return;
+    if (pair == pairs) {  // the slot that receives the total after the scan
+        if (!FILL) pair_ptr[pair] = 0;
+        return;
+    }
+    const uint64_t r0 = 2 * pair;
+    idx_t i0 = row_ptr[r0] - base;
+    const idx_t e0 = row_ptr[r0 + 1] - base;
+    idx_t i1 = e0;
+    const idx_t e1 = r0 + 1 < static_cast<uint64_t>(m) ? row_ptr[r0 + 2] - base : e0;
+    if (e1 - i0 > kSpmmMaxMergedPair) {
+        if (!FILL) pair_ptr[pair] = 0;
+        return;
+    }
+    const uint32_t out = FILL ? pair_ptr[pair] : 0;
+    uint32_t count = 0;
+    while (i0 < e0 || i1 < e1) {
+        const uint32_t h0 = i0 < e0 ? static_cast<uint32_t>(col[i0] - base) : kNoColumn;
+        const uint32_t h1 = i1 < e1 ? static_cast<uint32_t>(col[i1] - base) : kNoColumn;
+        const uint32_t lo = h0 < h1 ? h0 : h1;
+        const uint32_t t0 = h0 == lo, t1 = h1 == lo;
+        if (FILL) entries[out + count] = (lo << 2) | t0 | (t1 << 1);
+        ++count;
+        i0 += t0;
+        i1 += t1;
+    }
+    if (!FILL) pair_ptr[pair] = count;
+}
+
+// LR lanes (4..64) per row pair, V = 16 B / sizeof(T) adjacent columns per lane; blockIdx.y walks
+// panels of LR*V columns.  The lanes of a group fetch LR entries of the merged list at once, one
+// each, work out from the two flag bits which value of which row belongs to their entry, fetch
+// those, and pass row offsets, flags and values round in registers.
+template <typename T, int LR, bool WIDE>
+__global__ __launch_bounds__(kBlock) void spmm_pair_kernel(idx_t m, idx_t n, idx_t base,
+                                                           const idx_t* __restrict__ row_ptr,
+                                                           const idx_t* __restrict__ col, const T* __restrict__ val,
+                                                           const uint32_t* __restrict__ pair_ptr,
+                                                           const uint32_t* __restrict__ entries,
+                                                           const T* __restrict__ B, int64_t ldb, T* __restrict__ C,
+                                                           int64_t ldc, bool c_row_major, T alpha, T beta) {
+    typedef typename ByteOffset<WIDE>::type off_t;
+    constexpr int V = 16 / sizeof(T);
+    constexpr int kPairsPerBlock = kBlock / LR;
+    constexpr int kBatch = LR < 8 ? LR : 8;
+    const idx_t lane = threadIdx.x % LR;
+    const uint64_t pair = static_cast<uint64_t>(blockIdx.x) * kPairsPerBlock + threadIdx.x / LR;
+    const uint64_t r0 = 2 * pair;
+    if (r0 >= static_cast<uint64_t>(m)) return;  // whole lane groups
+    const uint64_t c_own = (static_cast<uint64_t>(blockIdx.y) * LR + lane) * V;
+    const bool stores = c_own < static_cast<uint64_t>(n);  // lanes past the last column only help fetching
+    const uint64_t c0 = stores ? c_own : 0;
+    const bool two_rows = r0 + 1 < static_cast<uint64_t>(m);
+
+    idx_t i0 = row_ptr[r0] - base;
+    const idx_t e0 = row_ptr[r0 + 1] - base;
+    idx_t i1 = e0;
+    const idx_t e1 = two_rows ? row_ptr[r0 + 2] - base : e0;
+
+    T acc0[V], acc1[V];
+#pragma unroll
+    for (int i = 0; i < V; ++i) acc0[i] = acc1[i] = T(0);
+    const char* B_bytes = reinterpret_cast<const char*>(B);
+    const off_t lane_off = static_cast<off_t>(c0 * sizeof(T));
+    const off_t ldb_bytes = static_cast<off_t>(ldb * sizeof(T));
+
+    if (e1 - i0 <= kSpmmMaxMergedPair) {
+        const uint32_t s_end = pair_ptr[pair + 1];
+        const unsigned group_first = (__lane_id() / LR) * LR;
+        const uint64_t group_bits = LR == kWave ? ~0ull : ((1ull << (LR % kWave)) - 1ull);
+        const uint64_t below = (1ull << lane) - 1ull;
+        for (uint32_t s = pair_ptr[pair]; s < s_end; s += LR) {
+            const uint32_t e = s + lane < s_end ? entries[s + lane] : 0u;
+            // this lane's entry is the p0-th of the chunk that row 2p takes part in, the p1-th for row 2p+1
+            const uint64_t in0 = (__ballot(e & 1u) >> group_first) & group_bits;
+            const uint64_t in1 = (__ballot(e & 2u) >> group_first) & group_bits;
+            const T v0 = (e & 1u) ? val[i0 + __popcll(in0 & below)] : T(0);
+            const T v1 = (e & 2u) ? val[i1 + __popcll(in1 & below)] : T(0);
+            i0 += __popcll(in0);
+            i1 += __popcll(in1);
+            const off_t roff = static_cast<off_t>(e >> 2) * ldb_bytes;
+            const uint32_t flags = e & 3u;
+            const uint32_t left = s_end - s;
+            auto chunk = [&](auto checked) {
+                constexpr bool kChecked = decltype(checked)::value;
+                static_for<LR / kBatch>([&](auto g) {
+                    constexpr int u0 = decltype(g)::value * kBatch;
+                    if (!kChecked || u0 < left) {
+                        Vec<T, V> b[kBatch];
+                        static_for<kBatch>([&](auto u) {
+                            constexpr int k = u0 + decltype(u)::value;
+                            if (!kChecked || k < left) {
+                                const off_t off = group_bcast<LR, k>(roff) + lane_off;
+                                b[decltype(u)::value] = load_vec<T, V>(reinterpret_cast<const T*>(B_bytes + off));
+                            }
+                        });
+                        static_for<kBatch>([&](auto u) {
+                            constexpr int k = u0 + decltype(u)::value;
+                            if (!kChecked || k < left) {
+                                const uint32_t fk = group_bcast<LR, k>(flags);
+                                // a row that lacks the column must not see it at all (0 * inf would be NaN)
+                                if (fk & 1u) {
+                                    const T a = group_bcast<LR, k>(v0);
+#pragma unroll
+                                    for (int i = 0; i < V; ++i) acc0[i] += a * b[decltype(u)::value].v[i];
+                                }
+                                if (fk & 2u) {
+                                    const T a = group_bcast<LR, k>(v1);
+#pragma unroll
+                                    for (int i = 0; i < V; ++i) acc1[i] += a * b[decltype(u)::value].v[i];
+                                }
+                            }
+                        });
+                    }
+                });
+            };
+            if (left >= LR) chunk(std::false_type{});
+            else chunk(std::true_type{});
+        }
+    } else {
+        // a pair too long to be worth merging: one row after the other
+        row_times_b<T, LR, V, WIDE>(i0, e0, lane, base, col, val, B_bytes, lane_off, ldb_bytes, acc0);
+        row_times_b<T, LR, V, WIDE>(i1, e1, lane, base, col, val, B_bytes, lane_off, ldb_bytes, acc1);
+    }
+
+    if (!stores) return;
+    store_c<T, V>(C, ldc, c_row_major, r0, c0, acc0, alpha, beta);
+    if (two_rows) store_c<T, V>(C, ldc, c_row_major, r0 + 1, c0, acc1, alpha, beta);
+}
+
+// op(B) lies within 4 GiB of its first element: byte offsets into it fit 32 bits
+bool narrow_offsets(const SpmmArgs& a, size_t value_bytes) {
+    const uint64_t last = (a.k == 0 ? 0 : static_cast<uint64_t>(a.k) - 1) * static_cast<uint64_t>(a.ldb) + a.n;
+    return last * value_bytes <= 0xffffffffull;
+}
+
+template <typename T, int LR>
+void launch_pair(hipStream_t stream, const SpmmArgs& a, const uint32_t* pair_ptr, const uint32_t* entries, T alpha,
+                 T beta) {
+    constexpr int V = 16 / sizeof(T);
+    const uint64_t pairs = (static_cast<uint64_t>(a.m) + 1) / 2;
+    const uint64_t pair_blocks = (pairs + (kBlock / LR) - 1) / (kBlock / LR);
+    const uint64_t panels = (static_cast<uint64_t>(a.n) + LR * V - 1) / (LR * V);
+    const dim3 grid(static_cast<uint32_t>(pair_blocks), static_cast<uint32_t>(panels));
+    const T* val = static_cast<const T*>(a.val);
+    const T* B = static_cast<const T*>(a.B);
+    T* C = static_cast<T*>(a.C);
+    if (narrow_offsets(a, sizeof(T))) {
+        hipLaunchKernelGGL((spmm_pair_kernel<T, LR, false>), grid, dim3(kBlock), 0, stream, a.m, a.n, a.base, a.row_ptr,
+                           a.col, val, pair_ptr, entries, B, a.ldb, C, a.ldc, a.c_row_major, alpha, beta);
+    } else {
+        hipLaunchKernelGGL((spmm_pair_kernel<T, LR, true>), grid, dim3(kBlock), 0, stream, a.m, a.n, a.base, a.row_ptr,
+                           a.col, val, pair_ptr, entries, B, a.ldb, C, a.ldc, a.c_row_major, alpha, beta);
+    }
+}
+
 template <typename T, int LR, int V>
 void launch_rowb(hipStream_t stream, const SpmmArgs& a, T alpha, T beta) {
     const uint64_t row_blocks = (static_cast<uint64_t>(a.m) + (kBlock / LR) - 1) / (kBlock / LR);
@@ -182,15 +428,13 @@ void launch_rowb(hipStream_t stream, const SpmmArgs& a, T alpha, T beta) {
     const T* val = static_cast<const T*>(a.val);
     const T* B = static_cast<const T*>(a.B);
     T* C = static_cast<T*>(a.C);
-    const bool beta0 = beta == T(0);
-#define MCSP_LAUNCH_ROWB(B0, CR)                                                                                   \
-    hipLaunchKernelGGL((spmm_rowb_kernel<T, LR, V, B0, CR>), grid, dim3(kBlock), 0, stream, a.m, a.n, a.base,       \
-                       a.row_ptr, a.col, val, B, a.ldb, C, a.ldc, alpha, beta)
-    if (beta0 && a.c_row_major) MCSP_LAUNCH_ROWB(true, true);
-    else if (beta0) MCSP_LAUNCH_ROWB(true, false);
-    else if (a.c_row_major) MCSP_LAUNCH_ROWB(false, true);
-    else MCSP_LAUNCH_ROWB(false, false);
-#undef MCSP_LAUNCH_ROWB
+    if (LR < 4 || narrow_offsets(a, sizeof(T))) {  // the narrow groups do not use byte offsets at all
+        hipLaunchKernelGGL((spmm_rowb_kernel<T, LR, V, false>), grid, dim3(kBlock), 0, stream, a.m, a.n, a.base,
+                           a.row_ptr, a.col, val, B, a.ldb, C, a.ldc, a.c_row_major, alpha, beta);
+    } else {
+        hipLaunchKernelGGL((spmm_rowb_kernel<T, LR, V, true>), grid, dim3(kBlock), 0, stream, a.m, a.n, a.base,
+                           a.row_ptr, a.col, val, B, a.ldb, C, a.ldc, a.c_row_major, alpha, beta);
+    }
 }
 
 template <typename T, int V>
@@ -236,6 +480,59 @@ void launch_spmm(hipStream_t stream, const SpmmArgs& a, T alpha, T beta) {
     }
 }
 
+SpmmScheduleLayout spmm_schedule_layout(idx_t m, idx_t nnz) {
+    SpmmScheduleLayout l;
+    const uint64_t slots = (static_cast<uint64_t>(m) + 1) / 2 + 1;
+    size_t off = 0;
+    l.pair_ptr = off; off += align_up(slots * sizeof(uint32_t));
+    l.entries = off; off += align_up(static_cast<size_t>(nnz) * sizeof(uint32_t));
+    l.scan_ws = off; off += exclusive_scan_workspace_bytes(slots);
+    l.total = off;
+    return l;
+}
+
+void launch_spmm_schedule(hipStream_t stream, idx_t m, idx_t nnz, idx_t base, const idx_t* row_ptr, const idx_t* col,
+                          void* schedule) {
+    const SpmmScheduleLayout l = spmm_schedule_layout(m, nnz);
+    char* w = static_cast<char*>(schedule);
+    uint32_t* pair_ptr = reinterpret_cast<uint32_t*>(w + l.pair_ptr);
+    uint32_t* entries = reinterpret_cast<uint32_t*>(w + l.entries);
+    const uint64_t slots = (static_cast<uint64_t>(m) + 1) / 2 + 1;
+    const dim3 grid(static_cast<uint32_t>((slots + kBlock - 1) / kBlock));
+    hipLaunchKernelGGL((pair_merge_kernel<false>), grid, dim3(kBlock), 0, stream, m, base, row_ptr, col, pair_ptr,
+                       entries);
+    launch_exclusive_scan_u32(stream, pair_ptr, slots, w + l.scan_ws);
+    hipLaunchKernelGGL((pair_merge_kernel<true>), grid, dim3(kBlock), 0, stream, m, base, row_ptr, col, pair_ptr,
+                       entries);
+}
+
+bool spmm_schedule_usable(const SpmmArgs& a, size_t value_bytes) {
+    const int64_t wide = static_cast<int64_t>(16 / value_bytes);
+    // narrower than four 128-bit vectors per row: too few lanes per pair to share the fetching
+    return a.b_row_major && a.n >= 3 * wide + 1 && a.k <= kSpmmMaxScheduledColumns &&
+           reinterpret_cast<uintptr_t>(a.B) % 16 == 0 &&
+           a.ldb % wide == 0 && a.n % wide == 0 &&
+           (!a.c_row_major || (reinterpret_cast<uintptr_t>(a.C) % 16 == 0 && a.ldc % wide == 0));
+}
+
+template <typename T>
+void launch_spmm_scheduled(hipStream_t stream, const SpmmArgs& a, const void* schedule, T alpha, T beta) {
+    if (a.m == 0 || a.n == 0) return;
+    constexpr int V = 16 / sizeof(T);
+    const SpmmScheduleLayout l = spmm_schedule_layout(a.m, a.nnz);
+    const char* w = static_cast<const char*>(schedule);
+    const uint32_t* pair_ptr = reinterpret_cast<const uint32_t*>(w + l.pair_ptr);
+    const uint32_t* entries = reinterpret_cast<const uint32_t*>(w + l.entries);
+    const uint64_t lanes_needed = (static_cast<uint64_t>(a.n) + V - 1) / V;
+    if (lanes_needed <= 4) launch_pair<T, 4>(stream, a, pair_ptr, entries, alpha, beta);
+    else if (lanes_needed <= 8) launch_pair<T, 8>(stream, a, pair_ptr, entries, alpha, beta);
+    else if (lanes_needed <= 16) launch_pair<T, 16>(stream, a, pair_ptr, entries, alpha, beta);
+    else if (lanes_needed <= 32) launch_pair<T, 32>(stream, a, pair_ptr, entries, alpha, beta);
+    else launch_pair<T, 64>(stream, a, pair_ptr, entries, alpha, beta);
+}
+
+template void launch_spmm_scheduled<float>(hipStream_t, const SpmmArgs&, const void*, float, float);
+template void launch_spmm_scheduled<double>(hipStream_t, const SpmmArgs&, const void*, double, double);
 template void launch_spmm<float>(hipStream_t, const SpmmArgs&, float, float);
 template void launch_spmm<double>(hipStream_t, const SpmmArgs&, double, double);
 

@@ -248,10 +248,19 @@ def test_spmm_argument_checks(lib):
     assert call(b=Bt) == api.STATUS_INVALID_VALUE  # B is 4 x 6 but op(B) must be 6 x 4
     size = ctypes.c_size_t()
     assert lib.mcsparseSpMM_bufferSize(o.h, 0, 0, o.pa, o.A, B, o.pa, C, api.R_32F, 0, ctypes.byref(size)) == 0
-    assert size.value == 128
+    # room for the row-pair schedule of mcsparseSpMM_preprocess: 4 + 1 offsets, 20 entries, scan scratch
+    assert size.value % 128 == 0 and size.value >= 128 + 128 and size.value < 4096
     assert lib.mcsparseSpMM_bufferSize(None, 0, 0, o.pa, o.A, B, o.pa, C, api.R_32F, 0, ctypes.byref(size)) == 1
     assert lib.mcsparseSpMM_bufferSize(o.h, 0, 0, o.pa, o.A, None, o.pa, C, api.R_32F, 0, ctypes.byref(size)) == 3
-    assert lib.mcsparseSpMM_preprocess(o.h, 0, 0, o.pa, o.A, B, o.pa, C, api.R_32F, 0, FAKE) == 0  # no-op (:965-970)
+    # preprocess (:965-970 is a no-op; here it checks its arguments like SpMM and builds a schedule for CSR)
+    assert lib.mcsparseSpMM_preprocess(None, 0, 0, o.pa, o.A, B, o.pa, C, api.R_32F, 0, FAKE) == 1
+    assert lib.mcsparseSpMM_preprocess(o.h, 0, 0, o.pa, o.A, B, o.pa, C, api.R_32F, 0, None) == 3
+    assert lib.mcsparseSpMM_preprocess(o.h, 0, 0, o.pa, None, B, o.pa, C, api.R_32F, 0, FAKE) == 3
+    assert lib.mcsparseSpMM_preprocess(o.h, api.OP_T, 0, o.pa, o.A, B, o.pa, C, api.R_32F, 0, FAKE) == 0  # nothing to do
+    state, entries = ctypes.c_int(-1), ctypes.c_int64(-1)
+    assert lib.mcsparseSpMatGetSpMMSchedule(o.A, ctypes.byref(state), ctypes.byref(entries)) == 0
+    assert state.value == 0 and entries.value == 0
+    assert lib.mcsparseSpMatGetSpMMSchedule(o.A, None, ctypes.byref(entries)) == 3
     for f, need in ((api.FORMAT_COO, 9 * 4), (api.FORMAT_CSC, (9 + 20) * 4 + 20 * 4)):
         o2 = Objs(lib, m=8, n=6, nnz=20, fmt=f)
         assert lib.mcsparseSpMM_bufferSize(o2.h, 0, 0, o2.pa, o2.A, B, o2.pa, C, api.R_32F, 0, ctypes.byref(size)) == 0
@@ -261,6 +270,9 @@ def test_spmm_argument_checks(lib):
     # nnz == 0 with beta == 1 returns before any launch (:110-114)
     e = Objs(lib, m=8, n=6, nnz=0)
     assert lib.mcsparseSpMM(e.h, 0, 0, e.pa, e.A, B, e.pa, C, api.R_32F, 0, FAKE) == 0
+    assert lib.mcsparseSpMM_preprocess(e.h, 0, 0, e.pa, e.A, B, e.pa, C, api.R_32F, 0, FAKE) == 0  # empty: no schedule
+    assert lib.mcsparseSpMM_bufferSize(e.h, 0, 0, e.pa, e.A, B, e.pa, C, api.R_32F, 0, ctypes.byref(size)) == 0
+    assert size.value == 128
 
 
 def test_conversion_argument_checks(lib):
