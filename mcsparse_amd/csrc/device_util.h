@@ -50,14 +50,17 @@ __device__ __forceinline__ T group_sum(T v) {
 template <int L, int U>
 __device__ __forceinline__ int group_bcast_bits(int v) {
     static_assert(L >= 4 && L <= kWave && (L & (L - 1)) == 0 && U >= 0 && U < L, "group shape");
+    // mov_dpp leaves the previous contents of the destination undefined, which is fine where
+    // every lane receives a value and lets the compiler fold the move into the instruction
+    // that uses it.
     if constexpr (L == 4) {
-        return __builtin_amdgcn_update_dpp(0, v, U | (U << 2) | (U << 4) | (U << 6), 0xF, 0xF, false);
+        return __builtin_amdgcn_mov_dpp(v, U | (U << 2) | (U << 4) | (U << 6), 0xF, 0xF, true);
     } else if constexpr (L == 8) {
         constexpr int kRowBcast = 0x150;  // row_newbcast:0
-        const int lower = __builtin_amdgcn_update_dpp(0, v, kRowBcast + U, 0xF, 0x3, false);
+        const int lower = __builtin_amdgcn_mov_dpp(v, kRowBcast + U, 0xF, 0xF, true);
         return __builtin_amdgcn_update_dpp(lower, v, kRowBcast + 8 + U, 0xF, 0xC, false);
     } else if constexpr (L == 16) {
-        return __builtin_amdgcn_update_dpp(0, v, 0x150 + U, 0xF, 0xF, false);
+        return __builtin_amdgcn_mov_dpp(v, 0x150 + U, 0xF, 0xF, true);
     } else if constexpr (L == 32) {
         const int lower = __builtin_amdgcn_readlane(v, U);
         const int upper = __builtin_amdgcn_readlane(v, 32 + U);

@@ -293,6 +293,14 @@ __global__ __launch_bounds__(kBlock) void pair_merge_kernel(idx_t m, idx_t base,
     if (!FILL) pair_ptr[pair] = count;
 }
 
+// Returns the top bit of w and shifts w left by one: an add whose carry is the answer.
+__device__ __forceinline__ bool shift_out_top(uint32_t& w) {
+    unsigned doubled;
+    const bool top = __builtin_uadd_overflow(w, w, &doubled);
+    w = doubled;
+    return top;
+}
+
 // LR lanes (4..64) per row pair, V = 16 B / sizeof(T) adjacent columns per lane; blockIdx.y walks
 // panels of LR*V columns.  The lanes of a group fetch LR entries of the merged list at once, one
 // each, work out from the two flag bits which value of which row belongs to their entry, fetch
@@ -345,6 +353,10 @@ __global__ __launch_bounds__(kBlock) void spmm_pair_kernel(idx_t m, idx_t n, idx
             i0 += __popcll(in0);
             i1 += __popcll(in1);
             const off_t roff = static_cast<off_t>(e >> 2) * ldb_bytes;
+            // Which entries each row takes part in, as one bit per entry with entry 0 in the top
+            // bit: doubling the word moves the next entry's bit into the carry, which is then the
+            // lane mask the multiply-adds of that entry run under.
+            uint32_t take0 = __brev(static_cast<uint32_t>(in0)), take1 = __brev(static_cast<uint32_t>(in1));
             const uint32_t flags = e & 3u;
             const uint32_t left = s_end - s;
             auto chunk = [&](auto checked) {
@@ -363,14 +375,22 @@ __global__ __launch_bounds__(kBlock) void spmm_pair_kernel(idx_t m, idx_t n, idx
                         static_for<kBatch>([&](auto u) {
                             constexpr int k = u0 + decltype(u)::value;
                             if (!kChecked || k < left) {
-                                const uint32_t fk = group_bcast<LR, k>(flags);
                                 // a row that lacks the column must not see it at all (0 * inf would be NaN)
-                                if (fk & 1u) {
+                                bool row0, row1;
+                                if constexpr (LR == kWave) {  // one group per wavefront: the flags are scalars
+                                    const uint32_t fk = group_bcast<LR, k>(flags);
+                                    row0 = fk & 1u;
+                                    row1 = fk & 2u;
+                                } else {
+                                    row0 = shift_out_top(take0);
+                                    row1 = shift_out_top(take1);
+                                }
+                                if (row0) {
                                     const T a = group_bcast<LR, k>(v0);
 #pragma unroll
                                     for (int i = 0; i < V; ++i) acc0[i] += a * b[decltype(u)::value].v[i];
                                 }
-                                if (fk & 2u) {
+                                if (row1) {
                                     const T a = group_bcast<LR, k>(v1);
 #pragma unroll
                                     for (int i = 0; i < V; ++i) acc1[i] += a * b[decltype(u)::value].v[i];
