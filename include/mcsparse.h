@@ -413,7 +413,7 @@ mcsparseStatus_t mcsparseSpMatSetSpMVPlan(mcsparseSpMatDescr_t spMatDescr, int f
 /* What mcsparseSpMM_preprocess left on a CSR descriptor:
  * state 0 = no schedule, 1 = built but the rows share too few columns for it to pay off
  * (SpMM ignores it), 2 = SpMM uses it when called with the same buffer and CSR arrays.
- * merged_entries = total length of the merged column lists of all row pairs (compare with nnz). */
+ * merged_entries = total length of the merged column lists of all row groups (compare with nnz). */
 mcsparseStatus_t mcsparseSpMatGetSpMMSchedule(mcsparseSpMatDescr_t spMatDescr, int* state, int64_t* merged_entries);
 
 #ifdef __cplusplus

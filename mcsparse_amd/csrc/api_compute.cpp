@@ -228,7 +228,7 @@ mcspStatus_t spmv_typed(mcsparseHandle_t h, mcsparseSpMatDescr* A, CsrView v, co
     return MCSP_STATUS_SUCCESS;
 }
 
-// Scratch layout of an SpMM call: CSR gets room for the row-pair schedule that
+// Scratch layout of an SpMM call: CSR gets room for the row-group schedule that
 // mcsparseSpMM_preprocess builds (SpMM itself writes nothing there); COO gets [row offsets m+1];
 // CSC gets the transposed copy [row_ptr m+1 | col_ind nnz][values][csr2csc workspace]
 // (mcsp_spmm_gpu.cpp:818-849).
@@ -424,7 +424,7 @@ mcsparseStatus_t mcsparseSpMM_bufferSize(mcsparseHandle_t handle, mcsparseOperat
 }
 
 // reference: src/kernels/level3/spmm/mcsp_spmm_gpu.cpp:965-970 -- a no-op there.  Here a CSR
-// matrix gets its row-pair schedule built into externalBuffer (sized by mcsparseSpMM_bufferSize);
+// matrix gets its row-group schedule built into externalBuffer (sized by mcsparseSpMM_bufferSize);
 // mcsparseSpMM uses it when it is handed the same buffer and the same CSR arrays, and falls back
 // to the schedule-free kernel otherwise.  Until then the caller must leave the buffer and the
 // structure of A alone; the values of A may change freely.
@@ -450,9 +450,9 @@ mcsparseStatus_t mcsparseSpMM_preprocess(mcsparseHandle_t handle, mcsparseOperat
                                static_cast<const idx_t*>(matA->rows), static_cast<const idx_t*>(matA->cols),
                                externalBuffer);
     const mcsp::SpmmScheduleLayout l = mcsp::spmm_schedule_layout(m, nnz);
-    const uint64_t pairs = (static_cast<uint64_t>(m) + 1) / 2;
+    const uint64_t groups = mcsp::spmm_groups(m);
     uint32_t entries = 0;
-    const char* total_slot = static_cast<const char*>(externalBuffer) + l.pair_ptr + pairs * sizeof(uint32_t);
+    const char* total_slot = static_cast<const char*>(externalBuffer) + l.group_ptr + groups * sizeof(uint32_t);
     if (hipMemcpyAsync(&entries, total_slot, sizeof(entries), hipMemcpyDeviceToHost, handle->stream) != hipSuccess ||
         hipStreamSynchronize(handle->stream) != hipSuccess)
         return to_public_status(MCSP_STATUS_INTERNAL_ERROR);
@@ -464,7 +464,7 @@ mcsparseStatus_t mcsparseSpMM_preprocess(mcsparseHandle_t handle, mcsparseOperat
     s.nnz = matA->nnz;
     s.base = static_cast<int>(matA->idxBase);
     s.entries = entries;
-    // Worth it when the merged lists are clearly shorter than the rows they replace; pairs too
+    // Worth it when the merged lists are clearly shorter than the rows they replace; groups too
     // long to merge contribute no entries and are not evidence either way.
     s.useful = entries != 0 && static_cast<uint64_t>(entries) * 100 <= static_cast<uint64_t>(matA->nnz) * 85;
     s.valid = true;

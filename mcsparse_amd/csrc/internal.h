@@ -71,7 +71,7 @@ struct SpmvPlan {
     int forced_lanes = 0;
 };
 
-// Row-pair schedule built by mcsparseSpMM_preprocess inside the caller's buffer.  Unlike the
+// Row-group schedule built by mcsparseSpMM_preprocess inside the caller's buffer.  Unlike the
 // SpMV plan it is part of the computation: SpMM uses it only while the buffer and the CSR
 // arrays it was built from are the ones of the call, and the caller must not change the
 // structure or the buffer's contents in between (the contract of a preprocess step).
@@ -202,21 +202,27 @@ struct SpmmArgs {
 template <typename T>
 void launch_spmm(hipStream_t stream, const SpmmArgs& a, T alpha, T beta);
 
-// Row-pair schedule of a CSR structure (spmm.hip): for rows 2p and 2p+1 the merged list of
-// their column indices, each entry = (zero-based column << 2) | bit 0: row 2p has it |
-// bit 1: row 2p+1 has it.  pair_ptr has pairs+1 offsets into entries.  Pairs holding more than
-// kSpmmMaxMergedPair nonzeros get no entries and are processed row by row.
-constexpr idx_t kSpmmMaxMergedPair = 1024;
-constexpr int64_t kSpmmMaxScheduledColumns = int64_t(1) << 30;
+// Row-group schedule of a CSR structure (spmm.hip): for every group of kSpmmGroupRows
+// consecutive rows the merged list of their column indices, each entry =
+// (zero-based column << kSpmmGroupRows) | one bit per row of the group that has the column.
+// group_ptr has groups+1 offsets into entries.  Groups holding more than kSpmmMaxMergedGroup
+// nonzeros get no entries and are processed row by row.
+#ifndef MCSP_GROUP_ROWS
+#define MCSP_GROUP_ROWS 4
+#endif
+constexpr int kSpmmGroupRows = MCSP_GROUP_ROWS;
+constexpr idx_t kSpmmMaxMergedGroup = 2048;
+constexpr int64_t kSpmmMaxScheduledColumns = int64_t(1) << (32 - kSpmmGroupRows);
+constexpr uint64_t spmm_groups(idx_t m) { return (static_cast<uint64_t>(m) + kSpmmGroupRows - 1) / kSpmmGroupRows; }
 struct SpmmScheduleLayout {
-    size_t pair_ptr, entries, scan_ws, total;
+    size_t group_ptr, entries, scan_ws, total;
 };
 SpmmScheduleLayout spmm_schedule_layout(idx_t m, idx_t nnz);
-// Fills pair_ptr and entries inside `schedule` (laid out as spmm_schedule_layout says).
+// Fills group_ptr and entries inside `schedule` (laid out as spmm_schedule_layout says).
 void launch_spmm_schedule(hipStream_t stream, idx_t m, idx_t nnz, idx_t base, const idx_t* row_ptr, const idx_t* col,
                           void* schedule);
 // Same result as launch_spmm for a row-major op(B) whose rows allow 128-bit accesses
-// (spmm_schedule_usable says so), reading every B row once per row pair.
+// (spmm_schedule_usable says so), reading every B row once per row group.
 bool spmm_schedule_usable(const SpmmArgs& a, size_t value_bytes);
 template <typename T>
 void launch_spmm_scheduled(hipStream_t stream, const SpmmArgs& a, const void* schedule, T alpha, T beta);

@@ -247,50 +247,69 @@ __global__ __launch_bounds__(kBlock) void spmm_colb_kernel(idx_t m, idx_t n, idx
     }
 }
 
-// ---- row pairs --------------------------------------------------------------------------
+// ---- row groups -------------------------------------------------------------------------
 // Neighbouring rows of a matrix from a mesh or a stencil share most of their columns.  A lane
-// group that owns rows 2p and 2p+1 together walks the merged column list of the pair (built
-// once per structure by launch_spmm_schedule) and feeds every row of op(B) it loads to both
-// accumulators, so the bytes pulled through the vector memory path -- what bounds this
-// kernel -- shrink by the overlap of the two rows.  Values are read from the CSR array on
-// every call: entry k of a row is its k-th nonzero in storage order, whatever the order is,
-// so unsorted rows only lose sharing, never correctness.
+// group that owns kSpmmGroupRows consecutive rows walks the merged column list of the group
+// (built once per structure by launch_spmm_schedule) and feeds every row of op(B) it loads to
+// the accumulators of all rows that have the column, so the bytes pulled through the vector
+// memory path -- what bounds this kernel -- shrink by the overlap of the rows.  Values are read
+// from the CSR array on every call: entry k of a row is its k-th nonzero in storage order,
+// whatever the order is, so unsorted rows only lose sharing, never correctness.
 constexpr uint32_t kNoColumn = 0xffffffffu;
+constexpr int R = kSpmmGroupRows;
+
+// Offsets of the rows of one group; rows past the end of the matrix are empty.
+__device__ __forceinline__ void group_row_ranges(idx_t m, idx_t base, const idx_t* __restrict__ row_ptr, uint64_t r0,
+                                                 idx_t (&begin)[R], idx_t (&end)[R]) {
+    idx_t next = row_ptr[r0] - base;
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        begin[r] = next;
+        if (r0 + r < static_cast<uint64_t>(m)) next = row_ptr[r0 + r + 1] - base;
+        end[r] = next;
+    }
+}
 
 template <bool FILL>
-__global__ __launch_bounds__(kBlock) void pair_merge_kernel(idx_t m, idx_t base, const idx_t* __restrict__ row_ptr,
-                                                            const idx_t* __restrict__ col,
-                                                            uint32_t* __restrict__ pair_ptr,
-                                                            uint32_t* __restrict__ entries) {
-    const uint64_t pairs = (static_cast<uint64_t>(m) + 1) / 2;
-    const uint64_t pair = static_cast<uint64_t>(blockIdx.x) * kBlock + threadIdx.x;
-    if (pair > pairs) return;
-    if (pair == pairs) {  // the slot that receives the total after the scan
-        if (!FILL) pair_ptr[pair] = 0;
+__global__ __launch_bounds__(kBlock) void group_merge_kernel(idx_t m, idx_t base, const idx_t* __restrict__ row_ptr,
+                                                             const idx_t* __restrict__ col,
+                                                             uint32_t* __restrict__ group_ptr,
+                                                             uint32_t* __restrict__ entries) {
+    const uint64_t groups = spmm_groups(m);
+    const uint64_t group = static_cast<uint64_t>(blockIdx.x) * kBlock + threadIdx.x;
+    if (group > groups) return;
+    if (group == groups) {  // the slot that receives the total after the scan
+        if (!FILL) group_ptr[group] = 0;
         return;
     }
-    const uint64_t r0 = 2 * pair;
-    idx_t i0 = row_ptr[r0] - base;
-    const idx_t e0 = row_ptr[r0 + 1] - base;
-    idx_t i1 = e0;
-    const idx_t e1 = r0 + 1 < static_cast<uint64_t>(m) ? row_ptr[r0 + 2] - base : e0;
-    if (e1 - i0 > kSpmmMaxMergedPair) {
-        if (!FILL) pair_ptr[pair] = 0;
+    idx_t i[R], e[R];
+    group_row_ranges(m, base, row_ptr, group * R, i, e);
+    if (e[R - 1] - i[0] > kSpmmMaxMergedGroup) {
+        if (!FILL) group_ptr[group] = 0;
         return;
     }
-    const uint32_t out = FILL ? pair_ptr[pair] : 0;
+    const uint32_t out = FILL ? group_ptr[group] : 0;
     uint32_t count = 0;
-    while (i0 < e0 || i1 < e1) {
-        const uint32_t h0 = i0 < e0 ? static_cast<uint32_t>(col[i0] - base) : kNoColumn;
-        const uint32_t h1 = i1 < e1 ? static_cast<uint32_t>(col[i1] - base) : kNoColumn;
-        const uint32_t lo = h0 < h1 ? h0 : h1;
-        const uint32_t t0 = h0 == lo, t1 = h1 == lo;
-        if (FILL) entries[out + count] = (lo << 2) | t0 | (t1 << 1);
+    while (true) {
+        uint32_t head[R];
+        uint32_t lo = kNoColumn;
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            head[r] = i[r] < e[r] ? static_cast<uint32_t>(col[i[r]] - base) : kNoColumn;
+            lo = head[r] < lo ? head[r] : lo;
+        }
+        if (lo == kNoColumn) break;
+        uint32_t flags = 0;
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const uint32_t takes = head[r] == lo;
+            flags |= takes << r;
+            i[r] += takes;
+        }
+        if (FILL) entries[out + count] = (lo << R) | flags;
         ++count;
-        i0 += t0;
-        i1 += t1;
     }
-    if (!FILL) pair_ptr[pair] = count;
+    if (!FILL) group_ptr[group] = count;
 }
 
 // Returns the top bit of w and shifts w left by one: an add whose carry is the answer.
@@ -301,63 +320,67 @@ __device__ __forceinline__ bool shift_out_top(uint32_t& w) {
     return top;
 }
 
-// LR lanes (4..64) per row pair, V = 16 B / sizeof(T) adjacent columns per lane; blockIdx.y walks
+// LR lanes (4..64) per row group, V = 16 B / sizeof(T) adjacent columns per lane; blockIdx.y walks
 // panels of LR*V columns.  The lanes of a group fetch LR entries of the merged list at once, one
-// each, work out from the two flag bits which value of which row belongs to their entry, fetch
+// each, work out from the flag bits which value of which row belongs to their entry, fetch
 // those, and pass row offsets, flags and values round in registers.
 template <typename T, int LR, bool WIDE>
-__global__ __launch_bounds__(kBlock) void spmm_pair_kernel(idx_t m, idx_t n, idx_t base,
-                                                           const idx_t* __restrict__ row_ptr,
-                                                           const idx_t* __restrict__ col, const T* __restrict__ val,
-                                                           const uint32_t* __restrict__ pair_ptr,
-                                                           const uint32_t* __restrict__ entries,
-                                                           const T* __restrict__ B, int64_t ldb, T* __restrict__ C,
-                                                           int64_t ldc, bool c_row_major, T alpha, T beta) {
+__global__ __launch_bounds__(kBlock) void spmm_group_kernel(idx_t m, idx_t n, idx_t base,
+                                                            const idx_t* __restrict__ row_ptr,
+                                                            const idx_t* __restrict__ col, const T* __restrict__ val,
+                                                            const uint32_t* __restrict__ group_ptr,
+                                                            const uint32_t* __restrict__ entries,
+                                                            const T* __restrict__ B, int64_t ldb, T* __restrict__ C,
+                                                            int64_t ldc, bool c_row_major, T alpha, T beta) {
     typedef typename ByteOffset<WIDE>::type off_t;
     constexpr int V = 16 / sizeof(T);
-    constexpr int kPairsPerBlock = kBlock / LR;
+    constexpr int kGroupsPerBlock = kBlock / LR;
     constexpr int kBatch = LR < 8 ? LR : 8;
     const idx_t lane = threadIdx.x % LR;
-    const uint64_t pair = static_cast<uint64_t>(blockIdx.x) * kPairsPerBlock + threadIdx.x / LR;
-    const uint64_t r0 = 2 * pair;
+    const uint64_t group = static_cast<uint64_t>(blockIdx.x) * kGroupsPerBlock + threadIdx.x / LR;
+    const uint64_t r0 = group * R;
     if (r0 >= static_cast<uint64_t>(m)) return;  // whole lane groups
     const uint64_t c_own = (static_cast<uint64_t>(blockIdx.y) * LR + lane) * V;
     const bool stores = c_own < static_cast<uint64_t>(n);  // lanes past the last column only help fetching
     const uint64_t c0 = stores ? c_own : 0;
-    const bool two_rows = r0 + 1 < static_cast<uint64_t>(m);
 
-    idx_t i0 = row_ptr[r0] - base;
-    const idx_t e0 = row_ptr[r0 + 1] - base;
-    idx_t i1 = e0;
-    const idx_t e1 = two_rows ? row_ptr[r0 + 2] - base : e0;
+    idx_t i[R], e[R];
+    group_row_ranges(m, base, row_ptr, r0, i, e);
 
-    T acc0[V], acc1[V];
+    T acc[R][V];
 #pragma unroll
-    for (int i = 0; i < V; ++i) acc0[i] = acc1[i] = T(0);
+    for (int r = 0; r < R; ++r) {
+#pragma unroll
+        for (int c = 0; c < V; ++c) acc[r][c] = T(0);
+    }
     const char* B_bytes = reinterpret_cast<const char*>(B);
     const off_t lane_off = static_cast<off_t>(c0 * sizeof(T));
     const off_t ldb_bytes = static_cast<off_t>(ldb * sizeof(T));
 
-    if (e1 - i0 <= kSpmmMaxMergedPair) {
-        const uint32_t s_end = pair_ptr[pair + 1];
+    if (e[R - 1] - i[0] <= kSpmmMaxMergedGroup) {
+        const uint32_t s_end = group_ptr[group + 1];
         const unsigned group_first = (__lane_id() / LR) * LR;
         const uint64_t group_bits = LR == kWave ? ~0ull : ((1ull << (LR % kWave)) - 1ull);
         const uint64_t below = (1ull << lane) - 1ull;
-        for (uint32_t s = pair_ptr[pair]; s < s_end; s += LR) {
-            const uint32_t e = s + lane < s_end ? entries[s + lane] : 0u;
-            // this lane's entry is the p0-th of the chunk that row 2p takes part in, the p1-th for row 2p+1
-            const uint64_t in0 = (__ballot(e & 1u) >> group_first) & group_bits;
-            const uint64_t in1 = (__ballot(e & 2u) >> group_first) & group_bits;
-            const T v0 = (e & 1u) ? val[i0 + __popcll(in0 & below)] : T(0);
-            const T v1 = (e & 2u) ? val[i1 + __popcll(in1 & below)] : T(0);
-            i0 += __popcll(in0);
-            i1 += __popcll(in1);
-            const off_t roff = static_cast<off_t>(e >> 2) * ldb_bytes;
-            // Which entries each row takes part in, as one bit per entry with entry 0 in the top
-            // bit: doubling the word moves the next entry's bit into the carry, which is then the
-            // lane mask the multiply-adds of that entry run under.
-            uint32_t take0 = __brev(static_cast<uint32_t>(in0)), take1 = __brev(static_cast<uint32_t>(in1));
-            const uint32_t flags = e & 3u;
+        for (uint32_t s = group_ptr[group]; s < s_end; s += LR) {
+            const uint32_t ent = s + lane < s_end ? entries[s + lane] : 0u;
+            // this lane's entry is the p-th of the chunk that row r takes part in: the p-th value of
+            // the row from where the row stands.  take[r] holds which entries of the chunk row r
+            // takes part in, one bit per entry with entry 0 in the top bit: doubling the word moves
+            // the next entry's bit into the carry, which is then the lane mask the multiply-adds of
+            // that entry run under.
+            T v[R];
+            uint32_t take[R];
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                const bool mine = (ent >> r) & 1u;
+                const uint64_t in = (__ballot(mine) >> group_first) & group_bits;
+                v[r] = mine ? val[i[r] + __popcll(in & below)] : T(0);
+                i[r] += __popcll(in);
+                take[r] = __brev(static_cast<uint32_t>(in));
+            }
+            const off_t roff = static_cast<off_t>(ent >> R) * ldb_bytes;
+            const uint32_t flags = ent & ((1u << R) - 1u);
             const uint32_t left = s_end - s;
             auto chunk = [&](auto checked) {
                 constexpr bool kChecked = decltype(checked)::value;
@@ -376,25 +399,19 @@ __global__ __launch_bounds__(kBlock) void spmm_pair_kernel(idx_t m, idx_t n, idx
                             constexpr int k = u0 + decltype(u)::value;
                             if (!kChecked || k < left) {
                                 // a row that lacks the column must not see it at all (0 * inf would be NaN)
-                                bool row0, row1;
-                                if constexpr (LR == kWave) {  // one group per wavefront: the flags are scalars
-                                    const uint32_t fk = group_bcast<LR, k>(flags);
-                                    row0 = fk & 1u;
-                                    row1 = fk & 2u;
-                                } else {
-                                    row0 = shift_out_top(take0);
-                                    row1 = shift_out_top(take1);
-                                }
-                                if (row0) {
-                                    const T a = group_bcast<LR, k>(v0);
+                                uint32_t fk = 0;
+                                if constexpr (LR == kWave) fk = group_bcast<LR, k>(flags);  // one group per wavefront: scalar
+                                static_for<R>([&](auto rc) {
+                                    constexpr int r = decltype(rc)::value;
+                                    bool has;
+                                    if constexpr (LR == kWave) has = (fk >> r) & 1u;
+                                    else has = shift_out_top(take[r]);
+                                    if (has) {
+                                        const T a = group_bcast<LR, k>(v[r]);
 #pragma unroll
-                                    for (int i = 0; i < V; ++i) acc0[i] += a * b[decltype(u)::value].v[i];
-                                }
-                                if (row1) {
-                                    const T a = group_bcast<LR, k>(v1);
-#pragma unroll
-                                    for (int i = 0; i < V; ++i) acc1[i] += a * b[decltype(u)::value].v[i];
-                                }
+                                        for (int c = 0; c < V; ++c) acc[r][c] += a * b[decltype(u)::value].v[c];
+                                    }
+                                });
                             }
                         });
                     }
@@ -404,14 +421,17 @@ __global__ __launch_bounds__(kBlock) void spmm_pair_kernel(idx_t m, idx_t n, idx
             else chunk(std::true_type{});
         }
     } else {
-        // a pair too long to be worth merging: one row after the other
-        row_times_b<T, LR, V, WIDE>(i0, e0, lane, base, col, val, B_bytes, lane_off, ldb_bytes, acc0);
-        row_times_b<T, LR, V, WIDE>(i1, e1, lane, base, col, val, B_bytes, lane_off, ldb_bytes, acc1);
+        // a group too long to be worth merging: one row after the other
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+            row_times_b<T, LR, V, WIDE>(i[r], e[r], lane, base, col, val, B_bytes, lane_off, ldb_bytes, acc[r]);
     }
 
     if (!stores) return;
-    store_c<T, V>(C, ldc, c_row_major, r0, c0, acc0, alpha, beta);
-    if (two_rows) store_c<T, V>(C, ldc, c_row_major, r0 + 1, c0, acc1, alpha, beta);
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        if (r0 + r < static_cast<uint64_t>(m)) store_c<T, V>(C, ldc, c_row_major, r0 + r, c0, acc[r], alpha, beta);
+    }
 }
 
 // op(B) lies within 4 GiB of its first element: byte offsets into it fit 32 bits
@@ -421,22 +441,22 @@ bool narrow_offsets(const SpmmArgs& a, size_t value_bytes) {
 }
 
 template <typename T, int LR>
-void launch_pair(hipStream_t stream, const SpmmArgs& a, const uint32_t* pair_ptr, const uint32_t* entries, T alpha,
-                 T beta) {
+void launch_group(hipStream_t stream, const SpmmArgs& a, const uint32_t* group_ptr, const uint32_t* entries, T alpha,
+                  T beta) {
     constexpr int V = 16 / sizeof(T);
-    const uint64_t pairs = (static_cast<uint64_t>(a.m) + 1) / 2;
-    const uint64_t pair_blocks = (pairs + (kBlock / LR) - 1) / (kBlock / LR);
+    const uint64_t groups = spmm_groups(a.m);
+    const uint64_t group_blocks = (groups + (kBlock / LR) - 1) / (kBlock / LR);
     const uint64_t panels = (static_cast<uint64_t>(a.n) + LR * V - 1) / (LR * V);
-    const dim3 grid(static_cast<uint32_t>(pair_blocks), static_cast<uint32_t>(panels));
+    const dim3 grid(static_cast<uint32_t>(group_blocks), static_cast<uint32_t>(panels));
     const T* val = static_cast<const T*>(a.val);
     const T* B = static_cast<const T*>(a.B);
     T* C = static_cast<T*>(a.C);
     if (narrow_offsets(a, sizeof(T))) {
-        hipLaunchKernelGGL((spmm_pair_kernel<T, LR, false>), grid, dim3(kBlock), 0, stream, a.m, a.n, a.base, a.row_ptr,
-                           a.col, val, pair_ptr, entries, B, a.ldb, C, a.ldc, a.c_row_major, alpha, beta);
+        hipLaunchKernelGGL((spmm_group_kernel<T, LR, false>), grid, dim3(kBlock), 0, stream, a.m, a.n, a.base, a.row_ptr,
+                           a.col, val, group_ptr, entries, B, a.ldb, C, a.ldc, a.c_row_major, alpha, beta);
     } else {
-        hipLaunchKernelGGL((spmm_pair_kernel<T, LR, true>), grid, dim3(kBlock), 0, stream, a.m, a.n, a.base, a.row_ptr,
-                           a.col, val, pair_ptr, entries, B, a.ldb, C, a.ldc, a.c_row_major, alpha, beta);
+        hipLaunchKernelGGL((spmm_group_kernel<T, LR, true>), grid, dim3(kBlock), 0, stream, a.m, a.n, a.base, a.row_ptr,
+                           a.col, val, group_ptr, entries, B, a.ldb, C, a.ldc, a.c_row_major, alpha, beta);
     }
 }
 
@@ -502,9 +522,9 @@ void launch_spmm(hipStream_t stream, const SpmmArgs& a, T alpha, T beta) {
 
 SpmmScheduleLayout spmm_schedule_layout(idx_t m, idx_t nnz) {
     SpmmScheduleLayout l;
-    const uint64_t slots = (static_cast<uint64_t>(m) + 1) / 2 + 1;
+    const uint64_t slots = spmm_groups(m) + 1;
     size_t off = 0;
-    l.pair_ptr = off; off += align_up(slots * sizeof(uint32_t));
+    l.group_ptr = off; off += align_up(slots * sizeof(uint32_t));
     l.entries = off; off += align_up(static_cast<size_t>(nnz) * sizeof(uint32_t));
     l.scan_ws = off; off += exclusive_scan_workspace_bytes(slots);
     l.total = off;
@@ -515,20 +535,20 @@ void launch_spmm_schedule(hipStream_t stream, idx_t m, idx_t nnz, idx_t base, co
                           void* schedule) {
     const SpmmScheduleLayout l = spmm_schedule_layout(m, nnz);
     char* w = static_cast<char*>(schedule);
-    uint32_t* pair_ptr = reinterpret_cast<uint32_t*>(w + l.pair_ptr);
+    uint32_t* group_ptr = reinterpret_cast<uint32_t*>(w + l.group_ptr);
     uint32_t* entries = reinterpret_cast<uint32_t*>(w + l.entries);
-    const uint64_t slots = (static_cast<uint64_t>(m) + 1) / 2 + 1;
+    const uint64_t slots = spmm_groups(m) + 1;
     const dim3 grid(static_cast<uint32_t>((slots + kBlock - 1) / kBlock));
-    hipLaunchKernelGGL((pair_merge_kernel<false>), grid, dim3(kBlock), 0, stream, m, base, row_ptr, col, pair_ptr,
+    hipLaunchKernelGGL((group_merge_kernel<false>), grid, dim3(kBlock), 0, stream, m, base, row_ptr, col, group_ptr,
                        entries);
-    launch_exclusive_scan_u32(stream, pair_ptr, slots, w + l.scan_ws);
-    hipLaunchKernelGGL((pair_merge_kernel<true>), grid, dim3(kBlock), 0, stream, m, base, row_ptr, col, pair_ptr,
+    launch_exclusive_scan_u32(stream, group_ptr, slots, w + l.scan_ws);
+    hipLaunchKernelGGL((group_merge_kernel<true>), grid, dim3(kBlock), 0, stream, m, base, row_ptr, col, group_ptr,
                        entries);
 }
 
 bool spmm_schedule_usable(const SpmmArgs& a, size_t value_bytes) {
     const int64_t wide = static_cast<int64_t>(16 / value_bytes);
-    // narrower than four 128-bit vectors per row: too few lanes per pair to share the fetching
+    // narrower than four 128-bit vectors per row: too few lanes per group to share the fetching
     return a.b_row_major && a.n >= 3 * wide + 1 && a.k <= kSpmmMaxScheduledColumns &&
            reinterpret_cast<uintptr_t>(a.B) % 16 == 0 &&
            a.ldb % wide == 0 && a.n % wide == 0 &&
@@ -541,14 +561,14 @@ void launch_spmm_scheduled(hipStream_t stream, const SpmmArgs& a, const void* sc
     constexpr int V = 16 / sizeof(T);
     const SpmmScheduleLayout l = spmm_schedule_layout(a.m, a.nnz);
     const char* w = static_cast<const char*>(schedule);
-    const uint32_t* pair_ptr = reinterpret_cast<const uint32_t*>(w + l.pair_ptr);
+    const uint32_t* group_ptr = reinterpret_cast<const uint32_t*>(w + l.group_ptr);
     const uint32_t* entries = reinterpret_cast<const uint32_t*>(w + l.entries);
     const uint64_t lanes_needed = (static_cast<uint64_t>(a.n) + V - 1) / V;
-    if (lanes_needed <= 4) launch_pair<T, 4>(stream, a, pair_ptr, entries, alpha, beta);
-    else if (lanes_needed <= 8) launch_pair<T, 8>(stream, a, pair_ptr, entries, alpha, beta);
-    else if (lanes_needed <= 16) launch_pair<T, 16>(stream, a, pair_ptr, entries, alpha, beta);
-    else if (lanes_needed <= 32) launch_pair<T, 32>(stream, a, pair_ptr, entries, alpha, beta);
-    else launch_pair<T, 64>(stream, a, pair_ptr, entries, alpha, beta);
+    if (lanes_needed <= 4) launch_group<T, 4>(stream, a, group_ptr, entries, alpha, beta);
+    else if (lanes_needed <= 8) launch_group<T, 8>(stream, a, group_ptr, entries, alpha, beta);
+    else if (lanes_needed <= 16) launch_group<T, 16>(stream, a, group_ptr, entries, alpha, beta);
+    else if (lanes_needed <= 32) launch_group<T, 32>(stream, a, group_ptr, entries, alpha, beta);
+    else launch_group<T, 64>(stream, a, group_ptr, entries, alpha, beta);
 }
 
 template void launch_spmm_scheduled<float>(hipStream_t, const SpmmArgs&, const void*, float, float);

@@ -248,7 +248,7 @@ def test_spmm_argument_checks(lib):
     assert call(b=Bt) == api.STATUS_INVALID_VALUE  # B is 4 x 6 but op(B) must be 6 x 4
     size = ctypes.c_size_t()
     assert lib.mcsparseSpMM_bufferSize(o.h, 0, 0, o.pa, o.A, B, o.pa, C, api.R_32F, 0, ctypes.byref(size)) == 0
-    # room for the row-pair schedule of mcsparseSpMM_preprocess: 4 + 1 offsets, 20 entries, scan scratch
+    # room for the row-group schedule of mcsparseSpMM_preprocess: group offsets, 20 entries, scan scratch
     assert size.value % 128 == 0 and size.value >= 128 + 128 and size.value < 4096
     assert lib.mcsparseSpMM_bufferSize(None, 0, 0, o.pa, o.A, B, o.pa, C, api.R_32F, 0, ctypes.byref(size)) == 1
     assert lib.mcsparseSpMM_bufferSize(o.h, 0, 0, o.pa, o.A, None, o.pa, C, api.R_32F, 0, ctypes.byref(size)) == 3

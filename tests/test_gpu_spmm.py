@@ -114,12 +114,12 @@ def test_exact_cases(torch_gpu, handle):
     assert st == 0 and np.array_equal(got, C0)
 
 
-# ---- row-pair schedule (mcsparseSpMM_preprocess) ------------------------------------------------
+# ---- row-group schedule (mcsparseSpMM_preprocess) ------------------------------------------------
 
 @pytest.mark.parametrize("n", [4, 8, 24, 64, 100, 256, 260])
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
 def test_preprocessed_stencil(torch_gpu, handle, oracle, n, dtype):
-    a = wl.stencil_27pt(13, dtype=dtype).with_base(1)  # odd row count: the last row has no partner
+    a = wl.stencil_27pt(13, dtype=dtype).with_base(1)  # row count not a multiple of the group size: the last group is short
     for c_order in (api.ORDER_ROW, api.ORDER_COL):
         check(torch_gpu, handle, oracle, a, n, 1.0, 0.0, preprocess=True, expect_schedule=2, c_order=c_order)
         check(torch_gpu, handle, oracle, a, n, -1.5, 0.75, preprocess=True, expect_schedule=2, c_order=c_order, pad_b=4,
@@ -127,7 +127,7 @@ def test_preprocessed_stencil(torch_gpu, handle, oracle, n, dtype):
 
 
 def test_preprocessed_ragged_rows_with_overlap(torch_gpu, handle, oracle):
-    """Rows of different lengths, empty rows, unsorted columns inside rows, a pair too long to merge."""
+    """Rows of different lengths, empty rows, unsorted columns inside rows, a group too long to merge."""
     rng = np.random.default_rng(12)
     m, k = 501, 3000
     rows = []
@@ -135,7 +135,7 @@ def test_preprocessed_ragged_rows_with_overlap(torch_gpu, handle, oracle):
         if r % 7 == 3:
             cols = np.zeros(0, np.int64)
         elif r in (100, 101):
-            cols = rng.choice(k, 700, replace=False)            # 1400 nonzeros in the pair: not merged
+            cols = rng.choice(k, 1100, replace=False)           # 2200 nonzeros in their group: not merged
         else:
             prev = rows[-1] if rows and len(rows[-1]) else rng.choice(k, 12, replace=False)
             keep = prev[rng.random(len(prev)) < 0.8]
