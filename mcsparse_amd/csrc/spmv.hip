@@ -25,7 +25,10 @@ constexpr int kBlock = 256;
 // ------------------------------------------------------------------------------------------
 // vector family
 // ------------------------------------------------------------------------------------------
-template <typename T, int L, int U, bool BETA0>
+// What a kernel does with a finished row sum s.
+enum YUpdate : int { kYSet = 0, kYScale = 1 };  // y = alpha*s | y = beta*y + alpha*s
+
+template <typename T, int L, int U, int UPDATE>
 __global__ __launch_bounds__(kBlock) void spmv_vector_kernel(idx_t m, idx_t base, const idx_t* __restrict__ row_ptr,
                                                              const idx_t* __restrict__ col,
                                                              const T* __restrict__ val, const T* __restrict__ x,
@@ -56,16 +59,19 @@ __global__ __launch_bounds__(kBlock) void spmv_vector_kernel(idx_t m, idx_t base
     do {
         idx_t c[U];
         T v[U];
+        bool act[U];
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-            const bool act = j[u] < e[u];
-            c[u] = act ? load_stream(col + j[u]) : base;
-            v[u] = act ? load_stream(val + j[u]) : T(0);
+            act[u] = j[u] < e[u];
+            c[u] = act[u] ? load_stream(col + j[u]) : base;
+            v[u] = act[u] ? load_stream(val + j[u]) : T(0);
         }
         more = false;
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-            s[u] += v[u] * x[c[u] - base];
+            // a lane without a nonzero must not touch the sum at all: 0 * x[..] is NaN for an infinite x
+            const T xv = x[c[u] - base];
+            if (act[u]) s[u] += v[u] * xv;
             j[u] += L;
             more |= j[u] < e[u];
         }
@@ -79,7 +85,7 @@ __global__ __launch_bounds__(kBlock) void spmv_vector_kernel(idx_t m, idx_t base
         for (int u = 0; u < U; ++u) {
             const uint64_t row = row0 + static_cast<uint64_t>(u) * kGroups;
             if (row < m) {
-                if constexpr (BETA0) {
+                if constexpr (UPDATE == kYSet) {
                     y[row] = alpha * s[u];
                 } else {
                     y[row] = beta * y[row] + alpha * s[u];
@@ -98,10 +104,10 @@ void launch_vector_lu(hipStream_t stream, const SpmvArgs& a, T alpha, T beta) {
     const T* x = static_cast<const T*>(a.x);
     T* y = static_cast<T*>(a.y);
     if (beta == T(0)) {
-        hipLaunchKernelGGL((spmv_vector_kernel<T, L, U, true>), grid, dim3(kBlock), 0, stream, a.m, a.base, a.row_ptr,
+        hipLaunchKernelGGL((spmv_vector_kernel<T, L, U, kYSet>), grid, dim3(kBlock), 0, stream, a.m, a.base, a.row_ptr,
                            a.col, val, x, y, alpha, beta);
     } else {
-        hipLaunchKernelGGL((spmv_vector_kernel<T, L, U, false>), grid, dim3(kBlock), 0, stream, a.m, a.base,
+        hipLaunchKernelGGL((spmv_vector_kernel<T, L, U, kYScale>), grid, dim3(kBlock), 0, stream, a.m, a.base,
                            a.row_ptr, a.col, val, x, y, alpha, beta);
     }
 }

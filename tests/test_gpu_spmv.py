@@ -154,6 +154,29 @@ def test_scalar_special_cases(torch_gpu, handle, oracle):
         assert_within(y, y_ref, bound, np.float32)
 
 
+def test_unreferenced_infinite_x_stays_out(torch_gpu, handle, oracle):
+    """x[0] = inf and x[last] = nan, columns no row but one names: only that row may see them.
+    (Lanes past the end of a short row once multiplied 0 by x[0].)"""
+    rng = np.random.default_rng(21)
+    m, n = 3000, 4000
+    rows = [np.sort(rng.choice(np.arange(1, n - 1), rng.integers(0, 40), replace=False)) for _ in range(m)]
+    rows[7] = np.array([0, 5, n - 1])
+    ptr = np.concatenate([[0], np.cumsum([len(c) for c in rows])]).astype(np.int32)
+    col = np.concatenate(rows).astype(np.int32)
+    for dt in (np.float32, np.float64):
+        a = wl.Csr(m, n, ptr, col, rng.uniform(-1, 1, len(col)).astype(dt))
+        x = rng.uniform(-1, 1, n).astype(dt)
+        x[0], x[n - 1] = np.inf, np.nan
+        for fam, lanes in ((api.FAMILY_VECTOR, 0), (api.FAMILY_VECTOR, 64), (api.FAMILY_VECTOR, 4), (api.FAMILY_MERGE, 0)):
+            st, y, _ = run_spmv(torch_gpu, handle, a, x, np.zeros(m, dt), 1.0, 0.0, family=fam, lanes=lanes)
+            assert st == 0
+            assert np.isnan(y[7]) and np.isfinite(np.delete(y, 7)).all(), (dt, fam, lanes)
+            xf = x.copy()
+            xf[0] = xf[n - 1] = 0
+            y_ref, bound = oracle.spmv(False, m, n, 0, ptr, col, a.val, 1.0, 0.0, xf, None)
+            assert_within(np.delete(y, 7), np.delete(y_ref, 7), np.delete(bound, 7), dt)
+
+
 def test_same_result_on_repeat_and_y_transpose_identity(torch_gpu, handle, oracle):
     # deterministic: two runs agree bit for bit, for both families; and y^T(Ax) = (A^T y)^T x
     a = wl.power_law(m=20000, max_len=9000, dtype=np.float64)
