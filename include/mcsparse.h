@@ -261,6 +261,16 @@ mcsparseStatus_t mcsparseDnMatGet(mcsparseDnMatDescr_t dnMatDescr, int64_t* rows
 mcsparseStatus_t mcsparseDnMatGetValues(mcsparseDnMatDescr_t dnMatDescr, void** values);
 mcsparseStatus_t mcsparseDnMatSetValues(mcsparseDnMatDescr_t dnMatDescr, void* values);
 
+/* ---- strided batches for SpMM: include/interface/mcsp_generic.h:178-185 ------------- */
+/* Batch b of a call uses the arrays moved on by b strides (in elements); all three operands
+ * of an SpMM must carry the same batch count (src/kernels/level3/spmm/mcsp_spmm_gpu.cpp:96-98).
+ * A stride of 0 shares the array between the batches. */
+mcsparseStatus_t mcsparseCooSetStridedBatch(mcsparseSpMatDescr_t spMatDescr, int batchCount, int64_t batchStride);
+mcsparseStatus_t mcsparseCsrSetStridedBatch(mcsparseSpMatDescr_t spMatDescr, int batchCount, int64_t offsetsBatchStride,
+                                            int64_t columnsValuesBatchStride);
+mcsparseStatus_t mcsparseDnMatSetStridedBatch(mcsparseDnMatDescr_t dnMatDescr, int batchCount, int64_t batchStride);
+mcsparseStatus_t mcsparseDnMatGetStridedBatch(mcsparseDnMatDescr_t dnMatDescr, int* batchCount, int64_t* batchStride);
+
 /* ---- y = alpha*op(A)*x + beta*y : include/interface/mcsp_generic.h:43-51 ---------- */
 /* externalBuffer is caller-allocated device scratch of at least *bufferSize bytes and must be
  * non-NULL even for op N (src/kernels/level2/spmv/mcsp_spmv_gpu.cpp:703-705).  Work is

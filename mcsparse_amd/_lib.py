@@ -51,6 +51,10 @@ PROTOTYPES = {
     "mcsparseDnMatGet": (c_int, [vp, P(c_i64), P(c_i64), P(c_i64), P(vp), P(c_int), P(c_int)]),
     "mcsparseDnMatGetValues": (c_int, [vp, P(vp)]),
     "mcsparseDnMatSetValues": (c_int, [vp, vp]),
+    "mcsparseCooSetStridedBatch": (c_int, [vp, c_int, c_i64]),
+    "mcsparseCsrSetStridedBatch": (c_int, [vp, c_int, c_i64, c_i64]),
+    "mcsparseDnMatSetStridedBatch": (c_int, [vp, c_int, c_i64]),
+    "mcsparseDnMatGetStridedBatch": (c_int, [vp, P(c_int), P(c_i64)]),
     "mcsparseSpMV": (c_int, [vp, c_int, vp, vp, vp, vp, vp, c_int, c_int, vp]),
     "mcsparseSpMV_bufferSize": (c_int, [vp, c_int, vp, vp, vp, vp, vp, c_int, c_int, P(c_size)]),
     "mcsparseSpMM_bufferSize": (c_int, [vp, c_int, c_int, vp, vp, vp, vp, vp, c_int, c_int, P(c_size)]),

@@ -37,21 +37,24 @@ struct CsrView {
     bool transpose;      // the call needs view^T
 };
 
-CsrView make_view(const mcsparseSpMatDescr* A, mcsparseOperation_t op) {
+CsrView make_view(const mcsparseSpMatDescr* A, mcsparseOperation_t op, const idx_t* rows32 = nullptr,
+                  const idx_t* cols32 = nullptr) {
+    const idx_t* a_rows = rows32 != nullptr ? rows32 : static_cast<const idx_t*>(A->rows);
+    const idx_t* a_cols = cols32 != nullptr ? cols32 : static_cast<const idx_t*>(A->cols);
     CsrView v;
     const bool op_t = op != MCSPARSE_OPERATION_NON_TRANSPOSE;
     v.coo_rows = nullptr;
     if (A->format == MCSPARSE_FORMAT_CSC) {
         v.m = A->col_num;
         v.n = A->row_num;
-        v.ptr = static_cast<const idx_t*>(A->cols);  // column offsets
-        v.ind = static_cast<const idx_t*>(A->rows);  // row indices
+        v.ptr = a_cols;  // column offsets
+        v.ind = a_rows;  // row indices
         v.transpose = !op_t;
     } else {
         v.m = A->row_num;
         v.n = A->col_num;
-        v.ptr = static_cast<const idx_t*>(A->rows);
-        v.ind = static_cast<const idx_t*>(A->cols);
+        v.ptr = a_rows;
+        v.ind = a_cols;
         v.transpose = op_t;
         if (A->format == MCSPARSE_FORMAT_COO) {
             v.coo_rows = v.ptr;
@@ -69,12 +72,13 @@ bool format_is_built(mcsparseFormat_t f) {
 // Scratch layout of an SpMV call, all parts aligned to 128 bytes:
 //   [analysis][merge workspace][COO only: row offsets m+1]
 //   transposing calls add [col_ptr n+1 | row_ind nnz][values][csr2csc workspace]
+//   64-bit index arrays add their narrowed copies at the end
 // (the transposed part is the reference's layout, mcsp_spmv_gpu.cpp:308 and :813-831).
 struct SpmvLayout {
-    size_t merge_ws, coo_ptr, col_ptr, row_ind, vals, csr2csc_ws, total;
+    size_t merge_ws, coo_ptr, col_ptr, row_ind, vals, csr2csc_ws, narrow, total;
 };
 
-SpmvLayout spmv_layout(const CsrView& v, int64_t nnz, size_t value_bytes) {
+SpmvLayout spmv_layout(const CsrView& v, int64_t nnz, size_t value_bytes, size_t narrow) {
     SpmvLayout l = {};
     const int64_t out_rows = v.transpose ? v.n : v.m;  // rows of the matrix the SpMV kernel sees
     size_t off = kAnalysisBytes;
@@ -93,6 +97,8 @@ SpmvLayout spmv_layout(const CsrView& v, int64_t nnz, size_t value_bytes) {
         off += align_up(mcsp::csr2csc_workspace_bytes(static_cast<idx_t>(v.m), static_cast<idx_t>(v.n),
                                                       static_cast<idx_t>(nnz), value_bytes));
     }
+    l.narrow = off;
+    off += narrow;
     l.total = off < kMinBuffer ? kMinBuffer : off;
     return l;
 }
@@ -122,10 +128,55 @@ mcspStatus_t check_spmv_args(mcsparseHandle_t handle, mcsparseOperation_t opA, c
 }
 
 // Row and column index types must agree; 32I and 64I are the two the reference dispatches on
-// (mcsp_spmv_gpu.cpp:1123-1133).  Only 32I is built here.
+// (mcsp_spmv_gpu.cpp:1123-1133).
 mcspStatus_t check_index_types(const mcsparseSpMatDescr* A) {
     if (A->rowIdxType == MCSPARSE_INDEX_32I && A->colIdxType == MCSPARSE_INDEX_32I) return MCSP_STATUS_SUCCESS;
+    if (A->rowIdxType == MCSPARSE_INDEX_64I && A->colIdxType == MCSPARSE_INDEX_64I) return MCSP_STATUS_SUCCESS;
     return MCSP_STATUS_NOT_IMPLEMENTED;
+}
+
+// The kernels work on 32-bit indices.  Every extent of a matrix is checked to be below 2^32
+// (as in the reference, mcsp_spmv_gpu.cpp:698-701), so the entries of 64-bit index arrays fit
+// 32 bits: a call on such a matrix first copies its two index arrays, narrowed, into the
+// scratch buffer and runs on the copies.  The reference instantiates its kernels for int64
+// instead (mcsp_spmv_gpu.cpp:1128-1129); the results are the same.
+bool wide_indices(const mcsparseSpMatDescr* A) { return A->rowIdxType == MCSPARSE_INDEX_64I; }
+
+// Lengths of the descriptor's `rows` and `cols` arrays.
+void index_array_lengths(const mcsparseSpMatDescr* A, size_t* rows_len, size_t* cols_len) {
+    const size_t nnz = static_cast<size_t>(A->nnz);
+    switch (A->format) {
+        case MCSPARSE_FORMAT_CSR: *rows_len = static_cast<size_t>(A->row_num) + 1; *cols_len = nnz; break;
+        case MCSPARSE_FORMAT_CSC: *rows_len = nnz; *cols_len = static_cast<size_t>(A->col_num) + 1; break;
+        default: *rows_len = nnz; *cols_len = nnz; break;  // COO
+    }
+}
+
+size_t narrow_bytes(const mcsparseSpMatDescr* A) {
+    if (!wide_indices(A)) return 0;
+    size_t rl, cl;
+    index_array_lengths(A, &rl, &cl);
+    return align_up(rl * sizeof(idx_t)) + align_up(cl * sizeof(idx_t));
+}
+
+// 32-bit `rows` and `cols` arrays of the descriptor: the caller's own, or narrowed copies
+// written to `region` (narrow_bytes(A) bytes).
+struct IndexArrays {
+    const idx_t* rows;
+    const idx_t* cols;
+};
+IndexArrays index_arrays(mcsparseHandle_t h, const mcsparseSpMatDescr* A, char* region) {
+    IndexArrays out = {static_cast<const idx_t*>(A->rows), static_cast<const idx_t*>(A->cols)};
+    if (!wide_indices(A)) return out;
+    size_t rl, cl;
+    index_array_lengths(A, &rl, &cl);
+    idx_t* r32 = reinterpret_cast<idx_t*>(region);
+    idx_t* c32 = reinterpret_cast<idx_t*>(region + align_up(rl * sizeof(idx_t)));
+    if (A->rows != nullptr) mcsp::launch_narrow_indices(h->stream, static_cast<const int64_t*>(A->rows), r32, rl);
+    if (A->cols != nullptr) mcsp::launch_narrow_indices(h->stream, static_cast<const int64_t*>(A->cols), c32, cl);
+    out.rows = A->rows != nullptr ? r32 : nullptr;
+    out.cols = A->cols != nullptr ? c32 : nullptr;
+    return out;
 }
 
 // Chooses the kernel family for a structure; runs the row-length analysis (one kernel, one
@@ -171,8 +222,8 @@ mcspStatus_t ensure_plan(mcsparseHandle_t h, mcsparseSpMatDescr* A, const idx_t*
 }
 
 template <typename T>
-mcspStatus_t spmv_typed(mcsparseHandle_t h, mcsparseSpMatDescr* A, CsrView v, const void* alpha, const void* beta,
-                        const mcsparseDnVecDescr* x, mcsparseDnVecDescr* y, void* buffer) {
+mcspStatus_t spmv_typed(mcsparseHandle_t h, mcsparseSpMatDescr* A, mcsparseOperation_t op, const void* alpha,
+                        const void* beta, const mcsparseDnVecDescr* x, mcsparseDnVecDescr* y, void* buffer) {
     T h_alpha, h_beta;
     if (!scalar_to_host(h, beta, &h_beta) || !scalar_to_host(h, alpha, &h_alpha)) return MCSP_STATUS_INTERNAL_ERROR;
     // reference: mcsp_spmv_gpu.cpp:235-237 -- y is left untouched in both cases
@@ -181,8 +232,14 @@ mcspStatus_t spmv_typed(mcsparseHandle_t h, mcsparseSpMatDescr* A, CsrView v, co
     const idx_t nnz = static_cast<idx_t>(A->nnz);
     const idx_t base = static_cast<idx_t>(A->idxBase);
     char* buf = static_cast<char*>(buffer);
-    const SpmvLayout l = spmv_layout(v, A->nnz, sizeof(T));
+    CsrView v = make_view(A, op);
+    const SpmvLayout l = spmv_layout(v, A->nnz, sizeof(T), narrow_bytes(A));
+    // what identifies the structure to the plan cache: the caller's own array
     const void* signature = v.coo_rows != nullptr ? static_cast<const void*>(v.coo_rows) : v.ptr;
+    if (wide_indices(A)) {
+        const IndexArrays ia = index_arrays(h, A, buf + l.narrow);
+        v = make_view(A, op, ia.rows, ia.cols);
+    }
     if (v.coo_rows != nullptr) {
         idx_t* built = reinterpret_cast<idx_t*>(buf + l.coo_ptr);
         mcsp::launch_coo2csr(h->stream, nnz, static_cast<idx_t>(v.m), v.coo_rows, base, built);
@@ -231,9 +288,9 @@ mcspStatus_t spmv_typed(mcsparseHandle_t h, mcsparseSpMatDescr* A, CsrView v, co
 // Scratch layout of an SpMM call: CSR gets room for the row-group schedule that
 // mcsparseSpMM_preprocess builds (SpMM itself writes nothing there); COO gets [row offsets m+1];
 // CSC gets the transposed copy [row_ptr m+1 | col_ind nnz][values][csr2csc workspace]
-// (mcsp_spmm_gpu.cpp:818-849).
+// (mcsp_spmm_gpu.cpp:818-849); 64-bit index arrays add their narrowed copies at the end.
 struct SpmmLayout {
-    size_t ptr, ind, vals, csr2csc_ws, total;
+    size_t ptr, ind, vals, csr2csc_ws, narrow, total;
 };
 
 bool schedulable(const mcsparseSpMatDescr* A) {
@@ -264,6 +321,8 @@ SpmmLayout spmm_layout(const mcsparseSpMatDescr* A, size_t value_bytes) {
         off += align_up(mcsp::csr2csc_workspace_bytes(static_cast<idx_t>(A->col_num), static_cast<idx_t>(A->row_num),
                                                       static_cast<idx_t>(A->nnz), value_bytes));
     }
+    l.narrow = off;
+    off += narrow_bytes(A);
     l.total = off < kMinBuffer ? kMinBuffer : off;
     return l;
 }
@@ -276,51 +335,68 @@ mcspStatus_t spmm_typed(mcsparseHandle_t h, const mcsparseSpMatDescr* A, mcspars
     // reference: mcsp_spmm_gpu.cpp:110-114
     if (A->nnz == 0 && h_beta == T(1)) return MCSP_STATUS_SUCCESS;
 
-    mcsp::SpmmArgs a;
-    a.m = static_cast<idx_t>(A->row_num);
-    a.n = static_cast<idx_t>(C->col_num);
-    a.k = static_cast<idx_t>(A->col_num);
-    a.nnz = static_cast<idx_t>(A->nnz);
-    a.base = static_cast<idx_t>(A->idxBase);
-    a.row_ptr = static_cast<const idx_t*>(A->rows);
-    a.col = static_cast<const idx_t*>(A->cols);
-    a.val = A->vals;
     char* buf = static_cast<char*>(buffer);
     const SpmmLayout l = spmm_layout(A, sizeof(T));
-    if (A->format == MCSPARSE_FORMAT_COO && A->nnz != 0) {
-        idx_t* built = reinterpret_cast<idx_t*>(buf + l.ptr);
-        mcsp::launch_coo2csr(h->stream, a.nnz, a.m, static_cast<const idx_t*>(A->rows), a.base, built);
-        a.row_ptr = built;
-    } else if (A->format == MCSPARSE_FORMAT_CSC && A->nnz != 0) {
-        // the CSC arrays are the CSR of A^T (col_num x row_num); transposing them gives the CSR of A
-        idx_t* t_ptr = reinterpret_cast<idx_t*>(buf + l.ptr);
-        idx_t* t_ind = reinterpret_cast<idx_t*>(buf + l.ind);
-        void* t_val = buf + l.vals;
-        mcsp::launch_csr2csc(h->stream, static_cast<idx_t>(A->col_num), static_cast<idx_t>(A->row_num), a.nnz, A->vals,
-                             static_cast<const idx_t*>(A->cols), static_cast<const idx_t*>(A->rows), t_val, t_ind,
-                             t_ptr, sizeof(T), a.base, buf + l.csr2csc_ws);
-        a.row_ptr = t_ptr;
-        a.col = t_ind;
-        a.val = t_val;
-    } else if (A->format != MCSPARSE_FORMAT_CSR) {
-        // no nonzeros: C = beta*C over m empty rows; coo2csr with nnz = 0 writes the m+1 offsets
-        idx_t* built = reinterpret_cast<idx_t*>(buf + l.ptr);
-        mcsp::launch_coo2csr(h->stream, 0, a.m, built, a.base, built);
-        a.row_ptr = built;
-    }
-    a.B = B->values;
-    a.ldb = B->ld;
-    // op(B)(kk, j) sits at kk*ldb + j for (N, row-major) and (T, column-major), else at j*ldb + kk;
-    // the reference copies the first kind into the second (mcsp_spmm_gpu.cpp:119-133).
-    const bool op_n = opB == MCSPARSE_OPERATION_NON_TRANSPOSE;
-    a.b_row_major = (op_n && B->order == MCSPARSE_ORDER_ROW) || (!op_n && B->order == MCSPARSE_ORDER_COL);
-    a.C = C->values;
-    a.ldc = C->ld;
-    a.c_row_major = C->order == MCSPARSE_ORDER_ROW;
-    if (schedule_matches(A, buffer) && mcsp::spmm_schedule_usable(a, sizeof(T))) {
-        mcsp::launch_spmm_scheduled<T>(h->stream, a, buffer, h_alpha, h_beta);
-    } else {
-        mcsp::launch_spmm<T>(h->stream, a, h_alpha, h_beta);
+    // Strided batches (csr_spmm_device.hpp:102-108): batch b works on the arrays moved on by b
+    // strides; the reference runs them as blockIdx.z of one launch, here they are launches in a
+    // row on the stream, sharing the scratch buffer.
+    const int64_t batches = C->batchCount;
+    const bool shared_structure = A->offsetsBatchStride == 0 && A->batchStride == 0;
+    const size_t idx_bytes = wide_indices(A) ? sizeof(int64_t) : sizeof(idx_t);
+    for (int64_t b = 0; b < batches; ++b) {
+        mcsparseSpMatDescr Ab = *A;  // this batch's view of A
+        const int64_t rows_stride = A->format == MCSPARSE_FORMAT_CSR ? A->offsetsBatchStride : A->batchStride;
+        const int64_t cols_stride = A->format == MCSPARSE_FORMAT_CSC ? A->offsetsBatchStride : A->batchStride;
+        if (A->rows != nullptr) Ab.rows = static_cast<char*>(A->rows) + b * rows_stride * static_cast<int64_t>(idx_bytes);
+        if (A->cols != nullptr) Ab.cols = static_cast<char*>(A->cols) + b * cols_stride * static_cast<int64_t>(idx_bytes);
+        if (A->vals != nullptr) Ab.vals = static_cast<char*>(A->vals) + b * A->batchStride * static_cast<int64_t>(sizeof(T));
+        const IndexArrays ia = index_arrays(h, &Ab, buf + l.narrow);
+
+        mcsp::SpmmArgs a;
+        a.m = static_cast<idx_t>(A->row_num);
+        a.n = static_cast<idx_t>(C->col_num);
+        a.k = static_cast<idx_t>(A->col_num);
+        a.nnz = static_cast<idx_t>(A->nnz);
+        a.base = static_cast<idx_t>(A->idxBase);
+        a.row_ptr = ia.rows;
+        a.col = ia.cols;
+        a.val = Ab.vals;
+        if (A->format == MCSPARSE_FORMAT_COO && A->nnz != 0) {
+            idx_t* built = reinterpret_cast<idx_t*>(buf + l.ptr);
+            mcsp::launch_coo2csr(h->stream, a.nnz, a.m, ia.rows, a.base, built);
+            a.row_ptr = built;
+        } else if (A->format == MCSPARSE_FORMAT_CSC && A->nnz != 0) {
+            // the CSC arrays are the CSR of A^T (col_num x row_num); transposing them gives the CSR of A
+            idx_t* t_ptr = reinterpret_cast<idx_t*>(buf + l.ptr);
+            idx_t* t_ind = reinterpret_cast<idx_t*>(buf + l.ind);
+            void* t_val = buf + l.vals;
+            mcsp::launch_csr2csc(h->stream, static_cast<idx_t>(A->col_num), static_cast<idx_t>(A->row_num), a.nnz,
+                                 Ab.vals, ia.cols, ia.rows, t_val, t_ind, t_ptr, sizeof(T), a.base,
+                                 buf + l.csr2csc_ws);
+            a.row_ptr = t_ptr;
+            a.col = t_ind;
+            a.val = t_val;
+        } else if (A->format != MCSPARSE_FORMAT_CSR) {
+            // no nonzeros: C = beta*C over m empty rows; coo2csr with nnz = 0 writes the m+1 offsets
+            idx_t* built = reinterpret_cast<idx_t*>(buf + l.ptr);
+            mcsp::launch_coo2csr(h->stream, 0, a.m, built, a.base, built);
+            a.row_ptr = built;
+        }
+        a.B = static_cast<const char*>(B->values) + b * B->batchStride * static_cast<int64_t>(sizeof(T));
+        a.ldb = B->ld;
+        // op(B)(kk, j) sits at kk*ldb + j for (N, row-major) and (T, column-major), else at j*ldb + kk;
+        // the reference copies the first kind into the second (mcsp_spmm_gpu.cpp:119-133).
+        const bool op_n = opB == MCSPARSE_OPERATION_NON_TRANSPOSE;
+        a.b_row_major = (op_n && B->order == MCSPARSE_ORDER_ROW) || (!op_n && B->order == MCSPARSE_ORDER_COL);
+        a.C = static_cast<char*>(C->values) + b * C->batchStride * static_cast<int64_t>(sizeof(T));
+        a.ldc = C->ld;
+        a.c_row_major = C->order == MCSPARSE_ORDER_ROW;
+        // the schedule was built from batch 0's structure
+        if ((b == 0 || shared_structure) && schedule_matches(A, buffer) && mcsp::spmm_schedule_usable(a, sizeof(T))) {
+            mcsp::launch_spmm_scheduled<T>(h->stream, a, buffer, h_alpha, h_beta);
+        } else {
+            mcsp::launch_spmm<T>(h->stream, a, h_alpha, h_beta);
+        }
     }
     return MCSP_STATUS_SUCCESS;
 }
@@ -360,7 +436,7 @@ mcsparseStatus_t mcsparseSpMV_bufferSize(mcsparseHandle_t handle, mcsparseOperat
 
     const size_t vb = value_size(matA->valueType);
     const CsrView v = make_view(matA, opA);
-    const SpmvLayout l = spmv_layout(v, matA->nnz, vb);
+    const SpmvLayout l = spmv_layout(v, matA->nnz, vb, narrow_bytes(matA));
     if (v.transpose) {
         matA->assist_index_buffer_size = l.vals - l.col_ptr;
         matA->fixed_length_buffer_size = l.csr2csc_ws;
@@ -390,13 +466,12 @@ mcsparseStatus_t mcsparseSpMV(mcsparseHandle_t handle, mcsparseOperation_t opA, 
     if (!(computeType == matA->valueType && computeType == vecY->valueType && computeType == vecX->valueType))
         return to_public_status(MCSP_STATUS_NOT_IMPLEMENTED);
 
-    const CsrView v = make_view(matA, opA);
     switch (computeType) {
         case MACA_R_32F:
-            st = spmv_typed<float>(handle, matA, v, alpha, beta, vecX, vecY, externalBuffer);
+            st = spmv_typed<float>(handle, matA, opA, alpha, beta, vecX, vecY, externalBuffer);
             break;
         case MACA_R_64F:
-            st = spmv_typed<double>(handle, matA, v, alpha, beta, vecX, vecY, externalBuffer);
+            st = spmv_typed<double>(handle, matA, opA, alpha, beta, vecX, vecY, externalBuffer);
             break;
         default:
             st = MCSP_STATUS_NOT_IMPLEMENTED;
@@ -446,8 +521,9 @@ mcsparseStatus_t mcsparseSpMM_preprocess(mcsparseHandle_t handle, mcsparseOperat
 
     const idx_t m = static_cast<idx_t>(matA->row_num);
     const idx_t nnz = static_cast<idx_t>(matA->nnz);
-    mcsp::launch_spmm_schedule(handle->stream, m, nnz, static_cast<idx_t>(matA->idxBase),
-                               static_cast<const idx_t*>(matA->rows), static_cast<const idx_t*>(matA->cols),
+    const IndexArrays ia = index_arrays(handle, matA, static_cast<char*>(externalBuffer) +
+                                                          spmm_layout(matA, value_size(matA->valueType)).narrow);
+    mcsp::launch_spmm_schedule(handle->stream, m, nnz, static_cast<idx_t>(matA->idxBase), ia.rows, ia.cols,
                                externalBuffer);
     const mcsp::SpmmScheduleLayout l = mcsp::spmm_schedule_layout(m, nnz);
     const uint64_t groups = mcsp::spmm_groups(m);
@@ -498,6 +574,9 @@ mcsparseStatus_t mcsparseSpMM(mcsparseHandle_t handle, mcsparseOperation_t opA, 
     const int64_t b_lead = matB->order == MCSPARSE_ORDER_ROW ? matB->col_num : matB->row_num;
     const int64_t c_lead = matC->order == MCSPARSE_ORDER_ROW ? matC->col_num : matC->row_num;
     if (matB->ld < b_lead || matC->ld < c_lead) return to_public_status(MCSP_STATUS_INVALID_SIZE);
+    // reference: mcsp_spmm_gpu.cpp:96-98
+    if (!(matC->batchCount == matA->batchCount && matC->batchCount == matB->batchCount))
+        return to_public_status(MCSP_STATUS_INVALID_SIZE);
 
     switch (computeType) {
         case MACA_R_32F: st = spmm_typed<float>(handle, matA, opB, alpha, beta, matB, matC, externalBuffer); break;

@@ -426,4 +426,41 @@ mcsparseStatus_t mcsparseDnMatSetValues(mcsparseDnMatDescr_t d, void* values) {
     return MCSPARSE_STATUS_SUCCESS;
 }
 
+// ---- strided batches: src/kernels/generic/mcsp_generic.cpp:686-743, :787-802 -----------------
+
+mcsparseStatus_t mcsparseCooSetStridedBatch(mcsparseSpMatDescr_t d, int batchCount, int64_t batchStride) {
+    if (d == nullptr) return to_public_status(MCSP_STATUS_INVALID_POINTER);
+    if (batchCount <= 0 || batchStride < 0) return to_public_status(MCSP_STATUS_INVALID_SIZE);
+    d->batchCount = batchCount;
+    d->batchStride = batchStride;
+    return MCSPARSE_STATUS_SUCCESS;
+}
+
+mcsparseStatus_t mcsparseCsrSetStridedBatch(mcsparseSpMatDescr_t d, int batchCount, int64_t offsetsBatchStride,
+                                            int64_t columnsValuesBatchStride) {
+    if (d == nullptr) return to_public_status(MCSP_STATUS_INVALID_POINTER);
+    if (batchCount <= 0 || offsetsBatchStride < 0 || columnsValuesBatchStride < 0)
+        return to_public_status(MCSP_STATUS_INVALID_SIZE);
+    d->batchCount = batchCount;
+    d->offsetsBatchStride = offsetsBatchStride;
+    d->batchStride = columnsValuesBatchStride;
+    return MCSPARSE_STATUS_SUCCESS;
+}
+
+mcsparseStatus_t mcsparseDnMatSetStridedBatch(mcsparseDnMatDescr_t d, int batchCount, int64_t batchStride) {
+    if (d == nullptr) return to_public_status(MCSP_STATUS_INVALID_POINTER);
+    if (batchCount <= 0 || batchStride < 0) return to_public_status(MCSP_STATUS_INVALID_SIZE);
+    d->batchCount = batchCount;
+    d->batchStride = batchStride;
+    return MCSPARSE_STATUS_SUCCESS;
+}
+
+mcsparseStatus_t mcsparseDnMatGetStridedBatch(mcsparseDnMatDescr_t d, int* batchCount, int64_t* batchStride) {
+    if (d == nullptr || batchCount == nullptr || batchStride == nullptr)
+        return to_public_status(MCSP_STATUS_INVALID_POINTER);
+    *batchCount = static_cast<int>(d->batchCount);
+    *batchStride = d->batchStride;
+    return MCSPARSE_STATUS_SUCCESS;
+}
+
 }  // extern "C"

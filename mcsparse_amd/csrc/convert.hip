@@ -630,6 +630,20 @@ void launch_gather(hipStream_t stream, idx_t nnz, const T* y, T* x_val, const id
                        stream, nnz, y, x_val, x_ind, base);
 }
 
+namespace {
+__global__ __launch_bounds__(kBlock) void narrow_indices_kernel(const int64_t* __restrict__ src, idx_t* __restrict__ dst,
+                                                                uint64_t n) {
+    const uint64_t i = static_cast<uint64_t>(blockIdx.x) * kBlock + threadIdx.x;
+    if (i < n) dst[i] = static_cast<idx_t>(load_stream(src + i));
+}
+}  // namespace
+
+void launch_narrow_indices(hipStream_t stream, const int64_t* src, idx_t* dst, uint64_t n) {
+    if (n == 0) return;
+    hipLaunchKernelGGL(narrow_indices_kernel, dim3(static_cast<uint32_t>((n + kBlock - 1) / kBlock)), dim3(kBlock), 0,
+                       stream, src, dst, n);
+}
+
 size_t exclusive_scan_workspace_bytes(uint64_t n) {
     return align_up(scan_workspace_elems(n) * sizeof(uint32_t)) + kAlign;
 }

@@ -39,7 +39,7 @@ struct mcsparseDnVecDescr {
     void* values = nullptr;
 };
 
-// reference: src/include/mcsp_internal_types.h:135-147 (batch fields are not on this path)
+// reference: src/include/mcsp_internal_types.h:135-147
 struct mcsparseDnMatDescr {
     macaDataType valueType = MACA_R_32F;
     mcsparseOrder_t order = MCSPARSE_ORDER_COL;
@@ -47,6 +47,8 @@ struct mcsparseDnMatDescr {
     int64_t col_num = 0;
     int64_t ld = 0;
     void* values = nullptr;
+    int64_t batchCount = 1;
+    int64_t batchStride = 0;
 };
 
 // Kernel family of an SpMV call.
@@ -101,6 +103,11 @@ struct mcsparseSpMatDescr {
     void* rows = nullptr;
     void* cols = nullptr;
     void* vals = nullptr;
+    // strided batches (:194-196): batchStride moves the index and value arrays, offsetsBatchStride
+    // the offsets array of CSR / CSC
+    int64_t batchCount = 1;
+    int64_t batchStride = 0;
+    int64_t offsetsBatchStride = 0;
     // sizes of the transpose scratch layout, filled by *_bufferSize
     // (reference: src/common/mcsp_internal_transpose_sparse.hpp:517-549)
     int is_buffersize_called = 0;
@@ -252,6 +259,8 @@ void launch_exclusive_scan_u32(hipStream_t stream, uint32_t* data, uint64_t n, v
 // x_val[i] = y[x_ind[i] - base]
 template <typename T>
 void launch_gather(hipStream_t stream, idx_t nnz, const T* y, T* x_val, const idx_t* x_ind, idx_t base);
+// dst[i] = low 32 bits of src[i]
+void launch_narrow_indices(hipStream_t stream, const int64_t* src, idx_t* dst, uint64_t n);
 
 }  // namespace mcsp
 

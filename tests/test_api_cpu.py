@@ -191,7 +191,11 @@ def test_spmv_argument_checks(lib):
     assert mixed.spmv() == api.STATUS_NOT_SUPPORTED  # row/col index types differ (:1126-1132)
     assert mixed.spmv(h=None) == api.STATUS_NOT_SUPPORTED  # the index-type dispatch comes first
     i64 = Objs(lib, idx=(3, 3))
-    assert i64.spmv() == api.STATUS_NOT_SUPPORTED  # 64-bit indices are not built
+    assert i64.spmv(h=None) == api.STATUS_NOT_INITIALIZED  # 64-bit indices pass the dispatch (:1128-1129)
+    assert i64.spmv(buf=None) == api.STATUS_INVALID_VALUE
+    assert i64.spmv_size()[0] == 0 and i64.spmv_size()[1] > o.spmv_size()[1]  # room for the narrowed copies
+    u16 = Objs(lib, idx=(1, 1))
+    assert u16.spmv() == api.STATUS_NOT_SUPPORTED  # 16-bit indices: not dispatched (:1130-1132)
     cplx = Objs(lib, vt=api.C_32F)
     assert cplx.spmv(ct=api.C_32F) == api.STATUS_NOT_SUPPORTED
 
@@ -358,3 +362,28 @@ def test_sort_argument_checks(lib):
         assert fn(o.h, 0, None, None, None, 0) == 0
         assert fn(o.h, 4, FAKE, None, FAKE, 0) == api.STATUS_INVALID_VALUE
     lib.mcsparseDestroyMatDescr(d)
+
+
+def test_strided_batch_setters(lib):
+    # src/kernels/generic/mcsp_generic.cpp:686-743: null descriptor, count <= 0, negative stride
+    o = Objs(lib)
+    assert lib.mcsparseCsrSetStridedBatch(None, 1, 0, 0) == api.STATUS_INVALID_VALUE
+    assert lib.mcsparseCsrSetStridedBatch(o.A, 0, 0, 0) == api.STATUS_INVALID_VALUE
+    assert lib.mcsparseCsrSetStridedBatch(o.A, 2, -1, 0) == api.STATUS_INVALID_VALUE
+    assert lib.mcsparseCsrSetStridedBatch(o.A, 2, 0, -1) == api.STATUS_INVALID_VALUE
+    assert lib.mcsparseCsrSetStridedBatch(o.A, 2, 8, 40) == 0
+    assert lib.mcsparseCooSetStridedBatch(None, 1, 0) == api.STATUS_INVALID_VALUE
+    assert lib.mcsparseCooSetStridedBatch(o.A, -3, 0) == api.STATUS_INVALID_VALUE
+    B = ctypes.c_void_p()
+    assert lib.mcsparseCreateDnMat(ctypes.byref(B), 6, 4, 4, FAKE, api.R_32F, api.ORDER_ROW) == 0
+    count, stride = ctypes.c_int(-1), ctypes.c_int64(-1)
+    assert lib.mcsparseDnMatGetStridedBatch(B, ctypes.byref(count), ctypes.byref(stride)) == 0
+    assert (count.value, stride.value) == (1, 0)  # defaults (src/include/mcsp_internal_types.h:143-144)
+    assert lib.mcsparseDnMatSetStridedBatch(B, 0, 24) == api.STATUS_INVALID_VALUE
+    assert lib.mcsparseDnMatSetStridedBatch(B, 3, -24) == api.STATUS_INVALID_VALUE
+    assert lib.mcsparseDnMatSetStridedBatch(None, 3, 24) == api.STATUS_INVALID_VALUE
+    assert lib.mcsparseDnMatSetStridedBatch(B, 3, 24) == 0
+    assert lib.mcsparseDnMatGetStridedBatch(B, ctypes.byref(count), ctypes.byref(stride)) == 0
+    assert (count.value, stride.value) == (3, 24)
+    assert lib.mcsparseDnMatGetStridedBatch(B, None, ctypes.byref(stride)) == api.STATUS_INVALID_VALUE
+    lib.mcsparseDestroyDnMat(B)
