@@ -115,21 +115,38 @@ __global__ __launch_bounds__(kBlock) void csr2coo_kernel(idx_t m, idx_t nnz, idx
 
 // Offsets from sorted row indices: boundary t (between entry t-1 and entry t, 0 <= t <= nnz) fills
 // the offsets of the rows that lie in between, so empty rows are covered.  Each thread takes four
-// consecutive boundaries and reads its entries once.
+// consecutive entries (one 128-bit load when the array allows it) and the boundaries in front of
+// them; the entry before its first one comes from the neighbouring lane.
 // Reference semantics: src/kernels/conversion/coo2csr_device.hpp:8-24.
 constexpr int kCooPerThread = 4;
+template <bool VEC>
 __global__ __launch_bounds__(kBlock) void coo2csr_kernel(idx_t nnz, idx_t m, idx_t base,
                                                          const idx_t* __restrict__ coo_rows,
                                                          idx_t* __restrict__ row_ptr) {
+    typedef idx_t idx4 __attribute__((ext_vector_type(4)));
     const uint64_t t0 = (static_cast<uint64_t>(blockIdx.x) * kBlock + threadIdx.x) * kCooPerThread;
+    // entries t0 .. t0+3; past the end they read as row m, which makes boundary nnz close the
+    // offsets up to m and the boundaries after it empty
+    idx_t r[kCooPerThread];
+    if (VEC && t0 + kCooPerThread <= nnz) {
+        const idx4 v = __builtin_nontemporal_load(reinterpret_cast<const idx4*>(coo_rows + t0));
+#pragma unroll
+        for (int e = 0; e < kCooPerThread; ++e) r[e] = v[e] - base;
+    } else {
+#pragma unroll
+        for (int e = 0; e < kCooPerThread; ++e) r[e] = t0 + e < nnz ? load_stream(coo_rows + t0 + e) - base : m;
+    }
+    // entry t0-1: the last entry of the lane below, a load for the first lane of a wavefront
+    idx_t before = __shfl_up(r[kCooPerThread - 1], 1, kWave);
+    if (threadIdx.x % kWave == 0 && t0 != 0 && t0 <= nnz) before = coo_rows[t0 - 1] - base;
     if (t0 > nnz) return;
-    // row (0-based, +1) of the entry before boundary t0; 0 in front of the first entry
-    uint64_t prev = t0 == 0 ? 0 : static_cast<uint64_t>(coo_rows[t0 - 1] - base) + 1;
+    // rows [prev, cur) get offset t: prev = row of entry t-1 plus one (0 in front of the first entry)
+    uint64_t prev = t0 == 0 ? 0 : static_cast<uint64_t>(before) + 1;
 #pragma unroll
     for (int e = 0; e < kCooPerThread; ++e) {
         const uint64_t t = t0 + e;
         if (t > nnz) break;
-        const uint64_t cur = t == nnz ? static_cast<uint64_t>(m) + 1 : static_cast<uint64_t>(coo_rows[t] - base) + 1;
+        const uint64_t cur = static_cast<uint64_t>(r[e]) + 1;  // t == nnz: m + 1
         for (uint64_t i = prev; i < cur; ++i) row_ptr[i] = static_cast<idx_t>(t) + base;
         prev = cur;
     }
@@ -249,9 +266,14 @@ __global__ __launch_bounds__(kHistBlock) void radix_hist_kernel(const idx_t* __r
     __shared__ uint32_t s_cnt[kMaxRadix];
     const uint32_t radix = 1u << bits;
     const uint32_t mask = radix - 1;
+    // The same tile order as the scatter kernel below: an XCD counts a contiguous range of tiles,
+    // so the sixteen neighbouring tiles whose counters share a cache line write it in one L2.
+    const uint32_t tiles_per_xcd = (tiles + kXcds - 1) / kXcds;
+    const uint32_t tile = (blockIdx.x % kXcds) * tiles_per_xcd + blockIdx.x / kXcds;
+    if (tile >= tiles) return;  // whole workgroup
     s_cnt[threadIdx.x] = 0;
     __syncthreads();
-    const uint64_t start = static_cast<uint64_t>(blockIdx.x) * kSortTile;
+    const uint64_t start = static_cast<uint64_t>(tile) * kSortTile;
 #pragma unroll
     for (int i = 0; i < kSortTile / (kHistBlock * 4); ++i) {
         const uint64_t p = start + (static_cast<uint64_t>(i) * kHistBlock + threadIdx.x) * 4;
@@ -264,7 +286,7 @@ __global__ __launch_bounds__(kHistBlock) void radix_hist_kernel(const idx_t* __r
         }
     }
     __syncthreads();
-    if (threadIdx.x < radix) counters[static_cast<uint64_t>(threadIdx.x) * tiles + blockIdx.x] = s_cnt[threadIdx.x];
+    if (threadIdx.x < radix) counters[static_cast<uint64_t>(threadIdx.x) * tiles + tile] = s_cnt[threadIdx.x];
 }
 
 // Exclusive scan over the kSortBlock threads of the scatter kernel.
@@ -444,7 +466,7 @@ void radix_sort_triples(hipStream_t stream, idx_t count, uint32_t key_bits, cons
         idx_t* k_out = last ? keys_out : t.keys[p & 1];
         idx_t* a_out = last ? aux_out : t.aux[p & 1];
         void* v_out = last ? vals_out : t.vals[p & 1];
-        hipLaunchKernelGGL(radix_hist_kernel, dim3(tiles), dim3(kHistBlock), 0, stream, keys_in, count, shift, bits,
+        hipLaunchKernelGGL(radix_hist_kernel, dim3(scatter_grid), dim3(kHistBlock), 0, stream, keys_in, count, shift, bits,
                            tiles, t.counters);
         launch_exclusive_scan(stream, t.counters, static_cast<uint64_t>(radix) * tiles, t.scan_ws);
         if (value_bytes == 0) {
@@ -558,8 +580,12 @@ void launch_csr2coo(hipStream_t stream, idx_t m, idx_t nnz, const idx_t* row_ptr
 
 void launch_coo2csr(hipStream_t stream, idx_t nnz, idx_t m, const idx_t* coo_rows, idx_t base, idx_t* row_ptr) {
     const uint64_t threads = (static_cast<uint64_t>(nnz) + kCooPerThread) / kCooPerThread;
-    hipLaunchKernelGGL(coo2csr_kernel, dim3(static_cast<uint32_t>((threads + kBlock - 1) / kBlock)), dim3(kBlock), 0,
-                       stream, nnz, m, base, coo_rows, row_ptr);
+    const dim3 grid(static_cast<uint32_t>((threads + kBlock - 1) / kBlock));
+    if (reinterpret_cast<uintptr_t>(coo_rows) % 16 == 0) {
+        hipLaunchKernelGGL(coo2csr_kernel<true>, grid, dim3(kBlock), 0, stream, nnz, m, base, coo_rows, row_ptr);
+    } else {
+        hipLaunchKernelGGL(coo2csr_kernel<false>, grid, dim3(kBlock), 0, stream, nnz, m, base, coo_rows, row_ptr);
+    }
 }
 
 size_t csr2csc_workspace_bytes(idx_t /*m*/, idx_t /*n*/, idx_t nnz, size_t value_bytes) {
