@@ -11,7 +11,9 @@ fp64 CSR SpMV, 1,048,576 rows x 16 nonzeros per row.  Prints one JSON line.
 
 Workloads: c1 (5-pt Laplacian 256^2 fp32), c2 (default), c3 / c3t (power-law fp32, op N / T),
 c4-8 / c4-64 / c4-256 (27-pt stencil 128^3 SpMM), c5 (csr2csc on the c3 matrix),
-c5-coo (csr2coo on it), c5-spmv (A^T x from the converted CSC).
+c5-coo (csr2coo on it), c5-spmv (A^T x from the converted CSC).  Probes: copy (a plain device copy, the
+yardstick of the traffic counters), gather-probe (16.8 M random 8-byte reads of an 8 MB table
+through mcsparseDgthr: what the x[col] reads of c2 cost on their own).
 """
 import argparse
 import json
@@ -106,6 +108,8 @@ def main():
         # plain device copy of known size: the yardstick the rocprofv3 FETCH_SIZE / WRITE_SIZE
         # counters are scaled by
         return copy_probe(torch, args)
+    elif name == "gather-probe":
+        return gather_probe(torch, api, handle, args)
     else:
         print("unknown workload %r" % name, file=sys.stderr)
         return 2
@@ -290,6 +294,35 @@ def copy_probe(torch, args):
     ms = (time.perf_counter() - t0) * 1e3 / steps
     print(json.dumps({"workload": "copy", "bytes_read_per_step": 4 * n, "bytes_written_per_step": 4 * n,
                       "steps": steps, "ms_per_step": round(ms, 4), "GBps": round(8 * n / ms / 1e6, 1)}))
+    return 0
+
+
+def gather_probe(torch, api, handle, args):
+    """x_val[i] = y[x_ind[i]] for as many uniformly random indices as c2 has nonzeros, from a table
+    the size of c2's x, and from one that fits every L2: the cost of the gathers of a random-column
+    SpMV with everything else (row offsets, values, sums) taken away."""
+    count = 1 << 24
+    steps = args.steps or 20
+    rng = np.random.default_rng(7)
+    out = {"workload": "gather-probe", "gathers": count, "element_bytes": 8, "steps": steps, "tables": []}
+    stream = torch.cuda.current_stream()
+    for table_elems in (1 << 17, 1 << 20):
+        ind = torch.from_numpy(rng.integers(0, table_elems, count, dtype=np.int32)).cuda()
+        table = torch.rand(table_elems, dtype=torch.float64, device="cuda")
+        dst = torch.zeros(count, dtype=torch.float64, device="cuda")
+        for _ in range(3):
+            api.check(api.gthr(handle, count, table, dst, ind, 0))
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(stream)
+        for _ in range(steps):
+            api.check(api.gthr(handle, count, table, dst, ind, 0))
+        e1.record(stream)
+        torch.cuda.synchronize()
+        us = e0.elapsed_time(e1) * 1e3 / steps
+        out["tables"].append({"table_MB": table_elems * 8 / 1e6, "us_per_call": round(us, 1),
+                              "gathers_per_us": round(count / us, 1),
+                              "streamed_bytes_per_call": count * (4 + 8)})
+    print(json.dumps(out))
     return 0
 
 

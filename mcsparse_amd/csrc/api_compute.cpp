@@ -393,7 +393,7 @@ mcspStatus_t spmm_typed(mcsparseHandle_t h, const mcsparseSpMatDescr* A, mcspars
         a.c_row_major = C->order == MCSPARSE_ORDER_ROW;
         // the schedule was built from batch 0's structure
         if ((b == 0 || shared_structure) && schedule_matches(A, buffer) && mcsp::spmm_schedule_usable(a, sizeof(T))) {
-            mcsp::launch_spmm_scheduled<T>(h->stream, a, buffer, h_alpha, h_beta);
+            mcsp::launch_spmm_scheduled<T>(h->stream, a, buffer, A->schedule.mean_span, h_alpha, h_beta);
         } else {
             mcsp::launch_spmm<T>(h->stream, a, h_alpha, h_beta);
         }
@@ -529,7 +529,10 @@ mcsparseStatus_t mcsparseSpMM_preprocess(mcsparseHandle_t handle, mcsparseOperat
     const uint64_t groups = mcsp::spmm_groups(m);
     uint32_t entries = 0;
     const char* total_slot = static_cast<const char*>(externalBuffer) + l.group_ptr + groups * sizeof(uint32_t);
+    unsigned long long span_sum = 0;
+    const char* span_slot = static_cast<const char*>(externalBuffer) + l.span_sum;
     if (hipMemcpyAsync(&entries, total_slot, sizeof(entries), hipMemcpyDeviceToHost, handle->stream) != hipSuccess ||
+        hipMemcpyAsync(&span_sum, span_slot, sizeof(span_sum), hipMemcpyDeviceToHost, handle->stream) != hipSuccess ||
         hipStreamSynchronize(handle->stream) != hipSuccess)
         return to_public_status(MCSP_STATUS_INTERNAL_ERROR);
     SpmmSchedule& s = matA->schedule;
@@ -540,6 +543,7 @@ mcsparseStatus_t mcsparseSpMM_preprocess(mcsparseHandle_t handle, mcsparseOperat
     s.nnz = matA->nnz;
     s.base = static_cast<int>(matA->idxBase);
     s.entries = entries;
+    s.mean_span = groups != 0 ? span_sum / groups : 0;
     // Worth it when the merged lists are clearly shorter than the rows they replace; groups too
     // long to merge contribute no entries and are not evidence either way.
     s.useful = entries != 0 && static_cast<uint64_t>(entries) * 100 <= static_cast<uint64_t>(matA->nnz) * 85;

@@ -86,6 +86,7 @@ struct SpmmSchedule {
     int64_t m = 0, nnz = 0;
     int base = 0;
     uint32_t entries = 0;  // length of all merged lists together
+    uint64_t mean_span = 0;  // mean distance between the first and the last column of a group
 };
 
 // reference: src/include/mcsp_internal_types.h:184-225.  rows/cols follow the reference's
@@ -212,7 +213,8 @@ void launch_spmm(hipStream_t stream, const SpmmArgs& a, T alpha, T beta);
 // Row-group schedule of a CSR structure (spmm.hip): for every group of kSpmmGroupRows
 // consecutive rows the merged list of their column indices, each entry =
 // (zero-based column << kSpmmGroupRows) | one bit per row of the group that has the column.
-// group_ptr has groups+1 offsets into entries.  Groups holding more than kSpmmMaxMergedGroup
+// group_ptr has groups+1 offsets into entries; span_sum (one u64) is the sum over the groups of
+// the distance between their first and last column.  Groups holding more than kSpmmMaxMergedGroup
 // nonzeros get no entries and are processed row by row.
 #ifndef MCSP_GROUP_ROWS
 #define MCSP_GROUP_ROWS 4
@@ -222,7 +224,7 @@ constexpr idx_t kSpmmMaxMergedGroup = 2048;
 constexpr int64_t kSpmmMaxScheduledColumns = int64_t(1) << (32 - kSpmmGroupRows);
 constexpr uint64_t spmm_groups(idx_t m) { return (static_cast<uint64_t>(m) + kSpmmGroupRows - 1) / kSpmmGroupRows; }
 struct SpmmScheduleLayout {
-    size_t group_ptr, entries, scan_ws, total;
+    size_t group_ptr, span_sum, entries, scan_ws, total;
 };
 SpmmScheduleLayout spmm_schedule_layout(idx_t m, idx_t nnz);
 // Fills group_ptr and entries inside `schedule` (laid out as spmm_schedule_layout says).
@@ -232,7 +234,8 @@ void launch_spmm_schedule(hipStream_t stream, idx_t m, idx_t nnz, idx_t base, co
 // (spmm_schedule_usable says so), reading every B row once per row group.
 bool spmm_schedule_usable(const SpmmArgs& a, size_t value_bytes);
 template <typename T>
-void launch_spmm_scheduled(hipStream_t stream, const SpmmArgs& a, const void* schedule, T alpha, T beta);
+void launch_spmm_scheduled(hipStream_t stream, const SpmmArgs& a, const void* schedule, uint64_t mean_span, T alpha,
+                           T beta);
 
 // ---- conversions (convert.hip) ----
 void launch_csr2coo(hipStream_t stream, idx_t m, idx_t nnz, const idx_t* row_ptr, idx_t base, idx_t* coo_rows);

@@ -63,6 +63,23 @@ struct ByteOffset { typedef uint32_t type; };
 template <>
 struct ByteOffset<true> { typedef uint64_t type; };
 
+// Workgroups are handed to the 8 XCDs round-robin (workgroup h runs on XCD h % 8), each XCD with
+// an L2 of its own.  Rows that are close in the matrix tend to read the same rows of op(B), so
+// an XCD should work on a contiguous stretch of rows: this maps the hardware's workgroup number
+// to a position such that every XCD takes `chunk` consecutive positions at a time.  chunk = 1
+// is the identity; positions past `count` (the grid is padded to whole rounds) do no work.
+constexpr uint32_t kXcds = 8;
+__device__ __forceinline__ uint64_t xcd_position(uint32_t hw_block, uint32_t chunk) {
+    const uint32_t per_round = kXcds * chunk;
+    const uint32_t round = hw_block / per_round;
+    const uint32_t rem = hw_block % per_round;
+    return static_cast<uint64_t>(round) * per_round + (rem % kXcds) * chunk + rem / kXcds;
+}
+inline uint32_t xcd_padded_grid(uint64_t count, uint32_t chunk) {
+    const uint64_t per_round = static_cast<uint64_t>(kXcds) * chunk;
+    return static_cast<uint32_t>((count + per_round - 1) / per_round * per_round);
+}
+
 // acc += sum over the nonzeros [begin, end) of one row of A of value * (V columns of the row of
 // op(B) the nonzero names), for a group of LR >= 4 lanes that all pass the same range.
 // B_bytes is the operand's first element, lane_off the byte offset of this lane's columns.
@@ -274,42 +291,50 @@ template <bool FILL>
 __global__ __launch_bounds__(kBlock) void group_merge_kernel(idx_t m, idx_t base, const idx_t* __restrict__ row_ptr,
                                                              const idx_t* __restrict__ col,
                                                              uint32_t* __restrict__ group_ptr,
-                                                             uint32_t* __restrict__ entries) {
+                                                             uint32_t* __restrict__ entries,
+                                                             unsigned long long* __restrict__ span_sum) {
     const uint64_t groups = spmm_groups(m);
     const uint64_t group = static_cast<uint64_t>(blockIdx.x) * kBlock + threadIdx.x;
-    if (group > groups) return;
-    if (group == groups) {  // the slot that receives the total after the scan
-        if (!FILL) group_ptr[group] = 0;
-        return;
-    }
-    idx_t i[R], e[R];
-    group_row_ranges(m, base, row_ptr, group * R, i, e);
-    if (e[R - 1] - i[0] > kSpmmMaxMergedGroup) {
-        if (!FILL) group_ptr[group] = 0;
-        return;
-    }
-    const uint32_t out = FILL ? group_ptr[group] : 0;
+    // slot `groups` receives the total after the scan; threads past it only take part in the
+    // wavefront's sum below
     uint32_t count = 0;
-    while (true) {
-        uint32_t head[R];
-        uint32_t lo = kNoColumn;
+    uint32_t first = kNoColumn, last = 0;
+    if (group < groups) {
+        idx_t i[R], e[R];
+        group_row_ranges(m, base, row_ptr, group * R, i, e);
+        if (e[R - 1] - i[0] <= kSpmmMaxMergedGroup) {
+            const uint32_t out = FILL ? group_ptr[group] : 0;
+            while (true) {
+                uint32_t head[R];
+                uint32_t lo = kNoColumn;
 #pragma unroll
-        for (int r = 0; r < R; ++r) {
-            head[r] = i[r] < e[r] ? static_cast<uint32_t>(col[i[r]] - base) : kNoColumn;
-            lo = head[r] < lo ? head[r] : lo;
-        }
-        if (lo == kNoColumn) break;
-        uint32_t flags = 0;
+                for (int r = 0; r < R; ++r) {
+                    head[r] = i[r] < e[r] ? static_cast<uint32_t>(col[i[r]] - base) : kNoColumn;
+                    lo = head[r] < lo ? head[r] : lo;
+                }
+                if (lo == kNoColumn) break;
+                if (first == kNoColumn) first = lo;
+                last = lo > last ? lo : last;
+                uint32_t flags = 0;
 #pragma unroll
-        for (int r = 0; r < R; ++r) {
-            const uint32_t takes = head[r] == lo;
-            flags |= takes << r;
-            i[r] += takes;
+                for (int r = 0; r < R; ++r) {
+                    const uint32_t takes = head[r] == lo;
+                    flags |= takes << r;
+                    i[r] += takes;
+                }
+                if (FILL) entries[out + count] = (lo << R) | flags;
+                ++count;
+            }
         }
-        if (FILL) entries[out + count] = (lo << R) | flags;
-        ++count;
     }
-    if (!FILL) group_ptr[group] = count;
+    if (!FILL) {
+        if (group <= groups) group_ptr[group] = count;
+        // how far apart the columns of a group lie, summed over the wavefront before it is added
+        unsigned long long span = count != 0 ? last - first : 0;
+#pragma unroll
+        for (int off = kWave / 2; off > 0; off >>= 1) span += __shfl_xor(span, off, kWave);
+        if (lane_id() == 0 && span != 0) atomicAdd(span_sum, span);
+    }
 }
 
 // Returns the top bit of w and shifts w left by one: an add whose carry is the answer.
@@ -331,13 +356,14 @@ __global__ __launch_bounds__(kBlock) void spmm_group_kernel(idx_t m, idx_t n, id
                                                             const uint32_t* __restrict__ group_ptr,
                                                             const uint32_t* __restrict__ entries,
                                                             const T* __restrict__ B, int64_t ldb, T* __restrict__ C,
-                                                            int64_t ldc, bool c_row_major, T alpha, T beta) {
+                                                            int64_t ldc, bool c_row_major, T alpha, T beta,
+                                                            uint32_t xcd_chunk) {
     typedef typename ByteOffset<WIDE>::type off_t;
     constexpr int V = 16 / sizeof(T);
     constexpr int kGroupsPerBlock = kBlock / LR;
     constexpr int kBatch = LR < 8 ? LR : 8;
     const idx_t lane = threadIdx.x % LR;
-    const uint64_t group = static_cast<uint64_t>(blockIdx.x) * kGroupsPerBlock + threadIdx.x / LR;
+    const uint64_t group = xcd_position(blockIdx.x, xcd_chunk) * kGroupsPerBlock + threadIdx.x / LR;
     const uint64_t r0 = group * R;
     if (r0 >= static_cast<uint64_t>(m)) return;  // whole lane groups
     const uint64_t c_own = (static_cast<uint64_t>(blockIdx.y) * LR + lane) * V;
@@ -442,21 +468,32 @@ bool narrow_offsets(const SpmmArgs& a, size_t value_bytes) {
 
 template <typename T, int LR>
 void launch_group(hipStream_t stream, const SpmmArgs& a, const uint32_t* group_ptr, const uint32_t* entries, T alpha,
-                  T beta) {
+                  T beta, uint64_t mean_span) {
     constexpr int V = 16 / sizeof(T);
     const uint64_t groups = spmm_groups(a.m);
     const uint64_t group_blocks = (groups + (kBlock / LR) - 1) / (kBlock / LR);
     const uint64_t panels = (static_cast<uint64_t>(a.n) + LR * V - 1) / (LR * V);
-    const dim3 grid(static_cast<uint32_t>(group_blocks), static_cast<uint32_t>(panels));
+    // Rows whose columns lie `mean_span` apart read rows of op(B) from a window of that many rows
+    // around them.  An XCD that works through mean_span / 16 consecutive rows at a time keeps the
+    // rows of op(B) it shares with the stretches before and after (the neighbouring grid lines of
+    // a stencil) in its own L2 -- as long as such a stretch of op(B) is small against the 4 MB of
+    // an L2; beyond that the plain round-robin does as well.
+    constexpr uint64_t kRowsPerBlock = static_cast<uint64_t>(kBlock / LR) * R;
+    uint32_t xcd_chunk = 1;
+    const uint64_t stretch_rows = mean_span / 16;
+    if (stretch_rows * a.n * sizeof(T) <= (1u << 20)) {
+        while (static_cast<uint64_t>(xcd_chunk) * 2 * kRowsPerBlock <= stretch_rows) xcd_chunk *= 2;
+    }
+    const dim3 grid(xcd_padded_grid(group_blocks, xcd_chunk), static_cast<uint32_t>(panels));
     const T* val = static_cast<const T*>(a.val);
     const T* B = static_cast<const T*>(a.B);
     T* C = static_cast<T*>(a.C);
     if (narrow_offsets(a, sizeof(T))) {
         hipLaunchKernelGGL((spmm_group_kernel<T, LR, false>), grid, dim3(kBlock), 0, stream, a.m, a.n, a.base, a.row_ptr,
-                           a.col, val, group_ptr, entries, B, a.ldb, C, a.ldc, a.c_row_major, alpha, beta);
+                           a.col, val, group_ptr, entries, B, a.ldb, C, a.ldc, a.c_row_major, alpha, beta, xcd_chunk);
     } else {
         hipLaunchKernelGGL((spmm_group_kernel<T, LR, true>), grid, dim3(kBlock), 0, stream, a.m, a.n, a.base, a.row_ptr,
-                           a.col, val, group_ptr, entries, B, a.ldb, C, a.ldc, a.c_row_major, alpha, beta);
+                           a.col, val, group_ptr, entries, B, a.ldb, C, a.ldc, a.c_row_major, alpha, beta, xcd_chunk);
     }
 }
 
@@ -525,6 +562,7 @@ SpmmScheduleLayout spmm_schedule_layout(idx_t m, idx_t nnz) {
     const uint64_t slots = spmm_groups(m) + 1;
     size_t off = 0;
     l.group_ptr = off; off += align_up(slots * sizeof(uint32_t));
+    l.span_sum = off; off += kAlign;
     l.entries = off; off += align_up(static_cast<size_t>(nnz) * sizeof(uint32_t));
     l.scan_ws = off; off += exclusive_scan_workspace_bytes(slots);
     l.total = off;
@@ -539,11 +577,13 @@ void launch_spmm_schedule(hipStream_t stream, idx_t m, idx_t nnz, idx_t base, co
     uint32_t* entries = reinterpret_cast<uint32_t*>(w + l.entries);
     const uint64_t slots = spmm_groups(m) + 1;
     const dim3 grid(static_cast<uint32_t>((slots + kBlock - 1) / kBlock));
+    unsigned long long* span_sum = reinterpret_cast<unsigned long long*>(w + l.span_sum);
+    (void)hipMemsetAsync(span_sum, 0, sizeof(*span_sum), stream);
     hipLaunchKernelGGL((group_merge_kernel<false>), grid, dim3(kBlock), 0, stream, m, base, row_ptr, col, group_ptr,
-                       entries);
+                       entries, span_sum);
     launch_exclusive_scan_u32(stream, group_ptr, slots, w + l.scan_ws);
     hipLaunchKernelGGL((group_merge_kernel<true>), grid, dim3(kBlock), 0, stream, m, base, row_ptr, col, group_ptr,
-                       entries);
+                       entries, span_sum);
 }
 
 bool spmm_schedule_usable(const SpmmArgs& a, size_t value_bytes) {
@@ -556,7 +596,8 @@ bool spmm_schedule_usable(const SpmmArgs& a, size_t value_bytes) {
 }
 
 template <typename T>
-void launch_spmm_scheduled(hipStream_t stream, const SpmmArgs& a, const void* schedule, T alpha, T beta) {
+void launch_spmm_scheduled(hipStream_t stream, const SpmmArgs& a, const void* schedule, uint64_t mean_span, T alpha,
+                           T beta) {
     if (a.m == 0 || a.n == 0) return;
     constexpr int V = 16 / sizeof(T);
     const SpmmScheduleLayout l = spmm_schedule_layout(a.m, a.nnz);
@@ -564,15 +605,15 @@ void launch_spmm_scheduled(hipStream_t stream, const SpmmArgs& a, const void* sc
     const uint32_t* group_ptr = reinterpret_cast<const uint32_t*>(w + l.group_ptr);
     const uint32_t* entries = reinterpret_cast<const uint32_t*>(w + l.entries);
     const uint64_t lanes_needed = (static_cast<uint64_t>(a.n) + V - 1) / V;
-    if (lanes_needed <= 4) launch_group<T, 4>(stream, a, group_ptr, entries, alpha, beta);
-    else if (lanes_needed <= 8) launch_group<T, 8>(stream, a, group_ptr, entries, alpha, beta);
-    else if (lanes_needed <= 16) launch_group<T, 16>(stream, a, group_ptr, entries, alpha, beta);
-    else if (lanes_needed <= 32) launch_group<T, 32>(stream, a, group_ptr, entries, alpha, beta);
-    else launch_group<T, 64>(stream, a, group_ptr, entries, alpha, beta);
+    if (lanes_needed <= 4) launch_group<T, 4>(stream, a, group_ptr, entries, alpha, beta, mean_span);
+    else if (lanes_needed <= 8) launch_group<T, 8>(stream, a, group_ptr, entries, alpha, beta, mean_span);
+    else if (lanes_needed <= 16) launch_group<T, 16>(stream, a, group_ptr, entries, alpha, beta, mean_span);
+    else if (lanes_needed <= 32) launch_group<T, 32>(stream, a, group_ptr, entries, alpha, beta, mean_span);
+    else launch_group<T, 64>(stream, a, group_ptr, entries, alpha, beta, mean_span);
 }
 
-template void launch_spmm_scheduled<float>(hipStream_t, const SpmmArgs&, const void*, float, float);
-template void launch_spmm_scheduled<double>(hipStream_t, const SpmmArgs&, const void*, double, double);
+template void launch_spmm_scheduled<float>(hipStream_t, const SpmmArgs&, const void*, uint64_t, float, float);
+template void launch_spmm_scheduled<double>(hipStream_t, const SpmmArgs&, const void*, uint64_t, double, double);
 template void launch_spmm<float>(hipStream_t, const SpmmArgs&, float, float);
 template void launch_spmm<double>(hipStream_t, const SpmmArgs&, double, double);
 
