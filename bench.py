@@ -28,11 +28,21 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 
-# HBM/fabric bytes per launch of the dominant kernel, from rocprofv3 FETCH_SIZE and WRITE_SIZE
-# (each scaled by what the same counter reads on a 1 GiB copy: 2 KiB and 1 KiB per count).
-# The counter summaries are kept under profiles/.
+# HBM/fabric bytes per call (all kernels of one step together), from rocprofv3 FETCH_SIZE and
+# WRITE_SIZE, each scaled by what the same counter reads on a 1 GiB copy: 2 KiB and 1 KiB per
+# count.  The counter summaries are kept under profiles/.
+def _traffic(fetch_counts, write_counts):
+    return int((fetch_counts * 2 + write_counts) * 1024)
+
+
 MEASURED_TRAFFIC_BYTES = {
-    "c2": int((654222.0 * 2 + 10263.5 * 1) * 1024),
+    "c2": _traffic(652676.1, 9147.2),                      # spmv_vector_kernel<double, 16, 4>
+    "c3": _traffic(5637867.2 + 6781.0 + 1857.9, 22218.4 + 231.8 + 817.9),   # merge kernel + partition + fix-up
+    "c4-64": _traffic(484944.7, 524288.0),                 # spmm_group_kernel<float, 16>
+    "c4-256": _traffic(3685140.3, 2097152.0),              # spmm_group_kernel<float, 64>
+    # csr2csc: 3 x (scatter + histogram + scans) + csr2coo + coo2csr
+    "c5": _traffic(3 * (701953.5 + 229171.1 + 3 * 4822.2 + 2 * 7174.2) + 83018.4 + 238051.1,
+                   3 * (1381473.1 + 28769.2 + 3 * 9552.7 + 2 * 56.0) + 459941.5 + 19514.6),
 }
 
 
