@@ -61,13 +61,22 @@ def test_config5_conversions_full_size(torch_gpu, handle, oracle, power_law_full
     assert_within(yt, yt_ref, bound_t, np.float32, what="C5 A^T x from CSC")
 
 
-@pytest.mark.parametrize("n", [8, 64, 256])
-def test_config4_stencil_full_size(torch_gpu, handle, oracle, n):
+@pytest.fixture(scope="module")
+def stencil_full():
     a = wl.stencil_27pt(128, dtype=np.float32)
     assert (a.m, a.nnz) == (2097152, 55742968)
+    return a
+
+
+# preprocess = True runs the row-group kernel (for N = 8 the schedule is built but too narrow to use)
+@pytest.mark.parametrize("preprocess", [False, True])
+@pytest.mark.parametrize("n", [8, 64, 256])
+def test_config4_stencil_full_size(torch_gpu, handle, oracle, stencil_full, n, preprocess):
+    a = stencil_full
     rng = np.random.default_rng(n)
     B = rng.uniform(-1, 1, (a.n, n)).astype(np.float32)
-    st, got, _ = run_spmm(torch_gpu, handle, a, B, np.zeros((a.m, n), np.float32), 1.0, 0.0)
+    st, got, _ = run_spmm(torch_gpu, handle, a, B, np.zeros((a.m, n), np.float32), 1.0, 0.0, preprocess=preprocess,
+                          expect_schedule=2 if preprocess else None)
     assert st == 0
     # oracle on a sample of rows: first/last planes, and random interior rows
     rows = np.unique(np.concatenate([np.arange(0, 300), np.arange(a.m - 300, a.m),

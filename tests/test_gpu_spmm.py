@@ -126,6 +126,16 @@ def test_preprocessed_stencil(torch_gpu, handle, oracle, n, dtype):
               pad_c=8)
 
 
+def test_preprocessed_stencil_in_xcd_stretches(torch_gpu, handle, oracle):
+    """A stencil large enough for the row-group kernel to hand every XCD stretches of several
+    workgroups (the column span of a 48^3 stencil is 4,706 rows), with a last round that is only
+    partly filled."""
+    a = wl.stencil_27pt(48, dtype=np.float32)
+    for n in (64, 40):
+        check(torch_gpu, handle, oracle, a, n, 1.0, 0.0, preprocess=True, expect_schedule=2)
+    check(torch_gpu, handle, oracle, a, 64, 0.5, -1.0, preprocess=True, expect_schedule=2, c_order=api.ORDER_COL)
+
+
 def test_preprocessed_ragged_rows_with_overlap(torch_gpu, handle, oracle):
     """Rows of different lengths, empty rows, unsorted columns inside rows, a group too long to merge."""
     rng = np.random.default_rng(12)
