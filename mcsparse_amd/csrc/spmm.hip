@@ -361,7 +361,10 @@ __global__ __launch_bounds__(kBlock) void spmm_group_kernel(idx_t m, idx_t n, id
     typedef typename ByteOffset<WIDE>::type off_t;
     constexpr int V = 16 / sizeof(T);
     constexpr int kGroupsPerBlock = kBlock / LR;
-    constexpr int kBatch = LR < 8 ? LR : 8;
+    // rows of op(B) a lane asks for at a time: pairs that alternate with the arithmetic of the pair
+    // before (measured best below a wavefront per group), eight at once for one group per wavefront
+    constexpr bool kAlternate = LR < kWave;
+    constexpr int kBatch = kAlternate ? 2 : 8;
     const idx_t lane = threadIdx.x % LR;
     const uint64_t group = xcd_position(blockIdx.x, xcd_chunk) * kGroupsPerBlock + threadIdx.x / LR;
     const uint64_t r0 = group * R;
@@ -408,39 +411,55 @@ __global__ __launch_bounds__(kBlock) void spmm_group_kernel(idx_t m, idx_t n, id
             const off_t roff = static_cast<off_t>(ent >> R) * ldb_bytes;
             const uint32_t flags = ent & ((1u << R) - 1u);
             const uint32_t left = s_end - s;
+            // With kAlternate two batches of rows of op(B) take turns: the loads of one are on their
+            // way while the multiply-adds of the other run, so a wavefront's arithmetic hides part
+            // of its own loads.
             auto chunk = [&](auto checked) {
                 constexpr bool kChecked = decltype(checked)::value;
-                static_for<LR / kBatch>([&](auto g) {
+                constexpr int kBatches = LR / kBatch;
+                Vec<T, V> b[kAlternate ? 2 : 1][kBatch];
+                auto load_batch = [&](auto g) {
                     constexpr int u0 = decltype(g)::value * kBatch;
-                    if (!kChecked || u0 < left) {
-                        Vec<T, V> b[kBatch];
-                        static_for<kBatch>([&](auto u) {
-                            constexpr int k = u0 + decltype(u)::value;
-                            if (!kChecked || k < left) {
-                                const off_t off = group_bcast<LR, k>(roff) + lane_off;
-                                b[decltype(u)::value] = load_vec<T, V>(reinterpret_cast<const T*>(B_bytes + off));
-                            }
-                        });
-                        static_for<kBatch>([&](auto u) {
-                            constexpr int k = u0 + decltype(u)::value;
-                            if (!kChecked || k < left) {
-                                // a row that lacks the column must not see it at all (0 * inf would be NaN)
-                                uint32_t fk = 0;
-                                if constexpr (LR == kWave) fk = group_bcast<LR, k>(flags);  // one group per wavefront: scalar
-                                static_for<R>([&](auto rc) {
-                                    constexpr int r = decltype(rc)::value;
-                                    bool has;
-                                    if constexpr (LR == kWave) has = (fk >> r) & 1u;
-                                    else has = shift_out_top(take[r]);
-                                    if (has) {
-                                        const T a = group_bcast<LR, k>(v[r]);
+                    static_for<kBatch>([&](auto u) {
+                        constexpr int k = u0 + decltype(u)::value;
+                        if (!kChecked || k < left) {
+                            const off_t off = group_bcast<LR, k>(roff) + lane_off;
+                            b[kAlternate ? decltype(g)::value & 1 : 0][decltype(u)::value] =
+                                load_vec<T, V>(reinterpret_cast<const T*>(B_bytes + off));
+                        }
+                    });
+                };
+                auto use_batch = [&](auto g) {
+                    constexpr int u0 = decltype(g)::value * kBatch;
+                    static_for<kBatch>([&](auto u) {
+                        constexpr int k = u0 + decltype(u)::value;
+                        if (!kChecked || k < left) {
+                            // a row that lacks the column must not see it at all (0 * inf would be NaN)
+                            uint32_t fk = 0;
+                            if constexpr (LR == kWave) fk = group_bcast<LR, k>(flags);  // one group per wavefront: scalar
+                            static_for<R>([&](auto rc) {
+                                constexpr int r = decltype(rc)::value;
+                                bool has;
+                                if constexpr (LR == kWave) has = (fk >> r) & 1u;
+                                else has = shift_out_top(take[r]);
+                                if (has) {
+                                    const T a = group_bcast<LR, k>(v[r]);
 #pragma unroll
-                                        for (int c = 0; c < V; ++c) acc[r][c] += a * b[decltype(u)::value].v[c];
-                                    }
-                                });
-                            }
-                        });
+                                    for (int c = 0; c < V; ++c) acc[r][c] += a * b[kAlternate ? decltype(g)::value & 1 : 0][decltype(u)::value].v[c];
+                                }
+                            });
+                        }
+                    });
+                };
+                if constexpr (kAlternate) load_batch(std::integral_constant<int, 0>{});
+                static_for<kBatches>([&](auto g) {
+                    constexpr int next = decltype(g)::value + 1;
+                    if constexpr (!kAlternate) {
+                        if (!kChecked || decltype(g)::value * kBatch < left) load_batch(g);
+                    } else if constexpr (next < kBatches) {
+                        if (!kChecked || next * kBatch < left) load_batch(std::integral_constant<int, next>{});
                     }
+                    if (!kChecked || decltype(g)::value * kBatch < left) use_batch(g);
                 });
             };
             if (left >= LR) chunk(std::false_type{});
