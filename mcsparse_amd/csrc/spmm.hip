@@ -182,40 +182,107 @@ __global__ __launch_bounds__(kBlock) void spmm_rowb_kernel(idx_t m, idx_t n, idx
 #pragma unroll
     for (int i = 0; i < V; ++i) acc[i] = T(0);
 
-    if constexpr (LR >= 4) {
-        row_times_b<T, LR, V, WIDE>(start, end, lane, base, col, val, reinterpret_cast<const char*>(B),
-                                    static_cast<off_t>(c0 * sizeof(T)), static_cast<off_t>(ldb * sizeof(T)), acc);
-    } else {
-        constexpr int kUnroll = 8;
-        const T* Bc = B + c0;
-        idx_t j = start;
-        for (; j + kUnroll <= end; j += kUnroll) {
-            idx_t c[kUnroll];
-            T a[kUnroll];
-            Vec<T, V> b[kUnroll];
-#pragma unroll
-            for (int u = 0; u < kUnroll; ++u) {
-                c[u] = col[j + u] - base;
-                a[u] = val[j + u];
-            }
-#pragma unroll
-            for (int u = 0; u < kUnroll; ++u) b[u] = load_vec<T, V>(Bc + static_cast<int64_t>(c[u]) * ldb);
-#pragma unroll
-            for (int u = 0; u < kUnroll; ++u) {
-#pragma unroll
-                for (int i = 0; i < V; ++i) acc[i] += a[u] * b[u].v[i];
-            }
-        }
-        for (; j < end; ++j) {
-            const idx_t c = col[j] - base;
-            const T a = val[j];
-            const Vec<T, V> b = load_vec<T, V>(Bc + static_cast<int64_t>(c) * ldb);
-#pragma unroll
-            for (int i = 0; i < V; ++i) acc[i] += a * b.v[i];
-        }
-    }
+    static_assert(LR >= 4, "narrower operands take spmm_narrow_kernel");
+    row_times_b<T, LR, V, WIDE>(start, end, lane, base, col, val, reinterpret_cast<const char*>(B),
+                                static_cast<off_t>(c0 * sizeof(T)), static_cast<off_t>(ldb * sizeof(T)), acc);
 
     if (stores) store_c<T, V>(C, ldc, c_row_major, row, c0, acc, alpha, beta);
+}
+
+// op(B) row-major with few columns (n <= 2 vectors of V).  A row of op(B) then takes only
+// C = 1 or 2 lanes, and what a row of A costs is the chain of dependent loads (offsets,
+// nonzeros, rows of op(B)) rather than bytes.  So 16 lanes share a row of A as P = 16 / C
+// phases x C column lanes: phase p takes the nonzeros p, p + P, ... of the row, kSteps of them in
+// flight at once, and the P partial sums are added up across the lanes at the end.
+template <typename T, int V, int C>
+__global__ __launch_bounds__(kBlock) void spmm_narrow_kernel(idx_t m, idx_t n, idx_t base,
+                                                             const idx_t* __restrict__ row_ptr,
+                                                             const idx_t* __restrict__ col,
+                                                             const T* __restrict__ val, const T* __restrict__ B,
+                                                             int64_t ldb, T* __restrict__ Cm, int64_t ldc,
+                                                             bool c_row_major, T alpha, T beta) {
+    constexpr int kLanes = 16;
+    constexpr int P = kLanes / C;
+    constexpr int kSteps = 4;  // measured on a 27-point stencil, n = 8: 1, 2, 4, 8 steps -> 305, 280, 260, 291 us
+    constexpr int kRows = 1;   // more rows per lane group in flight only cost registers (2 -> 352 us)
+    constexpr int kGroups = kBlock / kLanes;
+    const idx_t sub = threadIdx.x % kLanes;
+    const idx_t phase = sub / C;
+    const uint64_t c_own = static_cast<uint64_t>(sub % C) * V;
+    const bool in_panel = c_own < n;
+    const uint64_t c0 = in_panel ? c_own : 0;
+    const uint64_t first_row = (static_cast<uint64_t>(blockIdx.x) * kGroups + threadIdx.x / kLanes) * kRows;
+
+    idx_t at[kRows], end[kRows];
+    T acc[kRows][V];
+#pragma unroll
+    for (int w = 0; w < kRows; ++w) {
+        const uint64_t row = first_row + w;
+        at[w] = end[w] = 0;
+        if (row < m) {
+            at[w] = row_ptr[row] - base + phase;
+            end[w] = row_ptr[row + 1] - base;
+        }
+#pragma unroll
+        for (int i = 0; i < V; ++i) acc[w][i] = T(0);
+    }
+    bool more = true;
+    while (more) {
+        idx_t cc[kRows][kSteps];
+        T aa[kRows][kSteps];
+#pragma unroll
+        for (int w = 0; w < kRows; ++w) {
+#pragma unroll
+            for (int u = 0; u < kSteps; ++u) {
+                const idx_t j = at[w] + u * P;
+                if (j < end[w]) {
+                    cc[w][u] = col[j] - base;
+                    aa[w][u] = val[j];
+                }
+            }
+        }
+        Vec<T, V> b[kRows][kSteps];
+#pragma unroll
+        for (int w = 0; w < kRows; ++w) {
+#pragma unroll
+            for (int u = 0; u < kSteps; ++u) {
+                if (at[w] + u * P < end[w]) b[w][u] = load_vec<T, V>(B + static_cast<int64_t>(cc[w][u]) * ldb + c0);
+            }
+        }
+        more = false;
+#pragma unroll
+        for (int w = 0; w < kRows; ++w) {
+#pragma unroll
+            for (int u = 0; u < kSteps; ++u) {
+                if (at[w] + u * P < end[w]) {  // a lane without a nonzero stays out: 0 * inf would be NaN
+#pragma unroll
+                    for (int i = 0; i < V; ++i) acc[w][i] += aa[w][u] * b[w][u].v[i];
+                }
+            }
+            at[w] += kSteps * P;
+            more |= at[w] < end[w];
+        }
+        more = __any(more);  // the sums below need every lane of the wavefront
+    }
+#pragma unroll
+    for (int w = 0; w < kRows; ++w) {
+#pragma unroll
+        for (int stride = C; stride < kLanes; stride <<= 1) {
+#pragma unroll
+            for (int i = 0; i < V; ++i) acc[w][i] += __shfl_xor(acc[w][i], stride, kLanes);
+        }
+        const uint64_t row = first_row + w;
+        if (row < m && phase == 0 && in_panel) store_c<T, V>(Cm, ldc, c_row_major, row, c0, acc[w], alpha, beta);
+    }
+}
+
+template <typename T, int V, int C>
+void launch_narrow(hipStream_t stream, const SpmmArgs& a, T alpha, T beta) {
+    constexpr int kRowsPerBlock = kBlock / 16;
+    const uint64_t blocks = (static_cast<uint64_t>(a.m) + kRowsPerBlock - 1) / kRowsPerBlock;
+    hipLaunchKernelGGL((spmm_narrow_kernel<T, V, C>), dim3(static_cast<uint32_t>(blocks)), dim3(kBlock), 0, stream, a.m,
+                       a.n, a.base, a.row_ptr, a.col, static_cast<const T*>(a.val), static_cast<const T*>(a.B), a.ldb,
+                       static_cast<T*>(a.C), a.ldc, a.c_row_major, alpha, beta);
 }
 
 // op(B) column-major: element (kk, j) at j*ldb + kk.  One wavefront per row of A, lanes strided
@@ -524,7 +591,7 @@ void launch_rowb(hipStream_t stream, const SpmmArgs& a, T alpha, T beta) {
     const T* val = static_cast<const T*>(a.val);
     const T* B = static_cast<const T*>(a.B);
     T* C = static_cast<T*>(a.C);
-    if (LR < 4 || narrow_offsets(a, sizeof(T))) {  // the narrow groups do not use byte offsets at all
+    if (narrow_offsets(a, sizeof(T))) {
         hipLaunchKernelGGL((spmm_rowb_kernel<T, LR, V, false>), grid, dim3(kBlock), 0, stream, a.m, a.n, a.base,
                            a.row_ptr, a.col, val, B, a.ldb, C, a.ldc, a.c_row_major, alpha, beta);
     } else {
@@ -536,9 +603,9 @@ void launch_rowb(hipStream_t stream, const SpmmArgs& a, T alpha, T beta) {
 template <typename T, int V>
 void launch_rowb_v(hipStream_t stream, const SpmmArgs& a, T alpha, T beta) {
     const uint64_t lanes_needed = (static_cast<uint64_t>(a.n) + V - 1) / V;
-    if (lanes_needed <= 1) launch_rowb<T, 1, V>(stream, a, alpha, beta);
-    else if (lanes_needed <= 2) launch_rowb<T, 2, V>(stream, a, alpha, beta);
-    else if (lanes_needed <= 4) launch_rowb<T, 4, V>(stream, a, alpha, beta);
+    if (lanes_needed <= 1) launch_narrow<T, V, 1>(stream, a, alpha, beta);
+    else if (lanes_needed <= 2) launch_narrow<T, V, 2>(stream, a, alpha, beta);
+    else if (lanes_needed <= 4) launch_rowb<T, 4, V>(stream, a, alpha, beta);  // measured faster than four column lanes above
     else if (lanes_needed <= 8) launch_rowb<T, 8, V>(stream, a, alpha, beta);
     else if (lanes_needed <= 16) launch_rowb<T, 16, V>(stream, a, alpha, beta);
     else if (lanes_needed <= 32) launch_rowb<T, 32, V>(stream, a, alpha, beta);
