@@ -354,14 +354,29 @@ __device__ __forceinline__ void group_row_ranges(idx_t m, idx_t base, const idx_
     }
 }
 
+// One thread merges the rows of one group.  The column indices of the 64 groups of a wavefront
+// are one contiguous stretch of the CSR array; read thread by thread they would cost a cache
+// line per element, so the wavefront first copies the stretch into LDS (when it fits).
+constexpr uint32_t kMergeStage = 8192;  // column indices a wavefront keeps in LDS
 template <bool FILL>
-__global__ __launch_bounds__(kBlock) void group_merge_kernel(idx_t m, idx_t base, const idx_t* __restrict__ row_ptr,
-                                                             const idx_t* __restrict__ col,
-                                                             uint32_t* __restrict__ group_ptr,
-                                                             uint32_t* __restrict__ entries,
-                                                             unsigned long long* __restrict__ span_sum) {
+__global__ __launch_bounds__(kWave) void group_merge_kernel(idx_t m, idx_t base, const idx_t* __restrict__ row_ptr,
+                                                            const idx_t* __restrict__ col,
+                                                            uint32_t* __restrict__ group_ptr,
+                                                            uint32_t* __restrict__ entries,
+                                                            unsigned long long* __restrict__ span_sum) {
+    __shared__ idx_t s_col[kMergeStage];
     const uint64_t groups = spmm_groups(m);
-    const uint64_t group = static_cast<uint64_t>(blockIdx.x) * kBlock + threadIdx.x;
+    const uint64_t first_group = static_cast<uint64_t>(blockIdx.x) * kWave;
+    const uint64_t group = first_group + threadIdx.x;
+    const uint64_t first_row = first_group * R < m ? first_group * R : m;
+    const uint64_t end_row = (first_group + kWave) * R < m ? (first_group + kWave) * R : m;
+    const idx_t stretch_begin = row_ptr[first_row] - base;
+    const idx_t stretch_end = row_ptr[end_row] - base;
+    const bool staged = stretch_end - stretch_begin <= kMergeStage;
+    if (staged) {
+        for (idx_t t = threadIdx.x; t < stretch_end - stretch_begin; t += kWave) s_col[t] = col[stretch_begin + t];
+    }
+    __syncthreads();
     // slot `groups` receives the total after the scan; threads past it only take part in the
     // wavefront's sum below
     uint32_t count = 0;
@@ -376,7 +391,8 @@ __global__ __launch_bounds__(kBlock) void group_merge_kernel(idx_t m, idx_t base
                 uint32_t lo = kNoColumn;
 #pragma unroll
                 for (int r = 0; r < R; ++r) {
-                    head[r] = i[r] < e[r] ? static_cast<uint32_t>(col[i[r]] - base) : kNoColumn;
+                    head[r] = kNoColumn;
+                    if (i[r] < e[r]) head[r] = static_cast<uint32_t>((staged ? s_col[i[r] - stretch_begin] : col[i[r]]) - base);
                     lo = head[r] < lo ? head[r] : lo;
                 }
                 if (lo == kNoColumn) break;
@@ -662,13 +678,13 @@ void launch_spmm_schedule(hipStream_t stream, idx_t m, idx_t nnz, idx_t base, co
     uint32_t* group_ptr = reinterpret_cast<uint32_t*>(w + l.group_ptr);
     uint32_t* entries = reinterpret_cast<uint32_t*>(w + l.entries);
     const uint64_t slots = spmm_groups(m) + 1;
-    const dim3 grid(static_cast<uint32_t>((slots + kBlock - 1) / kBlock));
+    const dim3 grid(static_cast<uint32_t>((slots + kWave - 1) / kWave));
     unsigned long long* span_sum = reinterpret_cast<unsigned long long*>(w + l.span_sum);
     (void)hipMemsetAsync(span_sum, 0, sizeof(*span_sum), stream);
-    hipLaunchKernelGGL((group_merge_kernel<false>), grid, dim3(kBlock), 0, stream, m, base, row_ptr, col, group_ptr,
+    hipLaunchKernelGGL((group_merge_kernel<false>), grid, dim3(kWave), 0, stream, m, base, row_ptr, col, group_ptr,
                        entries, span_sum);
     launch_exclusive_scan_u32(stream, group_ptr, slots, w + l.scan_ws);
-    hipLaunchKernelGGL((group_merge_kernel<true>), grid, dim3(kBlock), 0, stream, m, base, row_ptr, col, group_ptr,
+    hipLaunchKernelGGL((group_merge_kernel<true>), grid, dim3(kWave), 0, stream, m, base, row_ptr, col, group_ptr,
                        entries, span_sum);
 }
 
