@@ -51,6 +51,30 @@ __device__ __forceinline__ idx_t wave_merge_search(uint64_t d, idx_t m, idx_t nn
     return static_cast<idx_t>(lo);
 }
 
+// Number of rows r in [0, m] whose first nonzero index row_ptr[r] - base is <= g, found like the
+// merge-path search above; with g a nonzero index the answer minus one is the row that holds g.
+// Every lane of the wave must call this; all lanes return the same value.
+__device__ __forceinline__ idx_t wave_count_row_starts(const idx_t* __restrict__ row_ptr, idx_t m, idx_t base, idx_t g) {
+    uint64_t lo = 0;
+    uint64_t hi = static_cast<uint64_t>(m) + 1;
+    const unsigned lane = lane_id();
+    while (lo < hi) {
+        const uint64_t span = hi - lo;
+        const uint64_t step = (span + kWave - 1) / kWave;
+        const uint64_t probe = lo + lane * step;
+        const bool pred = probe < hi && row_ptr[probe] - base <= g;
+        const unsigned count = __popcll(__ballot(pred));
+        if (count == 0) {
+            hi = lo;
+        } else {
+            const uint64_t new_hi = lo + static_cast<uint64_t>(count) * step;
+            lo = lo + static_cast<uint64_t>(count - 1) * step + 1;
+            hi = new_hi < hi ? new_hi : hi;
+        }
+    }
+    return static_cast<idx_t>(lo);
+}
+
 // coo_rows[j] = row of nonzero j (+ base).  One tile of the merged path per workgroup, so empty
 // rows, 1-nonzero rows and 200k-nonzero rows all cost one item each.
 // Reference semantics: src/kernels/conversion/coo2csr_device.hpp:26-41.
@@ -153,9 +177,9 @@ __global__ __launch_bounds__(kBlock) void coo2csr_kernel(idx_t nnz, idx_t m, idx
 }
 
 // ------------------------------------------------------------------------------------------
-// device-wide exclusive scan of uint32 (in place), chunks of 2048
+// device-wide exclusive scan of uint32 (in place), chunks of 4096
 // ------------------------------------------------------------------------------------------
-constexpr int kScanIpt = 8;
+constexpr int kScanIpt = 16;
 constexpr int kScanChunk = kBlock * kScanIpt;
 
 __device__ __forceinline__ uint32_t block_exclusive_scan(uint32_t v, uint32_t* s_wave, uint32_t* total) {
@@ -202,20 +226,44 @@ __global__ __launch_bounds__(kBlock) void scan_chunks_kernel(uint32_t* __restric
     __shared__ uint32_t s_wave[kBlock / kWave];
     // thread owns kScanIpt consecutive elements so that its local prefix is sequential
     const uint64_t start = static_cast<uint64_t>(blockIdx.x) * kScanChunk + static_cast<uint64_t>(threadIdx.x) * kScanIpt;
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    // whole runs of an aligned array move as 128-bit loads and stores
+    const bool whole = (reinterpret_cast<uintptr_t>(data) & 15u) == 0 && start + kScanIpt <= n;
     uint32_t v[kScanIpt];
     uint32_t sum = 0;
+    if (whole) {
 #pragma unroll
-    for (int i = 0; i < kScanIpt; ++i) {
-        v[i] = start + i < n ? data[start + i] : 0;
-        sum += v[i];
+        for (int q = 0; q < kScanIpt / 4; ++q) {
+            const u32x4 four = *reinterpret_cast<const u32x4*>(data + start + 4 * q);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[4 * q + e] = four[e];
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < kScanIpt; ++i) v[i] = start + i < n ? data[start + i] : 0;
     }
+#pragma unroll
+    for (int i = 0; i < kScanIpt; ++i) sum += v[i];
     uint32_t total;
     uint32_t off = block_exclusive_scan(sum, s_wave, &total);
     if (chunk_offsets != nullptr) off += chunk_offsets[blockIdx.x];
+    if (whole) {
 #pragma unroll
-    for (int i = 0; i < kScanIpt; ++i) {
-        if (start + i < n) data[start + i] = off;
-        off += v[i];
+        for (int q = 0; q < kScanIpt / 4; ++q) {
+            u32x4 four;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                four[e] = off;
+                off += v[4 * q + e];
+            }
+            *reinterpret_cast<u32x4*>(data + start + 4 * q) = four;
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < kScanIpt; ++i) {
+            if (start + i < n) data[start + i] = off;
+            off += v[i];
+        }
     }
 }
 
@@ -310,17 +358,20 @@ __device__ __forceinline__ uint32_t sort_block_exclusive_scan(uint32_t v, uint32
 }
 
 // VB = bytes per value (0 = no values).  counters hold, after the exclusive scan, the output
-// position of the first key of each (digit, tile).
+// position of the first key of each (digit, tile).  FROM_CSR: the triples are the nonzeros of a
+// CSR matrix in place -- rows_in is its row_ptr array (m + 1 offsets, index base `base`) and the
+// row of every nonzero (+ base) is worked out here instead of being read.
 template <int VB>
 struct ValueOf { typedef uint32_t type; };
 template <>
 struct ValueOf<8> { typedef uint64_t type; };
 
-template <int VB>
+template <int VB, bool FROM_CSR>
 __global__ __launch_bounds__(kSortBlock) void radix_scatter_kernel(
     const idx_t* __restrict__ keys_in, const idx_t* __restrict__ rows_in, const void* __restrict__ vals_in_v,
     idx_t* __restrict__ keys_out, idx_t* __restrict__ rows_out, void* __restrict__ vals_out_v, idx_t count,
-    uint32_t shift, uint32_t bits, uint32_t tiles, const uint32_t* __restrict__ counters) {
+    uint32_t shift, uint32_t bits, uint32_t tiles, const uint32_t* __restrict__ counters,
+    const idx_t* __restrict__ tile_rows, idx_t base) {
     typedef typename ValueOf<VB>::type val_t;
     const val_t* vals_in = static_cast<const val_t*>(vals_in_v);
     val_t* vals_out = static_cast<val_t*>(vals_out_v);
@@ -351,6 +402,23 @@ __global__ __launch_bounds__(kSortBlock) void radix_scatter_kernel(
     for (uint32_t i = tid; i < kSortWaves * kMaxRadix; i += kSortBlock) (&s_cnt[0][0])[i] = 0;
     __syncthreads();
 
+    // FROM_CSR: the row starts that fall inside the tile, relative to it, go to LDS (s_rows is
+    // free until the tile is sorted); the row of a nonzero is the row of the tile's first nonzero
+    // plus the number of starts at or before it.  They are asked for here and parked in LDS after
+    // the ranking below, which covers their latency.
+    idx_t first_row = 0, inside = 0, tile_first = 0;
+    const idx_t* starts_in = nullptr;
+    bool staged = false;
+    idx_t start_of[kSortIpt];
+    if constexpr (FROM_CSR) {
+        const idx_t before = tile_rows[tile];  // row starts at or before the tile's first nonzero
+        first_row = before - 1;
+        inside = tile_rows[tile + 1] - before;
+        starts_in = rows_in + before;
+        tile_first = static_cast<idx_t>(tile_start) + base;
+        staged = inside <= static_cast<idx_t>(kSortTile);
+    }
+
     // Position inside the tile of this thread's i-th triple: waves own consecutive slabs, lanes
     // are interleaved inside a slab, so (wave, i, lane) order is input order.
     idx_t key[kSortIpt], row[kSortIpt];
@@ -362,8 +430,15 @@ __global__ __launch_bounds__(kSortBlock) void radix_scatter_kernel(
         const uint32_t p = wave * kSortWaveItems + i * kWave + lane;
         const bool live = p < tile_count;
         key[i] = live ? load_stream(keys_in + tile_start + p) : 0;
-        row[i] = live ? load_stream(rows_in + tile_start + p) : 0;
+        if constexpr (!FROM_CSR) row[i] = live ? load_stream(rows_in + tile_start + p) : 0;
         if constexpr (VB != 0) val[i] = live ? load_stream(vals_in + tile_start + p) : val_t(0);
+    }
+    if constexpr (FROM_CSR) {
+#pragma unroll
+        for (int i = 0; i < kSortIpt; ++i) {
+            const idx_t j = i * kSortBlock + tid;
+            start_of[i] = staged && j < inside ? starts_in[j] : 0;
+        }
     }
 #pragma unroll
     for (int i = 0; i < kSortIpt; ++i) {
@@ -388,7 +463,35 @@ __global__ __launch_bounds__(kSortBlock) void radix_scatter_kernel(
             if ((peers & lanemask_lt) == 0) *counter = before + __popcll(peers);
         }
     }
+    if constexpr (FROM_CSR) {
+#pragma unroll
+        for (int i = 0; i < kSortIpt; ++i) {
+            const idx_t j = i * kSortBlock + tid;
+            if (staged && j < inside) s_rows[j] = start_of[i] - tile_first;
+        }
+    }
     __syncthreads();
+
+    if constexpr (FROM_CSR) {
+#pragma unroll
+        for (int i = 0; i < kSortIpt; ++i) {
+            const uint32_t p = wave * kSortWaveItems + i * kWave + lane;
+            idx_t lo = 0;
+            idx_t hi = inside;
+            if (staged) {
+                while (lo < hi) {
+                    const idx_t mid = (lo + hi) >> 1;
+                    if (s_rows[mid] <= p) lo = mid + 1; else hi = mid;
+                }
+            } else {  // more than a tile's worth of (mostly empty) rows: search the offsets in place
+                while (lo < hi) {
+                    const idx_t mid = (lo + hi) >> 1;
+                    if (starts_in[mid] - tile_first <= p) lo = mid + 1; else hi = mid;
+                }
+            }
+            row[i] = first_row + lo + base;
+        }
+    }
 
     // per digit: turn the wave counts into wave offsets, then lay the digits out in order
     uint32_t digit_total = 0;
@@ -435,6 +538,17 @@ __global__ __launch_bounds__(kSortBlock) void radix_scatter_kernel(
     }
 }
 
+// tile_rows[t] = number of rows that start at or before the first nonzero of sort tile t
+// (t = tiles: all m + 1 offsets).  One wavefront per entry.
+__global__ __launch_bounds__(kBlock) void tile_row_starts_kernel(const idx_t* __restrict__ row_ptr, idx_t m, idx_t base,
+                                                                 idx_t nnz, uint32_t tiles, idx_t* __restrict__ tile_rows) {
+    const uint32_t t = blockIdx.x * (kBlock / kWave) + threadIdx.x / kWave;
+    if (t > tiles) return;  // whole wavefront
+    const uint64_t first = static_cast<uint64_t>(t) * kSortTile;
+    const idx_t starts = wave_count_row_starts(row_ptr, m, base, first < nnz ? static_cast<idx_t>(first) : nnz);
+    if (threadIdx.x % kWave == 0) tile_rows[t] = starts;
+}
+
 uint32_t sort_tiles(idx_t nnz) { return static_cast<uint32_t>((static_cast<uint64_t>(nnz) + kSortTile - 1) / kSortTile); }
 
 size_t sort_counter_elems(idx_t count) { return static_cast<size_t>(kMaxRadix) * sort_tiles(count); }
@@ -447,6 +561,27 @@ struct SortScratch {
     void* vals[2];
     uint32_t* counters;
     uint32_t* scan_ws;
+    idx_t* tile_rows = nullptr;  // sort_tiles(count) + 1 entries, only for sorts that read a CSR matrix in place
+};
+
+template <int VB>
+void launch_scatter(hipStream_t stream, bool from_csr, uint32_t grid, const idx_t* keys_in, const idx_t* aux_in,
+                    const void* vals_in, idx_t* keys_out, idx_t* aux_out, void* vals_out, idx_t count, uint32_t shift,
+                    uint32_t bits, uint32_t tiles, const uint32_t* counters, const idx_t* tile_rows, idx_t base) {
+    if (from_csr) {
+        hipLaunchKernelGGL((radix_scatter_kernel<VB, true>), dim3(grid), dim3(kSortBlock), 0, stream, keys_in, aux_in,
+                           vals_in, keys_out, aux_out, vals_out, count, shift, bits, tiles, counters, tile_rows, base);
+    } else {
+        hipLaunchKernelGGL((radix_scatter_kernel<VB, false>), dim3(grid), dim3(kSortBlock), 0, stream, keys_in, aux_in,
+                           vals_in, keys_out, aux_out, vals_out, count, shift, bits, tiles, counters, tile_rows, base);
+    }
+}
+
+// A sort whose triples are the nonzeros of a CSR matrix where they lie.
+struct CsrSource {
+    idx_t rows = 0;  // > 0: aux_in is the row_ptr of a CSR matrix with this many rows, and the first
+                     // pass derives the aux of every triple, its row + base, from it
+    idx_t base = 0;  // index base of row_ptr
 };
 
 // Stable LSD radix sort of (key, aux, value) triples on the low key_bits of the keys, in
@@ -454,31 +589,30 @@ struct SortScratch {
 // which must not overlap the inputs.  value_bytes is 0 (no values), 4 or 8.
 void radix_sort_triples(hipStream_t stream, idx_t count, uint32_t key_bits, const idx_t* keys_in, const idx_t* aux_in,
                         const void* vals_in, idx_t* keys_out, idx_t* aux_out, void* vals_out, size_t value_bytes,
-                        const SortScratch& t) {
+                        const SortScratch& t, const CsrSource& csr = CsrSource()) {
     const uint32_t passes = key_bits == 0 ? 1 : (key_bits + 7) / 8;
     const uint32_t bits = key_bits == 0 ? 1 : (key_bits + passes - 1) / passes;
     const uint32_t radix = 1u << bits;
     const uint32_t tiles = sort_tiles(count);
     const uint32_t scatter_grid = (tiles + kXcds - 1) / kXcds * kXcds;
     uint32_t shift = 0;
+    if (csr.rows > 0) {
+        const uint32_t waves_per_block = kBlock / kWave;
+        hipLaunchKernelGGL(tile_row_starts_kernel, dim3((tiles + 1 + waves_per_block - 1) / waves_per_block), dim3(kBlock),
+                           0, stream, aux_in, csr.rows, csr.base, count, tiles, t.tile_rows);
+    }
     for (uint32_t p = 0; p < passes; ++p) {
         const bool last = p + 1 == passes;
+        const bool from_csr = p == 0 && csr.rows > 0;
         idx_t* k_out = last ? keys_out : t.keys[p & 1];
         idx_t* a_out = last ? aux_out : t.aux[p & 1];
         void* v_out = last ? vals_out : t.vals[p & 1];
         hipLaunchKernelGGL(radix_hist_kernel, dim3(scatter_grid), dim3(kHistBlock), 0, stream, keys_in, count, shift, bits,
                            tiles, t.counters);
         launch_exclusive_scan(stream, t.counters, static_cast<uint64_t>(radix) * tiles, t.scan_ws);
-        if (value_bytes == 0) {
-            hipLaunchKernelGGL((radix_scatter_kernel<0>), dim3(scatter_grid), dim3(kSortBlock), 0, stream, keys_in, aux_in,
-                               vals_in, k_out, a_out, v_out, count, shift, bits, tiles, t.counters);
-        } else if (value_bytes == 4) {
-            hipLaunchKernelGGL((radix_scatter_kernel<4>), dim3(scatter_grid), dim3(kSortBlock), 0, stream, keys_in, aux_in,
-                               vals_in, k_out, a_out, v_out, count, shift, bits, tiles, t.counters);
-        } else {
-            hipLaunchKernelGGL((radix_scatter_kernel<8>), dim3(scatter_grid), dim3(kSortBlock), 0, stream, keys_in, aux_in,
-                               vals_in, k_out, a_out, v_out, count, shift, bits, tiles, t.counters);
-        }
+        auto* launch = value_bytes == 0 ? launch_scatter<0> : value_bytes == 4 ? launch_scatter<4> : launch_scatter<8>;
+        launch(stream, from_csr, scatter_grid, keys_in, aux_in, vals_in, k_out, a_out, v_out, count, shift, bits, tiles,
+               t.counters, t.tile_rows, csr.base);
         keys_in = k_out;
         aux_in = a_out;
         vals_in = v_out;
@@ -487,7 +621,7 @@ void radix_sort_triples(hipStream_t stream, idx_t count, uint32_t key_bits, cons
 }
 
 struct Csr2CscLayout {
-    size_t coo_rows, sorted_keys, keys_a, rows_a, vals_a, keys_b, rows_b, vals_b, counters, scan_ws, total;
+    size_t sorted_keys, keys_a, rows_a, vals_a, keys_b, rows_b, vals_b, counters, scan_ws, tile_rows, total;
 };
 
 Csr2CscLayout csr2csc_layout(idx_t nnz, size_t value_bytes) {
@@ -496,7 +630,6 @@ Csr2CscLayout csr2csc_layout(idx_t nnz, size_t value_bytes) {
     const size_t val_bytes = align_up(static_cast<size_t>(nnz) * value_bytes);
     const size_t counter_elems = sort_counter_elems(nnz);
     size_t off = 0;
-    l.coo_rows = off; off += idx_bytes;
     l.sorted_keys = off; off += idx_bytes;
     l.keys_a = off; off += idx_bytes;
     l.rows_a = off; off += idx_bytes;
@@ -506,6 +639,7 @@ Csr2CscLayout csr2csc_layout(idx_t nnz, size_t value_bytes) {
     l.vals_b = off; off += val_bytes;
     l.counters = off; off += align_up(counter_elems * sizeof(uint32_t));
     l.scan_ws = off; off += align_up(scan_workspace_elems(counter_elems) * sizeof(uint32_t)) + kAlign;
+    l.tile_rows = off; off += align_up((static_cast<size_t>(sort_tiles(nnz)) + 1) * sizeof(idx_t));
     l.total = off;
     return l;
 }
@@ -592,33 +726,31 @@ size_t csr2csc_workspace_bytes(idx_t /*m*/, idx_t /*n*/, idx_t nnz, size_t value
     return csr2csc_layout(nnz, value_bytes).total;
 }
 
+// The nonzeros are sorted by column where they lie: the first pass reads col / val in place and
+// works the row indices out of row_ptr; the sorted columns then give the offsets.
 void launch_csr2csc(hipStream_t stream, idx_t m, idx_t n, idx_t nnz, const void* csr_val, const idx_t* row_ptr,
                     const idx_t* col, void* csc_val, idx_t* row_ind, idx_t* col_ptr, size_t value_bytes, idx_t base,
                     void* workspace) {
     if (m == 0 || n == 0 || nnz == 0) return;
     const Csr2CscLayout l = csr2csc_layout(nnz, value_bytes);
     char* w = static_cast<char*>(workspace);
-    idx_t* coo_rows = reinterpret_cast<idx_t*>(w + l.coo_rows);
     idx_t* sorted_keys = reinterpret_cast<idx_t*>(w + l.sorted_keys);
-    idx_t* keys_t[2] = {reinterpret_cast<idx_t*>(w + l.keys_a), reinterpret_cast<idx_t*>(w + l.keys_b)};
-    idx_t* rows_t[2] = {reinterpret_cast<idx_t*>(w + l.rows_a), reinterpret_cast<idx_t*>(w + l.rows_b)};
-    void* vals_t[2] = {w + l.vals_a, w + l.vals_b};
-    uint32_t* counters = reinterpret_cast<uint32_t*>(w + l.counters);
-    uint32_t* scan_ws = reinterpret_cast<uint32_t*>(w + l.scan_ws);
-
-    launch_csr2coo(stream, m, nnz, row_ptr, base, coo_rows);
-
-    // keys are the raw column indices (index base included), so the largest key is n - 1 + base
     SortScratch t;
-    for (int i = 0; i < 2; ++i) {
-        t.keys[i] = keys_t[i];
-        t.aux[i] = rows_t[i];
-        t.vals[i] = vals_t[i];
-    }
-    t.counters = counters;
-    t.scan_ws = scan_ws;
-    radix_sort_triples(stream, nnz, bit_length(n - 1 + base), col, coo_rows, csr_val, sorted_keys, row_ind, csc_val,
-                       value_bytes, t);
+    t.keys[0] = reinterpret_cast<idx_t*>(w + l.keys_a);
+    t.keys[1] = reinterpret_cast<idx_t*>(w + l.keys_b);
+    t.aux[0] = reinterpret_cast<idx_t*>(w + l.rows_a);
+    t.aux[1] = reinterpret_cast<idx_t*>(w + l.rows_b);
+    t.vals[0] = w + l.vals_a;
+    t.vals[1] = w + l.vals_b;
+    t.counters = reinterpret_cast<uint32_t*>(w + l.counters);
+    t.scan_ws = reinterpret_cast<uint32_t*>(w + l.scan_ws);
+    t.tile_rows = reinterpret_cast<idx_t*>(w + l.tile_rows);
+    CsrSource csr;
+    csr.rows = m;
+    csr.base = base;
+    // keys are the raw column indices (index base included), so the largest key is n - 1 + base
+    radix_sort_triples(stream, nnz, bit_length(n - 1 + base), col, row_ptr, csr_val, sorted_keys, row_ind, csc_val,
+                       value_bytes, t, csr);
     launch_coo2csr(stream, nnz, n, sorted_keys, base, col_ptr);
 }
 

@@ -56,6 +56,22 @@ def check_csr2csc(torch, handle, oracle, a, what):
     return cp, ri, cv
 
 
+def one_per_row(m, seed):
+    """A permutation matrix: every 4096-nonzero tile of the sort spans exactly 4096 rows."""
+    rng = np.random.default_rng(seed)
+    return wl.Csr(m, m, np.arange(m + 1), rng.permutation(m), rng.uniform(-1, 1, m).astype(np.float32))
+
+
+def empty_stretches(seed):
+    """Long runs of empty rows before, between and after a few long rows."""
+    rng = np.random.default_rng(seed)
+    lens = np.zeros(30000, np.int64)
+    lens[[7000, 7001, 19000, 24999]] = [5000, 1, 9000, 300]
+    ptr = np.concatenate([[0], np.cumsum(lens)])
+    col = np.concatenate([np.sort(rng.choice(12000, n, replace=False)) for n in lens if n])
+    return wl.Csr(30000, 12000, ptr, col, rng.uniform(-1, 1, int(ptr[-1])))
+
+
 CASES = {
     "ragged_f32": lambda: wl.random_ragged(5003, 4099, 23, dtype=np.float32, seed=1),
     "ragged_f64_base1": lambda: wl.random_ragged(5003, 4099, 23, dtype=np.float64, seed=2).with_base(1),
@@ -68,6 +84,9 @@ CASES = {
     "n_pow2_minus1_base1": lambda: wl.random_ragged(4096, 65535, 20, dtype=np.float32, seed=7).with_base(1),
     "n_small": lambda: wl.random_ragged(70000, 3, 2, dtype=np.float32, seed=8),
     "stencil": lambda: wl.stencil_27pt(20, dtype=np.float32),
+    "one_per_row": lambda: one_per_row(10000, 10),
+    "empty_stretches": lambda: empty_stretches(11),
+    "empty_stretches_base1": lambda: empty_stretches(12).with_base(1),
 }
 
 
