@@ -367,6 +367,32 @@ def cpu_baseline(kind, a, alpha, beta, n_cols, algo_bytes, op):
         def run():
             oracle.spmv_omp(a.m, a.base, a.ptr, a.col, a.val, alpha, beta, x, y, dynamic=dyn)
         sample = "whole workload per repetition"
+    elif kind == "spmv":
+        # op T as the library and the reference do it: transpose on every call, then the row loop
+        x = rng.uniform(-1, 1, a.m).astype(dt)
+        y = rng.uniform(-1, 1, a.n).astype(dt)
+
+        def run():
+            cp, ri, cv = oracle.csr2csc(a.m, a.n, a.base, a.ptr, a.col, a.val, method="omp")
+            oracle.spmv_omp(a.n, a.base, cp, ri, cv, alpha, beta, x, y, dynamic=True)
+        sample = "whole workload per repetition (csr2csc + row loop over the transpose)"
+    elif kind == "spmv-csc":
+        cp, ri, cv = oracle.csr2csc(a.m, a.n, a.base, a.ptr, a.col, a.val, method="omp")
+        x = rng.uniform(-1, 1, a.m).astype(dt)
+        y = rng.uniform(-1, 1, a.n).astype(dt)
+        dyn = int(np.diff(cp.astype(np.int64)).max()) > 4096
+
+        def run():
+            oracle.spmv_omp(a.n, a.base, cp, ri, cv, alpha, beta, x, y, dynamic=dyn)
+        sample = "whole workload per repetition (row loop over the transposed matrix)"
+    elif kind == "csr2csc":
+        def run():
+            oracle.csr2csc(a.m, a.n, a.base, a.ptr, a.col, a.val, method="omp")
+        sample = "whole workload per repetition (per-thread column counts, scan, stable placement)"
+    elif kind == "csr2coo":
+        def run():
+            oracle.csr2coo_omp(a.m, a.base, a.ptr, a.nnz)
+        sample = "whole workload per repetition"
     elif kind == "spmm":
         rows = min(a.m, max(1024, int(2e9 / max(1, 27 * n_cols * 4 * 10))))
         sub_ptr = a.ptr[:rows + 1]

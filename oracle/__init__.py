@@ -101,7 +101,8 @@ def coo2csr(nnz, m, base, coo_rows):
 def csr2csc(m, n, base, ptr, col, val=None, method="radix2"):
     """Returns (col_ptr, row_ind, csc_val); csc_val is None when val is None.
 
-    method "radix2" follows the reference step by step, "counting" is the fast equivalent."""
+    method "radix2" follows the reference step by step, "counting" is the fast equivalent, "omp" the
+    multi-threaded one that bench.py times as the CPU baseline."""
     ptr, col = _idx(ptr), _idx(col)
     nnz = int(col.shape[0])
     col_ptr = np.zeros(n + 1, dtype=np.uint32)
@@ -112,7 +113,8 @@ def csr2csc(m, n, base, ptr, col, val=None, method="radix2"):
         vb = val.dtype.itemsize
     else:
         csc_val, vb = None, 0
-    fn = {"radix2": lib().orc_csr2csc_radix2, "counting": lib().orc_csr2csc_counting}[method]
+    fn = {"radix2": lib().orc_csr2csc_radix2, "counting": lib().orc_csr2csc_counting,
+          "omp": lib().orc_csr2csc_omp}[method]
     fn.restype = _c_int
     rc = fn(_c_i64(m), _c_i64(n), _c_i64(nnz), _c_int(base), _p(ptr), _p(col), _p(val), _c_i64(vb), _p(col_ptr),
             _p(row_ind), _p(csc_val))
@@ -177,3 +179,11 @@ def spmm_omp_f32(m, n, base, ptr, col, val, alpha, beta, B, C):
     lib().orc_spmm_omp_f32.restype = None
     lib().orc_spmm_omp_f32(_c_i64(m), _c_i64(n), _c_int(base), _p(ptr), _p(col), _p(val), ctypes.c_float(alpha),
                            ctypes.c_float(beta), _p(B), _p(C))
+
+
+def csr2coo_omp(m, base, ptr, nnz):
+    ptr = _idx(ptr)
+    out = np.zeros(nnz, dtype=np.uint32)
+    lib().orc_csr2coo_omp.restype = None
+    lib().orc_csr2coo_omp(_c_i64(m), _c_int(base), _p(ptr), _p(out))
+    return out

@@ -321,3 +321,88 @@ int orc_max_threads(void) {
     return 1;
 #endif
 }
+
+/* csr2csc for the CPU baseline: the rows are cut into one block per thread (equal numbers of
+ * nonzeros), every block counts its columns, the counts become each block's first slot in every
+ * column (blocks in row order, so the order inside a column is the input order), then every block
+ * places its nonzeros.  Same result as orc_csr2csc_counting; tests pin them equal. */
+int orc_csr2csc_omp(int64_t m, int64_t n, int64_t nnz, int base, const idx_t* ptr, const idx_t* col, const void* val,
+                    int64_t value_bytes, idx_t* col_ptr, idx_t* row_ind, void* csc_val) {
+    if (m == 0 || n == 0 || nnz == 0) return 0;
+    const int blocks = orc_max_threads();
+    int64_t* first_row = (int64_t*)malloc(((size_t)blocks + 1) * sizeof(int64_t));
+    uint32_t* slot = (uint32_t*)malloc((size_t)blocks * (size_t)n * sizeof(uint32_t));
+    int64_t* start = (int64_t*)malloc(((size_t)n + 1) * sizeof(int64_t));
+    int64_t* part = (int64_t*)calloc((size_t)blocks + 1, sizeof(int64_t));
+    if (!first_row || !slot || !start || !part) {
+        free(first_row); free(slot); free(start); free(part);
+        return -1;
+    }
+    for (int b = 0; b <= blocks; ++b) { /* first row whose nonzeros start at or after b/blocks of all */
+        const int64_t want = nnz * b / blocks;
+        int64_t lo = 0, hi = m;
+        while (lo < hi) {
+            const int64_t mid = (lo + hi) / 2;
+            if ((int64_t)ptr[mid] - base < want) lo = mid + 1; else hi = mid;
+        }
+        first_row[b] = b == blocks ? m : lo;
+    }
+#pragma omp parallel for schedule(static, 1)
+    for (int b = 0; b < blocks; ++b) {
+        uint32_t* mine = slot + (size_t)b * (size_t)n;
+        memset(mine, 0, (size_t)n * sizeof(uint32_t));
+        for (int64_t j = (int64_t)ptr[first_row[b]] - base; j < (int64_t)ptr[first_row[b + 1]] - base; ++j)
+            ++mine[(int64_t)col[j] - base];
+    }
+#pragma omp parallel for schedule(static, 1)
+    for (int t = 0; t < blocks; ++t) { /* a range of columns per thread: counts -> first slots, column totals */
+        const int64_t c0 = n * t / blocks, c1 = n * (t + 1) / blocks;
+        int64_t sum = 0;
+        for (int64_t c = c0; c < c1; ++c) {
+            uint32_t running = 0;
+            for (int b = 0; b < blocks; ++b) {
+                const uint32_t count = slot[(size_t)b * (size_t)n + (size_t)c];
+                slot[(size_t)b * (size_t)n + (size_t)c] = running;
+                running += count;
+            }
+            start[c] = running;
+            sum += running;
+        }
+        part[t + 1] = sum;
+    }
+    for (int t = 0; t < blocks; ++t) part[t + 1] += part[t];
+#pragma omp parallel for schedule(static, 1)
+    for (int t = 0; t < blocks; ++t) {
+        const int64_t c0 = n * t / blocks, c1 = n * (t + 1) / blocks;
+        int64_t at = part[t];
+        for (int64_t c = c0; c < c1; ++c) {
+            const int64_t count = start[c];
+            start[c] = at;
+            col_ptr[c] = (idx_t)(at + base);
+            at += count;
+        }
+    }
+    start[n] = nnz;
+    col_ptr[n] = (idx_t)(nnz + base);
+#pragma omp parallel for schedule(static, 1)
+    for (int b = 0; b < blocks; ++b) {
+        uint32_t* mine = slot + (size_t)b * (size_t)n;
+        for (int64_t r = first_row[b]; r < first_row[b + 1]; ++r) {
+            for (int64_t j = (int64_t)ptr[r] - base; j < (int64_t)ptr[r + 1] - base; ++j) {
+                const int64_t c = (int64_t)col[j] - base;
+                const int64_t dst = start[c] + mine[c]++;
+                row_ind[dst] = (idx_t)(r + base);
+                if (value_bytes == 4) ((uint32_t*)csc_val)[dst] = ((const uint32_t*)val)[j];
+                else if (value_bytes == 8) ((uint64_t*)csc_val)[dst] = ((const uint64_t*)val)[j];
+            }
+        }
+    }
+    free(first_row); free(slot); free(start); free(part);
+    return 0;
+}
+
+void orc_csr2coo_omp(int64_t m, int base, const idx_t* ptr, idx_t* coo_rows) {
+#pragma omp parallel for schedule(dynamic, 4096)
+    for (int64_t r = 0; r < m; ++r)
+        for (int64_t j = (int64_t)ptr[r] - base; j < (int64_t)ptr[r + 1] - base; ++j) coo_rows[j] = (idx_t)(r + base);
+}

@@ -72,6 +72,16 @@ def empty_stretches(seed):
     return wl.Csr(30000, 12000, ptr, col, rng.uniform(-1, 1, int(ptr[-1])))
 
 
+def absent_columns(seed):
+    """Columns used only in the middle of a wide range: long stretches of equal offsets on both sides."""
+    rng = np.random.default_rng(seed)
+    m, n = 2000, 3_000_000
+    lens = rng.integers(0, 21, m)
+    ptr = np.concatenate([[0], np.cumsum(lens)])
+    col = np.concatenate([np.sort(rng.choice(np.arange(500_000, 2_500_000, 7), k, replace=False)) for k in lens])
+    return wl.Csr(m, n, ptr, col, rng.uniform(-1, 1, int(ptr[-1])).astype(np.float32))
+
+
 CASES = {
     "ragged_f32": lambda: wl.random_ragged(5003, 4099, 23, dtype=np.float32, seed=1),
     "ragged_f64_base1": lambda: wl.random_ragged(5003, 4099, 23, dtype=np.float64, seed=2).with_base(1),
@@ -87,6 +97,8 @@ CASES = {
     "one_per_row": lambda: one_per_row(10000, 10),
     "empty_stretches": lambda: empty_stretches(11),
     "empty_stretches_base1": lambda: empty_stretches(12).with_base(1),
+    "absent_columns": lambda: absent_columns(13),
+    "absent_columns_base1": lambda: absent_columns(14).with_base(1),
 }
 
 

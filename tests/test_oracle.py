@@ -49,7 +49,7 @@ def test_golden_spmv_spmm(oracle, path, base):
 
 @pytest.mark.parametrize("path", GOLDEN, ids=[os.path.basename(p) for p in GOLDEN])
 @pytest.mark.parametrize("base", [0, 1])
-@pytest.mark.parametrize("method", ["radix2", "counting"])
+@pytest.mark.parametrize("method", ["radix2", "counting", "omp"])
 def test_golden_conversions(oracle, path, base, method):
     g = load(path)
     m, n = int(g["m"]), int(g["n"])
@@ -134,7 +134,7 @@ def test_csr2csc_is_the_stable_sort(oracle):
     ptr = np.array([0, 4, 4, 7], dtype=np.int32)
     col = np.array([2, 0, 2, 2, 1, 2, 0], dtype=np.int32)  # unsorted, with repeats
     val = np.arange(10, 17, dtype=np.float64)
-    for method in ("radix2", "counting"):
+    for method in ("radix2", "counting", "omp"):
         cp, ri, cv = oracle.csr2csc(3, 3, 0, ptr, col, val, method=method)
         order = np.argsort(col, kind="stable")
         assert np.array_equal(cv, val[order])
@@ -147,8 +147,10 @@ def test_csr2csc_is_the_stable_sort(oracle):
         b = a.with_base(base)
         r1 = oracle.csr2csc(b.m, b.n, base, b.ptr, b.col, b.val, method="radix2")
         r2 = oracle.csr2csc(b.m, b.n, base, b.ptr, b.col, b.val, method="counting")
-        for u, v in zip(r1, r2):
-            assert np.array_equal(u, v)
+        r3 = oracle.csr2csc(b.m, b.n, base, b.ptr, b.col, b.val, method="omp")
+        for u, v, w in zip(r1, r2, r3):
+            assert np.array_equal(u, v) and np.array_equal(u, w)
+        assert np.array_equal(oracle.csr2coo_omp(b.m, base, b.ptr, b.nnz), oracle.csr2coo(b.m, base, b.ptr, b.nnz))
         cp, ri, cv = r1
         assert int(cp[-1]) - base == b.nnz and int(cp[0]) == base
         assert np.array_equal(np.sort(cv.view(np.uint32)), np.sort(b.val.view(np.uint32)))  # a permutation
