@@ -337,21 +337,35 @@ __global__ __launch_bounds__(kHistBlock) void radix_hist_kernel(const idx_t* __r
     if (threadIdx.x < radix) counters[static_cast<uint64_t>(threadIdx.x) * tiles + tile] = s_cnt[threadIdx.x];
 }
 
-// Exclusive scan over the kSortBlock threads of the scatter kernel.
-__device__ __forceinline__ uint32_t sort_block_exclusive_scan(uint32_t v, uint32_t* s_wave) {
+// Inclusive sum over the 64 lanes of a wavefront: four shifted adds inside each row of 16 lanes,
+// then the last lane of rows 0 and 2 is added to rows 1 and 3, then lane 31 to rows 2 and 3.
+__device__ __forceinline__ uint32_t wave_inclusive_sum(uint32_t v) {
+    constexpr int kRowShr = 0x110, kRowBcast15 = 0x142, kRowBcast31 = 0x143;
+    int x = static_cast<int>(v);
+    x += __builtin_amdgcn_update_dpp(0, x, kRowShr + 1, 0xF, 0xF, false);
+    x += __builtin_amdgcn_update_dpp(0, x, kRowShr + 2, 0xF, 0xF, false);
+    x += __builtin_amdgcn_update_dpp(0, x, kRowShr + 4, 0xF, 0xF, false);
+    x += __builtin_amdgcn_update_dpp(0, x, kRowShr + 8, 0xF, 0xF, false);
+    x += __builtin_amdgcn_update_dpp(0, x, kRowBcast15, 0xA, 0xF, false);
+    x += __builtin_amdgcn_update_dpp(0, x, kRowBcast31, 0xC, 0xF, false);
+    return static_cast<uint32_t>(x);
+}
+
+// Exclusive scan of one value per digit, held by the first kMaxRadix threads of the scatter
+// kernel; the other wavefronts only take part in the barrier.
+__device__ __forceinline__ uint32_t digit_exclusive_scan(uint32_t v, uint32_t* s_wave) {
+    constexpr unsigned kDigitWaves = kMaxRadix / kWave;
     const unsigned lane = threadIdx.x % kWave;
     const unsigned wave = threadIdx.x / kWave;
-    uint32_t inc = v;
-#pragma unroll
-    for (int off = 1; off < kWave; off <<= 1) {
-        const uint32_t up = __shfl_up(inc, off, kWave);
-        if (lane >= static_cast<unsigned>(off)) inc += up;
+    uint32_t inc = 0;
+    if (wave < kDigitWaves) {
+        inc = wave_inclusive_sum(v);
+        if (lane == kWave - 1) s_wave[wave] = inc;
     }
-    if (lane == kWave - 1) s_wave[wave] = inc;
     __syncthreads();
     uint32_t wave_off = 0;
 #pragma unroll
-    for (unsigned w = 0; w < kSortWaves; ++w) {
+    for (unsigned w = 0; w + 1 < kDigitWaves; ++w) {
         if (w < wave) wave_off += s_wave[w];
     }
     return wave_off + inc - v;
@@ -445,22 +459,29 @@ __global__ __launch_bounds__(kSortBlock) void radix_scatter_kernel(
         const uint32_t p = wave * kSortWaveItems + i * kWave + lane;
         const bool live = p < tile_count;
         const uint32_t d = (key[i] >> shift) & mask;
-        // lanes of this wave holding the same digit in this round
+        // lanes of this wave holding the same digit in this round: per bit of the digit, keep the
+        // lanes that voted as this lane did (vote xor own bit, spread over the word, is 0 there)
         uint64_t peers = __ballot(live);
-        for (uint32_t b = 0; b < bits; ++b) {
-            const bool bit = (d >> b) & 1u;
-            const uint64_t vote = __ballot(bit);
-            peers &= bit ? vote : ~vote;
+#pragma unroll
+        for (uint32_t b = 0; b < 8; ++b) {
+            if (b < bits) {
+                const uint32_t own = static_cast<uint32_t>(static_cast<int32_t>(d << (31 - b)) >> 31);  // bit b, spread
+                const uint64_t vote = __ballot(own != 0);
+                peers &= ~(vote ^ ((static_cast<uint64_t>(own) << 32) | own));
+            }
         }
         rank[i] = 0;
         if (live) {
-            // The counter is shared by the lanes of this wave across rounds, so it is accessed
-            // as volatile: every peer reads it, then the lowest peer alone adds the round's
-            // count.  LDS operations of one wave complete in program order.
-            volatile uint32_t* counter = &s_cnt[wave][d];
-            const uint32_t before = *counter;
+            // The counter is shared by the lanes of this wave across rounds: every peer reads it,
+            // then the lowest peer alone adds the round's count.  LDS operations of one wave
+            // complete in program order; the relaxed atomics keep the compiler from reordering or
+            // merging them and keep them LDS instructions.
+            uint32_t* counter = &s_cnt[wave][d];
+            const uint32_t before = __hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WAVEFRONT);
             rank[i] = before + __popcll(peers & lanemask_lt);
-            if ((peers & lanemask_lt) == 0) *counter = before + __popcll(peers);
+            if ((peers & lanemask_lt) == 0) {
+                __hip_atomic_store(counter, before + __popcll(peers), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WAVEFRONT);
+            }
         }
     }
     if constexpr (FROM_CSR) {
@@ -503,7 +524,7 @@ __global__ __launch_bounds__(kSortBlock) void radix_scatter_kernel(
             digit_total += c;
         }
     }
-    const uint32_t digit_start = sort_block_exclusive_scan(digit_total, s_wave);
+    const uint32_t digit_start = digit_exclusive_scan(digit_total, s_wave);
     if (tid < radix) {
         s_start[tid] = digit_start;
         s_dest[tid] = counters[static_cast<uint64_t>(tid) * tiles + tile];
