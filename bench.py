@@ -36,13 +36,14 @@ def _traffic(fetch_counts, write_counts):
 
 
 MEASURED_TRAFFIC_BYTES = {
-    "c2": _traffic(652670.2, 9150.2),                      # spmv_vector_kernel<double, 16, 4>
-    "c3": _traffic(5637867.2 + 6781.0 + 1857.9, 22218.4 + 231.8 + 817.9),   # merge kernel + partition + fix-up
-    "c4-64": _traffic(571013.1, 524288.0),                 # spmm_group_kernel<float, 16>
-    "c4-256": _traffic(3683533.2, 2097152.0),              # spmm_group_kernel<float, 64>
-    # csr2csc: 3 x (scatter + histogram + scans) + csr2coo + coo2csr
-    "c5": _traffic(3 * (701953.5 + 229171.1 + 3 * 4822.2 + 2 * 7174.2) + 83018.4 + 238051.1,
-                   3 * (1381473.1 + 28769.2 + 3 * 9552.7 + 2 * 56.0) + 459941.5 + 19514.6),
+    "c2": _traffic(652672.2, 9150.5),                      # spmv_vector_kernel<double, 16, 4>
+    "c3": _traffic(5638503.0 + 6781.0 + 1857.9, 22218.8 + 231.8 + 817.9),   # merge kernel + partition + fix-up
+    "c4-64": _traffic(612581.5, 524288.0),                 # spmm_group_kernel<float, 16>
+    "c4-256": _traffic(3673856.2, 2097152.0),              # spmm_group_kernel<float, 64>
+    # csr2csc: 2 x scatter + the scatter that reads the CSR arrays in place + 3 x (histogram + scans)
+    # + row starts per tile + coo2csr
+    "c5": _traffic(2 * 701979.3 + 481119.7 + 3 * (229171.1 + 2 * 7210.4 + 14341.0) + 21136.0 + 237160.4,
+                   2 * 1387277.8 + 1419195.4 + 3 * (28799.2 + 2 * 14331.3 + 56.0) + 223.8 + 19514.6),
 }
 
 
