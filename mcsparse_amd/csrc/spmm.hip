@@ -355,9 +355,11 @@ __device__ __forceinline__ void group_row_ranges(idx_t m, idx_t base, const idx_
 }
 
 // One thread merges the rows of one group.  The column indices of the 64 groups of a wavefront
-// are one contiguous stretch of the CSR array; read thread by thread they would cost a cache
-// line per element, so the wavefront first copies the stretch into LDS (when it fits).
+// are one contiguous stretch of the CSR array, and so are their merged lists; read or written
+// thread by thread they would cost a cache line per element, so the wavefront first copies the
+// stretch into LDS and collects the lists there before it writes them out (when they fit).
 constexpr uint32_t kMergeStage = 8192;  // column indices a wavefront keeps in LDS
+constexpr uint32_t kMergeOut = 4096;    // merged entries a wavefront collects in LDS
 template <bool FILL>
 __global__ __launch_bounds__(kWave) void group_merge_kernel(idx_t m, idx_t base, const idx_t* __restrict__ row_ptr,
                                                             const idx_t* __restrict__ col,
@@ -365,6 +367,7 @@ __global__ __launch_bounds__(kWave) void group_merge_kernel(idx_t m, idx_t base,
                                                             uint32_t* __restrict__ entries,
                                                             unsigned long long* __restrict__ span_sum) {
     __shared__ idx_t s_col[kMergeStage];
+    __shared__ uint32_t s_out[FILL ? kMergeOut : 1];
     const uint64_t groups = spmm_groups(m);
     const uint64_t first_group = static_cast<uint64_t>(blockIdx.x) * kWave;
     const uint64_t group = first_group + threadIdx.x;
@@ -374,8 +377,30 @@ __global__ __launch_bounds__(kWave) void group_merge_kernel(idx_t m, idx_t base,
     const idx_t stretch_end = row_ptr[end_row] - base;
     const bool staged = stretch_end - stretch_begin <= kMergeStage;
     if (staged) {
-        for (idx_t t = threadIdx.x; t < stretch_end - stretch_begin; t += kWave) s_col[t] = col[stretch_begin + t];
+        // sixteen loads on their way before the first is parked: the copy is bound by latency otherwise
+        constexpr int kAhead = 16;
+        const idx_t length = stretch_end - stretch_begin;
+        for (idx_t t0 = 0; t0 < length; t0 += kAhead * kWave) {
+            idx_t got[kAhead];
+#pragma unroll
+            for (int a = 0; a < kAhead; ++a) {
+                const idx_t t = t0 + a * kWave + threadIdx.x;
+                got[a] = t < length ? col[stretch_begin + t] : 0;
+            }
+#pragma unroll
+            for (int a = 0; a < kAhead; ++a) {
+                const idx_t t = t0 + a * kWave + threadIdx.x;
+                if (t < length) s_col[t] = got[a];
+            }
+        }
     }
+    // FILL: the lists of this wavefront's groups occupy entries[out_begin, out_end)
+    uint32_t out_begin = 0, out_end = 0;
+    if (FILL) {
+        out_begin = group_ptr[first_group < groups ? first_group : groups];
+        out_end = group_ptr[first_group + kWave < groups ? first_group + kWave : groups];
+    }
+    const bool collected = FILL && out_end - out_begin <= kMergeOut;
     __syncthreads();
     // slot `groups` receives the total after the scan; threads past it only take part in the
     // wavefront's sum below
@@ -386,28 +411,52 @@ __global__ __launch_bounds__(kWave) void group_merge_kernel(idx_t m, idx_t base,
         group_row_ranges(m, base, row_ptr, group * R, i, e);
         if (e[R - 1] - i[0] <= kSpmmMaxMergedGroup) {
             const uint32_t out = FILL ? group_ptr[group] : 0;
-            while (true) {
+            // the head of every row stays in a register and is read again only when the row moves on
+            auto merge = [&](auto staged_c, auto collected_c) {
+                constexpr bool kStaged = decltype(staged_c)::value;
+                constexpr bool kCollected = decltype(collected_c)::value;
+                auto head_of = [&](int r) -> uint32_t {
+                    if (i[r] >= e[r]) return kNoColumn;
+                    return static_cast<uint32_t>((kStaged ? s_col[i[r] - stretch_begin] : col[i[r]]) - base);
+                };
                 uint32_t head[R];
-                uint32_t lo = kNoColumn;
 #pragma unroll
-                for (int r = 0; r < R; ++r) {
-                    head[r] = kNoColumn;
-                    if (i[r] < e[r]) head[r] = static_cast<uint32_t>((staged ? s_col[i[r] - stretch_begin] : col[i[r]]) - base);
-                    lo = head[r] < lo ? head[r] : lo;
-                }
-                if (lo == kNoColumn) break;
-                if (first == kNoColumn) first = lo;
-                last = lo > last ? lo : last;
-                uint32_t flags = 0;
+                for (int r = 0; r < R; ++r) head[r] = head_of(r);
+                while (true) {
+                    uint32_t lo = kNoColumn;
 #pragma unroll
-                for (int r = 0; r < R; ++r) {
-                    const uint32_t takes = head[r] == lo;
-                    flags |= takes << r;
-                    i[r] += takes;
+                    for (int r = 0; r < R; ++r) lo = head[r] < lo ? head[r] : lo;
+                    if (lo == kNoColumn) break;
+                    if (first == kNoColumn) first = lo;
+                    last = lo > last ? lo : last;
+                    uint32_t flags = 0;
+#pragma unroll
+                    for (int r = 0; r < R; ++r) {
+                        if (head[r] == lo) {
+                            flags |= 1u << r;
+                            ++i[r];
+                            head[r] = head_of(r);
+                        }
+                    }
+                    if (FILL) {
+                        if (kCollected) s_out[out - out_begin + count] = (lo << R) | flags;
+                        else entries[out + count] = (lo << R) | flags;
+                    }
+                    ++count;
                 }
-                if (FILL) entries[out + count] = (lo << R) | flags;
-                ++count;
+            };
+            if (staged) {
+                if (collected) merge(std::true_type{}, std::true_type{});
+                else merge(std::true_type{}, std::false_type{});
+            } else {
+                merge(std::false_type{}, std::false_type{});
             }
+        }
+    }
+    if (FILL) {
+        __syncthreads();
+        if (collected && staged) {
+            for (uint32_t t = threadIdx.x; t < out_end - out_begin; t += kWave) entries[out_begin + t] = s_out[t];
         }
     }
     if (!FILL) {
