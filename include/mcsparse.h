@@ -414,7 +414,9 @@ mcsparseStatus_t mcsparseXcsrRowBins(mcsparseHandle_t handle, int m, const int* 
 
 /* Which SpMV kernel family a CSR op-N call on this descriptor runs:
  * 0 = not analysed yet, 1 = sub-wavefront vector kernel, 2 = merge-path kernel.
- * lanes_per_row is the sub-wavefront width for family 1 (0 otherwise). */
+ * lanes_per_row is the sub-wavefront width for family 1; for family 2 it is 1 when the tiles of
+ * the merge path run in the order of their first column (chosen for matrices with rows longer
+ * than a tile and an x too large for an L2) and 0 when they run in storage order. */
 mcsparseStatus_t mcsparseSpMatGetSpMVPlan(mcsparseSpMatDescr_t spMatDescr, int* family, int* lanes_per_row);
 
 /* Forces the SpMV kernel family for a descriptor (0 = automatic).  For tests and benchmarks. */

@@ -183,7 +183,7 @@ IndexArrays index_arrays(mcsparseHandle_t h, const mcsparseSpMatDescr* A, char* 
 // blocking 136-byte read-back) the first time a structure is seen.  `ptr` are the offsets to
 // analyse, `signature` the caller's array that identifies the structure.
 mcspStatus_t ensure_plan(mcsparseHandle_t h, mcsparseSpMatDescr* A, const idx_t* ptr, const void* signature,
-                         int64_t m, int64_t nnz, void* buffer) {
+                         int64_t m, int64_t nnz, int64_t x_bytes, void* buffer) {
     SpmvPlan& p = A->plan;
     if (p.valid && p.rows == signature && p.m == m && p.nnz == nnz && p.base == static_cast<int>(A->idxBase))
         return MCSP_STATUS_SUCCESS;
@@ -194,7 +194,8 @@ mcspStatus_t ensure_plan(mcsparseHandle_t h, mcsparseSpMatDescr* A, const idx_t*
     const int mean_lanes = mcsp::spmv_pick_lanes(static_cast<idx_t>(m), static_cast<idx_t>(nnz));
     if (p.forced_family != kFamilyAuto) {
         p.family = p.forced_family;
-        p.lanes = p.family == kFamilyVector ? (p.forced_lanes ? p.forced_lanes : mean_lanes) : 0;
+        // merge family: lanes != 0 asks for the tiles to run in the order of their first column
+        p.lanes = p.family == kFamilyVector ? (p.forced_lanes ? p.forced_lanes : mean_lanes) : (p.forced_lanes ? 1 : 0);
         p.max_row_len = 0;
         p.valid = true;
         return MCSP_STATUS_SUCCESS;
@@ -212,7 +213,10 @@ mcspStatus_t ensure_plan(mcsparseHandle_t h, mcsparseSpMatDescr* A, const idx_t*
     const uint32_t limit = static_cast<uint32_t>(32 * mean_lanes > 512 ? 32 * mean_lanes : 512);
     if (p.max_row_len > limit) {
         p.family = kFamilyMerge;
-        p.lanes = 0;
+        // Rows longer than a tile of the merge path put whole tiles inside one row; when x is too
+        // large to stay in an XCD's L2 next to the streamed matrix, those tiles run in the order of
+        // their first column (plan.lanes = 1), which costs two small kernels per call.
+        p.lanes = p.max_row_len >= kMergeTileItems && x_bytes > kMergeOrderMinVectorBytes ? 1 : 0;
     } else {
         p.family = kFamilyVector;
         p.lanes = p.forced_lanes ? p.forced_lanes : mean_lanes;
@@ -257,10 +261,11 @@ mcspStatus_t spmv_typed(mcsparseHandle_t h, mcsparseSpMatDescr* A, mcsparseOpera
         a.row_ptr = v.ptr;
         a.col = v.ind;
         a.val = v.val;
-        const mcspStatus_t st = ensure_plan(h, A, v.ptr, signature, v.m, A->nnz, buffer);
+        const mcspStatus_t st =
+            ensure_plan(h, A, v.ptr, signature, v.m, A->nnz, v.n * static_cast<int64_t>(sizeof(T)), buffer);
         if (st != MCSP_STATUS_SUCCESS) return st;
         if (A->plan.family == kFamilyMerge) {
-            mcsp::launch_spmv_merge<T>(h->stream, a, h_alpha, h_beta, buf + l.merge_ws);
+            mcsp::launch_spmv_merge<T>(h->stream, a, h_alpha, h_beta, buf + l.merge_ws, A->plan.lanes != 0);
         } else {
             mcsp::launch_spmv_vector<T>(h->stream, a, h_alpha, h_beta, A->plan.lanes);
         }
@@ -281,7 +286,7 @@ mcspStatus_t spmv_typed(mcsparseHandle_t h, mcsparseSpMatDescr* A, mcsparseOpera
     a.val = t_val;
     // no analysis of the freshly built structure (it would need a read-back): merge-path is
     // insensitive to the row-length distribution
-    mcsp::launch_spmv_merge<T>(h->stream, a, h_alpha, h_beta, buf + l.merge_ws);
+    mcsp::launch_spmv_merge<T>(h->stream, a, h_alpha, h_beta, buf + l.merge_ws, false);
     return MCSP_STATUS_SUCCESS;
 }
 

@@ -52,7 +52,7 @@ mcspStatus_t csrmv_impl(mcsparseHandle_t handle, int m, int n, int nnz, const T*
     a.x = x;
     a.y = y;
     if (workspace != nullptr) {
-        mcsp::launch_spmv_merge<T>(handle->stream, a, h_alpha, h_beta, workspace);
+        mcsp::launch_spmv_merge<T>(handle->stream, a, h_alpha, h_beta, workspace, false);
     } else {
         mcsp::launch_spmv_vector<T>(handle->stream, a, h_alpha, h_beta, mcsp::spmv_pick_lanes(a.m, a.nnz));
     }

@@ -53,6 +53,10 @@ struct mcsparseDnMatDescr {
 
 // Kernel family of an SpMV call.
 enum SpmvFamily : int { kFamilyAuto = 0, kFamilyVector = 1, kFamilyMerge = 2 };
+// Path items (row ends + nonzeros) per workgroup of the merge family, and the size of x from which
+// the analysis asks for its tiles to run in column order.
+constexpr uint32_t kMergeTileItems = 2048;
+constexpr int64_t kMergeOrderMinVectorBytes = 2 << 20;
 
 // Result of the row-length analysis of one CSR structure.  It only steers which kernel
 // runs; both kernel families are correct for any structure, so a stale plan costs time,
@@ -191,7 +195,7 @@ void launch_spmv_vector(hipStream_t stream, const SpmvArgs& a, T alpha, T beta, 
 // workspace: spmv_merge_workspace_bytes(m, nnz, sizeof(T)) bytes of device scratch.
 size_t spmv_merge_workspace_bytes(idx_t m, idx_t nnz, size_t value_bytes);
 template <typename T>
-void launch_spmv_merge(hipStream_t stream, const SpmvArgs& a, T alpha, T beta, void* workspace);
+void launch_spmv_merge(hipStream_t stream, const SpmvArgs& a, T alpha, T beta, void* workspace, bool order_tiles);
 int spmv_pick_lanes(idx_t m, idx_t nnz);
 
 // ---- SpMM (spmm.hip) ----

@@ -117,6 +117,7 @@ void launch_vector_lu(hipStream_t stream, const SpmvArgs& a, T alpha, T beta) {
 // ------------------------------------------------------------------------------------------
 constexpr int kItemsPerThread = 8;
 constexpr int kTile = kBlock * kItemsPerThread;  // path items per workgroup
+static_assert(kTile == static_cast<int>(kMergeTileItems), "the analysis compares row lengths with the tile size");
 
 // Path coordinate of diagonal d: how many row ends (x) precede it; nonzeros consumed = d - x.
 // A row end is consumed before a nonzero whenever row_end <= nonzero index.
@@ -136,15 +137,84 @@ __device__ __forceinline__ idx_t merge_search_global(uint64_t d, idx_t m, idx_t 
     return static_cast<idx_t>(lo);
 }
 
+// Tiles that lie inside long rows read x through a window that moves up with the tile's position in
+// the row.  Run in storage order, the tiles in flight at any moment belong to a few rows and their
+// windows are scattered over all of x; run in the order of their first column, all of them read
+// the same band of x, which then stays in L2 while the band moves once across the vector.  A coarse
+// order is enough: tiles are dropped into kOrderBuckets buckets by their first column and the
+// buckets run one after the other, in whatever order the tiles arrived inside them.  The result
+// does not depend on the order the tiles run in (carries are indexed by tile).
+constexpr int kOrderBuckets = kBlock;
+
+__global__ __launch_bounds__(kBlock) void zero_words_kernel(uint32_t* __restrict__ p, uint32_t n) {
+    const uint32_t i = blockIdx.x * kBlock + threadIdx.x;
+    if (i < n) p[i] = 0;
+}
+
+// tile_row[t] for t in [0, tiles]; with tile_bucket != nullptr also the bucket of every tile and the
+// number of tiles per bucket (bucket_count must be zero on entry).
 __global__ __launch_bounds__(kBlock) void merge_partition_kernel(idx_t m, idx_t nnz, idx_t base,
                                                                  const idx_t* __restrict__ row_ptr, uint32_t tiles,
-                                                                 idx_t* __restrict__ tile_row) {
+                                                                 idx_t* __restrict__ tile_row,
+                                                                 const idx_t* __restrict__ col, uint32_t key_shift,
+                                                                 uint32_t* __restrict__ tile_bucket,
+                                                                 uint32_t* __restrict__ bucket_count) {
+    __shared__ uint32_t s_count[kOrderBuckets];
+    const bool ordering = tile_bucket != nullptr;
+    if (ordering) {
+        s_count[threadIdx.x] = 0;
+        __syncthreads();
+    }
     const uint32_t t = blockIdx.x * kBlock + threadIdx.x;
-    if (t > tiles) return;
-    const uint64_t total = static_cast<uint64_t>(m) + nnz;
-    uint64_t d = static_cast<uint64_t>(t) * kTile;
-    if (d > total) d = total;
-    tile_row[t] = merge_search_global(d, m, nnz, base, row_ptr);
+    if (t <= tiles) {
+        const uint64_t total = static_cast<uint64_t>(m) + nnz;
+        uint64_t d = static_cast<uint64_t>(t) * kTile;
+        if (d > total) d = total;
+        const idx_t x = merge_search_global(d, m, nnz, base, row_ptr);
+        tile_row[t] = x;
+        if (ordering && t < tiles) {
+            const uint64_t first = d - x;  // the tile's first nonzero, if it has one
+            const uint32_t key = first < nnz ? col[first] - base : 0u;
+            const uint32_t bucket = min(key >> key_shift, static_cast<uint32_t>(kOrderBuckets - 1));
+            tile_bucket[t] = bucket;
+            atomicAdd(&s_count[bucket], 1u);
+        }
+    }
+    if (ordering) {
+        __syncthreads();
+        const uint32_t c = s_count[threadIdx.x];
+        if (c != 0) atomicAdd(&bucket_count[threadIdx.x], c);
+    }
+}
+
+// tile_order[position] = tile: bucket after bucket.  Every workgroup scans the bucket sizes for
+// itself; bucket_cursor (zero on entry) hands out the slots inside a bucket.
+__global__ __launch_bounds__(kBlock) void merge_order_kernel(uint32_t tiles, const uint32_t* __restrict__ tile_bucket,
+                                                             const uint32_t* __restrict__ bucket_count,
+                                                             uint32_t* __restrict__ bucket_cursor,
+                                                             uint32_t* __restrict__ tile_order) {
+    __shared__ uint32_t s_start[kOrderBuckets];
+    __shared__ uint32_t s_wave[kBlock / kWave];
+    const unsigned lane = threadIdx.x % kWave;
+    const unsigned wave = threadIdx.x / kWave;
+    const uint32_t size = bucket_count[threadIdx.x];
+    uint32_t inc = size;
+#pragma unroll
+    for (int off = 1; off < kWave; off <<= 1) {
+        const uint32_t up = __shfl_up(inc, off, kWave);
+        if (lane >= static_cast<unsigned>(off)) inc += up;
+    }
+    if (lane == kWave - 1) s_wave[wave] = inc;
+    __syncthreads();
+    uint32_t before = 0;
+    for (unsigned w = 0; w < wave; ++w) before += s_wave[w];
+    s_start[threadIdx.x] = before + inc - size;
+    __syncthreads();
+    const uint32_t t = blockIdx.x * kBlock + threadIdx.x;
+    if (t < tiles) {
+        const uint32_t bucket = tile_bucket[t];
+        tile_order[s_start[bucket] + atomicAdd(&bucket_cursor[bucket], 1u)] = t;
+    }
 }
 
 template <typename T, bool BETA0>
@@ -153,7 +223,8 @@ __global__ __launch_bounds__(kBlock) void spmv_merge_kernel(idx_t m, idx_t nnz, 
                                                             const idx_t* __restrict__ col, const T* __restrict__ val,
                                                             const T* __restrict__ x, T* __restrict__ y, T alpha,
                                                             T beta, const idx_t* __restrict__ tile_row,
-                                                            idx_t* __restrict__ carry_row, T* __restrict__ carry_val) {
+                                                            idx_t* __restrict__ carry_row, T* __restrict__ carry_val,
+                                                            const uint32_t* __restrict__ tile_order) {
     // s_row_end[i] = end offset of row x0+i; one extra slot closes the tile.
     __shared__ idx_t s_row_end[kTile + 1];
     // [0, tile_nnz) holds the products, [tile_nnz, tile_nnz + tile_rows) the finished row sums.
@@ -161,7 +232,7 @@ __global__ __launch_bounds__(kBlock) void spmv_merge_kernel(idx_t m, idx_t nnz, 
     __shared__ idx_t s_wave_key[kBlock / kWave];
     __shared__ T s_wave_val[kBlock / kWave];
 
-    const uint32_t tile = blockIdx.x;
+    const uint32_t tile = tile_order != nullptr ? tile_order[blockIdx.x] : blockIdx.x;
     const uint32_t tid = threadIdx.x;
     const uint64_t total = static_cast<uint64_t>(m) + nnz;
     const uint64_t d0 = static_cast<uint64_t>(tile) * kTile;
@@ -341,15 +412,17 @@ void launch_spmv_vector(hipStream_t stream, const SpmvArgs& a, T alpha, T beta, 
     }
 }
 
-// Workspace layout: [tile_row: tiles+1 idx][carry_row: tiles idx][carry_val: tiles T], each
+// Workspace layout: [tile_row: tiles+1 idx][carry_row: tiles idx][carry_val: tiles T]
+// [tile_bucket: tiles][tile_order: tiles][bucket sizes, bucket cursors: 2 * kOrderBuckets], each
 // sub-array aligned to 128 bytes.
 size_t spmv_merge_workspace_bytes(idx_t m, idx_t nnz, size_t value_bytes) {
     const size_t tiles = merge_tiles(m, nnz);
-    return align_up((tiles + 1) * sizeof(idx_t)) + align_up(tiles * sizeof(idx_t)) + align_up(tiles * value_bytes);
+    return align_up((tiles + 1) * sizeof(idx_t)) + align_up(tiles * sizeof(idx_t)) + align_up(tiles * value_bytes) +
+           2 * align_up(tiles * sizeof(uint32_t)) + align_up(2 * kOrderBuckets * sizeof(uint32_t));
 }
 
 template <typename T>
-void launch_spmv_merge(hipStream_t stream, const SpmvArgs& a, T alpha, T beta, void* workspace) {
+void launch_spmv_merge(hipStream_t stream, const SpmvArgs& a, T alpha, T beta, void* workspace, bool order_tiles) {
     if (a.m == 0) return;
     const uint32_t tiles = merge_tiles(a.m, a.nnz);
     char* w = static_cast<char*>(workspace);
@@ -358,19 +431,42 @@ void launch_spmv_merge(hipStream_t stream, const SpmvArgs& a, T alpha, T beta, v
     idx_t* carry_row = reinterpret_cast<idx_t*>(w);
     w += align_up(static_cast<size_t>(tiles) * sizeof(idx_t));
     T* carry_val = reinterpret_cast<T*>(w);
+    w += align_up(static_cast<size_t>(tiles) * sizeof(T));
+    uint32_t* tile_bucket = reinterpret_cast<uint32_t*>(w);
+    w += align_up(static_cast<size_t>(tiles) * sizeof(uint32_t));
+    uint32_t* tile_order = reinterpret_cast<uint32_t*>(w);
+    w += align_up(static_cast<size_t>(tiles) * sizeof(uint32_t));
+    uint32_t* bucket_count = reinterpret_cast<uint32_t*>(w);
+    uint32_t* bucket_cursor = bucket_count + kOrderBuckets;
 
     const T* val = static_cast<const T*>(a.val);
     const T* x = static_cast<const T*>(a.x);
     T* y = static_cast<T*>(a.y);
 
-    hipLaunchKernelGGL(merge_partition_kernel, dim3((tiles + 1 + kBlock - 1) / kBlock), dim3(kBlock), 0, stream, a.m,
-                       a.nnz, a.base, a.row_ptr, tiles, tile_row);
+    const dim3 per_tile((tiles + 1 + kBlock - 1) / kBlock);
+    if (order_tiles) {
+        // columns [0, n) fall into kOrderBuckets buckets of 2^key_shift columns
+        uint32_t key_shift = 0;
+        while ((static_cast<uint64_t>(kOrderBuckets) << key_shift) < a.n) ++key_shift;
+        hipLaunchKernelGGL(zero_words_kernel, dim3(2), dim3(kBlock), 0, stream, bucket_count, 2u * kOrderBuckets);
+        hipLaunchKernelGGL(merge_partition_kernel, per_tile, dim3(kBlock), 0, stream, a.m, a.nnz, a.base, a.row_ptr, tiles,
+                           tile_row, a.col, key_shift, tile_bucket, bucket_count);
+        hipLaunchKernelGGL(merge_order_kernel, per_tile, dim3(kBlock), 0, stream, tiles,
+                           static_cast<const uint32_t*>(tile_bucket), static_cast<const uint32_t*>(bucket_count),
+                           bucket_cursor, tile_order);
+    } else {
+        hipLaunchKernelGGL(merge_partition_kernel, per_tile, dim3(kBlock), 0, stream, a.m, a.nnz, a.base, a.row_ptr, tiles,
+                           tile_row, a.col, 0u, static_cast<uint32_t*>(nullptr), static_cast<uint32_t*>(nullptr));
+        tile_order = nullptr;
+    }
     if (beta == T(0)) {
         hipLaunchKernelGGL((spmv_merge_kernel<T, true>), dim3(tiles), dim3(kBlock), 0, stream, a.m, a.nnz, a.base,
-                           a.row_ptr, a.col, val, x, y, alpha, beta, tile_row, carry_row, carry_val);
+                           a.row_ptr, a.col, val, x, y, alpha, beta, tile_row, carry_row, carry_val,
+                           static_cast<const uint32_t*>(tile_order));
     } else {
         hipLaunchKernelGGL((spmv_merge_kernel<T, false>), dim3(tiles), dim3(kBlock), 0, stream, a.m, a.nnz, a.base,
-                           a.row_ptr, a.col, val, x, y, alpha, beta, tile_row, carry_row, carry_val);
+                           a.row_ptr, a.col, val, x, y, alpha, beta, tile_row, carry_row, carry_val,
+                           static_cast<const uint32_t*>(tile_order));
     }
     hipLaunchKernelGGL((spmv_merge_fixup_kernel<T>), dim3((tiles + kBlock - 1) / kBlock), dim3(kBlock), 0, stream, a.m,
                        tiles, carry_row, carry_val, y, alpha);
@@ -378,7 +474,7 @@ void launch_spmv_merge(hipStream_t stream, const SpmvArgs& a, T alpha, T beta, v
 
 template void launch_spmv_vector<float>(hipStream_t, const SpmvArgs&, float, float, int);
 template void launch_spmv_vector<double>(hipStream_t, const SpmvArgs&, double, double, int);
-template void launch_spmv_merge<float>(hipStream_t, const SpmvArgs&, float, float, void*);
-template void launch_spmv_merge<double>(hipStream_t, const SpmvArgs&, double, double, void*);
+template void launch_spmv_merge<float>(hipStream_t, const SpmvArgs&, float, float, void*, bool);
+template void launch_spmv_merge<double>(hipStream_t, const SpmvArgs&, double, double, void*, bool);
 
 }  // namespace mcsp

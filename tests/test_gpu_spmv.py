@@ -87,6 +87,9 @@ def test_merge_family_shapes(torch_gpu, handle, oracle, dtype, shape):
         pytest.skip("empty draw")
     check(torch_gpu, handle, oracle, a, 1.0, 0.0, family=api.FAMILY_MERGE, what="merge %r" % (shape,))
     check(torch_gpu, handle, oracle, a, 0.5, -2.0, family=api.FAMILY_MERGE, what="merge beta %r" % (shape,))
+    # lanes = 1: the tiles run in the order of their first column; same results
+    check(torch_gpu, handle, oracle, a, 1.0, 0.0, family=api.FAMILY_MERGE, lanes=1, what="ordered merge %r" % (shape,))
+    check(torch_gpu, handle, oracle, a, 0.5, -2.0, family=api.FAMILY_MERGE, lanes=1, what="ordered merge beta")
 
 
 def test_merge_family_one_huge_row_and_many_empty(torch_gpu, handle, oracle):
@@ -99,10 +102,10 @@ def test_merge_family_one_huge_row_and_many_empty(torch_gpu, handle, oracle):
     col = np.concatenate([np.sort(rng.choice(n, size=l, replace=False)) for l in lens if l])
     val = rng.uniform(-1, 1, int(ptr[-1])).astype(np.float32)
     a = wl.Csr(m, n, ptr, col, val)
-    for fam in (api.FAMILY_MERGE, api.FAMILY_AUTO):
-        worst, plan = check(torch_gpu, handle, oracle, a, 1.0, 0.0, family=fam, what="huge rows")
-        check(torch_gpu, handle, oracle, a, 3.0, 0.25, family=fam, what="huge rows beta")
-    assert plan[0] == api.FAMILY_MERGE
+    for fam, lanes in ((api.FAMILY_MERGE, 0), (api.FAMILY_MERGE, 1), (api.FAMILY_AUTO, 0)):
+        worst, plan = check(torch_gpu, handle, oracle, a, 1.0, 0.0, family=fam, lanes=lanes, what="huge rows")
+        check(torch_gpu, handle, oracle, a, 3.0, 0.25, family=fam, lanes=lanes, what="huge rows beta")
+    assert plan == (api.FAMILY_MERGE, 0)  # x (1.2 MB) fits an L2: storage order
 
 
 @pytest.mark.parametrize("base", [0, 1])
