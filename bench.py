@@ -36,10 +36,11 @@ def _traffic(fetch_counts, write_counts):
 
 
 MEASURED_TRAFFIC_BYTES = {
-    "c2": _traffic(652672.2, 9150.5),                      # spmv_vector_kernel<double, 16, 4>
-    "c3": _traffic(5638503.0 + 6781.0 + 1857.9, 22218.8 + 231.8 + 817.9),   # merge kernel + partition + fix-up
-    "c4-64": _traffic(612581.5, 524288.0),                 # spmm_group_kernel<float, 16>
-    "c4-256": _traffic(3673856.2, 2097152.0),              # spmm_group_kernel<float, 64>
+    "c2": _traffic(652646.9, 9147.7),                      # spmv_vector_kernel<double, 16, 4>
+    # merge kernel (tiles in column order) + partition + tile order + fix-up
+    "c3": _traffic(3818524.4 + 10496.0 + 135.4 + 1857.9, 20886.2 + 695.5 + 2216.5 + 817.9),
+    "c4-64": _traffic(614289.0, 524288.0),                 # spmm_group_kernel<float, 16>
+    "c4-256": _traffic(3674369.0, 2097152.0),              # spmm_group_kernel<float, 64>
     # csr2csc: 2 x scatter + the scatter that reads the CSR arrays in place + 3 x (histogram + scans)
     # + row starts per tile + coo2csr
     "c5": _traffic(2 * 701979.3 + 481119.7 + 3 * (229171.1 + 2 * 7210.4 + 14341.0) + 21136.0 + 237160.4,
