@@ -266,10 +266,18 @@ __global__ __launch_bounds__(kBlock) void spmm_narrow_kernel(idx_t m, idx_t n, i
     }
 #pragma unroll
     for (int w = 0; w < kRows; ++w) {
+        // sum over the nonzero phases: the lanes of a 16-lane DPP row that serve the same columns
 #pragma unroll
-        for (int stride = C; stride < kLanes; stride <<= 1) {
-#pragma unroll
-            for (int i = 0; i < V; ++i) acc[w][i] += __shfl_xor(acc[w][i], stride, kLanes);
+        for (int i = 0; i < V; ++i) {
+            if constexpr (C == 1) {
+                acc[w][i] = group_sum<kLanes>(acc[w][i]);
+            } else {
+                static_assert(C == 2, "column lanes per row");
+                constexpr int kQuadXor2 = 0x4E, kRowRor4 = 0x124, kRowRor8 = 0x128;  // lanes 2, 4 and 8 away
+                acc[w][i] += dpp_mov<kQuadXor2>(acc[w][i]);
+                acc[w][i] += dpp_mov<kRowRor4>(acc[w][i]);
+                acc[w][i] += dpp_mov<kRowRor8>(acc[w][i]);
+            }
         }
         const uint64_t row = first_row + w;
         if (row < m && phase == 0 && in_panel) store_c<T, V>(Cm, ldc, c_row_major, row, c0, acc[w], alpha, beta);
