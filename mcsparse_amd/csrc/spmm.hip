@@ -195,7 +195,7 @@ __global__ __launch_bounds__(kBlock) void spmm_rowb_kernel(idx_t m, idx_t n, idx
 // phases x C column lanes: phase p takes the nonzeros p, p + P, ... of the row, kSteps of them in
 // flight at once, and the P partial sums are added up across the lanes at the end.
 template <typename T, int V, int C>
-__global__ __launch_bounds__(kBlock) void spmm_narrow_kernel(idx_t m, idx_t n, idx_t base,
+__global__ __launch_bounds__(kBlock) void spmm_narrow_kernel(idx_t m, idx_t n, idx_t nnz, idx_t base,
                                                              const idx_t* __restrict__ row_ptr,
                                                              const idx_t* __restrict__ col,
                                                              const T* __restrict__ val, const T* __restrict__ B,
@@ -226,7 +226,11 @@ __global__ __launch_bounds__(kBlock) void spmm_narrow_kernel(idx_t m, idx_t n, i
 #pragma unroll
         for (int i = 0; i < V; ++i) acc[w][i] = T(0);
     }
-    bool more = true;
+    // Loads that sit under a test of their own are waited for one by one; so the nonzeros of all
+    // steps are read without one, from an index clamped to the last nonzero of the matrix, and
+    // whether a step really has a nonzero is only asked where its product would be added.
+    const idx_t last_nonzero = nnz - 1;
+    bool more = nnz != 0;  // without nonzeros there is nothing to read, only C to scale
     while (more) {
         idx_t cc[kRows][kSteps];
         T aa[kRows][kSteps];
@@ -234,11 +238,9 @@ __global__ __launch_bounds__(kBlock) void spmm_narrow_kernel(idx_t m, idx_t n, i
         for (int w = 0; w < kRows; ++w) {
 #pragma unroll
             for (int u = 0; u < kSteps; ++u) {
-                const idx_t j = at[w] + u * P;
-                if (j < end[w]) {
-                    cc[w][u] = col[j] - base;
-                    aa[w][u] = val[j];
-                }
+                const idx_t j = min(at[w] + u * P, last_nonzero);
+                cc[w][u] = col[j];
+                aa[w][u] = val[j];
             }
         }
         Vec<T, V> b[kRows][kSteps];
@@ -246,7 +248,7 @@ __global__ __launch_bounds__(kBlock) void spmm_narrow_kernel(idx_t m, idx_t n, i
         for (int w = 0; w < kRows; ++w) {
 #pragma unroll
             for (int u = 0; u < kSteps; ++u) {
-                if (at[w] + u * P < end[w]) b[w][u] = load_vec<T, V>(B + static_cast<int64_t>(cc[w][u]) * ldb + c0);
+                b[w][u] = load_vec<T, V>(B + static_cast<int64_t>(cc[w][u] - base) * ldb + c0);
             }
         }
         more = false;
@@ -289,7 +291,7 @@ void launch_narrow(hipStream_t stream, const SpmmArgs& a, T alpha, T beta) {
     constexpr int kRowsPerBlock = kBlock / 16;
     const uint64_t blocks = (static_cast<uint64_t>(a.m) + kRowsPerBlock - 1) / kRowsPerBlock;
     hipLaunchKernelGGL((spmm_narrow_kernel<T, V, C>), dim3(static_cast<uint32_t>(blocks)), dim3(kBlock), 0, stream, a.m,
-                       a.n, a.base, a.row_ptr, a.col, static_cast<const T*>(a.val), static_cast<const T*>(a.B), a.ldb,
+                       a.n, a.nnz, a.base, a.row_ptr, a.col, static_cast<const T*>(a.val), static_cast<const T*>(a.B), a.ldb,
                        static_cast<T*>(a.C), a.ldc, a.c_row_major, alpha, beta);
 }
 
