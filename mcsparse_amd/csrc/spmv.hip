@@ -38,19 +38,27 @@ __global__ __launch_bounds__(kBlock) void spmv_vector_kernel(idx_t m, idx_t base
     const idx_t group = threadIdx.x / L;
     const uint64_t row0 = static_cast<uint64_t>(blockIdx.x) * (kGroups * U) + group;
 
+    // A load that sits under a test of its own, or whose only use does, is waited for on the spot,
+    // one latency after the other.  So the loads of the U rows are written without tests (from
+    // clamped indices), each kind back to back, and the tests come where the values are used.
     idx_t j[U], e[U];
     T s[U];
+    {
+        idx_t begin_raw[U], end_raw[U];
 #pragma unroll
-    for (int u = 0; u < U; ++u) {
-        const uint64_t row = row0 + static_cast<uint64_t>(u) * kGroups;
-        if (row < m) {
-            j[u] = row_ptr[row] - base + lane;
-            e[u] = row_ptr[row + 1] - base;
-        } else {
-            j[u] = 0;
-            e[u] = 0;
+        for (int u = 0; u < U; ++u) {
+            const uint64_t row = row0 + static_cast<uint64_t>(u) * kGroups;
+            const uint64_t r = row < m ? row : m - 1;  // m != 0 here
+            begin_raw[u] = row_ptr[r];
+            end_raw[u] = row_ptr[r + 1];
         }
-        s[u] = T(0);
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const uint64_t row = row0 + static_cast<uint64_t>(u) * kGroups;
+            j[u] = row < m ? begin_raw[u] - base + lane : 0;
+            e[u] = row < m ? end_raw[u] - base : 0;
+            s[u] = T(0);
+        }
     }
 
     // All lanes stay in the loop until every row of the wave is done, so that the loads of the
@@ -66,12 +74,17 @@ __global__ __launch_bounds__(kBlock) void spmv_vector_kernel(idx_t m, idx_t base
             c[u] = act[u] ? load_stream(col + j[u]) : base;
             v[u] = act[u] ? load_stream(val + j[u]) : T(0);
         }
+        T xv[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) xv[u] = x[c[u] - base];
+        // every gather is asked for before the first one is needed
+#pragma unroll
+        for (int u = 0; u < U; ++u) asm volatile("" : "+v"(xv[u]));
         more = false;
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             // a lane without a nonzero must not touch the sum at all: 0 * x[..] is NaN for an infinite x
-            const T xv = x[c[u] - base];
-            if (act[u]) s[u] += v[u] * xv;
+            if (act[u]) s[u] += v[u] * xv[u];
             j[u] += L;
             more |= j[u] < e[u];
         }
