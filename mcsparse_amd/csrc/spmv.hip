@@ -258,17 +258,47 @@ __global__ __launch_bounds__(kBlock) void spmv_merge_kernel(idx_t m, idx_t nnz, 
     const idx_t tile_nnz = y1 - y0;
     const idx_t tile_items = tile_rows + tile_nnz;
 
-    for (idx_t i = tid; i <= tile_rows; i += kBlock) {
-        const idx_t r = x0 + i;
-        s_row_end[i] = r < m ? row_ptr[r + 1] - base : 0xFFFFFFFFu;
-    }
+    // A load that sits under a test of its own is waited for on the spot.  The loads of a thread's
+    // items are therefore written without tests, from clamped indices, each kind back to back: the
+    // row ends, the nonzeros, then the gathers from x; the tests come where the values are stored.
+    idx_t ends[kItemsPerThread + 1];
 #pragma unroll
-    for (int i = 0; i < kItemsPerThread; ++i) {
-        const idx_t k = tid + i * kBlock;
-        if (k < tile_nnz) {
-            const idx_t c = load_stream(col + y0 + k) - base;
-            const T v = load_stream(val + y0 + k);
-            s_data[k] = v * x[c];
+    for (int i = 0; i <= kItemsPerThread; ++i) {
+        // rows past the tile's last one are not needed: they all read that one's end again
+        const idx_t r = min(x0 + tid + static_cast<idx_t>(i) * kBlock, min(x1, m - 1));  // m != 0 here
+        ends[i] = row_ptr[r + 1];
+    }
+    const idx_t last_item = tile_nnz != 0 ? tile_nnz - 1 : 0;
+    const idx_t* tile_col = tile_nnz != 0 ? col + y0 : row_ptr;  // a tile of row ends only reads a valid word
+    const T* tile_val = tile_nnz != 0 ? val + y0 : x;
+#pragma unroll
+    for (int i = 0; i <= kItemsPerThread; ++i) {
+        const idx_t k = tid + static_cast<idx_t>(i) * kBlock;
+        if (k <= tile_rows) s_row_end[k] = x0 + k < m ? ends[i] - base : 0xFFFFFFFFu;
+    }
+    constexpr int kGatherBatch = kItemsPerThread;  // items whose loads are in flight together
+#pragma unroll
+    for (int i0 = 0; i0 < kItemsPerThread; i0 += kGatherBatch) {
+        idx_t c[kGatherBatch];
+        T v[kGatherBatch], xv[kGatherBatch];
+#pragma unroll
+        for (int i = 0; i < kGatherBatch; ++i) {
+            const idx_t k = min(tid + static_cast<idx_t>(i0 + i) * kBlock, last_item);
+            c[i] = load_stream(tile_col + k);
+            v[i] = load_stream(tile_val + k);
+        }
+#pragma unroll
+        for (int i = 0; i < kGatherBatch; ++i) {
+            const idx_t k = tid + static_cast<idx_t>(i0 + i) * kBlock;
+            xv[i] = x[k < tile_nnz ? c[i] - base : 0];
+        }
+        // every gather of the batch is asked for before the first one is needed
+#pragma unroll
+        for (int i = 0; i < kGatherBatch; ++i) asm volatile("" : "+v"(xv[i]));
+#pragma unroll
+        for (int i = 0; i < kGatherBatch; ++i) {
+            const idx_t k = tid + static_cast<idx_t>(i0 + i) * kBlock;
+            if (k < tile_nnz) s_data[k] = v[i] * xv[i];
         }
     }
     __syncthreads();
