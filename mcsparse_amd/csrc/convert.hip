@@ -209,11 +209,18 @@ __global__ __launch_bounds__(kBlock) void scan_reduce_kernel(const uint32_t* __r
                                                              uint32_t* __restrict__ chunk_sums) {
     __shared__ uint32_t s_wave[kBlock / kWave];
     const uint64_t start = static_cast<uint64_t>(blockIdx.x) * kScanChunk;
+    // loads without a test of their own (clamped index), so that they are all on their way at once
+    uint32_t got[kScanIpt];
+#pragma unroll
+    for (int i = 0; i < kScanIpt; ++i) {
+        const uint64_t p = start + static_cast<uint64_t>(i) * kBlock + threadIdx.x;
+        got[i] = data[p < n ? p : n - 1];  // n != 0: the grid has no workgroup otherwise
+    }
     uint32_t v = 0;
 #pragma unroll
     for (int i = 0; i < kScanIpt; ++i) {
         const uint64_t p = start + static_cast<uint64_t>(i) * kBlock + threadIdx.x;
-        if (p < n) v += data[p];
+        v += p < n ? got[i] : 0u;
     }
     uint32_t total;
     block_exclusive_scan(v, s_wave, &total);
