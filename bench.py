@@ -36,15 +36,15 @@ def _traffic(fetch_counts, write_counts):
 
 
 MEASURED_TRAFFIC_BYTES = {
-    "c2": _traffic(652646.9, 9147.7),                      # spmv_vector_kernel<double, 16, 4>
+    "c2": _traffic(653890.5, 10048.5),                      # spmv_vector_kernel<double, 16, 4>
     # merge kernel (tiles in column order) + partition + tile order + fix-up
-    "c3": _traffic(3818524.4 + 10496.0 + 135.4 + 1857.9, 20886.2 + 695.5 + 2216.5 + 817.9),
-    "c4-64": _traffic(614289.0, 524288.0),                 # spmm_group_kernel<float, 16>
-    "c4-256": _traffic(3674369.0, 2097152.0),              # spmm_group_kernel<float, 64>
+    "c3": _traffic(3832220.9 + 10496.0 + 135.1 + 1857.9, 20915.7 + 695.5 + 2220.8 + 817.9),
+    "c4-64": _traffic(613893.3, 524288.0),                 # spmm_group_kernel<float, 16>
+    "c4-256": _traffic(3673719.8, 2097152.0),              # spmm_group_kernel<float, 64>
     # csr2csc: 2 x scatter + the scatter that reads the CSR arrays in place + 3 x (histogram + scans)
     # + row starts per tile + coo2csr
-    "c5": _traffic(2 * 701979.3 + 481119.7 + 3 * (229171.1 + 2 * 7210.4 + 14341.0) + 21136.0 + 237160.4,
-                   2 * 1387277.8 + 1419195.4 + 3 * (28799.2 + 2 * 14331.3 + 56.0) + 223.8 + 19514.6),
+    "c5": _traffic(2 * 701979.0 + 481119.4 + 3 * (229171.1 + 2 * 7206.6 + 14342.5) + 21136.0 + 237161.6,
+                   2 * 1387754.6 + 1421432.8 + 3 * (28789.0 + 2 * 14326.3 + 56.0) + 223.8 + 19514.6),
 }
 
 
