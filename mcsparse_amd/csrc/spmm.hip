@@ -318,9 +318,14 @@ __global__ __launch_bounds__(kBlock) void spmm_colb_kernel(idx_t m, idx_t n, idx
         for (idx_t e = start + lane; e < end; e += kWave) {
             const idx_t c = col[e] - base;
             const T a = val[e];
+            // the JB gathers without a test per load (a column past n reads column n - 1 again), so that
+            // they are on their way together; the test comes where the product is added
+            T b[JB];
+#pragma unroll
+            for (int jj = 0; jj < JB; ++jj) b[jj] = B[static_cast<int64_t>(min(j0 + jj, n - 1)) * ldb + c];
 #pragma unroll
             for (int jj = 0; jj < JB; ++jj) {
-                if (j0 + jj < n) s[jj] += a * B[static_cast<int64_t>(j0 + jj) * ldb + c];
+                if (j0 + jj < n) s[jj] += a * b[jj];
             }
         }
 #pragma unroll
