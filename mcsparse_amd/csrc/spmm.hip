@@ -484,6 +484,8 @@ __global__ __launch_bounds__(kWave) void group_merge_kernel(idx_t m, idx_t base,
     }
 }
 
+__global__ void zero_u64_kernel(unsigned long long* p) { *p = 0; }
+
 // Returns the top bit of w and shifts w left by one: an add whose carry is the answer.
 __device__ __forceinline__ bool shift_out_top(uint32_t& w) {
     unsigned doubled;
@@ -747,7 +749,8 @@ void launch_spmm_schedule(hipStream_t stream, idx_t m, idx_t nnz, idx_t base, co
     const uint64_t slots = spmm_groups(m) + 1;
     const dim3 grid(static_cast<uint32_t>((slots + kWave - 1) / kWave));
     unsigned long long* span_sum = reinterpret_cast<unsigned long long*>(w + l.span_sum);
-    (void)hipMemsetAsync(span_sum, 0, sizeof(*span_sum), stream);
+    // a fill kernel rather than a memset node, so that the sequence can be captured in a HIP graph
+    hipLaunchKernelGGL(zero_u64_kernel, dim3(1), dim3(1), 0, stream, span_sum);
     hipLaunchKernelGGL((group_merge_kernel<false>), grid, dim3(kWave), 0, stream, m, base, row_ptr, col, group_ptr,
                        entries, span_sum);
     launch_exclusive_scan_u32(stream, group_ptr, slots, w + l.scan_ws);
