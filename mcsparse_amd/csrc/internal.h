@@ -53,9 +53,9 @@ struct mcsparseDnMatDescr {
 
 // Kernel family of an SpMV call.
 enum SpmvFamily : int { kFamilyAuto = 0, kFamilyVector = 1, kFamilyMerge = 2 };
-// Path items (row ends + nonzeros) per workgroup of the merge family, and the size of x from which
-// the analysis asks for its tiles to run in column order.
-constexpr uint32_t kMergeTileItems = 2048;
+// Path items (row ends + nonzeros) per workgroup of the merge family when its tiles run in column
+// order, and the size of x from which the analysis asks for that order.
+constexpr uint32_t kMergeTileItems = 1024;
 constexpr int64_t kMergeOrderMinVectorBytes = 2 << 20;
 
 // Result of the row-length analysis of one CSR structure.  It only steers which kernel

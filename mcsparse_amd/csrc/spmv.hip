@@ -128,9 +128,15 @@ void launch_vector_lu(hipStream_t stream, const SpmvArgs& a, T alpha, T beta) {
 // ------------------------------------------------------------------------------------------
 // merge family
 // ------------------------------------------------------------------------------------------
-constexpr int kItemsPerThread = 8;
-constexpr int kTile = kBlock * kItemsPerThread;  // path items per workgroup
-static_assert(kTile == static_cast<int>(kMergeTileItems), "the analysis compares row lengths with the tile size");
+// Path items per thread, IPT, times kBlock threads make a tile, the share of one workgroup.  Tiles that
+// run in storage order take 8 items per thread.  Tiles that run in the order of their first column
+// take 4: the shorter a tile, the narrower the window of x it reads inside a long row, so rows from
+// half the length on keep their gathers within the band in flight (measured on a power-law matrix
+// of 4 M rows: 1.09 ms with 8 items, 1.00 ms with 4, 1.01 ms with 2).
+constexpr int kItemsInOrder = 8;
+constexpr int kItemsByColumn = 4;
+static_assert(kBlock * kItemsByColumn == static_cast<int>(kMergeTileItems),
+              "the analysis compares row lengths with the size of a tile that runs in column order");
 
 // Path coordinate of diagonal d: how many row ends (x) precede it; nonzeros consumed = d - x.
 // A row end is consumed before a nonzero whenever row_end <= nonzero index.
@@ -166,12 +172,14 @@ __global__ __launch_bounds__(kBlock) void zero_words_kernel(uint32_t* __restrict
 
 // tile_row[t] for t in [0, tiles]; with tile_bucket != nullptr also the bucket of every tile and the
 // number of tiles per bucket (bucket_count must be zero on entry).
+template <int IPT>
 __global__ __launch_bounds__(kBlock) void merge_partition_kernel(idx_t m, idx_t nnz, idx_t base,
                                                                  const idx_t* __restrict__ row_ptr, uint32_t tiles,
                                                                  idx_t* __restrict__ tile_row,
                                                                  const idx_t* __restrict__ col, uint32_t key_shift,
                                                                  uint32_t* __restrict__ tile_bucket,
                                                                  uint32_t* __restrict__ bucket_count) {
+    constexpr int kTile = kBlock * IPT;
     __shared__ uint32_t s_count[kOrderBuckets];
     const bool ordering = tile_bucket != nullptr;
     if (ordering) {
@@ -230,7 +238,7 @@ __global__ __launch_bounds__(kBlock) void merge_order_kernel(uint32_t tiles, con
     }
 }
 
-template <typename T, bool BETA0>
+template <typename T, bool BETA0, int IPT>
 __global__ __launch_bounds__(kBlock) void spmv_merge_kernel(idx_t m, idx_t nnz, idx_t base,
                                                             const idx_t* __restrict__ row_ptr,
                                                             const idx_t* __restrict__ col, const T* __restrict__ val,
@@ -238,6 +246,8 @@ __global__ __launch_bounds__(kBlock) void spmv_merge_kernel(idx_t m, idx_t nnz, 
                                                             T beta, const idx_t* __restrict__ tile_row,
                                                             idx_t* __restrict__ carry_row, T* __restrict__ carry_val,
                                                             const uint32_t* __restrict__ tile_order) {
+    constexpr int kItemsPerThread = IPT;
+    constexpr int kTile = kBlock * IPT;
     // s_row_end[i] = end offset of row x0+i; one extra slot closes the tile.
     __shared__ idx_t s_row_end[kTile + 1];
     // [0, tile_nnz) holds the products, [tile_nnz, tile_nnz + tile_rows) the finished row sums.
@@ -424,9 +434,10 @@ __global__ __launch_bounds__(kBlock) void spmv_merge_fixup_kernel(idx_t m, uint3
     if (sum != T(0)) y[r] += alpha * sum;
 }
 
-inline uint32_t merge_tiles(idx_t m, idx_t nnz) {
+inline uint32_t merge_tiles(idx_t m, idx_t nnz, int items_per_thread) {
+    const uint64_t tile = static_cast<uint64_t>(kBlock) * items_per_thread;
     const uint64_t total = static_cast<uint64_t>(m) + nnz;
-    return static_cast<uint32_t>((total + kTile - 1) / kTile);
+    return static_cast<uint32_t>((total + tile - 1) / tile);
 }
 
 }  // namespace
@@ -459,15 +470,14 @@ void launch_spmv_vector(hipStream_t stream, const SpmvArgs& a, T alpha, T beta, 
 // [tile_bucket: tiles][tile_order: tiles][bucket sizes, bucket cursors: 2 * kOrderBuckets], each
 // sub-array aligned to 128 bytes.
 size_t spmv_merge_workspace_bytes(idx_t m, idx_t nnz, size_t value_bytes) {
-    const size_t tiles = merge_tiles(m, nnz);
+    const size_t tiles = merge_tiles(m, nnz, kItemsByColumn);  // the shorter tiles: room for either kind
     return align_up((tiles + 1) * sizeof(idx_t)) + align_up(tiles * sizeof(idx_t)) + align_up(tiles * value_bytes) +
            2 * align_up(tiles * sizeof(uint32_t)) + align_up(2 * kOrderBuckets * sizeof(uint32_t));
 }
 
-template <typename T>
-void launch_spmv_merge(hipStream_t stream, const SpmvArgs& a, T alpha, T beta, void* workspace, bool order_tiles) {
-    if (a.m == 0) return;
-    const uint32_t tiles = merge_tiles(a.m, a.nnz);
+template <typename T, int IPT>
+void launch_spmv_merge_tiles(hipStream_t stream, const SpmvArgs& a, T alpha, T beta, void* workspace, bool order_tiles) {
+    const uint32_t tiles = merge_tiles(a.m, a.nnz, IPT);
     char* w = static_cast<char*>(workspace);
     idx_t* tile_row = reinterpret_cast<idx_t*>(w);
     w += align_up((static_cast<size_t>(tiles) + 1) * sizeof(idx_t));
@@ -492,27 +502,34 @@ void launch_spmv_merge(hipStream_t stream, const SpmvArgs& a, T alpha, T beta, v
         uint32_t key_shift = 0;
         while ((static_cast<uint64_t>(kOrderBuckets) << key_shift) < a.n) ++key_shift;
         hipLaunchKernelGGL(zero_words_kernel, dim3(2), dim3(kBlock), 0, stream, bucket_count, 2u * kOrderBuckets);
-        hipLaunchKernelGGL(merge_partition_kernel, per_tile, dim3(kBlock), 0, stream, a.m, a.nnz, a.base, a.row_ptr, tiles,
+        hipLaunchKernelGGL(merge_partition_kernel<IPT>, per_tile, dim3(kBlock), 0, stream, a.m, a.nnz, a.base, a.row_ptr, tiles,
                            tile_row, a.col, key_shift, tile_bucket, bucket_count);
         hipLaunchKernelGGL(merge_order_kernel, per_tile, dim3(kBlock), 0, stream, tiles,
                            static_cast<const uint32_t*>(tile_bucket), static_cast<const uint32_t*>(bucket_count),
                            bucket_cursor, tile_order);
     } else {
-        hipLaunchKernelGGL(merge_partition_kernel, per_tile, dim3(kBlock), 0, stream, a.m, a.nnz, a.base, a.row_ptr, tiles,
+        hipLaunchKernelGGL(merge_partition_kernel<IPT>, per_tile, dim3(kBlock), 0, stream, a.m, a.nnz, a.base, a.row_ptr, tiles,
                            tile_row, a.col, 0u, static_cast<uint32_t*>(nullptr), static_cast<uint32_t*>(nullptr));
         tile_order = nullptr;
     }
     if (beta == T(0)) {
-        hipLaunchKernelGGL((spmv_merge_kernel<T, true>), dim3(tiles), dim3(kBlock), 0, stream, a.m, a.nnz, a.base,
+        hipLaunchKernelGGL((spmv_merge_kernel<T, true, IPT>), dim3(tiles), dim3(kBlock), 0, stream, a.m, a.nnz, a.base,
                            a.row_ptr, a.col, val, x, y, alpha, beta, tile_row, carry_row, carry_val,
                            static_cast<const uint32_t*>(tile_order));
     } else {
-        hipLaunchKernelGGL((spmv_merge_kernel<T, false>), dim3(tiles), dim3(kBlock), 0, stream, a.m, a.nnz, a.base,
+        hipLaunchKernelGGL((spmv_merge_kernel<T, false, IPT>), dim3(tiles), dim3(kBlock), 0, stream, a.m, a.nnz, a.base,
                            a.row_ptr, a.col, val, x, y, alpha, beta, tile_row, carry_row, carry_val,
                            static_cast<const uint32_t*>(tile_order));
     }
     hipLaunchKernelGGL((spmv_merge_fixup_kernel<T>), dim3((tiles + kBlock - 1) / kBlock), dim3(kBlock), 0, stream, a.m,
                        tiles, carry_row, carry_val, y, alpha);
+}
+
+template <typename T>
+void launch_spmv_merge(hipStream_t stream, const SpmvArgs& a, T alpha, T beta, void* workspace, bool order_tiles) {
+    if (a.m == 0) return;
+    if (order_tiles) launch_spmv_merge_tiles<T, kItemsByColumn>(stream, a, alpha, beta, workspace, true);
+    else launch_spmv_merge_tiles<T, kItemsInOrder>(stream, a, alpha, beta, workspace, false);
 }
 
 template void launch_spmv_vector<float>(hipStream_t, const SpmvArgs&, float, float, int);
