@@ -209,13 +209,17 @@ __global__ __launch_bounds__(kBlock) void merge_partition_kernel(idx_t m, idx_t 
 }
 
 // tile_order[position] = tile: bucket after bucket.  Every workgroup scans the bucket sizes for
-// itself; bucket_cursor (zero on entry) hands out the slots inside a bucket.
+// itself; bucket_cursor (zero on entry) hands out the slots inside a bucket, one stretch per
+// workgroup and bucket: the tiles of a workgroup are first counted per bucket in LDS, so that the
+// device-wide cursor of a bucket is moved once by each workgroup instead of once by each tile.
 __global__ __launch_bounds__(kBlock) void merge_order_kernel(uint32_t tiles, const uint32_t* __restrict__ tile_bucket,
                                                              const uint32_t* __restrict__ bucket_count,
                                                              uint32_t* __restrict__ bucket_cursor,
                                                              uint32_t* __restrict__ tile_order) {
     __shared__ uint32_t s_start[kOrderBuckets];
+    __shared__ uint32_t s_mine[kOrderBuckets];
     __shared__ uint32_t s_wave[kBlock / kWave];
+    s_mine[threadIdx.x] = 0;
     const unsigned lane = threadIdx.x % kWave;
     const unsigned wave = threadIdx.x / kWave;
     const uint32_t size = bucket_count[threadIdx.x];
@@ -229,13 +233,15 @@ __global__ __launch_bounds__(kBlock) void merge_order_kernel(uint32_t tiles, con
     __syncthreads();
     uint32_t before = 0;
     for (unsigned w = 0; w < wave; ++w) before += s_wave[w];
-    s_start[threadIdx.x] = before + inc - size;
-    __syncthreads();
     const uint32_t t = blockIdx.x * kBlock + threadIdx.x;
-    if (t < tiles) {
-        const uint32_t bucket = tile_bucket[t];
-        tile_order[s_start[bucket] + atomicAdd(&bucket_cursor[bucket], 1u)] = t;
-    }
+    const uint32_t bucket = t < tiles ? tile_bucket[t] : 0u;
+    uint32_t slot = 0;
+    if (t < tiles) slot = atomicAdd(&s_mine[bucket], 1u);
+    __syncthreads();
+    const uint32_t mine = s_mine[threadIdx.x];
+    s_start[threadIdx.x] = before + inc - size + (mine != 0 ? atomicAdd(&bucket_cursor[threadIdx.x], mine) : 0u);
+    __syncthreads();
+    if (t < tiles) tile_order[s_start[bucket] + slot] = t;
 }
 
 template <typename T, bool BETA0, int IPT>
@@ -429,8 +435,27 @@ __global__ __launch_bounds__(kBlock) void spmv_merge_fixup_kernel(idx_t m, uint3
     const idx_t r = carry_row[t];
     if (r >= m) return;
     if (t > 0 && carry_row[t - 1] == r) return;
+    // A long row leaves a run of hundreds of carries to one thread.  Read one at a time, each costs a
+    // trip to memory before the next is asked for; so they are read eight at a time from clamped
+    // positions and added in the same order as before.
+    constexpr uint32_t kAhead = 8;
     T sum = carry_val[t];
-    for (uint32_t u = t + 1; u < tiles && carry_row[u] == r; ++u) sum += carry_val[u];
+    bool open = true;
+    for (uint32_t u = t + 1; open && u < tiles; u += kAhead) {
+        idx_t rows[kAhead];
+        T vals[kAhead];
+#pragma unroll
+        for (uint32_t i = 0; i < kAhead; ++i) {
+            const uint32_t at = min(u + i, tiles - 1);
+            rows[i] = carry_row[at];
+            vals[i] = carry_val[at];
+        }
+#pragma unroll
+        for (uint32_t i = 0; i < kAhead; ++i) {
+            open = open && u + i < tiles && rows[i] == r;
+            if (open) sum += vals[i];
+        }
+    }
     if (sum != T(0)) y[r] += alpha * sum;
 }
 
