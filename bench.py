@@ -38,7 +38,7 @@ def _traffic(fetch_counts, write_counts):
 MEASURED_TRAFFIC_BYTES = {
     "c2": _traffic(653890.5, 10048.5),                      # spmv_vector_kernel<double, 16, 4>
     # merge kernel (tiles in column order) + partition + tile order + fix-up
-    "c3": _traffic(3305934.9 + 17231.3 + 251.4 + 3136.4, 25164.6 + 1391.2 + 4304.9 + 1375.1),
+    "c3": _traffic(3305285.9 + 17229.2 + 251.2 + 3154.3, 25157.0 + 1391.2 + 1994.3 + 1375.1),
     "c4-64": _traffic(613893.3, 524288.0),                 # spmm_group_kernel<float, 16>
     "c4-256": _traffic(3673719.8, 2097152.0),              # spmm_group_kernel<float, 64>
     # csr2csc: 2 x scatter + the scatter that reads the CSR arrays in place + 3 x (histogram + scans)
