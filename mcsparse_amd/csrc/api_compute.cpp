@@ -272,21 +272,23 @@ mcspStatus_t spmv_typed(mcsparseHandle_t h, mcsparseSpMatDescr* A, mcsparseOpera
         return MCSP_STATUS_SUCCESS;
     }
 
-    // Transposing call: materialise the transpose in the scratch buffer on every call, as the
-    // reference does (mcsp_spmv_gpu.cpp:797-845) -- the caller may have changed the values.
+    // Transposing call.  The reference materialises the transpose in the scratch buffer on every call
+    // (mcsp_spmv_gpu.cpp:797-845) -- the caller may have changed the values -- and then runs its row
+    // kernel on it.  Here every call sorts (column, value * x[row]) pairs by column with the machinery
+    // of csr2csc, which is a stable sort of one array less, and then sums the products of each column:
+    // the sum of a column adds the same products in the same order (row order) as a row kernel on the
+    // transpose would, without the gathers from x.
     idx_t* t_ptr = reinterpret_cast<idx_t*>(buf + l.col_ptr);
-    idx_t* t_ind = reinterpret_cast<idx_t*>(buf + l.row_ind);
     void* t_val = buf + l.vals;
-    mcsp::launch_csr2csc(h->stream, static_cast<idx_t>(v.m), static_cast<idx_t>(v.n), nnz, v.val, v.ptr, v.ind, t_val,
-                         t_ind, t_ptr, sizeof(T), base, buf + l.csr2csc_ws);
+    mcsp::launch_transposed_products(h->stream, static_cast<idx_t>(v.m), static_cast<idx_t>(v.n), nnz, v.val, v.ptr, v.ind,
+                                     x->values, t_val, t_ptr, sizeof(T), base, buf + l.csr2csc_ws);
     a.m = static_cast<idx_t>(v.n);
     a.n = static_cast<idx_t>(v.m);
     a.row_ptr = t_ptr;
-    a.col = t_ind;
+    a.col = nullptr;
     a.val = t_val;
-    // no analysis of the freshly built structure (it would need a read-back): merge-path is
-    // insensitive to the row-length distribution
-    mcsp::launch_spmv_merge<T>(h->stream, a, h_alpha, h_beta, buf + l.merge_ws, false);
+    a.x = nullptr;
+    mcsp::launch_row_sums_merge<T>(h->stream, a, h_alpha, h_beta, buf + l.merge_ws);
     return MCSP_STATUS_SUCCESS;
 }
 

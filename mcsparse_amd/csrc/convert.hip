@@ -387,12 +387,21 @@ struct ValueOf { typedef uint32_t type; };
 template <>
 struct ValueOf<8> { typedef uint64_t type; };
 
-template <int VB, bool FROM_CSR>
+// AUX = false: (key, value) pairs, rows_out is not written.  TIMES_X (with FROM_CSR, without AUX): the
+// value that travels is value * x[row of the nonzero], in the floating-point type of VB bytes.
+template <int VB>
+struct RealOf { typedef float type; };
+template <>
+struct RealOf<8> { typedef double type; };
+
+template <int VB, bool FROM_CSR, bool AUX, bool TIMES_X>
 __global__ __launch_bounds__(kSortBlock) void radix_scatter_kernel(
     const idx_t* __restrict__ keys_in, const idx_t* __restrict__ rows_in, const void* __restrict__ vals_in_v,
     idx_t* __restrict__ keys_out, idx_t* __restrict__ rows_out, void* __restrict__ vals_out_v, idx_t count,
     uint32_t shift, uint32_t bits, uint32_t tiles, const uint32_t* __restrict__ counters,
-    const idx_t* __restrict__ tile_rows, idx_t base) {
+    const idx_t* __restrict__ tile_rows, idx_t base, const void* __restrict__ x_v) {
+    static_assert(AUX || VB != 0, "pairs carry a value");
+    static_assert(!TIMES_X || (FROM_CSR && !AUX), "products are formed where the rows are worked out");
     typedef typename ValueOf<VB>::type val_t;
     const val_t* vals_in = static_cast<const val_t*>(vals_in_v);
     val_t* vals_out = static_cast<val_t*>(vals_out_v);
@@ -402,7 +411,7 @@ __global__ __launch_bounds__(kSortBlock) void radix_scatter_kernel(
     __shared__ uint32_t s_dest[kMaxRadix];             // global position of that slot
     __shared__ uint32_t s_wave[kSortWaves];
     __shared__ idx_t s_keys[kSortTile];
-    __shared__ idx_t s_rows[kSortTile];
+    __shared__ idx_t s_rows[(AUX || FROM_CSR) ? kSortTile : 1];
     __shared__ val_t s_vals[VB ? kSortTile : 1];
 
     const uint32_t tid = threadIdx.x;
@@ -451,7 +460,7 @@ __global__ __launch_bounds__(kSortBlock) void radix_scatter_kernel(
         const uint32_t p = wave * kSortWaveItems + i * kWave + lane;
         const bool live = p < tile_count;
         key[i] = live ? load_stream(keys_in + tile_start + p) : 0;
-        if constexpr (!FROM_CSR) row[i] = live ? load_stream(rows_in + tile_start + p) : 0;
+        if constexpr (!FROM_CSR && AUX) row[i] = live ? load_stream(rows_in + tile_start + p) : 0;
         if constexpr (VB != 0) val[i] = live ? load_stream(vals_in + tile_start + p) : val_t(0);
     }
     if constexpr (FROM_CSR) {
@@ -519,6 +528,20 @@ __global__ __launch_bounds__(kSortBlock) void radix_scatter_kernel(
             }
             row[i] = first_row + lo + base;
         }
+        if constexpr (TIMES_X) {
+            typedef typename RealOf<VB>::type real_t;
+            const real_t* x = static_cast<const real_t*>(x_v);
+            real_t xr[kSortIpt];
+#pragma unroll
+            for (int i = 0; i < kSortIpt; ++i) {
+                const uint32_t p = wave * kSortWaveItems + i * kWave + lane;
+                xr[i] = x[p < tile_count ? row[i] - base : first_row];  // first_row: a row of the matrix
+            }
+#pragma unroll
+            for (int i = 0; i < kSortIpt; ++i) {
+                val[i] = __builtin_bit_cast(val_t, __builtin_bit_cast(real_t, val[i]) * xr[i]);
+            }
+        }
     }
 
     // per digit: turn the wave counts into wave offsets, then lay the digits out in order
@@ -545,7 +568,7 @@ __global__ __launch_bounds__(kSortBlock) void radix_scatter_kernel(
             const uint32_t d = (key[i] >> shift) & mask;
             const uint32_t slot = s_start[d] + s_cnt[wave][d] + rank[i];
             s_keys[slot] = key[i];
-            s_rows[slot] = row[i];
+            if constexpr (AUX) s_rows[slot] = row[i];
             if constexpr (VB != 0) s_vals[slot] = val[i];
         }
     }
@@ -560,7 +583,7 @@ __global__ __launch_bounds__(kSortBlock) void radix_scatter_kernel(
             const uint32_t d = (k >> shift) & mask;
             const uint64_t out = static_cast<uint64_t>(s_dest[d]) + (slot - s_start[d]);
             keys_out[out] = k;
-            rows_out[out] = s_rows[slot];
+            if constexpr (AUX) rows_out[out] = s_rows[slot];
             if constexpr (VB != 0) vals_out[out] = s_vals[slot];
         }
     }
@@ -595,13 +618,31 @@ struct SortScratch {
 template <int VB>
 void launch_scatter(hipStream_t stream, bool from_csr, uint32_t grid, const idx_t* keys_in, const idx_t* aux_in,
                     const void* vals_in, idx_t* keys_out, idx_t* aux_out, void* vals_out, idx_t count, uint32_t shift,
-                    uint32_t bits, uint32_t tiles, const uint32_t* counters, const idx_t* tile_rows, idx_t base) {
+                    uint32_t bits, uint32_t tiles, const uint32_t* counters, const idx_t* tile_rows, idx_t base,
+                    bool pairs, const void* x) {
+    const void* none = nullptr;
+    if constexpr (VB != 0) {
+        if (pairs && from_csr) {
+            hipLaunchKernelGGL((radix_scatter_kernel<VB, true, false, true>), dim3(grid), dim3(kSortBlock), 0, stream, keys_in,
+                               aux_in, vals_in, keys_out, aux_out, vals_out, count, shift, bits, tiles, counters, tile_rows,
+                               base, x);
+            return;
+        }
+        if (pairs) {
+            hipLaunchKernelGGL((radix_scatter_kernel<VB, false, false, false>), dim3(grid), dim3(kSortBlock), 0, stream, keys_in,
+                               aux_in, vals_in, keys_out, aux_out, vals_out, count, shift, bits, tiles, counters, tile_rows,
+                               base, none);
+            return;
+        }
+    }
     if (from_csr) {
-        hipLaunchKernelGGL((radix_scatter_kernel<VB, true>), dim3(grid), dim3(kSortBlock), 0, stream, keys_in, aux_in,
-                           vals_in, keys_out, aux_out, vals_out, count, shift, bits, tiles, counters, tile_rows, base);
+        hipLaunchKernelGGL((radix_scatter_kernel<VB, true, true, false>), dim3(grid), dim3(kSortBlock), 0, stream, keys_in,
+                           aux_in, vals_in, keys_out, aux_out, vals_out, count, shift, bits, tiles, counters, tile_rows, base,
+                           none);
     } else {
-        hipLaunchKernelGGL((radix_scatter_kernel<VB, false>), dim3(grid), dim3(kSortBlock), 0, stream, keys_in, aux_in,
-                           vals_in, keys_out, aux_out, vals_out, count, shift, bits, tiles, counters, tile_rows, base);
+        hipLaunchKernelGGL((radix_scatter_kernel<VB, false, true, false>), dim3(grid), dim3(kSortBlock), 0, stream, keys_in,
+                           aux_in, vals_in, keys_out, aux_out, vals_out, count, shift, bits, tiles, counters, tile_rows, base,
+                           none);
     }
 }
 
@@ -610,6 +651,9 @@ struct CsrSource {
     idx_t rows = 0;  // > 0: aux_in is the row_ptr of a CSR matrix with this many rows, and the first
                      // pass derives the aux of every triple, its row + base, from it
     idx_t base = 0;  // index base of row_ptr
+    // != nullptr: no aux travels; the value of every triple is multiplied by x[its row] in the first
+    // pass (x in the floating-point type of the values), and (key, product) pairs are sorted
+    const void* times_x = nullptr;
 };
 
 // Stable LSD radix sort of (key, aux, value) triples on the low key_bits of the keys, in
@@ -640,7 +684,7 @@ void radix_sort_triples(hipStream_t stream, idx_t count, uint32_t key_bits, cons
         launch_exclusive_scan(stream, t.counters, static_cast<uint64_t>(radix) * tiles, t.scan_ws);
         auto* launch = value_bytes == 0 ? launch_scatter<0> : value_bytes == 4 ? launch_scatter<4> : launch_scatter<8>;
         launch(stream, from_csr, scatter_grid, keys_in, aux_in, vals_in, k_out, a_out, v_out, count, shift, bits, tiles,
-               t.counters, t.tile_rows, csr.base);
+               t.counters, t.tile_rows, csr.base, csr.times_x != nullptr, csr.times_x);
         keys_in = k_out;
         aux_in = a_out;
         vals_in = v_out;
@@ -778,6 +822,35 @@ void launch_csr2csc(hipStream_t stream, idx_t m, idx_t n, idx_t nnz, const void*
     csr.base = base;
     // keys are the raw column indices (index base included), so the largest key is n - 1 + base
     radix_sort_triples(stream, nnz, bit_length(n - 1 + base), col, row_ptr, csr_val, sorted_keys, row_ind, csc_val,
+                       value_bytes, t, csr);
+    launch_coo2csr(stream, nnz, n, sorted_keys, base, col_ptr);
+}
+
+// What a transposing SpMV needs of A^T: the products value * x[row] of all nonzeros in the order of a
+// stable sort by column, and the column offsets.  (column, product) pairs are sorted instead of
+// (column, row, value) triples, so the later passes move 8 or 12 bytes per nonzero instead of 12 or
+// 16, and the sums over the columns then need no gather from x.  workspace: csr2csc_workspace_bytes.
+void launch_transposed_products(hipStream_t stream, idx_t m, idx_t n, idx_t nnz, const void* csr_val, const idx_t* row_ptr,
+                                const idx_t* col, const void* x, void* products, idx_t* col_ptr, size_t value_bytes,
+                                idx_t base, void* workspace) {
+    if (m == 0 || n == 0 || nnz == 0) return;
+    const Csr2CscLayout l = csr2csc_layout(nnz, value_bytes);
+    char* w = static_cast<char*>(workspace);
+    idx_t* sorted_keys = reinterpret_cast<idx_t*>(w + l.sorted_keys);
+    SortScratch t;
+    t.keys[0] = reinterpret_cast<idx_t*>(w + l.keys_a);
+    t.keys[1] = reinterpret_cast<idx_t*>(w + l.keys_b);
+    t.aux[0] = t.aux[1] = nullptr;
+    t.vals[0] = w + l.vals_a;
+    t.vals[1] = w + l.vals_b;
+    t.counters = reinterpret_cast<uint32_t*>(w + l.counters);
+    t.scan_ws = reinterpret_cast<uint32_t*>(w + l.scan_ws);
+    t.tile_rows = reinterpret_cast<idx_t*>(w + l.tile_rows);
+    CsrSource csr;
+    csr.rows = m;
+    csr.base = base;
+    csr.times_x = x;
+    radix_sort_triples(stream, nnz, bit_length(n - 1 + base), col, row_ptr, csr_val, sorted_keys, nullptr, products,
                        value_bytes, t, csr);
     launch_coo2csr(stream, nnz, n, sorted_keys, base, col_ptr);
 }

@@ -194,8 +194,12 @@ template <typename T>
 void launch_spmv_vector(hipStream_t stream, const SpmvArgs& a, T alpha, T beta, int lanes);
 // workspace: spmv_merge_workspace_bytes(m, nnz, sizeof(T)) bytes of device scratch.
 size_t spmv_merge_workspace_bytes(idx_t m, idx_t nnz, size_t value_bytes);
+// order_tiles: the tiles run in the order of their first column.
 template <typename T>
 void launch_spmv_merge(hipStream_t stream, const SpmvArgs& a, T alpha, T beta, void* workspace, bool order_tiles);
+// The same sums over rows when a.val already holds the products value * x (a.col and a.x unused).
+template <typename T>
+void launch_row_sums_merge(hipStream_t stream, const SpmvArgs& a, T alpha, T beta, void* workspace);
 int spmv_pick_lanes(idx_t m, idx_t nnz);
 
 // ---- SpMM (spmm.hip) ----
@@ -249,6 +253,12 @@ size_t csr2csc_workspace_bytes(idx_t m, idx_t n, idx_t nnz, size_t value_bytes);
 void launch_csr2csc(hipStream_t stream, idx_t m, idx_t n, idx_t nnz, const void* csr_val, const idx_t* row_ptr,
                     const idx_t* col, void* csc_val, idx_t* row_ind, idx_t* col_ptr, size_t value_bytes,
                     idx_t base, void* workspace);
+// products[nnz] = value * x[row] of every nonzero in the order of a stable sort by column, and
+// col_ptr[n+1] (+ base): what op(A) = A^T needs of the transpose.  value_bytes is 4 (fp32 values and
+// x) or 8 (fp64); workspace as for launch_csr2csc.
+void launch_transposed_products(hipStream_t stream, idx_t m, idx_t n, idx_t nnz, const void* csr_val, const idx_t* row_ptr,
+                                const idx_t* col, const void* x, void* products, idx_t* col_ptr, size_t value_bytes,
+                                idx_t base, void* workspace);
 
 // ---- index sorts (convert.hip) --------------------------------------------------------------
 size_t index_sort_workspace_bytes(idx_t nnz);

@@ -244,7 +244,8 @@ __global__ __launch_bounds__(kBlock) void merge_order_kernel(uint32_t tiles, con
     if (t < tiles) tile_order[s_start[bucket] + slot] = t;
 }
 
-template <typename T, bool BETA0, int IPT>
+// PRODUCTS: val holds value * x already (col and x are not read); the kernel only sums the rows.
+template <typename T, bool BETA0, int IPT, bool PRODUCTS>
 __global__ __launch_bounds__(kBlock) void spmv_merge_kernel(idx_t m, idx_t nnz, idx_t base,
                                                             const idx_t* __restrict__ row_ptr,
                                                             const idx_t* __restrict__ col, const T* __restrict__ val,
@@ -285,8 +286,8 @@ __global__ __launch_bounds__(kBlock) void spmv_merge_kernel(idx_t m, idx_t nnz, 
         ends[i] = row_ptr[r + 1];
     }
     const idx_t last_item = tile_nnz != 0 ? tile_nnz - 1 : 0;
-    const idx_t* tile_col = tile_nnz != 0 ? col + y0 : row_ptr;  // a tile of row ends only reads a valid word
-    const T* tile_val = tile_nnz != 0 ? val + y0 : x;
+    const idx_t* tile_col = tile_nnz != 0 && !PRODUCTS ? col + y0 : row_ptr;  // a tile of row ends only reads a valid word
+    const T* tile_val = tile_nnz != 0 ? val + y0 : (PRODUCTS ? val : x);
 #pragma unroll
     for (int i = 0; i <= kItemsPerThread; ++i) {
         const idx_t k = tid + static_cast<idx_t>(i) * kBlock;
@@ -300,13 +301,14 @@ __global__ __launch_bounds__(kBlock) void spmv_merge_kernel(idx_t m, idx_t nnz, 
 #pragma unroll
         for (int i = 0; i < kGatherBatch; ++i) {
             const idx_t k = min(tid + static_cast<idx_t>(i0 + i) * kBlock, last_item);
-            c[i] = load_stream(tile_col + k);
+            if constexpr (!PRODUCTS) c[i] = load_stream(tile_col + k);
             v[i] = load_stream(tile_val + k);
         }
 #pragma unroll
         for (int i = 0; i < kGatherBatch; ++i) {
             const idx_t k = tid + static_cast<idx_t>(i0 + i) * kBlock;
-            xv[i] = x[k < tile_nnz ? c[i] - base : 0];
+            if constexpr (PRODUCTS) xv[i] = T(1);
+            else xv[i] = x[k < tile_nnz ? c[i] - base : 0];
         }
         // every gather of the batch is asked for before the first one is needed
 #pragma unroll
@@ -314,7 +316,7 @@ __global__ __launch_bounds__(kBlock) void spmv_merge_kernel(idx_t m, idx_t nnz, 
 #pragma unroll
         for (int i = 0; i < kGatherBatch; ++i) {
             const idx_t k = tid + static_cast<idx_t>(i0 + i) * kBlock;
-            if (k < tile_nnz) s_data[k] = v[i] * xv[i];
+            if (k < tile_nnz) s_data[k] = PRODUCTS ? v[i] : v[i] * xv[i];
         }
     }
     __syncthreads();
@@ -500,7 +502,7 @@ size_t spmv_merge_workspace_bytes(idx_t m, idx_t nnz, size_t value_bytes) {
            2 * align_up(tiles * sizeof(uint32_t)) + align_up(2 * kOrderBuckets * sizeof(uint32_t));
 }
 
-template <typename T, int IPT>
+template <typename T, int IPT, bool PRODUCTS = false>
 void launch_spmv_merge_tiles(hipStream_t stream, const SpmvArgs& a, T alpha, T beta, void* workspace, bool order_tiles) {
     const uint32_t tiles = merge_tiles(a.m, a.nnz, IPT);
     char* w = static_cast<char*>(workspace);
@@ -538,11 +540,11 @@ void launch_spmv_merge_tiles(hipStream_t stream, const SpmvArgs& a, T alpha, T b
         tile_order = nullptr;
     }
     if (beta == T(0)) {
-        hipLaunchKernelGGL((spmv_merge_kernel<T, true, IPT>), dim3(tiles), dim3(kBlock), 0, stream, a.m, a.nnz, a.base,
+        hipLaunchKernelGGL((spmv_merge_kernel<T, true, IPT, PRODUCTS>), dim3(tiles), dim3(kBlock), 0, stream, a.m, a.nnz, a.base,
                            a.row_ptr, a.col, val, x, y, alpha, beta, tile_row, carry_row, carry_val,
                            static_cast<const uint32_t*>(tile_order));
     } else {
-        hipLaunchKernelGGL((spmv_merge_kernel<T, false, IPT>), dim3(tiles), dim3(kBlock), 0, stream, a.m, a.nnz, a.base,
+        hipLaunchKernelGGL((spmv_merge_kernel<T, false, IPT, PRODUCTS>), dim3(tiles), dim3(kBlock), 0, stream, a.m, a.nnz, a.base,
                            a.row_ptr, a.col, val, x, y, alpha, beta, tile_row, carry_row, carry_val,
                            static_cast<const uint32_t*>(tile_order));
     }
@@ -557,6 +559,14 @@ void launch_spmv_merge(hipStream_t stream, const SpmvArgs& a, T alpha, T beta, v
     else launch_spmv_merge_tiles<T, kItemsInOrder>(stream, a, alpha, beta, workspace, false);
 }
 
+template <typename T>
+void launch_row_sums_merge(hipStream_t stream, const SpmvArgs& a, T alpha, T beta, void* workspace) {
+    if (a.m == 0) return;
+    launch_spmv_merge_tiles<T, kItemsInOrder, true>(stream, a, alpha, beta, workspace, false);
+}
+
+template void launch_row_sums_merge<float>(hipStream_t, const SpmvArgs&, float, float, void*);
+template void launch_row_sums_merge<double>(hipStream_t, const SpmvArgs&, double, double, void*);
 template void launch_spmv_vector<float>(hipStream_t, const SpmvArgs&, float, float, int);
 template void launch_spmv_vector<double>(hipStream_t, const SpmvArgs&, double, double, int);
 template void launch_spmv_merge<float>(hipStream_t, const SpmvArgs&, float, float, void*, bool);
