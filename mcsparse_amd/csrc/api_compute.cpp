@@ -71,11 +71,11 @@ bool format_is_built(mcsparseFormat_t f) {
 
 // Scratch layout of an SpMV call, all parts aligned to 128 bytes:
 //   [analysis][merge workspace][COO only: row offsets m+1]
-//   transposing calls add [col_ptr n+1 | row_ind nnz][values][csr2csc workspace]
+//   transposing calls add [col_ptr n+1][products nnz][workspace of the sort by column]
 //   64-bit index arrays add their narrowed copies at the end
-// (the transposed part is the reference's layout, mcsp_spmv_gpu.cpp:308 and :813-831).
+// (the reference keeps the whole transpose there, mcsp_spmv_gpu.cpp:308 and :813-831).
 struct SpmvLayout {
-    size_t merge_ws, coo_ptr, col_ptr, row_ind, vals, csr2csc_ws, narrow, total;
+    size_t merge_ws, coo_ptr, col_ptr, vals, csr2csc_ws, narrow, total;
 };
 
 SpmvLayout spmv_layout(const CsrView& v, int64_t nnz, size_t value_bytes, size_t narrow) {
@@ -89,13 +89,11 @@ SpmvLayout spmv_layout(const CsrView& v, int64_t nnz, size_t value_bytes, size_t
     if (v.coo_rows != nullptr) off += align_up(static_cast<size_t>(v.m + 1) * sizeof(idx_t));
     if (v.transpose) {
         l.col_ptr = off;
-        l.row_ind = off + static_cast<size_t>(v.n + 1) * sizeof(idx_t);
-        off += align_up(static_cast<size_t>(v.n + 1 + nnz) * sizeof(idx_t));
+        off += align_up(static_cast<size_t>(v.n + 1) * sizeof(idx_t));
         l.vals = off;
         off += align_up(static_cast<size_t>(nnz) * value_bytes);
         l.csr2csc_ws = off;
-        off += align_up(mcsp::csr2csc_workspace_bytes(static_cast<idx_t>(v.m), static_cast<idx_t>(v.n),
-                                                      static_cast<idx_t>(nnz), value_bytes));
+        off += align_up(mcsp::transposed_products_workspace_bytes(static_cast<idx_t>(nnz), value_bytes));
     }
     l.narrow = off;
     off += narrow;

@@ -696,18 +696,20 @@ struct Csr2CscLayout {
     size_t sorted_keys, keys_a, rows_a, vals_a, keys_b, rows_b, vals_b, counters, scan_ws, tile_rows, total;
 };
 
-Csr2CscLayout csr2csc_layout(idx_t nnz, size_t value_bytes) {
+// pairs: no row arrays (the sort of a transposing SpMV, which carries no rows)
+Csr2CscLayout csr2csc_layout(idx_t nnz, size_t value_bytes, bool pairs = false) {
     Csr2CscLayout l;
     const size_t idx_bytes = align_up(static_cast<size_t>(nnz) * sizeof(idx_t));
+    const size_t row_bytes = pairs ? 0 : idx_bytes;
     const size_t val_bytes = align_up(static_cast<size_t>(nnz) * value_bytes);
     const size_t counter_elems = sort_counter_elems(nnz);
     size_t off = 0;
     l.sorted_keys = off; off += idx_bytes;
     l.keys_a = off; off += idx_bytes;
-    l.rows_a = off; off += idx_bytes;
+    l.rows_a = off; off += row_bytes;
     l.vals_a = off; off += val_bytes;
     l.keys_b = off; off += idx_bytes;
-    l.rows_b = off; off += idx_bytes;
+    l.rows_b = off; off += row_bytes;
     l.vals_b = off; off += val_bytes;
     l.counters = off; off += align_up(counter_elems * sizeof(uint32_t));
     l.scan_ws = off; off += align_up(scan_workspace_elems(counter_elems) * sizeof(uint32_t)) + kAlign;
@@ -798,6 +800,10 @@ size_t csr2csc_workspace_bytes(idx_t /*m*/, idx_t /*n*/, idx_t nnz, size_t value
     return csr2csc_layout(nnz, value_bytes).total;
 }
 
+size_t transposed_products_workspace_bytes(idx_t nnz, size_t value_bytes) {
+    return csr2csc_layout(nnz, value_bytes, true).total;
+}
+
 // The nonzeros are sorted by column where they lie: the first pass reads col / val in place and
 // works the row indices out of row_ptr; the sorted columns then give the offsets.
 void launch_csr2csc(hipStream_t stream, idx_t m, idx_t n, idx_t nnz, const void* csr_val, const idx_t* row_ptr,
@@ -829,12 +835,13 @@ void launch_csr2csc(hipStream_t stream, idx_t m, idx_t n, idx_t nnz, const void*
 // What a transposing SpMV needs of A^T: the products value * x[row] of all nonzeros in the order of a
 // stable sort by column, and the column offsets.  (column, product) pairs are sorted instead of
 // (column, row, value) triples, so the later passes move 8 or 12 bytes per nonzero instead of 12 or
-// 16, and the sums over the columns then need no gather from x.  workspace: csr2csc_workspace_bytes.
+// 16, and the sums over the columns then need no gather from x.
+// workspace: transposed_products_workspace_bytes.
 void launch_transposed_products(hipStream_t stream, idx_t m, idx_t n, idx_t nnz, const void* csr_val, const idx_t* row_ptr,
                                 const idx_t* col, const void* x, void* products, idx_t* col_ptr, size_t value_bytes,
                                 idx_t base, void* workspace) {
     if (m == 0 || n == 0 || nnz == 0) return;
-    const Csr2CscLayout l = csr2csc_layout(nnz, value_bytes);
+    const Csr2CscLayout l = csr2csc_layout(nnz, value_bytes, true);
     char* w = static_cast<char*>(workspace);
     idx_t* sorted_keys = reinterpret_cast<idx_t*>(w + l.sorted_keys);
     SortScratch t;

@@ -255,7 +255,8 @@ void launch_csr2csc(hipStream_t stream, idx_t m, idx_t n, idx_t nnz, const void*
                     idx_t base, void* workspace);
 // products[nnz] = value * x[row] of every nonzero in the order of a stable sort by column, and
 // col_ptr[n+1] (+ base): what op(A) = A^T needs of the transpose.  value_bytes is 4 (fp32 values and
-// x) or 8 (fp64); workspace as for launch_csr2csc.
+// x) or 8 (fp64); workspace of transposed_products_workspace_bytes(nnz, value_bytes) bytes.
+size_t transposed_products_workspace_bytes(idx_t nnz, size_t value_bytes);
 void launch_transposed_products(hipStream_t stream, idx_t m, idx_t n, idx_t nnz, const void* csr_val, const idx_t* row_ptr,
                                 const idx_t* col, const void* x, void* products, idx_t* col_ptr, size_t value_bytes,
                                 idx_t base, void* workspace);
