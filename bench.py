@@ -370,7 +370,7 @@ def cpu_baseline(kind, a, alpha, beta, n_cols, algo_bytes, op):
             oracle.spmv_omp(a.m, a.base, a.ptr, a.col, a.val, alpha, beta, x, y, dynamic=dyn)
         sample = "whole workload per repetition"
     elif kind == "spmv":
-        # op T as the library and the reference do it: transpose on every call, then the row loop
+        # op T as the reference does it: transpose on every call, then the row loop
         x = rng.uniform(-1, 1, a.m).astype(dt)
         y = rng.uniform(-1, 1, a.n).astype(dt)
 
