@@ -193,7 +193,11 @@ __global__ __launch_bounds__(kBlock) void spmm_rowb_kernel(idx_t m, idx_t n, idx
 // C = 1 or 2 lanes, and what a row of A costs is the chain of dependent loads (offsets,
 // nonzeros, rows of op(B)) rather than bytes.  So 16 lanes share a row of A as P = 16 / C
 // phases x C column lanes: phase p takes the nonzeros p, p + P, ... of the row, kSteps of them in
-// flight at once, and the P partial sums are added up across the lanes at the end.
+// flight at once, and the P partial sums are added up across the lanes at the end.  A lane group
+// works through kNarrowRowsPerGroup rows one after the other and asks for the offsets of the row
+// after next and the nonzeros of the next row while the rows of op(B) of the current one are on
+// their way, so that a row costs one trip to memory instead of three.
+constexpr int kNarrowRowsPerGroup = 8;
 template <typename T, int V, int C>
 __global__ __launch_bounds__(kBlock) void spmm_narrow_kernel(idx_t m, idx_t n, idx_t nnz, idx_t base,
                                                              const idx_t* __restrict__ row_ptr,
@@ -204,95 +208,131 @@ __global__ __launch_bounds__(kBlock) void spmm_narrow_kernel(idx_t m, idx_t n, i
     constexpr int kLanes = 16;
     constexpr int P = kLanes / C;
     constexpr int kSteps = 4;  // measured on a 27-point stencil, n = 8: 1, 2, 4, 8 steps -> 305, 280, 260, 291 us
-    constexpr int kRows = 1;   // more rows per lane group in flight only cost registers (2 -> 352 us)
     constexpr int kGroups = kBlock / kLanes;
     const idx_t sub = threadIdx.x % kLanes;
     const idx_t phase = sub / C;
     const uint64_t c_own = static_cast<uint64_t>(sub % C) * V;
     const bool in_panel = c_own < n;
     const uint64_t c0 = in_panel ? c_own : 0;
-    const uint64_t first_row = (static_cast<uint64_t>(blockIdx.x) * kGroups + threadIdx.x / kLanes) * kRows;
+    // the groups of a workgroup take neighbouring rows in every round
+    const uint64_t first_row = static_cast<uint64_t>(blockIdx.x) * (kGroups * kNarrowRowsPerGroup) + threadIdx.x / kLanes;
+    const uint64_t last_row = static_cast<uint64_t>(m) - 1;  // m != 0 here
 
-    idx_t at[kRows], end[kRows];
-    T acc[kRows][V];
+    if (nnz == 0) {  // nothing to read, only C to scale
+        T zero[V];
 #pragma unroll
-    for (int w = 0; w < kRows; ++w) {
-        const uint64_t row = first_row + w;
-        at[w] = end[w] = 0;
-        if (row < m) {
-            at[w] = row_ptr[row] - base + phase;
-            end[w] = row_ptr[row + 1] - base;
+        for (int i = 0; i < V; ++i) zero[i] = T(0);
+        for (int it = 0; it < kNarrowRowsPerGroup; ++it) {
+            const uint64_t row = first_row + static_cast<uint64_t>(it) * kGroups;
+            if (row < m && phase == 0 && in_panel) store_c<T, V>(Cm, ldc, c_row_major, row, c0, zero, alpha, beta);
         }
-#pragma unroll
-        for (int i = 0; i < V; ++i) acc[w][i] = T(0);
+        return;
     }
-    // Loads that sit under a test of their own are waited for one by one; so the nonzeros of all
-    // steps are read without one, from an index clamped to the last nonzero of the matrix, and
-    // whether a step really has a nonzero is only asked where its product would be added.
+    // Loads that sit under a test of their own are waited for one by one; so offsets are read from a
+    // row clamped to the last one and nonzeros from an index clamped to the last nonzero, and whether
+    // a row or a nonzero is really there is only asked where its product would be added.
     const idx_t last_nonzero = nnz - 1;
-    bool more = nnz != 0;  // without nonzeros there is nothing to read, only C to scale
-    while (more) {
-        idx_t cc[kRows][kSteps];
-        T aa[kRows][kSteps];
+    auto range_of = [&](uint64_t row, idx_t& at, idx_t& end) {
+        const uint64_t r = row < last_row ? row : last_row;
+        const idx_t b = row_ptr[r] - base;
+        const idx_t e = row_ptr[r + 1] - base;
+        at = b + phase;
+        end = row < m ? e : b;  // a row past the end is empty
+    };
+    idx_t at, end, at_next, end_next;
+    range_of(first_row, at, end);
+    range_of(first_row + kGroups, at_next, end_next);
+    idx_t cc[kSteps];
+    T aa[kSteps];
 #pragma unroll
-        for (int w = 0; w < kRows; ++w) {
+    for (int u = 0; u < kSteps; ++u) {
+        const idx_t j = min(at + u * P, last_nonzero);
+        cc[u] = col[j];
+        aa[u] = val[j];
+    }
+    for (int it = 0; it < kNarrowRowsPerGroup; ++it) {
+        const uint64_t row = first_row + static_cast<uint64_t>(it) * kGroups;
+        if (__all(row >= m)) break;  // the same for all lanes of the wavefront from here on
+        T acc[V];
 #pragma unroll
-            for (int u = 0; u < kSteps; ++u) {
-                const idx_t j = min(at[w] + u * P, last_nonzero);
-                cc[w][u] = col[j];
-                aa[w][u] = val[j];
+        for (int i = 0; i < V; ++i) acc[i] = T(0);
+        Vec<T, V> b[kSteps];
+#pragma unroll
+        for (int u = 0; u < kSteps; ++u) b[u] = load_vec<T, V>(B + static_cast<int64_t>(cc[u] - base) * ldb + c0);
+        // the next row's nonzeros and the offsets of the row after it, while those are on their way
+        idx_t cc_next[kSteps];
+        T aa_next[kSteps];
+#pragma unroll
+        for (int u = 0; u < kSteps; ++u) {
+            const idx_t j = min(at_next + u * P, last_nonzero);
+            cc_next[u] = col[j];
+            aa_next[u] = val[j];
+        }
+        idx_t at_after, end_after;
+        range_of(row + 2 * kGroups, at_after, end_after);
+#pragma unroll
+        for (int u = 0; u < kSteps; ++u) {
+            if (at + u * P < end) {  // a lane without a nonzero stays out: 0 * inf would be NaN
+#pragma unroll
+                for (int i = 0; i < V; ++i) acc[i] += aa[u] * b[u].v[i];
             }
         }
-        Vec<T, V> b[kRows][kSteps];
-#pragma unroll
-        for (int w = 0; w < kRows; ++w) {
+        // a row with more than kSteps * P nonzeros: the rest, kSteps * P at a time
+        at += kSteps * P;
+        while (__any(at < end)) {
+            idx_t c2[kSteps];
+            T a2[kSteps];
 #pragma unroll
             for (int u = 0; u < kSteps; ++u) {
-                b[w][u] = load_vec<T, V>(B + static_cast<int64_t>(cc[w][u] - base) * ldb + c0);
+                const idx_t j = min(at + u * P, last_nonzero);
+                c2[u] = col[j];
+                a2[u] = val[j];
             }
-        }
-        more = false;
+            Vec<T, V> b2[kSteps];
 #pragma unroll
-        for (int w = 0; w < kRows; ++w) {
+            for (int u = 0; u < kSteps; ++u) b2[u] = load_vec<T, V>(B + static_cast<int64_t>(c2[u] - base) * ldb + c0);
 #pragma unroll
             for (int u = 0; u < kSteps; ++u) {
-                if (at[w] + u * P < end[w]) {  // a lane without a nonzero stays out: 0 * inf would be NaN
+                if (at + u * P < end) {
 #pragma unroll
-                    for (int i = 0; i < V; ++i) acc[w][i] += aa[w][u] * b[w][u].v[i];
+                    for (int i = 0; i < V; ++i) acc[i] += a2[u] * b2[u].v[i];
                 }
             }
-            at[w] += kSteps * P;
-            more |= at[w] < end[w];
+            at += kSteps * P;
         }
-        more = __any(more);  // the sums below need every lane of the wavefront
-    }
-#pragma unroll
-    for (int w = 0; w < kRows; ++w) {
         // sum over the nonzero phases: the lanes of a 16-lane DPP row that serve the same columns
 #pragma unroll
         for (int i = 0; i < V; ++i) {
             if constexpr (C == 1) {
-                acc[w][i] = group_sum<kLanes>(acc[w][i]);
+                acc[i] = group_sum<kLanes>(acc[i]);
             } else {
                 static_assert(C == 2, "column lanes per row");
                 constexpr int kQuadXor2 = 0x4E, kRowRor4 = 0x124, kRowRor8 = 0x128;  // lanes 2, 4 and 8 away
-                acc[w][i] += dpp_mov<kQuadXor2>(acc[w][i]);
-                acc[w][i] += dpp_mov<kRowRor4>(acc[w][i]);
-                acc[w][i] += dpp_mov<kRowRor8>(acc[w][i]);
+                acc[i] += dpp_mov<kQuadXor2>(acc[i]);
+                acc[i] += dpp_mov<kRowRor4>(acc[i]);
+                acc[i] += dpp_mov<kRowRor8>(acc[i]);
             }
         }
-        const uint64_t row = first_row + w;
-        if (row < m && phase == 0 && in_panel) store_c<T, V>(Cm, ldc, c_row_major, row, c0, acc[w], alpha, beta);
+        if (row < m && phase == 0 && in_panel) store_c<T, V>(Cm, ldc, c_row_major, row, c0, acc, alpha, beta);
+        at = at_next;
+        end = end_next;
+        at_next = at_after;
+        end_next = end_after;
+#pragma unroll
+        for (int u = 0; u < kSteps; ++u) {
+            cc[u] = cc_next[u];
+            aa[u] = aa_next[u];
+        }
     }
 }
 
 template <typename T, int V, int C>
 void launch_narrow(hipStream_t stream, const SpmmArgs& a, T alpha, T beta) {
-    constexpr int kRowsPerBlock = kBlock / 16;
+    constexpr int kRowsPerBlock = kBlock / 16 * kNarrowRowsPerGroup;
     const uint64_t blocks = (static_cast<uint64_t>(a.m) + kRowsPerBlock - 1) / kRowsPerBlock;
     hipLaunchKernelGGL((spmm_narrow_kernel<T, V, C>), dim3(static_cast<uint32_t>(blocks)), dim3(kBlock), 0, stream, a.m,
-                       a.n, a.nnz, a.base, a.row_ptr, a.col, static_cast<const T*>(a.val), static_cast<const T*>(a.B), a.ldb,
-                       static_cast<T*>(a.C), a.ldc, a.c_row_major, alpha, beta);
+                       a.n, a.nnz, a.base, a.row_ptr, a.col, static_cast<const T*>(a.val),
+                       static_cast<const T*>(a.B), a.ldb, static_cast<T*>(a.C), a.ldc, a.c_row_major, alpha, beta);
 }
 
 // op(B) column-major: element (kk, j) at j*ldb + kk.  One wavefront per row of A, lanes strided
