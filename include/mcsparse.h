@@ -20,6 +20,11 @@
 extern "C" {
 #endif
 
+/* The library is built with hidden visibility; what this header declares is its exported surface. */
+#if defined(__GNUC__)
+#pragma GCC visibility push(default)
+#endif
+
 /* HIP stream handle.  Re-declaring the typedef is legal when <hip/hip_runtime_api.h>
  * is also included; mcStream_t is kept as the name the reference's users spell. */
 struct ihipStream_t;
@@ -427,6 +432,41 @@ mcsparseStatus_t mcsparseSpMatSetSpMVPlan(mcsparseSpMatDescr_t spMatDescr, int f
  * (SpMM ignores it), 2 = SpMM uses it when called with the same buffer and CSR arrays.
  * merged_entries = total length of the merged column lists of all row groups (compare with nnz). */
 mcsparseStatus_t mcsparseSpMatGetSpMMSchedule(mcsparseSpMatDescr_t spMatDescr, int* state, int64_t* merged_entries);
+
+/* Optional preparation of y = alpha*A*x + beta*y for a CSR matrix that is multiplied many times (the
+ * reference has no such step: include/interface/mcsp_generic.h:43-51).  It copies A into externalBuffer
+ * in a column-banded layout in which the reads of x hit in cache; mcsparseSpMV then uses that copy
+ * whenever it is called with the same externalBuffer, the same three CSR arrays and extents, op N.
+ *   - externalBuffer needs mcsparseSpMV_preprocess_bufferSize bytes (about twice the matrix), is
+ *     passed to both calls, and must be left alone in between, like the structure of A.
+ *   - The copy includes the values.  After changing values in place call mcsparseSpMV_preprocess
+ *     again; mcsparseSpMatSetValues and mcsparseCsrSetPointers drop the copy.
+ *   - Matrices the layout cannot help (x fits in cache as it is, rows longer than a few hundred
+ *     nonzeros, formats other than 32-bit CSR) are left to the ordinary kernels; the call still
+ *     returns SUCCESS.  mcsparseSpMatGetSpMVPreprocess tells which case applies.
+ *   - Results stay within the same bound as mcsparseSpMV's and are bit-reproducible from run to run.
+ * The call blocks the host until the copy is built. */
+mcsparseStatus_t mcsparseSpMV_preprocess_bufferSize(mcsparseHandle_t handle, mcsparseOperation_t opA,
+                                                    const void* alpha, mcsparseSpMatDescr_t matA,
+                                                    mcsparseDnVecDescr_t vecX, const void* beta,
+                                                    mcsparseDnVecDescr_t vecY, macaDataType computeType,
+                                                    mcsparseSpMVAlg_t alg, size_t* bufferSize);
+mcsparseStatus_t mcsparseSpMV_preprocess(mcsparseHandle_t handle, mcsparseOperation_t opA, const void* alpha,
+                                         mcsparseSpMatDescr_t matA, mcsparseDnVecDescr_t vecX, const void* beta,
+                                         mcsparseDnVecDescr_t vecY, macaDataType computeType, mcsparseSpMVAlg_t alg,
+                                         void* externalBuffer);
+/* state 0 = not preprocessed, 1 = preprocessed and left to the ordinary kernels, 2 = banded copy in
+ * use; bands and rows_per_tile describe the copy (0 unless state is 2). */
+mcsparseStatus_t mcsparseSpMatGetSpMVPreprocess(mcsparseSpMatDescr_t spMatDescr, int* state, int* bands,
+                                                int* rows_per_tile);
+
+/* Width, in bytes of x, of the column bands mcsparseSpMV_preprocess cuts (0 = the default, 2 MiB;
+ * rounded down to a power of two).  Drops a banded copy already built.  For tests and benchmarks. */
+mcsparseStatus_t mcsparseSpMatSetSpMVBandBytes(mcsparseSpMatDescr_t spMatDescr, size_t band_bytes);
+
+#if defined(__GNUC__)
+#pragma GCC visibility pop
+#endif
 
 #ifdef __cplusplus
 }

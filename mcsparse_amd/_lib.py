@@ -56,6 +56,10 @@ PROTOTYPES = {
     "mcsparseDnMatSetStridedBatch": (c_int, [vp, c_int, c_i64]),
     "mcsparseDnMatGetStridedBatch": (c_int, [vp, P(c_int), P(c_i64)]),
     "mcsparseSpMV": (c_int, [vp, c_int, vp, vp, vp, vp, vp, c_int, c_int, vp]),
+    "mcsparseSpMV_preprocess_bufferSize": (c_int, [vp, c_int, vp, vp, vp, vp, vp, c_int, c_int, P(c_size)]),
+    "mcsparseSpMV_preprocess": (c_int, [vp, c_int, vp, vp, vp, vp, vp, c_int, c_int, vp]),
+    "mcsparseSpMatSetSpMVBandBytes": (c_int, [vp, c_size]),
+    "mcsparseSpMatGetSpMVPreprocess": (c_int, [vp, P(c_int), P(c_int), P(c_int)]),
     "mcsparseSpMV_bufferSize": (c_int, [vp, c_int, vp, vp, vp, vp, vp, c_int, c_int, P(c_size)]),
     "mcsparseSpMM_bufferSize": (c_int, [vp, c_int, c_int, vp, vp, vp, vp, vp, c_int, c_int, P(c_size)]),
     "mcsparseSpMM_preprocess": (c_int, [vp, c_int, c_int, vp, vp, vp, vp, vp, c_int, c_int, vp]),

@@ -17,6 +17,7 @@ STATUS_ALLOC_FAILED = 2
 STATUS_INVALID_VALUE = 3
 STATUS_INTERNAL_ERROR = 7
 STATUS_NOT_SUPPORTED = 10
+STATUS_INSUFFICIENT_RESOURCES = 11
 
 OP_N, OP_T, OP_C = 0, 1, 2
 BASE_ZERO, BASE_ONE = 0, 1
@@ -133,6 +134,16 @@ class SpMat:
         check(self.lib.mcsparseSpMatGetSpMVPlan(self._d, ctypes.byref(fam), ctypes.byref(lanes)))
         return fam.value, lanes.value
 
+    def set_band_bytes(self, band_bytes):
+        check(self.lib.mcsparseSpMatSetSpMVBandBytes(self._d, band_bytes), "mcsparseSpMatSetSpMVBandBytes")
+
+    def spmv_preprocess_state(self):
+        """(state, bands, rows_per_tile) left by mcsparseSpMV_preprocess; state 2 = banded copy in use."""
+        state, bands, rows = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
+        check(self.lib.mcsparseSpMatGetSpMVPreprocess(self._d, ctypes.byref(state), ctypes.byref(bands),
+                                                      ctypes.byref(rows)))
+        return state.value, bands.value, rows.value
+
     def spmm_schedule(self):
         """(state, merged_entries) left by mcsparseSpMM_preprocess; state 2 = in use."""
         state, entries = ctypes.c_int(), ctypes.c_int64()
@@ -224,6 +235,21 @@ def spmv(handle, op, alpha, mat, x, beta, y, compute_type, buffer):
                                  _ptr(buffer))
     del keep
     return st
+
+
+def spmv_preprocess_buffer_size(handle, op, alpha, mat, x, beta, y, compute_type):
+    size = ctypes.c_size_t(0)
+    a, b = _scalar(alpha, compute_type), _scalar(beta, compute_type)
+    st = handle.lib.mcsparseSpMV_preprocess_bufferSize(handle.ptr, op, ctypes.addressof(a), mat.ptr, x.ptr,
+                                                       ctypes.addressof(b), y.ptr, compute_type, SPMV_ALG_DEFAULT,
+                                                       ctypes.byref(size))
+    return st, size.value
+
+
+def spmv_preprocess(handle, op, alpha, mat, x, beta, y, compute_type, buffer):
+    a, b = _scalar(alpha, compute_type), _scalar(beta, compute_type)
+    return handle.lib.mcsparseSpMV_preprocess(handle.ptr, op, ctypes.addressof(a), mat.ptr, x.ptr, ctypes.addressof(b),
+                                              y.ptr, compute_type, SPMV_ALG_DEFAULT, _ptr(buffer))
 
 
 def spmm_buffer_size(handle, op_a, op_b, alpha, mat, B, beta, C, compute_type):

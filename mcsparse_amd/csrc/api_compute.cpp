@@ -181,10 +181,18 @@ IndexArrays index_arrays(mcsparseHandle_t h, const mcsparseSpMatDescr* A, char* 
 // blocking 136-byte read-back) the first time a structure is seen.  `ptr` are the offsets to
 // analyse, `signature` the caller's array that identifies the structure.
 mcspStatus_t ensure_plan(mcsparseHandle_t h, mcsparseSpMatDescr* A, const idx_t* ptr, const void* signature,
-                         int64_t m, int64_t nnz, int64_t x_bytes, void* buffer) {
+                         int64_t m, int64_t nnz, int64_t x_bytes, void* buffer, bool may_read_back) {
     SpmvPlan& p = A->plan;
     if (p.valid && p.rows == signature && p.m == m && p.nnz == nnz && p.base == static_cast<int>(A->idxBase))
         return MCSP_STATUS_SUCCESS;
+    if (!may_read_back && p.forced_family == kFamilyAuto) {
+        // No analysis without its read-back: the merge family in storage order is correct and balanced
+        // for every structure.  The plan stays invalid, so a later call that may read back analyses.
+        p.valid = false;
+        p.family = kFamilyMerge;
+        p.lanes = 0;
+        return MCSP_STATUS_SUCCESS;
+    }
     p.rows = signature;
     p.m = m;
     p.nnz = nnz;
@@ -223,9 +231,34 @@ mcspStatus_t ensure_plan(mcsparseHandle_t h, mcsparseSpMatDescr* A, const idx_t*
     return MCSP_STATUS_SUCCESS;
 }
 
+// Where the banded copy of mcsparseSpMV_preprocess sits in its buffer: behind the scratch of a plain
+// SpMV call, which mcsparseSpMV may still write (row-length analysis) when handed the same buffer.
+size_t banded_region_offset(const mcsparseSpMatDescr* A, size_t value_bytes) {
+    const CsrView v = make_view(A, MCSPARSE_OPERATION_NON_TRANSPOSE);
+    return align_up(spmv_layout(v, A->nnz, value_bytes, narrow_bytes(A)).total);
+}
+
+// CSR, 32-bit indices, fp32 / fp64: what mcsparseSpMV_preprocess builds a banded copy for.
+bool banded_candidate(const mcsparseSpMatDescr* A, mcsparseOperation_t op, BandedShape* shape) {
+    if (A->format != MCSPARSE_FORMAT_CSR || op != MCSPARSE_OPERATION_NON_TRANSPOSE || wide_indices(A)) return false;
+    if (A->valueType != MACA_R_32F && A->valueType != MACA_R_64F) return false;
+    return mcsp::banded_shape(static_cast<idx_t>(A->row_num), static_cast<idx_t>(A->col_num), static_cast<idx_t>(A->nnz),
+                              static_cast<idx_t>(A->idxBase), value_size(A->valueType),
+                              A->banded.band_bytes != 0 ? A->banded.band_bytes : mcsp::kBandedBandBytes, shape);
+}
+
+// The banded copy on the descriptor belongs to this call: same buffer, same arrays, same extents.
+bool banded_matches(const mcsparseSpMatDescr* A, const void* buffer, size_t value_bytes) {
+    const SpmvBanded& b = A->banded;
+    return b.valid && b.useful && b.buffer == buffer && b.rows == A->rows && b.cols == A->cols && b.vals == A->vals &&
+           b.m == A->row_num && b.n == A->col_num && b.nnz == A->nnz && b.base == static_cast<int>(A->idxBase) &&
+           b.type == A->valueType && value_size(b.type) == value_bytes && A->format == MCSPARSE_FORMAT_CSR;
+}
+
 template <typename T>
 mcspStatus_t spmv_typed(mcsparseHandle_t h, mcsparseSpMatDescr* A, mcsparseOperation_t op, const void* alpha,
-                        const void* beta, const mcsparseDnVecDescr* x, mcsparseDnVecDescr* y, void* buffer) {
+                        const void* beta, const mcsparseDnVecDescr* x, mcsparseDnVecDescr* y, void* buffer,
+                        bool may_read_back) {
     T h_alpha, h_beta;
     if (!scalar_to_host(h, beta, &h_beta) || !scalar_to_host(h, alpha, &h_alpha)) return MCSP_STATUS_INTERNAL_ERROR;
     // reference: mcsp_spmv_gpu.cpp:235-237 -- y is left untouched in both cases
@@ -260,8 +293,14 @@ mcspStatus_t spmv_typed(mcsparseHandle_t h, mcsparseSpMatDescr* A, mcsparseOpera
         a.col = v.ind;
         a.val = v.val;
         const mcspStatus_t st =
-            ensure_plan(h, A, v.ptr, signature, v.m, A->nnz, v.n * static_cast<int64_t>(sizeof(T)), buffer);
+            ensure_plan(h, A, v.ptr, signature, v.m, A->nnz, v.n * static_cast<int64_t>(sizeof(T)), buffer,
+                        may_read_back);
         if (st != MCSP_STATUS_SUCCESS) return st;
+        if (A->plan.forced_family == kFamilyAuto && banded_matches(A, buffer, sizeof(T))) {
+            mcsp::launch_spmv_banded<T>(h->stream, A->banded.shape, A->banded.grid, a, h_alpha, h_beta,
+                                        buf + A->banded.region);
+            return MCSP_STATUS_SUCCESS;
+        }
         if (A->plan.family == kFamilyMerge) {
             mcsp::launch_spmv_merge<T>(h->stream, a, h_alpha, h_beta, buf + l.merge_ws, A->plan.lanes != 0);
         } else {
@@ -423,6 +462,54 @@ mcspStatus_t check_spmm_args(mcsparseHandle_t handle, const void* alpha, const m
 
 }  // namespace
 
+namespace mcsp {
+
+// The argument checks of mcsparseSpMV in the reference's order, then the ones this build adds.
+mcspStatus_t spmv_check(mcsparseHandle_t handle, mcsparseOperation_t opA, const void* alpha, mcsparseSpMatDescr_t matA,
+                        mcsparseDnVecDescr_t vecX, const void* beta, mcsparseDnVecDescr_t vecY,
+                        macaDataType computeType, const void* buffer, size_t buffer_bytes, bool may_read_back) {
+    if (matA != nullptr) {
+        const mcspStatus_t it = check_index_types(matA);
+        if (it != MCSP_STATUS_SUCCESS) return it;
+    }
+    const mcspStatus_t st = check_spmv_args(handle, opA, alpha, matA, vecX, beta, vecY, true, true, buffer);
+    if (st != MCSP_STATUS_SUCCESS) return st;
+    const bool real_type = computeType == MACA_R_32F || computeType == MACA_R_64F || computeType == MACA_R_16F ||
+                           computeType == MACA_R_16BF;
+    if (real_type && opA == MCSPARSE_OPERATION_CONJUGATE_TRANSPOSE) return MCSP_STATUS_INVALID_VALUE;
+    if (!format_is_built(matA->format)) return MCSP_STATUS_NOT_IMPLEMENTED;  // COO_AOS
+    // Same-type real fp32/fp64 only; the reference's mixed-precision and complex routes
+    // (:848-860) are outside this path.  x is checked too, which the reference omits.
+    if (!(computeType == matA->valueType && computeType == vecY->valueType && computeType == vecX->valueType))
+        return MCSP_STATUS_NOT_IMPLEMENTED;
+    if (computeType != MACA_R_32F && computeType != MACA_R_64F) return MCSP_STATUS_NOT_IMPLEMENTED;
+    if (!may_read_back && handle->ptr_mode != MCSPARSE_POINTER_MODE_HOST) return MCSP_STATUS_NOT_IMPLEMENTED;
+    if (buffer_bytes != 0) {
+        const CsrView v = make_view(matA, opA);
+        if (spmv_layout(v, matA->nnz, value_size(computeType), narrow_bytes(matA)).total > buffer_bytes)
+            return MCSP_STATUS_INSUFFICIENT_RESOURCES;
+    }
+    // The reference hands NULL arrays back as INVALID_POINTER (mcsp_spmv_gpu.cpp:217-220); a kernel
+    // would fault on them.  A call without nonzeros reads none of them.
+    if (matA->nnz != 0 && (matA->rows == nullptr || matA->cols == nullptr || matA->vals == nullptr ||
+                           vecX->values == nullptr || vecY->values == nullptr))
+        return MCSP_STATUS_INVALID_POINTER;
+    return MCSP_STATUS_SUCCESS;
+}
+
+mcspStatus_t spmv_call(mcsparseHandle_t handle, mcsparseOperation_t opA, const void* alpha, mcsparseSpMatDescr_t matA,
+                       mcsparseDnVecDescr_t vecX, const void* beta, mcsparseDnVecDescr_t vecY,
+                       macaDataType computeType, void* buffer, size_t buffer_bytes, bool may_read_back) {
+    const mcspStatus_t st =
+        spmv_check(handle, opA, alpha, matA, vecX, beta, vecY, computeType, buffer, buffer_bytes, may_read_back);
+    if (st != MCSP_STATUS_SUCCESS) return st;
+    if (computeType == MACA_R_32F)
+        return spmv_typed<float>(handle, matA, opA, alpha, beta, vecX, vecY, buffer, may_read_back);
+    return spmv_typed<double>(handle, matA, opA, alpha, beta, vecX, vecY, buffer, may_read_back);
+}
+
+}  // namespace mcsp
+
 extern "C" {
 
 // reference: src/kernels/level2/spmv/mcsp_spmv_gpu.cpp:309-352, :1108-1121
@@ -456,32 +543,80 @@ mcsparseStatus_t mcsparseSpMV(mcsparseHandle_t handle, mcsparseOperation_t opA, 
                               mcsparseSpMatDescr_t matA, mcsparseDnVecDescr_t vecX, const void* beta,
                               mcsparseDnVecDescr_t vecY, macaDataType computeType, mcsparseSpMVAlg_t /*alg*/,
                               void* externalBuffer) {
-    if (matA != nullptr) {
-        const mcspStatus_t it = check_index_types(matA);
-        if (it != MCSP_STATUS_SUCCESS) return to_public_status(it);
-    }
-    mcspStatus_t st = check_spmv_args(handle, opA, alpha, matA, vecX, beta, vecY, true, true, externalBuffer);
-    if (st != MCSP_STATUS_SUCCESS) return to_public_status(st);
-    const bool real_type = computeType == MACA_R_32F || computeType == MACA_R_64F || computeType == MACA_R_16F ||
-                           computeType == MACA_R_16BF;
-    if (real_type && opA == MCSPARSE_OPERATION_CONJUGATE_TRANSPOSE) return to_public_status(MCSP_STATUS_INVALID_VALUE);
-    if (!format_is_built(matA->format)) return to_public_status(MCSP_STATUS_NOT_IMPLEMENTED);  // COO_AOS
-    // Same-type real fp32/fp64 only; the reference's mixed-precision and complex routes
-    // (:848-860) are outside this path.  x is checked too, which the reference omits.
-    if (!(computeType == matA->valueType && computeType == vecY->valueType && computeType == vecX->valueType))
-        return to_public_status(MCSP_STATUS_NOT_IMPLEMENTED);
+    return to_public_status(
+        mcsp::spmv_call(handle, opA, alpha, matA, vecX, beta, vecY, computeType, externalBuffer, 0, true));
+}
 
-    switch (computeType) {
-        case MACA_R_32F:
-            st = spmv_typed<float>(handle, matA, opA, alpha, beta, vecX, vecY, externalBuffer);
-            break;
-        case MACA_R_64F:
-            st = spmv_typed<double>(handle, matA, opA, alpha, beta, vecX, vecY, externalBuffer);
-            break;
-        default:
-            st = MCSP_STATUS_NOT_IMPLEMENTED;
+// EXTENSION
+mcsparseStatus_t mcsparseSpMV_preprocess_bufferSize(mcsparseHandle_t handle, mcsparseOperation_t opA, const void* alpha,
+                                                    mcsparseSpMatDescr_t matA, mcsparseDnVecDescr_t vecX,
+                                                    const void* beta, mcsparseDnVecDescr_t vecY,
+                                                    macaDataType computeType, mcsparseSpMVAlg_t alg,
+                                                    size_t* bufferSize) {
+    const mcsparseStatus_t st =
+        mcsparseSpMV_bufferSize(handle, opA, alpha, matA, vecX, beta, vecY, computeType, alg, bufferSize);
+    if (st != MCSPARSE_STATUS_SUCCESS) return st;
+    BandedShape shape;
+    if (banded_candidate(matA, opA, &shape)) {
+        const size_t vb = value_size(matA->valueType);
+        *bufferSize = banded_region_offset(matA, vb) +
+                      mcsp::banded_layout(shape, static_cast<idx_t>(matA->row_num), static_cast<idx_t>(matA->nnz), vb).total;
     }
-    return to_public_status(st);
+    return MCSPARSE_STATUS_SUCCESS;
+}
+
+// EXTENSION
+mcsparseStatus_t mcsparseSpMV_preprocess(mcsparseHandle_t handle, mcsparseOperation_t opA, const void* alpha,
+                                         mcsparseSpMatDescr_t matA, mcsparseDnVecDescr_t vecX, const void* beta,
+                                         mcsparseDnVecDescr_t vecY, macaDataType computeType,
+                                         mcsparseSpMVAlg_t /*alg*/, void* externalBuffer) {
+    const mcspStatus_t st =
+        mcsp::spmv_check(handle, opA, alpha, matA, vecX, beta, vecY, computeType, externalBuffer, 0, true);
+    if (st != MCSP_STATUS_SUCCESS) return to_public_status(st);
+    matA->banded.valid = false;
+    BandedShape shape;
+    if (matA->nnz == 0 || !banded_candidate(matA, opA, &shape)) return MCSPARSE_STATUS_SUCCESS;  // nothing to prepare
+
+    // the row-length analysis says whether the rows are short enough for the banded kernel
+    const idx_t m = static_cast<idx_t>(matA->row_num);
+    const idx_t nnz = static_cast<idx_t>(matA->nnz);
+    const idx_t base = static_cast<idx_t>(matA->idxBase);
+    const size_t vb = value_size(matA->valueType);
+    const idx_t* row_ptr = static_cast<const idx_t*>(matA->rows);
+    const mcspStatus_t ps = ensure_plan(handle, matA, row_ptr, matA->rows, matA->row_num, matA->nnz,
+                                        matA->col_num * static_cast<int64_t>(vb), externalBuffer, true);
+    if (ps != MCSP_STATUS_SUCCESS) return to_public_status(ps);
+    SpmvBanded& b = matA->banded;
+    b.buffer = externalBuffer;
+    b.rows = matA->rows;
+    b.cols = matA->cols;
+    b.vals = matA->vals;
+    b.m = matA->row_num;
+    b.n = matA->col_num;
+    b.nnz = matA->nnz;
+    b.base = static_cast<int>(matA->idxBase);
+    b.type = matA->valueType;
+    b.shape = shape;
+    b.region = banded_region_offset(matA, vb);
+    b.grid = 0;
+    if (matA->plan.forced_family == kFamilyAuto && matA->plan.max_row_len > mcsp::kBandedMaxRowLength) {
+        b.useful = false;
+        b.valid = true;
+        return MCSPARSE_STATUS_SUCCESS;
+    }
+    char* region = static_cast<char*>(externalBuffer) + b.region;
+    mcsp::launch_banded_build(handle->stream, shape, m, nnz, base, row_ptr, static_cast<const idx_t*>(matA->cols),
+                              matA->vals, vb, region);
+    uint32_t xcd_start[9];
+    const mcsp::BandedLayout l = mcsp::banded_layout(shape, m, nnz, vb);
+    if (hipMemcpyAsync(xcd_start, region + l.xcd_start, sizeof(xcd_start), hipMemcpyDeviceToHost, handle->stream) !=
+            hipSuccess ||
+        hipStreamSynchronize(handle->stream) != hipSuccess)
+        return to_public_status(MCSP_STATUS_INTERNAL_ERROR);
+    b.grid = mcsp::banded_grid(xcd_start);
+    b.useful = true;
+    b.valid = true;
+    return MCSPARSE_STATUS_SUCCESS;
 }
 
 // reference: src/kernels/level3/spmm/mcsp_spmm_gpu.cpp:309-342, :950-963
@@ -586,6 +721,12 @@ mcsparseStatus_t mcsparseSpMM(mcsparseHandle_t handle, mcsparseOperation_t opA, 
     // reference: mcsp_spmm_gpu.cpp:96-98
     if (!(matC->batchCount == matA->batchCount && matC->batchCount == matB->batchCount))
         return to_public_status(MCSP_STATUS_INVALID_SIZE);
+    // the reference hands NULL arrays back as INVALID_POINTER (mcsp_spmm_gpu.cpp:100-103); a kernel
+    // would fault on them.  Arrays that a call without nonzeros never reads may be NULL.
+    if (matC->values == nullptr || (matA->format == MCSPARSE_FORMAT_CSR && matA->rows == nullptr) ||
+        (matA->nnz != 0 && (matA->rows == nullptr || matA->cols == nullptr || matA->vals == nullptr ||
+                            matB->values == nullptr)))
+        return to_public_status(MCSP_STATUS_INVALID_POINTER);
 
     switch (computeType) {
         case MACA_R_32F: st = spmm_typed<float>(handle, matA, opB, alpha, beta, matB, matC, externalBuffer); break;

@@ -298,6 +298,7 @@ mcsparseStatus_t mcsparseCsrSetPointers(mcsparseSpMatDescr_t d, void* csrRowOffs
     d->vals = csrValues;
     d->plan.valid = false;  // new structure, new analysis
     d->schedule.valid = false;
+    d->banded.valid = false;
     return MCSPARSE_STATUS_SUCCESS;
 }
 
@@ -308,6 +309,7 @@ mcsparseStatus_t mcsparseCscSetPointers(mcsparseSpMatDescr_t d, void* cscColOffs
     d->cols = cscColOffsets;
     d->vals = cscValues;
     d->plan.valid = false;
+    d->banded.valid = false;
     return MCSPARSE_STATUS_SUCCESS;
 }
 
@@ -346,6 +348,7 @@ mcsparseStatus_t mcsparseSpMatGetValues(mcsparseSpMatDescr_t d, void** values) {
 mcsparseStatus_t mcsparseSpMatSetValues(mcsparseSpMatDescr_t d, void* values) {
     if (d == nullptr) return to_public_status(MCSP_STATUS_INVALID_POINTER);
     d->vals = values;
+    d->banded.valid = false;  // the banded copy holds the old values
     return MCSPARSE_STATUS_SUCCESS;
 }
 
@@ -362,6 +365,24 @@ mcsparseStatus_t mcsparseSpMatGetSpMMSchedule(mcsparseSpMatDescr_t d, int* state
         return to_public_status(MCSP_STATUS_INVALID_POINTER);
     *state = !d->schedule.valid ? 0 : (d->schedule.useful ? 2 : 1);
     *merged_entries = d->schedule.valid ? static_cast<int64_t>(d->schedule.entries) : 0;
+    return MCSPARSE_STATUS_SUCCESS;
+}
+
+mcsparseStatus_t mcsparseSpMatGetSpMVPreprocess(mcsparseSpMatDescr_t d, int* state, int* bands, int* rows_per_tile) {
+    if (d == nullptr || state == nullptr || bands == nullptr || rows_per_tile == nullptr)
+        return to_public_status(MCSP_STATUS_INVALID_POINTER);
+    *state = !d->banded.valid ? 0 : (d->banded.useful ? 2 : 1);
+    *bands = d->banded.valid && d->banded.useful ? static_cast<int>(d->banded.shape.bands) : 0;
+    *rows_per_tile = d->banded.valid && d->banded.useful ? static_cast<int>(d->banded.shape.rows_per_tile) : 0;
+    return MCSPARSE_STATUS_SUCCESS;
+}
+
+mcsparseStatus_t mcsparseSpMatSetSpMVBandBytes(mcsparseSpMatDescr_t d, size_t band_bytes) {
+    if (d == nullptr) return to_public_status(MCSP_STATUS_INVALID_POINTER);
+    if (band_bytes != 0 && (band_bytes < 16 || band_bytes > (size_t(1) << 30)))
+        return to_public_status(MCSP_STATUS_INVALID_VALUE);
+    d->banded.band_bytes = band_bytes;
+    d->banded.valid = false;
     return MCSPARSE_STATUS_SUCCESS;
 }
 

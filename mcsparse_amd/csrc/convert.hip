@@ -654,6 +654,8 @@ struct CsrSource {
     // != nullptr: no aux travels; the value of every triple is multiplied by x[its row] in the first
     // pass (x in the floating-point type of the values), and (key, product) pairs are sorted
     const void* times_x = nullptr;
+    // lowest key bit the sort looks at: the keys are ordered by bits [first_bit, first_bit + key_bits)
+    uint32_t first_bit = 0;
 };
 
 // Stable LSD radix sort of (key, aux, value) triples on the low key_bits of the keys, in
@@ -667,7 +669,7 @@ void radix_sort_triples(hipStream_t stream, idx_t count, uint32_t key_bits, cons
     const uint32_t radix = 1u << bits;
     const uint32_t tiles = sort_tiles(count);
     const uint32_t scatter_grid = (tiles + kXcds - 1) / kXcds * kXcds;
-    uint32_t shift = 0;
+    uint32_t shift = csr.first_bit;
     if (csr.rows > 0) {
         const uint32_t waves_per_block = kBlock / kWave;
         hipLaunchKernelGGL(tile_row_starts_kernel, dim3((tiles + 1 + waves_per_block - 1) / waves_per_block), dim3(kBlock),
@@ -860,6 +862,46 @@ void launch_transposed_products(hipStream_t stream, idx_t m, idx_t n, idx_t nnz,
     radix_sort_triples(stream, nnz, bit_length(n - 1 + base), col, row_ptr, csr_val, sorted_keys, nullptr, products,
                        value_bytes, t, csr);
     launch_coo2csr(stream, nnz, n, sorted_keys, base, col_ptr);
+}
+
+// Scratch of launch_sort_by_column_band: the counters of one pass, their scan, the row starts per tile.
+namespace {
+struct BandSortLayout {
+    size_t counters, scan_ws, tile_rows, total;
+};
+BandSortLayout band_sort_layout(idx_t nnz) {
+    BandSortLayout l;
+    const size_t counter_elems = sort_counter_elems(nnz);
+    size_t off = 0;
+    l.counters = off; off += align_up(counter_elems * sizeof(uint32_t));
+    l.scan_ws = off; off += align_up(scan_workspace_elems(counter_elems) * sizeof(uint32_t)) + kAlign;
+    l.tile_rows = off; off += align_up((static_cast<size_t>(sort_tiles(nnz)) + 1) * sizeof(idx_t));
+    l.total = off;
+    return l;
+}
+}  // namespace
+
+size_t band_sort_workspace_bytes(idx_t nnz) { return band_sort_layout(nnz).total; }
+
+void launch_sort_by_column_band(hipStream_t stream, idx_t m, idx_t nnz, idx_t base, const idx_t* row_ptr, const idx_t* col,
+                                const void* val, size_t value_bytes, uint32_t band_shift, uint32_t band_bits,
+                                idx_t* cols_out, idx_t* rows_out, void* vals_out, void* workspace) {
+    if (m == 0 || nnz == 0) return;
+    const BandSortLayout l = band_sort_layout(nnz);
+    char* w = static_cast<char*>(workspace);
+    SortScratch t;  // one pass writes the outputs directly: no alternating sets
+    t.keys[0] = t.keys[1] = nullptr;
+    t.aux[0] = t.aux[1] = nullptr;
+    t.vals[0] = t.vals[1] = nullptr;
+    t.counters = reinterpret_cast<uint32_t*>(w + l.counters);
+    t.scan_ws = reinterpret_cast<uint32_t*>(w + l.scan_ws);
+    t.tile_rows = reinterpret_cast<idx_t*>(w + l.tile_rows);
+    CsrSource csr;
+    csr.rows = m;
+    csr.base = base;
+    csr.first_bit = band_shift;
+    radix_sort_triples(stream, nnz, band_bits > 8 ? 8 : band_bits, col, row_ptr, val, cols_out, rows_out, vals_out,
+                       value_bytes, t, csr);
 }
 
 size_t index_sort_workspace_bytes(idx_t nnz) { return index_sort_layout(nnz).total; }

@@ -93,6 +93,34 @@ struct SpmmSchedule {
     uint64_t mean_span = 0;  // mean distance between the first and the last column of a group
 };
 
+// Column-banded copy of a CSR matrix built by mcsparseSpMV_preprocess inside the caller's buffer
+// (spmv_banded.hip).  Like the SpMM schedule it is part of the computation, and it holds a copy of the
+// values: SpMV uses it only while the buffer, the three CSR arrays and the extents of the call are the
+// ones it was built from.
+struct BandedShape {
+    uint32_t band_shift;     // a band holds 2^band_shift keys (column index + index base)
+    uint32_t band_bits;      // bits needed to number the bands
+    uint32_t bands;
+    uint32_t rows_per_tile;
+    uint32_t chunks;         // row chunks = tiles per band
+    uint32_t tiles;
+};
+struct SpmvBanded {
+    bool valid = false;
+    bool useful = false;     // false: preprocess looked at the matrix and left it to the row kernels
+    const void* buffer = nullptr;
+    const void* rows = nullptr;
+    const void* cols = nullptr;
+    const void* vals = nullptr;
+    int64_t m = 0, n = 0, nnz = 0;
+    int base = 0;
+    macaDataType type = MACA_R_32F;
+    size_t region = 0;       // offset of the banded copy inside the buffer
+    BandedShape shape = {};
+    uint32_t grid = 0;       // workgroups of the SpMV kernel
+    size_t band_bytes = 0;   // user override of the band width (mcsparseSpMatSetSpMVBandBytes); 0 = default
+};
+
 // reference: src/include/mcsp_internal_types.h:184-225.  rows/cols follow the reference's
 // convention: for CSR rows = row offsets, cols = column indices; for CSC rows = row indices,
 // cols = column offsets (src/common/mcsp_helper.cpp:447-452).
@@ -120,6 +148,7 @@ struct mcsparseSpMatDescr {
     size_t fixed_length_buffer_size = 0;
     SpmvPlan plan;
     SpmmSchedule schedule;
+    SpmvBanded banded;
 };
 
 // Internal status, mapped to the public one exactly as the reference's wrapper does
@@ -174,6 +203,18 @@ namespace mcsp {
 
 typedef uint32_t idx_t;
 
+// ---- host layer shared between entry points (api_compute.cpp) ----
+// spmv_check: the argument checks of mcsparseSpMV.  buffer_bytes != 0 states how large `buffer` is:
+// a call that needs more is refused with INSUFFICIENT_RESOURCES.  may_read_back = false asks for a
+// call free of device-to-host copies: no row-length analysis (a structure without a plan runs the
+// merge family) and host scalars only.  spmv_call: the checks, then the launches.
+mcspStatus_t spmv_check(mcsparseHandle_t handle, mcsparseOperation_t opA, const void* alpha, mcsparseSpMatDescr_t matA,
+                        mcsparseDnVecDescr_t vecX, const void* beta, mcsparseDnVecDescr_t vecY,
+                        macaDataType computeType, const void* buffer, size_t buffer_bytes, bool may_read_back);
+mcspStatus_t spmv_call(mcsparseHandle_t handle, mcsparseOperation_t opA, const void* alpha, mcsparseSpMatDescr_t matA,
+                       mcsparseDnVecDescr_t vecX, const void* beta, mcsparseDnVecDescr_t vecY,
+                       macaDataType computeType, void* buffer, size_t buffer_bytes, bool may_read_back);
+
 // ---- row-length analysis (analysis.hip) ----
 // hist_out: MCSPARSE_ROW_BIN_COUNT counters followed by the longest row length (34 x u32),
 // zeroed by this call.  row_bins may be null.
@@ -202,6 +243,28 @@ template <typename T>
 void launch_row_sums_merge(hipStream_t stream, const SpmvArgs& a, T alpha, T beta, void* workspace);
 int spmv_pick_lanes(idx_t m, idx_t nnz);
 
+// ---- column-banded SpMV (spmv_banded.hip) ----
+// Rows of a tile (one workgroup's share of a band), the width of a band of x in bytes, and the
+// longest row the banded kernel takes (it adds up a row's run inside a tile with one thread).
+constexpr int kBandedMaxRowsPerTile = 1024;
+constexpr size_t kBandedBandBytes = size_t(2) << 20;
+constexpr uint32_t kBandedMaxRowLength = 256;
+struct BandedLayout {
+    // kept between preprocess and SpMV: [0, keep); scratch of the build: [keep, total)
+    size_t tile_ptr, xcd_start, entries, vals, partials, keep, tmp_keys, tmp_rows, sort_ws, total;
+};
+// False when the banded copy cannot help or cannot be built: x fits one band, more than 256 bands.
+bool banded_shape(idx_t m, idx_t n, idx_t nnz, idx_t base, size_t value_bytes, size_t band_bytes, BandedShape* out);
+BandedLayout banded_layout(const BandedShape& s, idx_t m, idx_t nnz, size_t value_bytes);
+// Builds the banded copy in `region` (banded_layout(...).total bytes); xcd_start (9 x u32 at
+// region + layout.xcd_start) is then read back by the caller and turned into the grid by banded_grid.
+void launch_banded_build(hipStream_t stream, const BandedShape& s, idx_t m, idx_t nnz, idx_t base, const idx_t* row_ptr,
+                         const idx_t* col, const void* val, size_t value_bytes, void* region);
+uint32_t banded_grid(const uint32_t* xcd_start_host);
+template <typename T>
+void launch_spmv_banded(hipStream_t stream, const BandedShape& s, uint32_t grid, const SpmvArgs& a, T alpha, T beta,
+                        void* region);
+
 // ---- SpMM (spmm.hip) ----
 struct SpmmArgs {
     idx_t m, n, k, nnz, base;   // C is m x n, A is m x k
@@ -224,10 +287,7 @@ void launch_spmm(hipStream_t stream, const SpmmArgs& a, T alpha, T beta);
 // group_ptr has groups+1 offsets into entries; span_sum (one u64) is the sum over the groups of
 // the distance between their first and last column.  Groups holding more than kSpmmMaxMergedGroup
 // nonzeros get no entries and are processed row by row.
-#ifndef MCSP_GROUP_ROWS
-#define MCSP_GROUP_ROWS 4
-#endif
-constexpr int kSpmmGroupRows = MCSP_GROUP_ROWS;
+constexpr int kSpmmGroupRows = 4;
 constexpr idx_t kSpmmMaxMergedGroup = 2048;
 constexpr int64_t kSpmmMaxScheduledColumns = int64_t(1) << (32 - kSpmmGroupRows);
 constexpr uint64_t spmm_groups(idx_t m) { return (static_cast<uint64_t>(m) + kSpmmGroupRows - 1) / kSpmmGroupRows; }
@@ -260,6 +320,14 @@ size_t transposed_products_workspace_bytes(idx_t nnz, size_t value_bytes);
 void launch_transposed_products(hipStream_t stream, idx_t m, idx_t n, idx_t nnz, const void* csr_val, const idx_t* row_ptr,
                                 const idx_t* col, const void* x, void* products, idx_t* col_ptr, size_t value_bytes,
                                 idx_t base, void* workspace);
+
+// One stable radix pass over the nonzeros of a CSR matrix where they lie, on band_bits (<= 8) bits
+// of the keys from bit band_shift on (key = column index, index base included): cols_out / rows_out
+// (row + base) / vals_out hold the nonzeros band by band, inside a band in CSR order.
+size_t band_sort_workspace_bytes(idx_t nnz);
+void launch_sort_by_column_band(hipStream_t stream, idx_t m, idx_t nnz, idx_t base, const idx_t* row_ptr, const idx_t* col,
+                                const void* val, size_t value_bytes, uint32_t band_shift, uint32_t band_bits,
+                                idx_t* cols_out, idx_t* rows_out, void* vals_out, void* workspace);
 
 // ---- index sorts (convert.hip) --------------------------------------------------------------
 size_t index_sort_workspace_bytes(idx_t nnz);

@@ -1,0 +1,320 @@
+// Column-banded CSR SpMV for gfx950: y = alpha*A*x + beta*y on a copy of A that is laid out so that
+// the gathers from x hit in L2.
+//
+// A gather x[col] costs one 128-byte line fill from L2 when the line is there and a trip over the
+// fabric when it is not; with x larger than an XCD's 4 MB L2 and columns spread over all of it, most
+// gathers of the row kernels (spmv.hip) miss.  mcsparseSpMV_preprocess therefore re-lays the matrix
+// out once: the columns are cut into bands narrow enough for a band of x to stay in L2, the rows
+// into chunks, and the nonzeros are stored tile by tile (band-major, chunk-minor), inside a tile in
+// CSR order.  An entry keeps (row inside the chunk, column inside the band) in one 32-bit word, so
+// the stream is as long as CSR's.  The SpMV kernel hands every XCD a contiguous stretch of that
+// tile list: an XCD works inside one band at a time and only that band of x lives in its L2.  A tile
+// leaves one partial sum per row and band; a second kernel adds a row's partial sums in band order.
+// No atomics: every sum is formed in a fixed order, so results are bit-reproducible run to run.
+//
+// Stands in, like spmv.hip, for the gather loop of the reference's row kernel
+// (src/kernels/level2/spmv/csr_vector_device.hpp:40-57).
+#include "device_util.h"
+#include "internal.h"
+
+namespace mcsp {
+
+namespace {
+
+constexpr int kBlock = 256;
+constexpr int kIpt = 8;
+constexpr int kSlab = kBlock * kIpt;  // entries a workgroup stages at a time
+constexpr int kRowsPerThread = kBandedMaxRowsPerTile / kBlock;
+constexpr uint32_t kXcds = 8;  // accelerator complex dies of an MI355X; workgroup i runs on XCD i % 8
+static_assert(kBandedMaxRowsPerTile % kBlock == 0, "rows of a tile are dealt to the threads in rounds");
+static_assert(kSlab <= 65536 && kBandedMaxRowsPerTile <= 65536, "16-bit positions in LDS");
+
+// ------------------------------------------------------------------------------------------
+// build
+// ------------------------------------------------------------------------------------------
+// Entry k of the band-sorted nonzeros becomes (row inside its chunk << band_shift) | (key inside the
+// band); key = column index with the index base left in.  Tile of an entry = band * chunks + chunk;
+// the entries are sorted by tile, and boundary k (between entries k-1 and k, 0 <= k <= nnz) writes
+// the offsets of the tiles that begin there, so empty tiles are covered.
+__global__ __launch_bounds__(kBlock) void banded_pack_kernel(idx_t nnz, idx_t base, uint32_t band_shift,
+                                                             uint32_t rows_per_tile, uint32_t chunks, uint32_t tiles,
+                                                             const idx_t* __restrict__ keys,
+                                                             const idx_t* __restrict__ rows,
+                                                             idx_t* __restrict__ entries,
+                                                             idx_t* __restrict__ tile_ptr) {
+    const uint64_t k = static_cast<uint64_t>(blockIdx.x) * kBlock + threadIdx.x;
+    if (k > nnz) return;
+    const idx_t band_mask = (1u << band_shift) - 1u;
+    uint32_t tile = tiles;  // boundary nnz closes every remaining tile
+    if (k < nnz) {
+        const idx_t key = keys[k];
+        const idx_t row = rows[k] - base;
+        const uint32_t chunk = row / rows_per_tile;
+        tile = (key >> band_shift) * chunks + chunk;
+        entries[k] = ((row - chunk * rows_per_tile) << band_shift) | (key & band_mask);
+    }
+    uint32_t first = 0;  // first tile whose offset this boundary writes
+    if (k != 0) {
+        const uint32_t prev_chunk = (rows[k - 1] - base) / rows_per_tile;
+        first = (keys[k - 1] >> band_shift) * chunks + prev_chunk + 1;
+    }
+    for (uint32_t t = first; t <= tile && t <= tiles; ++t) tile_ptr[t] = static_cast<idx_t>(k);
+}
+
+// xcd_start[i], i = 0..8: first tile of XCD i's stretch of the tile list, cut so that the stretches
+// hold about the same number of nonzeros.
+__global__ void banded_split_kernel(idx_t nnz, uint32_t tiles, const idx_t* __restrict__ tile_ptr,
+                                    uint32_t* __restrict__ xcd_start) {
+    const uint32_t i = threadIdx.x;
+    if (i > kXcds) return;
+    const uint64_t target = static_cast<uint64_t>(nnz) * i / kXcds;
+    uint32_t lo = 0, hi = tiles;  // first tile whose offset is >= target
+    while (lo < hi) {
+        const uint32_t mid = (lo + hi) >> 1;
+        if (tile_ptr[mid] < target) lo = mid + 1; else hi = mid;
+    }
+    xcd_start[i] = i == 0 ? 0u : (i == kXcds ? tiles : lo);
+}
+
+// ------------------------------------------------------------------------------------------
+// SpMV
+// ------------------------------------------------------------------------------------------
+// One tile per workgroup.  The tile's entries are staged a slab at a time: coalesced loads of the
+// packed entries and values, the gathers from the band of x, products and row numbers to LDS; the
+// ends of every row's run are found where neighbouring entries differ; then thread r adds up the run
+// of row r (and r + 256, ...) in storage order and keeps the sum in a register across slabs.
+// Every index that comes out of the layout is clamped, so a layout the caller has overwritten gives
+// wrong numbers but never an access outside the arrays.
+template <typename T>
+__global__ __launch_bounds__(kBlock) void spmv_banded_kernel(idx_t m, idx_t n, idx_t nnz, idx_t base, uint32_t band_shift,
+                                                             uint32_t rows_per_tile, uint32_t chunks, uint32_t tiles,
+                                                             const uint32_t* __restrict__ xcd_start,
+                                                             const idx_t* __restrict__ tile_ptr,
+                                                             const idx_t* __restrict__ entries,
+                                                             const T* __restrict__ vals, const T* __restrict__ x,
+                                                             T* __restrict__ partials) {
+    __shared__ T s_prod[kSlab];
+    __shared__ uint16_t s_row[kSlab];
+    __shared__ uint16_t s_beg[kBandedMaxRowsPerTile];
+    __shared__ uint16_t s_end[kBandedMaxRowsPerTile];
+
+    const uint32_t tid = threadIdx.x;
+    const uint32_t xcd = blockIdx.x % kXcds;
+    const uint32_t tile = xcd_start[xcd] + blockIdx.x / kXcds;
+    if (tile >= xcd_start[xcd + 1] || tile >= tiles) return;  // whole workgroup
+    const uint32_t band = tile / chunks;
+    const uint32_t chunk = tile - band * chunks;
+    const uint64_t row0 = static_cast<uint64_t>(chunk) * rows_per_tile;
+    if (row0 >= m) return;
+    const uint32_t tile_rows = static_cast<uint32_t>(m - row0 < rows_per_tile ? m - row0 : rows_per_tile);
+    idx_t e0 = tile_ptr[tile];
+    idx_t e1 = tile_ptr[tile + 1];
+    e0 = e0 < nnz ? e0 : nnz;
+    e1 = e1 < nnz ? e1 : nnz;
+    e1 = e1 > e0 ? e1 : e0;
+    const idx_t band_mask = (1u << band_shift) - 1u;
+    const idx_t band_key = band << band_shift;
+
+#pragma unroll
+    for (int q = 0; q < kRowsPerThread; ++q) {
+        s_beg[q * kBlock + tid] = 0;
+        s_end[q * kBlock + tid] = 0;
+    }
+    T acc[kRowsPerThread];
+#pragma unroll
+    for (int q = 0; q < kRowsPerThread; ++q) acc[q] = T(0);
+
+    for (idx_t slab = e0; slab < e1; slab += kSlab) {
+        const uint32_t cnt = e1 - slab < static_cast<idx_t>(kSlab) ? e1 - slab : kSlab;
+        // Loads without tests of their own (clamped positions), each kind back to back, so that all of
+        // a thread's loads are on their way before the first is waited for.
+        idx_t packed[kIpt];
+        T v[kIpt], xv[kIpt];
+#pragma unroll
+        for (int i = 0; i < kIpt; ++i) {
+            const uint32_t k = min(static_cast<uint32_t>(i) * kBlock + tid, cnt - 1);
+            packed[i] = load_stream(entries + slab + k);
+            v[i] = load_stream(vals + slab + k);
+        }
+#pragma unroll
+        for (int i = 0; i < kIpt; ++i) {
+            idx_t key = band_key | (packed[i] & band_mask);  // column + base
+            key = key > base ? key : base;
+            const idx_t c = min(key - base, n - 1);
+            xv[i] = x[c];
+        }
+#pragma unroll
+        for (int i = 0; i < kIpt; ++i) asm volatile("" : "+v"(xv[i]));
+#pragma unroll
+        for (int i = 0; i < kIpt; ++i) {
+            const uint32_t k = static_cast<uint32_t>(i) * kBlock + tid;
+            if (k < cnt) {
+                s_prod[k] = v[i] * xv[i];
+                s_row[k] = static_cast<uint16_t>(packed[i] >> band_shift);
+            }
+        }
+        __syncthreads();
+        // the run of row r is [s_beg[r], s_end[r]): entries of a tile are sorted by row
+#pragma unroll
+        for (int i = 0; i < kIpt; ++i) {
+            const uint32_t k = static_cast<uint32_t>(i) * kBlock + tid;
+            if (k < cnt) {
+                const uint32_t r = s_row[k];
+                if (r < tile_rows) {
+                    if (k == 0 || s_row[k - 1] != r) s_beg[r] = static_cast<uint16_t>(k);
+                    if (k + 1 == cnt || s_row[k + 1] != r) s_end[r] = static_cast<uint16_t>(k + 1);
+                }
+            }
+        }
+        __syncthreads();
+#pragma unroll
+        for (int q = 0; q < kRowsPerThread; ++q) {
+            const uint32_t r = q * kBlock + tid;
+            if (r < tile_rows) {
+                uint32_t end = s_end[r];
+                uint32_t j = s_beg[r];
+                end = end < cnt ? end : cnt;
+                T sum = T(0);
+                for (; j < end; ++j) sum += s_prod[j];
+                acc[q] += sum;
+                s_beg[r] = 0;
+                s_end[r] = 0;
+            }
+        }
+        __syncthreads();
+    }
+
+    T* out = partials + static_cast<uint64_t>(band) * m + row0;
+#pragma unroll
+    for (int q = 0; q < kRowsPerThread; ++q) {
+        const uint32_t r = q * kBlock + tid;
+        if (r < tile_rows) out[r] = acc[q];
+    }
+}
+
+// y[r] = beta*y[r] + alpha * (partials[0][r] + partials[1][r] + ...), the bands in order.
+template <typename T, bool BETA0>
+__global__ __launch_bounds__(kBlock) void banded_reduce_kernel(idx_t m, uint32_t bands, const T* __restrict__ partials,
+                                                               T* __restrict__ y, T alpha, T beta) {
+    const uint64_t r = static_cast<uint64_t>(blockIdx.x) * kBlock + threadIdx.x;
+    if (r >= m) return;
+    constexpr uint32_t kAhead = 8;
+    T sum = T(0);
+    for (uint32_t b0 = 0; b0 < bands; b0 += kAhead) {
+        T p[kAhead];
+#pragma unroll
+        for (uint32_t i = 0; i < kAhead; ++i) {
+            const uint32_t b = min(b0 + i, bands - 1);
+            p[i] = load_stream(partials + static_cast<uint64_t>(b) * m + r);
+        }
+#pragma unroll
+        for (uint32_t i = 0; i < kAhead; ++i) {
+            if (b0 + i < bands) sum = (b0 + i == 0) ? p[i] : sum + p[i];
+        }
+    }
+    if constexpr (BETA0) {
+        y[r] = alpha * sum;
+    } else {
+        y[r] = beta * y[r] + alpha * sum;
+    }
+}
+
+}  // namespace
+
+bool banded_shape(idx_t m, idx_t n, idx_t nnz, idx_t base, size_t value_bytes, size_t band_bytes, BandedShape* out) {
+    if (m == 0 || n == 0 || nnz == 0 || (value_bytes != 4 && value_bytes != 8)) return false;
+    uint32_t shift = 0;
+    while ((static_cast<size_t>(value_bytes) << (shift + 1)) <= band_bytes) ++shift;  // keys per band = 2^shift
+    const uint64_t max_key = static_cast<uint64_t>(n) - 1 + base;
+    const uint64_t bands = (max_key >> shift) + 1;
+    if (bands < 2 || bands > 256) return false;  // one band: x fits as it is; more than a sort pass orders
+    // rows per tile: a typical tile fills three quarters of a slab
+    const double per_row_and_band = static_cast<double>(nnz) / (static_cast<double>(m) * static_cast<double>(bands));
+    double rows = 0.75 * kSlab / (per_row_and_band > 1e-9 ? per_row_and_band : 1e-9);
+    if (rows > kBandedMaxRowsPerTile) rows = kBandedMaxRowsPerTile;
+    if (rows < 32) rows = 32;
+    uint32_t rows_per_tile = static_cast<uint32_t>(rows);
+    if (rows_per_tile > m) rows_per_tile = m;
+    if (bit_length(rows_per_tile - 1) + shift > 32) return false;
+    const uint64_t chunks = (static_cast<uint64_t>(m) + rows_per_tile - 1) / rows_per_tile;
+    if (bands * chunks >= (1ull << 31)) return false;
+    out->band_shift = shift;
+    out->band_bits = bit_length(static_cast<uint32_t>(bands - 1));
+    out->bands = static_cast<uint32_t>(bands);
+    out->rows_per_tile = rows_per_tile;
+    out->chunks = static_cast<uint32_t>(chunks);
+    out->tiles = static_cast<uint32_t>(bands * chunks);
+    return true;
+}
+
+BandedLayout banded_layout(const BandedShape& s, idx_t m, idx_t nnz, size_t value_bytes) {
+    BandedLayout l;
+    const size_t idx_bytes = align_up(static_cast<size_t>(nnz) * sizeof(idx_t));
+    size_t off = 0;
+    l.tile_ptr = off; off += align_up((static_cast<size_t>(s.tiles) + 1) * sizeof(idx_t));
+    l.xcd_start = off; off += align_up((kXcds + 1) * sizeof(uint32_t));
+    l.entries = off; off += idx_bytes;
+    l.vals = off; off += align_up(static_cast<size_t>(nnz) * value_bytes);
+    l.partials = off; off += align_up(static_cast<size_t>(s.bands) * m * value_bytes);
+    l.keep = off;
+    l.tmp_keys = off; off += idx_bytes;
+    l.tmp_rows = off; off += idx_bytes;
+    l.sort_ws = off; off += align_up(band_sort_workspace_bytes(nnz));
+    l.total = off;
+    return l;
+}
+
+void launch_banded_build(hipStream_t stream, const BandedShape& s, idx_t m, idx_t nnz, idx_t base, const idx_t* row_ptr,
+                         const idx_t* col, const void* val, size_t value_bytes, void* region) {
+    const BandedLayout l = banded_layout(s, m, nnz, value_bytes);
+    char* w = static_cast<char*>(region);
+    idx_t* tmp_keys = reinterpret_cast<idx_t*>(w + l.tmp_keys);
+    idx_t* tmp_rows = reinterpret_cast<idx_t*>(w + l.tmp_rows);
+    launch_sort_by_column_band(stream, m, nnz, base, row_ptr, col, val, value_bytes, s.band_shift, s.band_bits, tmp_keys,
+                               tmp_rows, w + l.vals, w + l.sort_ws);
+    const uint64_t boundaries = static_cast<uint64_t>(nnz) + 1;
+    hipLaunchKernelGGL(banded_pack_kernel, dim3(static_cast<uint32_t>((boundaries + kBlock - 1) / kBlock)), dim3(kBlock), 0,
+                       stream, nnz, base, s.band_shift, s.rows_per_tile, s.chunks, s.tiles,
+                       static_cast<const idx_t*>(tmp_keys), static_cast<const idx_t*>(tmp_rows),
+                       reinterpret_cast<idx_t*>(w + l.entries), reinterpret_cast<idx_t*>(w + l.tile_ptr));
+    hipLaunchKernelGGL(banded_split_kernel, dim3(1), dim3(kWave), 0, stream, nnz, s.tiles,
+                       reinterpret_cast<const idx_t*>(w + l.tile_ptr), reinterpret_cast<uint32_t*>(w + l.xcd_start));
+}
+
+uint32_t banded_grid(const uint32_t* xcd_start_host) {
+    uint32_t longest = 0;
+    for (uint32_t i = 0; i < kXcds; ++i) {
+        const uint32_t len = xcd_start_host[i + 1] > xcd_start_host[i] ? xcd_start_host[i + 1] - xcd_start_host[i] : 0;
+        longest = len > longest ? len : longest;
+    }
+    return longest * kXcds;
+}
+
+template <typename T>
+void launch_spmv_banded(hipStream_t stream, const BandedShape& s, uint32_t grid, const SpmvArgs& a, T alpha, T beta,
+                        void* region) {
+    if (a.m == 0) return;
+    const BandedLayout l = banded_layout(s, a.m, a.nnz, sizeof(T));
+    char* w = static_cast<char*>(region);
+    T* partials = reinterpret_cast<T*>(w + l.partials);
+    if (grid != 0) {
+        hipLaunchKernelGGL((spmv_banded_kernel<T>), dim3(grid), dim3(kBlock), 0, stream, a.m, a.n, a.nnz, a.base,
+                           s.band_shift, s.rows_per_tile, s.chunks, s.tiles,
+                           reinterpret_cast<const uint32_t*>(w + l.xcd_start),
+                           reinterpret_cast<const idx_t*>(w + l.tile_ptr), reinterpret_cast<const idx_t*>(w + l.entries),
+                           reinterpret_cast<const T*>(w + l.vals), static_cast<const T*>(a.x), partials);
+    }
+    const dim3 rows_grid((a.m + kBlock - 1) / kBlock);
+    if (beta == T(0)) {
+        hipLaunchKernelGGL((banded_reduce_kernel<T, true>), rows_grid, dim3(kBlock), 0, stream, a.m, s.bands,
+                           static_cast<const T*>(partials), static_cast<T*>(a.y), alpha, beta);
+    } else {
+        hipLaunchKernelGGL((banded_reduce_kernel<T, false>), rows_grid, dim3(kBlock), 0, stream, a.m, s.bands,
+                           static_cast<const T*>(partials), static_cast<T*>(a.y), alpha, beta);
+    }
+}
+
+template void launch_spmv_banded<float>(hipStream_t, const BandedShape&, uint32_t, const SpmvArgs&, float, float, void*);
+template void launch_spmv_banded<double>(hipStream_t, const BandedShape&, uint32_t, const SpmvArgs&, double, double, void*);
+
+}  // namespace mcsp

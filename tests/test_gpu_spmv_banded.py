@@ -1,0 +1,155 @@
+"""GPU parity of the column-banded SpMV (mcsparseSpMV_preprocess, then mcsparseSpMV on the same buffer)
+against the CPU oracle, within 8*u*(|alpha| * |A||x| + |beta*y|) as for every other SpMV family."""
+import glob
+import os
+
+import numpy as np
+import pytest
+
+from mcsparse_amd import api
+from mcsparse_amd import workloads as wl
+
+from gpu_util import assert_within, dev
+
+pytestmark = pytest.mark.gpu
+
+GOLDEN = sorted(glob.glob(os.path.join(os.path.dirname(__file__), "golden", "csr_*.npz")))
+
+
+def run_banded(torch, handle, oracle, a, alpha, beta, band_bytes=0, seed=1, expect_state=2, what="", calls=1):
+    rng = np.random.default_rng(seed)
+    dt = a.val.dtype
+    ct = api.maca_type(dt)
+    x = rng.uniform(-1, 1, a.n).astype(dt)
+    y = rng.uniform(-1, 1, a.m).astype(dt)
+    d_ptr, d_col, d_val, d_x, d_y = (dev(torch, v) for v in (a.ptr, a.col, a.val, x, y))
+    mat = api.SpMat(a.m, a.n, a.nnz, d_ptr, d_col, d_val, base=a.base)
+    if band_bytes:
+        mat.set_band_bytes(band_bytes)
+    vx, vy = api.DnVec(d_x), api.DnVec(d_y)
+    st, size = api.spmv_preprocess_buffer_size(handle, api.OP_N, alpha, mat, vx, beta, vy, ct)
+    assert st == api.STATUS_SUCCESS
+    buf = torch.empty(size, dtype=torch.uint8, device="cuda")
+    assert api.spmv_preprocess(handle, api.OP_N, alpha, mat, vx, beta, vy, ct, buf) == api.STATUS_SUCCESS
+    state, bands, rows = mat.spmv_preprocess_state()
+    assert state == expect_state, (state, bands, rows)
+    y_ref, bound = oracle.spmv(False, a.m, a.n, a.base, a.ptr, a.col, a.val, alpha, beta, x, y)
+    first = None
+    for _ in range(calls):
+        d_y.copy_(torch.from_numpy(y))
+        assert api.spmv(handle, api.OP_N, alpha, mat, vx, beta, vy, ct, buf) == api.STATUS_SUCCESS
+        torch.cuda.synchronize()
+        got = d_y.cpu().numpy()
+        assert_within(got, y_ref, bound, dt, what=what or "banded spmv")
+        if first is None:
+            first = got
+        else:  # fixed summation order: the same bits every time
+            assert np.array_equal(first.view(np.uint8), got.view(np.uint8))
+    return state, bands, rows
+
+
+@pytest.mark.parametrize("path", GOLDEN, ids=[os.path.basename(p)[:-4] for p in GOLDEN])
+@pytest.mark.parametrize("base", [0, 1])
+def test_golden_fixtures_banded(torch_gpu, handle, path, base):
+    """Integer-valued fixtures: every summation order is exact, so the result must equal the fixture's."""
+    torch = torch_gpu
+    with np.load(path) as z:
+        g = {k: z[k] for k in z.files}
+    for dt in (np.float32, np.float64):
+        a = wl.Csr(int(g["m"]), int(g["n"]), g["ptr"], g["col"], g["val"].astype(dt)).with_base(base)
+        ct = api.maca_type(dt)
+        alpha, beta = float(g["alpha"]), float(g["beta"])
+        d_ptr, d_col, d_val, d_x, d_y = (dev(torch, v) for v in (a.ptr, a.col, a.val, g["x"].astype(dt),
+                                                                   g["y0"].astype(dt)))
+        mat = api.SpMat(a.m, a.n, a.nnz, d_ptr, d_col, d_val, base=base)
+        mat.set_band_bytes(64)  # 16 or 8 columns per band: even these small fixtures are cut into several
+        vx, vy = api.DnVec(d_x), api.DnVec(d_y)
+        st, size = api.spmv_preprocess_buffer_size(handle, api.OP_N, alpha, mat, vx, beta, vy, ct)
+        assert st == api.STATUS_SUCCESS
+        buf = torch.empty(size, dtype=torch.uint8, device="cuda")
+        assert api.spmv_preprocess(handle, api.OP_N, alpha, mat, vx, beta, vy, ct, buf) == api.STATUS_SUCCESS
+        assert api.spmv(handle, api.OP_N, alpha, mat, vx, beta, vy, ct, buf) == api.STATUS_SUCCESS
+        torch.cuda.synchronize()
+        assert np.array_equal(d_y.cpu().numpy().astype(np.float64), g["y_n"])
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("base", [0, 1])
+@pytest.mark.parametrize("band_bytes", [1024, 8192, 1 << 16])
+def test_ragged_rows_small_bands(torch_gpu, handle, oracle, dtype, base, band_bytes):
+    # empty rows, rows that straddle bands, several bands per XCD and bands without entries in a chunk
+    a = wl.random_ragged(5003, 30011, 23, dtype=dtype, seed=band_bytes % 97, base=base)
+    state, bands, rows = run_banded(torch_gpu, handle, oracle, a, -0.75, 1.25, band_bytes=band_bytes, calls=2)
+    assert bands >= 2
+    run_banded(torch_gpu, handle, oracle, a, 2.0, 0.0, band_bytes=band_bytes)
+
+
+@pytest.mark.parametrize("per_row", [1, 3, 16, 61])
+def test_tiles_of_every_fill(torch_gpu, handle, oracle, per_row):
+    # per_row steers the rows per tile (32 .. 1024) and whether tiles need more than one slab
+    a = wl.uniform_rows(m=6000, n=50000, per_row=per_row, dtype=np.float64, config_id=20 + per_row)
+    run_banded(torch_gpu, handle, oracle, a, 1.5, 0.5, band_bytes=1 << 15)
+    b = wl.uniform_rows(m=3000, n=4000, per_row=min(per_row * 4, 200), dtype=np.float32, config_id=40 + per_row)
+    run_banded(torch_gpu, handle, oracle, b, 1.0, 0.0, band_bytes=4096)
+
+
+def test_default_band_width_config2_reduced(torch_gpu, handle, oracle):
+    a = wl.uniform_rows(m=1 << 16, n=1 << 20, per_row=16, dtype=np.float64)
+    state, bands, rows = run_banded(torch_gpu, handle, oracle, a, 1.5, 0.5, calls=2)
+    assert bands == 4
+
+
+def test_declined_structures_fall_back(torch_gpu, handle, oracle):
+    # x fits one band: nothing to do; long rows: left to the merge family.  SpMV still answers.
+    small = wl.random_ragged(2000, 3000, 9, dtype=np.float32, seed=3)
+    run_banded(torch_gpu, handle, oracle, small, 1.0, 0.0, expect_state=0)
+    long_rows = wl.power_law(m=1 << 14, n=1 << 20, max_len=20000, dtype=np.float32)
+    run_banded(torch_gpu, handle, oracle, long_rows, 1.0, 0.0, expect_state=1)
+
+
+def test_copy_is_dropped_with_the_arrays(torch_gpu, handle, oracle):
+    torch = torch_gpu
+    a = wl.uniform_rows(m=4000, n=30000, per_row=8, dtype=np.float32, config_id=77)
+    rng = np.random.default_rng(5)
+    x = rng.uniform(-1, 1, a.n).astype(np.float32)
+    d_ptr, d_col, d_val, d_x = (dev(torch, v) for v in (a.ptr, a.col, a.val, x))
+    d_y = torch.zeros(a.m, dtype=torch.float32, device="cuda")
+    mat = api.SpMat(a.m, a.n, a.nnz, d_ptr, d_col, d_val)
+    mat.set_band_bytes(8192)
+    vx, vy = api.DnVec(d_x), api.DnVec(d_y)
+    st, size = api.spmv_preprocess_buffer_size(handle, api.OP_N, 1.0, mat, vx, 0.0, vy, api.R_32F)
+    buf = torch.empty(size, dtype=torch.uint8, device="cuda")
+    assert api.spmv_preprocess(handle, api.OP_N, 1.0, mat, vx, 0.0, vy, api.R_32F, buf) == api.STATUS_SUCCESS
+    assert mat.spmv_preprocess_state()[0] == 2
+    # new values through the descriptor: the copy (which holds the old ones) must not be used
+    new_val = rng.uniform(-1, 1, a.nnz).astype(np.float32)
+    d_new = dev(torch, new_val)
+    assert mat.lib.mcsparseSpMatSetValues(mat.ptr, d_new.data_ptr()) == 0
+    assert mat.spmv_preprocess_state()[0] == 0
+    assert api.spmv(handle, api.OP_N, 1.0, mat, vx, 0.0, vy, api.R_32F, buf) == api.STATUS_SUCCESS
+    torch.cuda.synchronize()
+    y_ref, bound = oracle.spmv(False, a.m, a.n, 0, a.ptr, a.col, new_val, 1.0, 0.0, x, np.zeros(a.m, np.float32))
+    assert_within(d_y.cpu().numpy(), y_ref, bound, np.float32, what="after SetValues")
+
+
+def test_overwritten_buffer_stays_in_bounds(torch_gpu, handle, oracle):
+    """A caller that scribbles over the buffer after preprocess gets wrong numbers, not a fault."""
+    torch = torch_gpu
+    a = wl.uniform_rows(m=4000, n=30000, per_row=8, dtype=np.float64, config_id=78)
+    d_ptr, d_col, d_val = (dev(torch, v) for v in (a.ptr, a.col, a.val))
+    d_x = torch.ones(a.n, dtype=torch.float64, device="cuda")
+    d_y = torch.zeros(a.m, dtype=torch.float64, device="cuda")
+    mat = api.SpMat(a.m, a.n, a.nnz, d_ptr, d_col, d_val)
+    mat.set_band_bytes(1 << 14)
+    vx, vy = api.DnVec(d_x), api.DnVec(d_y)
+    st, size = api.spmv_preprocess_buffer_size(handle, api.OP_N, 1.0, mat, vx, 0.0, vy, api.R_64F)
+    buf = torch.empty(size, dtype=torch.uint8, device="cuda")
+    assert api.spmv_preprocess(handle, api.OP_N, 1.0, mat, vx, 0.0, vy, api.R_64F, buf) == api.STATUS_SUCCESS
+    buf.fill_(0xFF)
+    assert api.spmv(handle, api.OP_N, 1.0, mat, vx, 0.0, vy, api.R_64F, buf) == api.STATUS_SUCCESS
+    torch.cuda.synchronize()
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(1)
+    buf.copy_(torch.randint(0, 256, (size,), dtype=torch.uint8, device="cuda", generator=gen))
+    assert api.spmv(handle, api.OP_N, 1.0, mat, vx, 0.0, vy, api.R_64F, buf) == api.STATUS_SUCCESS
+    torch.cuda.synchronize()
