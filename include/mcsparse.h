@@ -464,6 +464,22 @@ mcsparseStatus_t mcsparseSpMatGetSpMVPreprocess(mcsparseSpMatDescr_t spMatDescr,
  * rounded down to a power of two).  Drops a banded copy already built.  For tests and benchmarks. */
 mcsparseStatus_t mcsparseSpMatSetSpMVBandBytes(mcsparseSpMatDescr_t spMatDescr, size_t band_bytes);
 
+/* mcsparseSpMV without an externalBuffer, for callers that cannot allocate device memory: code
+ * under HIP graph capture, serving loops and harnesses that forbid hipMalloc.  No counterpart in
+ * the reference.  The scratch lives in a device array of MCSPARSE_SPMV_STATIC_BUFFER_BYTES inside
+ * the library (one copy per GPU the library runs on, held until the process ends); a call whose
+ * scratch need (what mcsparseSpMV_bufferSize reports) exceeds it returns
+ * MCSPARSE_STATUS_INSUFFICIENT_RESOURCES and launches nothing.  The call allocates nothing and
+ * copies nothing to the host: it needs MCSPARSE_POINTER_MODE_HOST (NOT_SUPPORTED otherwise), and a
+ * structure that has no SpMV plan yet runs the merge-path family instead of being analysed.
+ * Results are those of mcsparseSpMV with the same kernel family.  All calls on one GPU share the
+ * array: calls that overlap in time on one GPU (different streams or threads) race. */
+#define MCSPARSE_SPMV_STATIC_BUFFER_BYTES (4u << 20)
+mcsparseStatus_t mcsparseSpMV_staticBuffer(mcsparseHandle_t handle, mcsparseOperation_t opA, const void* alpha,
+                                           mcsparseSpMatDescr_t matA, mcsparseDnVecDescr_t vecX, const void* beta,
+                                           mcsparseDnVecDescr_t vecY, macaDataType computeType,
+                                           mcsparseSpMVAlg_t alg);
+
 #if defined(__GNUC__)
 #pragma GCC visibility pop
 #endif

@@ -56,6 +56,7 @@ PROTOTYPES = {
     "mcsparseDnMatSetStridedBatch": (c_int, [vp, c_int, c_i64]),
     "mcsparseDnMatGetStridedBatch": (c_int, [vp, P(c_int), P(c_i64)]),
     "mcsparseSpMV": (c_int, [vp, c_int, vp, vp, vp, vp, vp, c_int, c_int, vp]),
+    "mcsparseSpMV_staticBuffer": (c_int, [vp, c_int, vp, vp, vp, vp, vp, c_int, c_int]),
     "mcsparseSpMV_preprocess_bufferSize": (c_int, [vp, c_int, vp, vp, vp, vp, vp, c_int, c_int, P(c_size)]),
     "mcsparseSpMV_preprocess": (c_int, [vp, c_int, vp, vp, vp, vp, vp, c_int, c_int, vp]),
     "mcsparseSpMatSetSpMVBandBytes": (c_int, [vp, c_size]),

@@ -252,6 +252,13 @@ def spmv_preprocess(handle, op, alpha, mat, x, beta, y, compute_type, buffer):
                                               y.ptr, compute_type, SPMV_ALG_DEFAULT, _ptr(buffer))
 
 
+def spmv_static_buffer(handle, op, alpha, mat, x, beta, y, compute_type):
+    """mcsparseSpMV_staticBuffer: host scalars only, scratch inside the library."""
+    a, b = _scalar(alpha, compute_type), _scalar(beta, compute_type)
+    return handle.lib.mcsparseSpMV_staticBuffer(handle.ptr, op, ctypes.addressof(a), mat.ptr, x.ptr,
+                                                ctypes.addressof(b), y.ptr, compute_type, SPMV_ALG_DEFAULT)
+
+
 def spmm_buffer_size(handle, op_a, op_b, alpha, mat, B, beta, C, compute_type):
     size = ctypes.c_size_t(0)
     a, b = _scalar(alpha, compute_type), _scalar(beta, compute_type)
