@@ -7,13 +7,16 @@ A step is one pass of the hot path (one mcsparseSpMV / mcsparseSpMM / mcsparseCs
 through the C ABI) over one synthetic operand set that is already resident in HBM.  Several
 independent copies of all operands are rotated so the 256 MB Infinity Cache cannot hold a
 matrix between steps.  The default workload is the configuration the metric is quoted on:
-fp64 CSR SpMV, 1,048,576 rows x 16 nonzeros per row.  Prints one JSON line.
+fp64 CSR SpMV, 1,048,576 rows x 16 nonzeros per row.  Prints one JSON line; the default
+invocation also measures the other configurations (fewer steps each, inside a wall-clock budget)
+and reports them under "others" of the same line.
 
 Workloads: c1 (5-pt Laplacian 256^2 fp32), c2 (default), c3 / c3t (power-law fp32, op N / T),
-c4-8 / c4-64 / c4-256 (27-pt stencil 128^3 SpMM), c5 (csr2csc on the c3 matrix),
-c5-coo (csr2coo on it), c5-spmv (A^T x from the converted CSC).  Probes: copy (a plain device copy, the
-yardstick of the traffic counters), gather-probe (16.8 M random 8-byte reads of an 8 MB table
-through mcsparseDgthr: what the x[col] reads of c2 cost on their own).
+c4-8 / c4-64 / c4-256 (27-pt stencil 128^3 SpMM, row-major B and C), c4-64-col (the same with
+column-major B and C, the layout of csrmm2), c5 (csr2csc on the c3 matrix), c5-coo (csr2coo on it),
+c5-spmv (A^T x from the converted CSC).  Probes: copy (a plain device copy, the yardstick of the
+traffic counters), gather-probe (16.8 M random 8-byte reads through mcsparseDgthr: what the x[col]
+reads of c2 cost on their own, from an 8 MB table and from one that fits every L2).
 """
 import argparse
 import json
@@ -28,23 +31,31 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 
+OTHERS = ["c4-64", "c3", "c3t", "c5", "c5-spmv", "c5-coo", "c4-8", "c4-256", "c4-64-col", "c1"]
+OTHERS_BUDGET_S = 200.0  # wall-clock budget of the default invocation for the workloads above
+
+
 # HBM/fabric bytes per call (all kernels of one step together), from rocprofv3 FETCH_SIZE and
 # WRITE_SIZE, each scaled by what the same counter reads on a 1 GiB copy: 2 KiB and 1 KiB per
-# count.  The counter summaries are kept under profiles/.
+# count.  These are constants taken from the counter summaries under profiles/ (named beside each),
+# not counters read during the run.
 def _traffic(fetch_counts, write_counts):
     return int((fetch_counts * 2 + write_counts) * 1024)
 
 
-MEASURED_TRAFFIC_BYTES = {
-    "c2": _traffic(653890.5, 10048.5),                      # spmv_vector_kernel<double, 16, 4>
+MEASURED_TRAFFIC = {
+    # spmv_banded_kernel<double> + banded_reduce_kernel<double>
+    "c2": (_traffic(111459.5 + 20554.1, 32768.0 + 8192.0), "profiles/spmv_banded_f64_c2_1Mx16.txt"),
     # merge kernel (tiles in column order) + partition + tile order + fix-up
-    "c3": _traffic(3305285.9 + 17229.2 + 251.2 + 3154.3, 25157.0 + 1391.2 + 1994.3 + 1375.1),
-    "c4-64": _traffic(613893.3, 524288.0),                 # spmm_group_kernel<float, 16>
-    "c4-256": _traffic(3673719.8, 2097152.0),              # spmm_group_kernel<float, 64>
+    "c3": (_traffic(3305285.9 + 17229.2 + 251.2 + 3154.3, 25157.0 + 1391.2 + 1994.3 + 1375.1),
+           "profiles/spmv_merge_f32_c3_powerlaw.txt"),
+    "c4-64": (_traffic(613893.3, 524288.0), "profiles/spmm_group_f32_c4_stencil128.txt"),
+    "c4-256": (_traffic(3673719.8, 2097152.0), "profiles/spmm_group_f32_c4_stencil128.txt"),
     # csr2csc: 2 x scatter + the scatter that reads the CSR arrays in place + 3 x (histogram + scans)
     # + row starts per tile + coo2csr
-    "c5": _traffic(2 * 701979.0 + 481119.4 + 3 * (229171.1 + 2 * 7206.6 + 14342.5) + 21136.0 + 237161.6,
-                   2 * 1387754.6 + 1421432.8 + 3 * (28789.0 + 2 * 14326.3 + 56.0) + 223.8 + 19514.6),
+    "c5": (_traffic(2 * 701979.0 + 481119.4 + 3 * (229171.1 + 2 * 7206.6 + 14342.5) + 21136.0 + 237161.6,
+                    2 * 1387754.6 + 1421432.8 + 3 * (28789.0 + 2 * 14326.3 + 56.0) + 223.8 + 19514.6),
+           "profiles/csr2csc_radix_f32_c5_powerlaw.txt"),
 }
 
 
@@ -57,75 +68,79 @@ def parse():
     p.add_argument("--copies", type=int, default=None, help="independent operand sets rotated between steps")
     p.add_argument("--scale", type=float, default=1.0, help="shrink the workload (for dry runs); 1.0 = as specified")
     p.add_argument("--no-cpu-baseline", action="store_true")
-    p.add_argument("--no-preprocess", action="store_true", help="SpMM workloads: skip mcsparseSpMM_preprocess")
+    p.add_argument("--no-preprocess", action="store_true",
+                   help="skip mcsparseSpMV_preprocess / mcsparseSpMM_preprocess (the reference has neither)")
+    p.add_argument("--no-others", action="store_true", help="default invocation: measure the headline workload only")
     p.add_argument("--family", type=int, default=0, help="force the SpMV kernel family (1 vector, 2 merge)")
     p.add_argument("--lanes", type=int, default=0, help="force lanes per row of the vector family")
+    p.add_argument("--band-bytes", type=int, default=0, help="band width of mcsparseSpMV_preprocess (0 = default)")
     p.add_argument("--cache", default=None, help="directory to keep generated matrices in between runs")
     return p.parse_args()
 
 
-def main():
-    args = parse()
-    if args.gpus != 1:
-        print("bench.py measures one GPU: this path has no multi-GPU part (got --gpus %d)" % args.gpus,
-              file=sys.stderr)
-        return 2
+class Matrices:
+    """Generated matrices, kept for the workloads that share one (c3, c3t, c5*)."""
 
-    import torch
-    from mcsparse_amd import api
-    from mcsparse_amd import workloads as wl
+    def __init__(self, wl, scale, cache):
+        self.wl, self.s, self.cache, self.have = wl, scale, cache, {}
 
-    if not torch.cuda.is_available():
-        print("bench.py needs a GPU", file=sys.stderr)
-        return 2
-    torch.cuda.set_device(0)
-    stream = torch.cuda.current_stream()
-    handle = api.Handle(stream=stream.cuda_stream)
-    name = args.workload
+    def get(self, key):
+        if key in self.have:
+            return self.have[key]
+        wl, s = self.wl, self.s
+        if key == "laplacian":
+            a = wl.laplacian_5pt(max(4, int(256 * s)), dtype=np.float32)
+        elif key == "uniform":
+            a = wl.uniform_rows(m=max(64, int((1 << 20) * s)), per_row=16, dtype=np.float64)
+        elif key == "power_law":
+            a = cached(self.cache, "power_law_%g" % s, lambda: wl.power_law(
+                m=max(64, int((1 << 22) * s)), max_len=max(8, int(200000 * min(1.0, s * 4))), dtype=np.float32))
+        elif key == "stencil":
+            a = wl.stencil_27pt(max(4, int(round(128 * s ** (1 / 3)))), dtype=np.float32)
+        else:
+            raise KeyError(key)
+        self.have = {key: a}  # one at a time: the power-law matrix alone is 1.4 GB on the host
+        return a
+
+
+def describe(name):
+    """(matrix key, kind, op is T, dense columns, alpha, beta, description) of a workload."""
+    if name == "c1":
+        return "laplacian", "spmv", False, 0, 1.0, 0.0, "fp32 CSR SpMV, 5-pt Laplacian 256x256"
+    if name == "c2":
+        return "uniform", "spmv", False, 0, 1.5, 0.5, "fp64 CSR SpMV, 1048576 rows x 16 nnz/row uniform"
+    pl = "fp32 CSR SpMV, 4194304 rows power-law (Zipf 1.8, <=200000 nnz/row)"
+    if name == "c3":
+        return "power_law", "spmv", False, 0, 1.0, 0.0, pl
+    if name == "c3t":
+        return "power_law", "spmv", True, 0, 1.0, 0.0, pl + ", op T"
+    if name == "c5":
+        return "power_law", "csr2csc", False, 0, 1.0, 0.0, "csr2csc (values + structure) of the fp32 power-law matrix"
+    if name == "c5-coo":
+        return "power_law", "csr2coo", False, 0, 1.0, 0.0, "csr2coo of the power-law matrix"
+    if name == "c5-spmv":
+        return ("power_law", "spmv-csc", False, 0, 1.0, 0.0,
+                "fp32 SpMV op T from the CSC produced by csr2csc (power-law matrix)")
+    if name.startswith("c4-"):
+        parts = name.split("-")
+        n_cols = int(parts[1])
+        col_major = len(parts) > 2 and parts[2] == "col"
+        return ("stencil", "spmm-col" if col_major else "spmm", False, n_cols, 1.0, 0.0,
+                "fp32 CSR SpMM, 27-pt stencil 128^3, B and C %s N=%d" % ("column-major" if col_major else "row-major",
+                                                                      n_cols))
+    raise KeyError(name)
+
+
+def run_workload(name, args, ctx, steps=None, warmup=None, with_cpu=True):
+    """Measures one workload; returns the JSON object of its line."""
+    torch, api, wl, handle, stream = ctx["torch"], ctx["api"], ctx["wl"], ctx["handle"], ctx["stream"]
+    key, kind, op_t, n_cols, alpha, beta, desc = describe(name)
+    a = ctx["matrices"].get(key)
+    op = api.OP_T if op_t else api.OP_N
     s = args.scale
 
-    def dev(a):
-        return torch.from_numpy(np.ascontiguousarray(a)).cuda()
-
-    t_gen = time.time()
-    kind = "spmv"
-    op = api.OP_N
-    n_cols = 0
-    if name == "c1":
-        a = wl.laplacian_5pt(max(4, int(256 * s)), dtype=np.float32)
-        alpha, beta, desc = 1.0, 0.0, "fp32 CSR SpMV, 5-pt Laplacian 256x256"
-    elif name == "c2":
-        a = wl.uniform_rows(m=max(64, int((1 << 20) * s)), per_row=16, dtype=np.float64)
-        alpha, beta, desc = 1.5, 0.5, "fp64 CSR SpMV, 1048576 rows x 16 nnz/row uniform"
-    elif name in ("c3", "c3t", "c5", "c5-coo", "c5-spmv"):
-        a = cached(args.cache, "power_law_%g" % s, lambda: wl.power_law(
-            m=max(64, int((1 << 22) * s)), max_len=max(8, int(200000 * min(1.0, s * 4))), dtype=np.float32))
-        alpha, beta = 1.0, 0.0
-        desc = "fp32 CSR SpMV, 4194304 rows power-law (Zipf 1.8, <=200000 nnz/row)"
-        if name == "c3t":
-            op = api.OP_T
-            desc += ", op T"
-        if name == "c5":
-            kind, desc = "csr2csc", "csr2csc (values + structure) of the fp32 power-law matrix"
-        if name == "c5-coo":
-            kind, desc = "csr2coo", "csr2coo of the power-law matrix"
-        if name == "c5-spmv":
-            kind, desc = "spmv-csc", "fp32 SpMV op T from the CSC produced by csr2csc (power-law matrix)"
-    elif name.startswith("c4-"):
-        n_cols = int(name.split("-")[1])
-        a = wl.stencil_27pt(max(4, int(round(128 * s ** (1 / 3)))), dtype=np.float32)
-        alpha, beta, kind = 1.0, 0.0, "spmm"
-        desc = "fp32 CSR SpMM, 27-pt stencil 128^3, B row-major N=%d" % n_cols
-    elif name == "copy":
-        # plain device copy of known size: the yardstick the rocprofv3 FETCH_SIZE / WRITE_SIZE
-        # counters are scaled by
-        return copy_probe(torch, args)
-    elif name == "gather-probe":
-        return gather_probe(torch, api, handle, args)
-    else:
-        print("unknown workload %r" % name, file=sys.stderr)
-        return 2
-    gen_s = time.time() - t_gen
+    def dev(v):
+        return torch.from_numpy(np.ascontiguousarray(v)).cuda()
 
     dt = a.val.dtype
     vb = dt.itemsize
@@ -135,7 +150,7 @@ def main():
         algo_bytes = wl.spmv_bytes(a, vb)
         flops = 2 * a.nnz
         extra_read = a.m * vb if beta != 0 else 0
-    elif kind == "spmm":
+    elif kind in ("spmm", "spmm-col"):
         algo_bytes = wl.spmm_bytes(a, n_cols, vb)
         flops = 2 * a.nnz * n_cols
         extra_read = 0
@@ -150,12 +165,36 @@ def main():
     copies = args.copies or max(2, min(8, int(np.ceil(1.2e9 / max(algo_bytes, 1)))))
     if algo_bytes > 8e8:
         copies = args.copies or 2
-    steps = args.steps if args.steps is not None else (200 if algo_bytes < 6e8 else 40)
-    warmup = args.warmup if args.warmup is not None else (20 if algo_bytes < 6e8 else 5)
+    if steps is None:
+        steps = args.steps if args.steps is not None else (200 if algo_bytes < 6e8 else 40)
+    if warmup is None:
+        warmup = args.warmup if args.warmup is not None else (20 if algo_bytes < 6e8 else 5)
 
     rng = np.random.default_rng(12345)
     sets = []
     preprocess_ms = []
+
+    def timed(call, what):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        api.check(call(), what)
+        torch.cuda.synchronize()
+        preprocess_ms.append((time.perf_counter() - t0) * 1e3)
+
+    def spmv_buffer(st, the_op, fmt_is_csr):
+        """Scratch of an SpMV set: with preprocessing, the larger buffer the banded copy lives in."""
+        direct = (the_op == api.OP_N) == fmt_is_csr  # CSR op N or CSC op T: the row kernels run as the arrays lie
+        use_pre = not args.no_preprocess and direct and not (args.family or args.lanes)
+        if use_pre:
+            rc, size = api.spmv_preprocess_buffer_size(handle, the_op, alpha, st["mat"], st["vx"], beta, st["vy"], ct)
+        else:
+            rc, size = api.spmv_buffer_size(handle, the_op, alpha, st["mat"], st["vx"], beta, st["vy"], ct)
+        api.check(rc, "mcsparseSpMV_bufferSize")
+        st["buf"] = torch.empty(size, dtype=torch.uint8, device="cuda")
+        if use_pre:
+            timed(lambda: api.spmv_preprocess(handle, the_op, alpha, st["mat"], st["vx"], beta, st["vy"], ct, st["buf"]),
+                  "mcsparseSpMV_preprocess")
+
     for c in range(copies):
         st = {"ptr": dev(a.ptr), "col": dev(a.col), "val": dev(a.val)}
         if kind == "spmv":
@@ -165,26 +204,25 @@ def main():
             st["mat"] = api.SpMat(a.m, a.n, a.nnz, st["ptr"], st["col"], st["val"], base=a.base)
             if args.family or args.lanes:
                 st["mat"].set_plan(args.family, args.lanes)
+            if args.band_bytes:
+                st["mat"].set_band_bytes(args.band_bytes)
             st["vx"], st["vy"] = api.DnVec(st["x"]), api.DnVec(st["y"])
-            rc, size = api.spmv_buffer_size(handle, op, alpha, st["mat"], st["vx"], beta, st["vy"], ct)
-            api.check(rc, "mcsparseSpMV_bufferSize")
-            st["buf"] = torch.empty(size, dtype=torch.uint8, device="cuda")
-        elif kind == "spmm":
-            st["B"] = dev(rng.uniform(-1, 1, (a.n, n_cols)).astype(dt))
-            st["C"] = torch.zeros((a.m, n_cols), dtype=tdt, device="cuda")
+            spmv_buffer(st, op, True)
+        elif kind in ("spmm", "spmm-col"):
+            row_major = kind == "spmm"
+            order = api.ORDER_ROW if row_major else api.ORDER_COL
+            shape_b, shape_c = ((a.n, n_cols), (a.m, n_cols)) if row_major else ((n_cols, a.n), (n_cols, a.m))
+            st["B"] = dev(rng.uniform(-1, 1, shape_b).astype(dt))
+            st["C"] = torch.zeros(shape_c, dtype=tdt, device="cuda")
             st["mat"] = api.SpMat(a.m, a.n, a.nnz, st["ptr"], st["col"], st["val"], base=a.base)
-            st["mB"] = api.DnMat(a.n, n_cols, n_cols, st["B"], order=api.ORDER_ROW)
-            st["mC"] = api.DnMat(a.m, n_cols, n_cols, st["C"], order=api.ORDER_ROW)
+            st["mB"] = api.DnMat(a.n, n_cols, n_cols if row_major else a.n, st["B"], order=order)
+            st["mC"] = api.DnMat(a.m, n_cols, n_cols if row_major else a.m, st["C"], order=order)
             rc, size = api.spmm_buffer_size(handle, api.OP_N, api.OP_N, alpha, st["mat"], st["mB"], beta, st["mC"], ct)
             api.check(rc, "mcsparseSpMM_bufferSize")
             st["buf"] = torch.empty(size, dtype=torch.uint8, device="cuda")
             if not args.no_preprocess:
-                torch.cuda.synchronize()
-                t_pre = time.perf_counter()
-                api.check(api.spmm_preprocess(handle, api.OP_N, api.OP_N, alpha, st["mat"], st["mB"], beta, st["mC"],
-                                              ct, st["buf"]), "mcsparseSpMM_preprocess")
-                torch.cuda.synchronize()
-                preprocess_ms.append((time.perf_counter() - t_pre) * 1e3)
+                timed(lambda: api.spmm_preprocess(handle, api.OP_N, api.OP_N, alpha, st["mat"], st["mB"], beta,
+                                                  st["mC"], ct, st["buf"]), "mcsparseSpMM_preprocess")
         elif kind in ("csr2csc", "spmv-csc"):
             st["o_val"] = torch.zeros(a.nnz, dtype=tdt, device="cuda")
             st["o_ptr"] = torch.zeros(a.n + 1, dtype=torch.int32, device="cuda")
@@ -197,17 +235,17 @@ def main():
                 api.check(api.csr2csc(handle, a.m, a.n, a.nnz, st["val"], st["ptr"], st["col"], st["o_val"],
                                       st["o_ptr"], st["o_row"], ct, api.ACTION_NUMERIC, a.base, st["buf"]))
                 torch.cuda.synchronize()
-                del st["buf"]
+                del st["buf"], st["ptr"], st["col"], st["val"]
                 st["x"] = dev(rng.uniform(-1, 1, a.m).astype(dt))
                 st["y"] = dev(rng.uniform(-1, 1, a.n).astype(dt))
                 st["mat"] = api.SpMat(a.m, a.n, a.nnz, st["o_ptr"], st["o_row"], st["o_val"], base=a.base,
                                       fmt=api.FORMAT_CSC)
                 if args.family or args.lanes:
                     st["mat"].set_plan(args.family, args.lanes)
+                if args.band_bytes:
+                    st["mat"].set_band_bytes(args.band_bytes)
                 st["vx"], st["vy"] = api.DnVec(st["x"]), api.DnVec(st["y"])
-                rc, size = api.spmv_buffer_size(handle, api.OP_T, alpha, st["mat"], st["vx"], beta, st["vy"], ct)
-                api.check(rc)
-                st["buf"] = torch.empty(size, dtype=torch.uint8, device="cuda")
+                spmv_buffer(st, api.OP_T, False)
         else:
             st["coo"] = torch.zeros(a.nnz, dtype=torch.int32, device="cuda")
         sets.append(st)
@@ -218,7 +256,7 @@ def main():
             rc = api.spmv(handle, op, alpha, st["mat"], st["vx"], beta, st["vy"], ct, st["buf"])
         elif kind == "spmv-csc":
             rc = api.spmv(handle, api.OP_T, alpha, st["mat"], st["vx"], beta, st["vy"], ct, st["buf"])
-        elif kind == "spmm":
+        elif kind in ("spmm", "spmm-col"):
             rc = api.spmm(handle, api.OP_N, api.OP_N, alpha, st["mat"], st["mB"], beta, st["mC"], ct, st["buf"])
         elif kind == "csr2csc":
             rc = api.csr2csc(handle, a.m, a.n, a.nnz, st["val"], st["ptr"], st["col"], st["o_val"], st["o_ptr"],
@@ -228,7 +266,7 @@ def main():
         if rc != 0:
             raise api.McsparseError(rc, "step")
 
-    # one-time preprocessing (row-length analysis per descriptor), timed apart from the steady state
+    # the first call on a structure (row-length analysis of a descriptor that has no plan yet)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for i in range(copies):
@@ -255,7 +293,12 @@ def main():
 
     value = algo_bytes / (ms_per_step * 1e-3) / 1e9
     achieved = algo_bytes / (dev_avg_ms * 1e-3) / 1e9
-    plan = sets[0]["mat"].plan() if "mat" in sets[0] and kind != "spmm" else None
+    mat0 = sets[0].get("mat")
+    plan = mat0.plan() if mat0 is not None and kind in ("spmv", "spmv-csc") else None
+    banded = mat0.spmv_preprocess_state() if mat0 is not None and kind in ("spmv", "spmv-csc") else None
+    traffic = MEASURED_TRAFFIC.get(name) if s == 1.0 else None
+    if traffic is not None and name == "c2" and not (banded and banded[0] == 2):
+        traffic = None  # the constant belongs to the banded kernels
 
     out = {
         "metric": "CSR SpMV/SpMM achieved HBM GB/s (% of MI355X peak) + GFLOP/s at 1 GPU",
@@ -278,17 +321,78 @@ def main():
         "algorithmic_bytes_per_step": int(algo_bytes),
         "extra_bytes_not_counted": int(extra_read),
         "first_call_ms": round(first_pass_ms, 4),
-        "spmm_preprocess_ms": round(min(preprocess_ms), 4) if preprocess_ms else None,
+        "preprocess_ms": round(min(preprocess_ms), 4) if preprocess_ms else None,
         "device_ms_per_step": {"mean": round(dev_avg_ms, 5), "median": round(float(np.median(dev_ms)), 5),
                                "min": round(float(dev_ms.min()), 5)},
         "spmv_plan": {"family": plan[0], "lanes_per_row": plan[1]} if plan else None,
+        "spmv_preprocess": {"state": banded[0], "bands": banded[1], "rows_per_tile": banded[2]} if banded else None,
         "roofline": {"bound": "hbm", "achieved": round(achieved, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4),
-                     "traffic": MEASURED_TRAFFIC_BYTES.get(name) if s == 1.0 else None},
+                     "traffic": traffic[0] if traffic else None,
+                     "traffic_source": ("constant from " + traffic[1]) if traffic else None},
     }
+    del sets
+    torch.cuda.empty_cache()
+    if with_cpu and not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(kind, a, alpha, beta, n_cols, algo_bytes, op_t)
+    return out
 
-    if not args.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline(kind, a, alpha, beta, n_cols, algo_bytes, op)
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this path has no multi-GPU part (got --gpus %d)" % args.gpus,
+              file=sys.stderr)
+        return 2
+
+    import torch
+    from mcsparse_amd import api
+    from mcsparse_amd import workloads as wl
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        return 2
+    torch.cuda.set_device(0)
+    stream = torch.cuda.current_stream()
+    handle = api.Handle(stream=stream.cuda_stream)
+    name = args.workload
+    if name == "copy":
+        # plain device copy of known size: the yardstick the rocprofv3 FETCH_SIZE / WRITE_SIZE
+        # counters are scaled by
+        return copy_probe(torch, args)
+    if name == "gather-probe":
+        return gather_probe(torch, api, handle, args)
+    try:
+        describe(name)
+    except (KeyError, ValueError, IndexError):
+        print("unknown workload %r" % name, file=sys.stderr)
+        return 2
+
+    ctx = {"torch": torch, "api": api, "wl": wl, "handle": handle, "stream": stream,
+           "matrices": Matrices(wl, args.scale, args.cache)}
+    t_start = time.perf_counter()
+    out = run_workload(name, args, ctx)
+
+    # The default invocation also measures the other configurations, each with fewer steps, while the
+    # wall-clock budget lasts; what does not fit is named under "others_skipped".
+    default_run = (name == "c2" and args.steps is None and args.warmup is None and not args.no_others and
+                   not (args.family or args.lanes or args.band_bytes or args.copies))
+    if default_run:
+        others, skipped = {}, []
+        for w in OTHERS:
+            if time.perf_counter() - t_start > OTHERS_BUDGET_S:
+                skipped.append(w)
+                continue
+            r = run_workload(w, args, ctx, steps=12, warmup=3)
+            others[w] = {k: r[k] for k in ("value", "unit", "ms_per_step", "pct_of_hbm_peak", "gflops", "steps",
+                                           "algorithmic_bytes_per_step", "device_ms_per_step", "preprocess_ms",
+                                           "first_call_ms", "spmv_plan", "spmv_preprocess", "roofline") if k in r}
+            others[w]["workload"] = r["config"]["workload"]
+            others[w]["nnz"] = r["config"]["nnz"]
+            if "cpu_baseline" in r:
+                others[w]["cpu_baseline"] = r["cpu_baseline"]
+        out["others"] = others
+        out["others_skipped"] = skipped
     print(json.dumps(out))
     return 0
 
@@ -311,14 +415,15 @@ def copy_probe(torch, args):
 
 def gather_probe(torch, api, handle, args):
     """x_val[i] = y[x_ind[i]] for as many uniformly random indices as c2 has nonzeros, from a table
-    the size of c2's x, and from one that fits every L2: the cost of the gathers of a random-column
-    SpMV with everything else (row offsets, values, sums) taken away."""
+    the size of c2's x, from one band of the banded layout (2 MiB) and from one that fits every L2:
+    the cost of the gathers of a random-column SpMV with everything else (row offsets, values, sums)
+    taken away.  mcsparseDgthr runs eight independent gathers per thread, like the SpMV kernels."""
     count = 1 << 24
     steps = args.steps or 20
     rng = np.random.default_rng(7)
     out = {"workload": "gather-probe", "gathers": count, "element_bytes": 8, "steps": steps, "tables": []}
     stream = torch.cuda.current_stream()
-    for table_elems in (1 << 17, 1 << 20):
+    for table_elems in (1 << 17, 1 << 18, 1 << 20):
         ind = torch.from_numpy(rng.integers(0, table_elems, count, dtype=np.int32)).cuda()
         table = torch.rand(table_elems, dtype=torch.float64, device="cuda")
         dst = torch.zeros(count, dtype=torch.float64, device="cuda")
@@ -353,35 +458,52 @@ def cached(directory, key, make):
     return a
 
 
-def cpu_baseline(kind, a, alpha, beta, n_cols, algo_bytes, op):
-    """Times the oracle's OpenMP port of the same semantics on the host cores (reported only)."""
+def host_cpu_model():
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+def cpu_baseline(kind, a, alpha, beta, n_cols, algo_bytes, op_t):
+    """Times the oracle's OpenMP port of the same semantics on the host cores (reported only).
+
+    The port is compiled for the host it runs on (-march=native) when a compiler is at hand, and
+    the operands are copied into pages that the OpenMP threads touch first, with the schedule of
+    the compute loops."""
     import oracle
-    from mcsparse_amd import api
-    oracle.build()
+    tuned = oracle.use_native_build()
     threads = oracle.max_threads()
     rng = np.random.default_rng(1)
     dt = a.val.dtype
-    if kind == "spmv" and op == api.OP_N:
-        x = rng.uniform(-1, 1, a.n).astype(dt)
-        y = rng.uniform(-1, 1, a.m).astype(dt)
+    ft = oracle.first_touch_copy
+    ptr, col, val = ft(a.ptr), ft(a.col), ft(a.val)
+    if kind == "spmv" and not op_t:
+        x = ft(rng.uniform(-1, 1, a.n).astype(dt))
+        y = ft(rng.uniform(-1, 1, a.m).astype(dt))
         dyn = int(a.row_lengths().max()) > 4096
 
         def run():
-            oracle.spmv_omp(a.m, a.base, a.ptr, a.col, a.val, alpha, beta, x, y, dynamic=dyn)
+            oracle.spmv_omp(a.m, a.base, ptr, col, val, alpha, beta, x, y, dynamic=dyn)
         sample = "whole workload per repetition"
     elif kind == "spmv":
         # op T as the reference does it: transpose on every call, then the row loop
-        x = rng.uniform(-1, 1, a.m).astype(dt)
-        y = rng.uniform(-1, 1, a.n).astype(dt)
+        x = ft(rng.uniform(-1, 1, a.m).astype(dt))
+        y = ft(rng.uniform(-1, 1, a.n).astype(dt))
 
         def run():
-            cp, ri, cv = oracle.csr2csc(a.m, a.n, a.base, a.ptr, a.col, a.val, method="omp")
+            cp, ri, cv = oracle.csr2csc(a.m, a.n, a.base, ptr, col, val, method="omp")
             oracle.spmv_omp(a.n, a.base, cp, ri, cv, alpha, beta, x, y, dynamic=True)
         sample = "whole workload per repetition (csr2csc + row loop over the transpose)"
     elif kind == "spmv-csc":
-        cp, ri, cv = oracle.csr2csc(a.m, a.n, a.base, a.ptr, a.col, a.val, method="omp")
-        x = rng.uniform(-1, 1, a.m).astype(dt)
-        y = rng.uniform(-1, 1, a.n).astype(dt)
+        cp, ri, cv = oracle.csr2csc(a.m, a.n, a.base, ptr, col, val, method="omp")
+        cp, ri, cv = ft(cp), ft(ri), ft(cv)
+        x = ft(rng.uniform(-1, 1, a.m).astype(dt))
+        y = ft(rng.uniform(-1, 1, a.n).astype(dt))
         dyn = int(np.diff(cp.astype(np.int64)).max()) > 4096
 
         def run():
@@ -389,20 +511,20 @@ def cpu_baseline(kind, a, alpha, beta, n_cols, algo_bytes, op):
         sample = "whole workload per repetition (row loop over the transposed matrix)"
     elif kind == "csr2csc":
         def run():
-            oracle.csr2csc(a.m, a.n, a.base, a.ptr, a.col, a.val, method="omp")
+            oracle.csr2csc(a.m, a.n, a.base, ptr, col, val, method="omp")
         sample = "whole workload per repetition (per-thread column counts, scan, stable placement)"
     elif kind == "csr2coo":
         def run():
-            oracle.csr2coo_omp(a.m, a.base, a.ptr, a.nnz)
+            oracle.csr2coo_omp(a.m, a.base, ptr, a.nnz)
         sample = "whole workload per repetition"
     elif kind == "spmm":
         rows = min(a.m, max(1024, int(2e9 / max(1, 27 * n_cols * 4 * 10))))
-        sub_ptr = a.ptr[:rows + 1]
-        B = rng.uniform(-1, 1, (a.n, n_cols)).astype(dt)
-        C = np.zeros((rows, n_cols), dtype=dt)
+        sub_ptr = ptr[:rows + 1]
+        B = ft(rng.uniform(-1, 1, (a.n, n_cols)).astype(dt))
+        C = ft(np.zeros((rows, n_cols), dtype=dt))
 
         def run():
-            oracle.spmm_omp_f32(rows, n_cols, a.base, sub_ptr, a.col, a.val, alpha, beta, B, C)
+            oracle.spmm_omp_f32(rows, n_cols, a.base, sub_ptr, col, val, alpha, beta, B, C)
         frac = rows / a.m
         algo_bytes = algo_bytes * frac
         sample = "first %d of %d rows per repetition, rate scaled by bytes" % (rows, a.m)
@@ -412,14 +534,16 @@ def cpu_baseline(kind, a, alpha, beta, n_cols, algo_bytes, op):
     for _ in range(2):
         run()
     times = []
-    t_end = time.perf_counter() + 10.0
+    t_end = time.perf_counter() + 8.0
     while len(times) < 10 and (time.perf_counter() < t_end or len(times) < 3):
         t0 = time.perf_counter()
         run()
         times.append(time.perf_counter() - t0)
     med = float(np.median(times))
     return {"value": round(algo_bytes / med / 1e9, 3), "unit": "GB/s", "cores": threads, "kind": "port",
-            "sample": "%s; median of %d (%.3f ms)" % (sample, len(times), med * 1e3)}
+            "host_cpu": host_cpu_model(), "build": "-O3 -march=native" if tuned else "-O3 -march=x86-64-v3",
+            "sample": "%s; median of %d (%.3f ms); operands first touched by the OpenMP threads" % (
+                sample, len(times), med * 1e3)}
 
 
 if __name__ == "__main__":

@@ -233,16 +233,19 @@ mcspStatus_t ensure_plan(mcsparseHandle_t h, mcsparseSpMatDescr* A, const idx_t*
 
 // Where the banded copy of mcsparseSpMV_preprocess sits in its buffer: behind the scratch of a plain
 // SpMV call, which mcsparseSpMV may still write (row-length analysis) when handed the same buffer.
-size_t banded_region_offset(const mcsparseSpMatDescr* A, size_t value_bytes) {
-    const CsrView v = make_view(A, MCSPARSE_OPERATION_NON_TRANSPOSE);
+size_t banded_region_offset(const mcsparseSpMatDescr* A, mcsparseOperation_t op, size_t value_bytes) {
+    const CsrView v = make_view(A, op);
     return align_up(spmv_layout(v, A->nnz, value_bytes, narrow_bytes(A)).total);
 }
 
-// CSR, 32-bit indices, fp32 / fp64: what mcsparseSpMV_preprocess builds a banded copy for.
+// What mcsparseSpMV_preprocess builds a banded copy for: calls that run the row kernels on the arrays
+// as they lie (CSR with op N, CSC with op T), 32-bit indices, fp32 / fp64.
 bool banded_candidate(const mcsparseSpMatDescr* A, mcsparseOperation_t op, BandedShape* shape) {
-    if (A->format != MCSPARSE_FORMAT_CSR || op != MCSPARSE_OPERATION_NON_TRANSPOSE || wide_indices(A)) return false;
+    if ((A->format != MCSPARSE_FORMAT_CSR && A->format != MCSPARSE_FORMAT_CSC) || wide_indices(A)) return false;
     if (A->valueType != MACA_R_32F && A->valueType != MACA_R_64F) return false;
-    return mcsp::banded_shape(static_cast<idx_t>(A->row_num), static_cast<idx_t>(A->col_num), static_cast<idx_t>(A->nnz),
+    const CsrView v = make_view(A, op);
+    if (v.transpose) return false;
+    return mcsp::banded_shape(static_cast<idx_t>(v.m), static_cast<idx_t>(v.n), static_cast<idx_t>(A->nnz),
                               static_cast<idx_t>(A->idxBase), value_size(A->valueType),
                               A->banded.band_bytes != 0 ? A->banded.band_bytes : mcsp::kBandedBandBytes, shape);
 }
@@ -252,7 +255,7 @@ bool banded_matches(const mcsparseSpMatDescr* A, const void* buffer, size_t valu
     const SpmvBanded& b = A->banded;
     return b.valid && b.useful && b.buffer == buffer && b.rows == A->rows && b.cols == A->cols && b.vals == A->vals &&
            b.m == A->row_num && b.n == A->col_num && b.nnz == A->nnz && b.base == static_cast<int>(A->idxBase) &&
-           b.type == A->valueType && value_size(b.type) == value_bytes && A->format == MCSPARSE_FORMAT_CSR;
+           b.type == A->valueType && value_size(b.type) == value_bytes && b.format == A->format;
 }
 
 template <typename T>
@@ -559,8 +562,9 @@ mcsparseStatus_t mcsparseSpMV_preprocess_bufferSize(mcsparseHandle_t handle, mcs
     BandedShape shape;
     if (banded_candidate(matA, opA, &shape)) {
         const size_t vb = value_size(matA->valueType);
-        *bufferSize = banded_region_offset(matA, vb) +
-                      mcsp::banded_layout(shape, static_cast<idx_t>(matA->row_num), static_cast<idx_t>(matA->nnz), vb).total;
+        const CsrView v = make_view(matA, opA);
+        *bufferSize = banded_region_offset(matA, opA, vb) +
+                      mcsp::banded_layout(shape, static_cast<idx_t>(v.m), static_cast<idx_t>(matA->nnz), vb).total;
     }
     return MCSPARSE_STATUS_SUCCESS;
 }
@@ -578,13 +582,13 @@ mcsparseStatus_t mcsparseSpMV_preprocess(mcsparseHandle_t handle, mcsparseOperat
     if (matA->nnz == 0 || !banded_candidate(matA, opA, &shape)) return MCSPARSE_STATUS_SUCCESS;  // nothing to prepare
 
     // the row-length analysis says whether the rows are short enough for the banded kernel
-    const idx_t m = static_cast<idx_t>(matA->row_num);
+    const CsrView v = make_view(matA, opA);
+    const idx_t m = static_cast<idx_t>(v.m);
     const idx_t nnz = static_cast<idx_t>(matA->nnz);
     const idx_t base = static_cast<idx_t>(matA->idxBase);
     const size_t vb = value_size(matA->valueType);
-    const idx_t* row_ptr = static_cast<const idx_t*>(matA->rows);
-    const mcspStatus_t ps = ensure_plan(handle, matA, row_ptr, matA->rows, matA->row_num, matA->nnz,
-                                        matA->col_num * static_cast<int64_t>(vb), externalBuffer, true);
+    const mcspStatus_t ps =
+        ensure_plan(handle, matA, v.ptr, v.ptr, v.m, matA->nnz, v.n * static_cast<int64_t>(vb), externalBuffer, true);
     if (ps != MCSP_STATUS_SUCCESS) return to_public_status(ps);
     SpmvBanded& b = matA->banded;
     b.buffer = externalBuffer;
@@ -596,8 +600,9 @@ mcsparseStatus_t mcsparseSpMV_preprocess(mcsparseHandle_t handle, mcsparseOperat
     b.nnz = matA->nnz;
     b.base = static_cast<int>(matA->idxBase);
     b.type = matA->valueType;
+    b.format = matA->format;
     b.shape = shape;
-    b.region = banded_region_offset(matA, vb);
+    b.region = banded_region_offset(matA, opA, vb);
     b.grid = 0;
     if (matA->plan.forced_family == kFamilyAuto && matA->plan.max_row_len > mcsp::kBandedMaxRowLength) {
         b.useful = false;
@@ -605,8 +610,7 @@ mcsparseStatus_t mcsparseSpMV_preprocess(mcsparseHandle_t handle, mcsparseOperat
         return MCSPARSE_STATUS_SUCCESS;
     }
     char* region = static_cast<char*>(externalBuffer) + b.region;
-    mcsp::launch_banded_build(handle->stream, shape, m, nnz, base, row_ptr, static_cast<const idx_t*>(matA->cols),
-                              matA->vals, vb, region);
+    mcsp::launch_banded_build(handle->stream, shape, m, nnz, base, v.ptr, v.ind, matA->vals, vb, region);
     uint32_t xcd_start[9];
     const mcsp::BandedLayout l = mcsp::banded_layout(shape, m, nnz, vb);
     if (hipMemcpyAsync(xcd_start, region + l.xcd_start, sizeof(xcd_start), hipMemcpyDeviceToHost, handle->stream) !=

@@ -115,6 +115,7 @@ struct SpmvBanded {
     int64_t m = 0, n = 0, nnz = 0;
     int base = 0;
     macaDataType type = MACA_R_32F;
+    mcsparseFormat_t format = MCSPARSE_FORMAT_CSR;
     size_t region = 0;       // offset of the banded copy inside the buffer
     BandedShape shape = {};
     uint32_t grid = 0;       // workgroups of the SpMV kernel

@@ -27,6 +27,40 @@ def build(force=False):
 _lib = None
 
 
+def use_native_build():
+    """Switches this binding to a copy of oracle.c compiled for the host it runs on
+    (-O3 -march=native), for the timed CPU baseline.  The committed build recipe targets a generic
+    x86-64-v3 machine because its output travels between hosts.  Returns False, and keeps the
+    portable library, when no compiler is at hand."""
+    global _lib, _native
+    if _native is not None:
+        return _native
+    import tempfile
+    out = os.path.join(tempfile.mkdtemp(prefix="oracle_native_"), "liboracle_native.so")
+    cmd = ["gcc", "-O3", "-march=native", "-fopenmp", "-fPIC", "-std=c11", "-shared", "-o", out,
+           os.path.join(_HERE, "oracle.c"), "-lm"]
+    try:
+        subprocess.check_call(cmd, stdout=subprocess.DEVNULL, stderr=subprocess.DEVNULL)
+        _lib = ctypes.CDLL(out)
+        _native = True
+    except (OSError, subprocess.CalledProcessError):
+        _native = False
+    return _native
+
+
+_native = None
+
+
+def first_touch_copy(a):
+    """A copy of `a` whose pages are first written by the OpenMP threads (static schedule)."""
+    a = np.ascontiguousarray(a)
+    out = np.empty_like(a)
+    if a.nbytes:
+        lib().orc_first_touch_copy.restype = None
+        lib().orc_first_touch_copy(_p(out), _p(a), _c_i64(a.nbytes))
+    return out
+
+
 def lib():
     global _lib
     if _lib is None:

@@ -313,6 +313,20 @@ void orc_spmm_omp_f32(int64_t m, int64_t n, int base, const idx_t* ptr, const id
     }
 }
 
+/* dst <- src in pages of 4 KiB dealt to the OpenMP threads as schedule(static) deals rows: a page
+ * of a freshly mapped dst is then first touched, and so placed, next to the thread that will
+ * read it in the loops above. */
+void orc_first_touch_copy(void* dst, const void* src, int64_t bytes) {
+    const int64_t page = 4096;
+    const int64_t pages = (bytes + page - 1) / page;
+#pragma omp parallel for schedule(static)
+    for (int64_t p = 0; p < pages; ++p) {
+        const int64_t off = p * page;
+        const int64_t len = bytes - off < page ? bytes - off : page;
+        memcpy((char*)dst + off, (const char*)src + off, (size_t)len);
+    }
+}
+
 int orc_max_threads(void) {
 #ifdef _OPENMP
     extern int omp_get_max_threads(void);

@@ -16,28 +16,35 @@ pytestmark = pytest.mark.gpu
 GOLDEN = sorted(glob.glob(os.path.join(os.path.dirname(__file__), "golden", "csr_*.npz")))
 
 
-def run_banded(torch, handle, oracle, a, alpha, beta, band_bytes=0, seed=1, expect_state=2, what="", calls=1):
+def run_banded(torch, handle, oracle, a, alpha, beta, band_bytes=0, seed=1, expect_state=2, what="", calls=1,
+               as_csc=False):
+    """as_csc: the arrays are handed over as the CSC of the n x m transpose and applied with op T."""
     rng = np.random.default_rng(seed)
     dt = a.val.dtype
     ct = api.maca_type(dt)
     x = rng.uniform(-1, 1, a.n).astype(dt)
     y = rng.uniform(-1, 1, a.m).astype(dt)
     d_ptr, d_col, d_val, d_x, d_y = (dev(torch, v) for v in (a.ptr, a.col, a.val, x, y))
-    mat = api.SpMat(a.m, a.n, a.nnz, d_ptr, d_col, d_val, base=a.base)
+    if as_csc:
+        mat = api.SpMat(a.n, a.m, a.nnz, d_ptr, d_col, d_val, base=a.base, fmt=api.FORMAT_CSC)
+        op = api.OP_T
+    else:
+        mat = api.SpMat(a.m, a.n, a.nnz, d_ptr, d_col, d_val, base=a.base)
+        op = api.OP_N
     if band_bytes:
         mat.set_band_bytes(band_bytes)
     vx, vy = api.DnVec(d_x), api.DnVec(d_y)
-    st, size = api.spmv_preprocess_buffer_size(handle, api.OP_N, alpha, mat, vx, beta, vy, ct)
+    st, size = api.spmv_preprocess_buffer_size(handle, op, alpha, mat, vx, beta, vy, ct)
     assert st == api.STATUS_SUCCESS
     buf = torch.empty(size, dtype=torch.uint8, device="cuda")
-    assert api.spmv_preprocess(handle, api.OP_N, alpha, mat, vx, beta, vy, ct, buf) == api.STATUS_SUCCESS
+    assert api.spmv_preprocess(handle, op, alpha, mat, vx, beta, vy, ct, buf) == api.STATUS_SUCCESS
     state, bands, rows = mat.spmv_preprocess_state()
     assert state == expect_state, (state, bands, rows)
     y_ref, bound = oracle.spmv(False, a.m, a.n, a.base, a.ptr, a.col, a.val, alpha, beta, x, y)
     first = None
     for _ in range(calls):
         d_y.copy_(torch.from_numpy(y))
-        assert api.spmv(handle, api.OP_N, alpha, mat, vx, beta, vy, ct, buf) == api.STATUS_SUCCESS
+        assert api.spmv(handle, op, alpha, mat, vx, beta, vy, ct, buf) == api.STATUS_SUCCESS
         torch.cuda.synchronize()
         got = d_y.cpu().numpy()
         assert_within(got, y_ref, bound, dt, what=what or "banded spmv")
@@ -91,6 +98,32 @@ def test_tiles_of_every_fill(torch_gpu, handle, oracle, per_row):
     run_banded(torch_gpu, handle, oracle, a, 1.5, 0.5, band_bytes=1 << 15)
     b = wl.uniform_rows(m=3000, n=4000, per_row=min(per_row * 4, 200), dtype=np.float32, config_id=40 + per_row)
     run_banded(torch_gpu, handle, oracle, b, 1.0, 0.0, band_bytes=4096)
+
+
+def test_csc_applied_transposed(torch_gpu, handle, oracle):
+    # CSC with op T runs the row kernels on the arrays as they lie, so it can be banded like CSR op N
+    a = wl.random_ragged(4001, 20011, 17, dtype=np.float32, seed=21, base=1)
+    run_banded(torch_gpu, handle, oracle, a, 1.25, -0.5, band_bytes=4096, as_csc=True, calls=2)
+    # the transposing directions are not banded: preprocess leaves them alone and SpMV still answers
+    torch = torch_gpu
+    rng = np.random.default_rng(2)
+    x = rng.uniform(-1, 1, a.m).astype(np.float32)
+    d_ptr, d_col, d_val, d_x = (dev(torch, v) for v in (a.ptr, a.col, a.val, x))
+    d_y = torch.zeros(a.n, dtype=torch.float32, device="cuda")
+    mat = api.SpMat(a.m, a.n, a.nnz, d_ptr, d_col, d_val, base=1)
+    mat.set_band_bytes(4096)
+    vx, vy = api.DnVec(d_x), api.DnVec(d_y)
+    st, size = api.spmv_preprocess_buffer_size(handle, api.OP_T, 1.0, mat, vx, 0.0, vy, api.R_32F)
+    assert st == api.STATUS_SUCCESS
+    st2, plain = api.spmv_buffer_size(handle, api.OP_T, 1.0, mat, vx, 0.0, vy, api.R_32F)
+    assert size == plain
+    buf = torch.empty(size, dtype=torch.uint8, device="cuda")
+    assert api.spmv_preprocess(handle, api.OP_T, 1.0, mat, vx, 0.0, vy, api.R_32F, buf) == api.STATUS_SUCCESS
+    assert mat.spmv_preprocess_state()[0] == 0
+    assert api.spmv(handle, api.OP_T, 1.0, mat, vx, 0.0, vy, api.R_32F, buf) == api.STATUS_SUCCESS
+    torch.cuda.synchronize()
+    y_ref, bound = oracle.spmv(True, a.m, a.n, 1, a.ptr, a.col, a.val, 1.0, 0.0, x, None)
+    assert_within(d_y.cpu().numpy(), y_ref, bound, np.float32, what="op T after preprocess")
 
 
 def test_default_band_width_config2_reduced(torch_gpu, handle, oracle):

@@ -224,3 +224,42 @@ def test_csrsort_sorts_inside_rows_only(oracle, base):
     assert np.array_equal(col[perm.view(np.int32)], a.col)   # perm[i] = old position of the entry now at i
     rows = np.repeat(np.arange(a.m), a.row_lengths())
     assert np.array_equal(rows[perm.view(np.int32)], rows)   # nothing left its row
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("dynamic", [False, True])
+def test_openmp_spmv_port_is_the_serial_oracle(oracle, dtype, dynamic):
+    """The OpenMP port that bench.py times computes what the pinned serial oracle computes."""
+    a = wl.random_ragged(3000, 2500, 12, dtype=dtype, seed=8, base=1)
+    rng = np.random.default_rng(3)
+    x = rng.uniform(-1, 1, a.n).astype(dtype)
+    y0 = rng.uniform(-1, 1, a.m).astype(dtype)
+    y = oracle.first_touch_copy(y0)
+    assert np.array_equal(y, y0)
+    oracle.spmv_omp(a.m, a.base, a.ptr, a.col, a.val, 1.5, -0.5, x, y, dynamic=dynamic)
+    y_ref, bound = oracle.spmv(False, a.m, a.n, a.base, a.ptr, a.col, a.val, 1.5, -0.5, x, y0)
+    u = 2.0 ** -24 if dtype == np.float32 else 2.0 ** -53
+    # sequential working-precision sums: error below (row length + 2) * u * bound
+    assert (np.abs(y.astype(np.longdouble) - y_ref) <= (a.row_lengths().max() + 2) * u * bound).all()
+    # integer data: exact, whatever the order
+    ai = wl.Csr(a.m, a.n, a.ptr, a.col, np.round(a.val * 4).astype(dtype), a.base)
+    xi = np.round(x * 8).astype(dtype)
+    yi = np.round(y0 * 8).astype(dtype)
+    want, _ = oracle.spmv(False, ai.m, ai.n, ai.base, ai.ptr, ai.col, ai.val, 2.0, 3.0, xi, yi)
+    got = yi.copy()
+    oracle.spmv_omp(ai.m, ai.base, ai.ptr, ai.col, ai.val, 2.0, 3.0, xi, got, dynamic=dynamic)
+    assert np.array_equal(got.astype(np.longdouble), want)
+
+
+def test_openmp_spmm_port_is_the_serial_oracle(oracle):
+    a = wl.random_ragged(700, 600, 9, dtype=np.float32, seed=9)
+    rng = np.random.default_rng(4)
+    n = 24
+    vals = np.round(a.val * 4).astype(np.float32)
+    B = np.round(rng.uniform(-1, 1, (a.n, n)) * 8).astype(np.float32)
+    C0 = np.round(rng.uniform(-1, 1, (a.m, n)) * 8).astype(np.float32)
+    want, _ = oracle.spmm(a.m, n, a.base, a.ptr, a.col, vals, 2.0, -1.0, B.ravel(), n, True, C0.ravel(), n, True)
+    got = C0.copy()
+    oracle.spmm_omp_f32(a.m, n, a.base, a.ptr, a.col, vals, 2.0, -1.0, B, got)
+    assert np.array_equal(got.astype(np.longdouble), want)
+    assert np.array_equal(oracle.csr2coo_omp(a.m, a.base, a.ptr, a.nnz), oracle.csr2coo(a.m, a.base, a.ptr, a.nnz))
