@@ -417,6 +417,13 @@ mcsparseStatus_t mcsparseDgthr(mcsparseHandle_t handle, int nnz, const double* y
 mcsparseStatus_t mcsparseXcsrRowBins(mcsparseHandle_t handle, int m, const int* csr_rows,
                                      mcsparseIndexBase_t idx_base, uint8_t* row_bins, uint32_t* bin_hist);
 
+/* The kernel choice mcsparseSpMV derives from such a histogram (host arrays, no GPU work): family and
+ * lanes_per_row as mcsparseSpMatGetSpMVPlan reports them.  m rows, nnz nonzeros, x_bytes = bytes of
+ * the dense vector.  The dispatch is per matrix: the bins say how well rows of this spread fill the
+ * lanes of the sub-wavefront kernel, and the merge-path kernel takes over when they fill under half. */
+mcsparseStatus_t mcsparseXcsrRowBinsPlan(const uint32_t* bin_hist, int64_t m, int64_t nnz, int64_t x_bytes, int* family,
+                                         int* lanes_per_row);
+
 /* Which SpMV kernel family a CSR op-N call on this descriptor runs:
  * 0 = not analysed yet, 1 = sub-wavefront vector kernel, 2 = merge-path kernel.
  * lanes_per_row is the sub-wavefront width for family 1; for family 2 it is 1 when the tiles of

@@ -105,6 +105,7 @@ PROTOTYPES = {
                                 c_int]),
     "mcsparseScsrmm": (c_int, [vp, c_int, c_int, c_int, c_int, c_int, vp, vp, vp, vp, vp, vp, c_int, vp, vp, c_int]),
     "mcsparseDcsrmm": (c_int, [vp, c_int, c_int, c_int, c_int, c_int, vp, vp, vp, vp, vp, vp, c_int, vp, vp, c_int]),
+    "mcsparseXcsrRowBinsPlan": (c_int, [vp, c_i64, c_i64, c_i64, P(c_int), P(c_int)]),
     "mcsparseXcsrRowBins": (c_int, [vp, c_int, vp, c_int, vp, vp]),
     "mcsparseSpMatGetSpMVPlan": (c_int, [vp, P(c_int), P(c_int)]),
     "mcsparseSpMatSetSpMVPlan": (c_int, [vp, c_int, c_int]),

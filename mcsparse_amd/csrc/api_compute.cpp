@@ -1,5 +1,6 @@
 // mcsparseSpMV / mcsparseSpMM / conversion entry points: argument validation in the order of the
 // reference's host drivers, scratch-buffer carving, kernel-family choice and launches.
+#include <cmath>
 #include <cstring>
 
 #include "internal.h"
@@ -13,6 +14,13 @@ constexpr size_t kAnalysisBytes = align_up((MCSPARSE_ROW_BIN_COUNT + 1) * sizeof
 
 bool fits_32(int64_t v) { return (v >> 32) == 0; }
 
+// A stream that is being captured into a HIP graph cannot be synchronised: trying to would fail and
+// invalidate the caller's capture.
+bool stream_is_capturing(hipStream_t stream) {
+    hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+    return hipStreamIsCapturing(stream, &status) == hipSuccess && status != hipStreamCaptureStatusNone;
+}
+
 // Reads a scalar of the compute type.  Device pointer mode costs one blocking copy, like the
 // reference (src/include/mcsp_internal_host_utils.hpp:34-63).
 template <typename T>
@@ -21,6 +29,7 @@ bool scalar_to_host(mcsparseHandle_t h, const void* p, T* out) {
         std::memcpy(out, p, sizeof(T));
         return true;
     }
+    if (stream_is_capturing(h->stream)) return false;  // a blocking read cannot be captured
     if (hipMemcpyAsync(out, p, sizeof(T), hipMemcpyDeviceToHost, h->stream) != hipSuccess) return false;
     return hipStreamSynchronize(h->stream) == hipSuccess;
 }
@@ -185,6 +194,9 @@ mcspStatus_t ensure_plan(mcsparseHandle_t h, mcsparseSpMatDescr* A, const idx_t*
     SpmvPlan& p = A->plan;
     if (p.valid && p.rows == signature && p.m == m && p.nnz == nnz && p.base == static_cast<int>(A->idxBase))
         return MCSP_STATUS_SUCCESS;
+    // The analysis ends in a blocking read-back, which a stream under graph capture cannot do: the
+    // plan only steers speed, so such a call goes without one.
+    if (may_read_back && p.forced_family == kFamilyAuto && stream_is_capturing(h->stream)) may_read_back = false;
     if (!may_read_back && p.forced_family == kFamilyAuto) {
         // No analysis without its read-back: the merge family in storage order is correct and balanced
         // for every structure.  The plan stays invalid, so a later call that may read back analyses.
@@ -214,19 +226,8 @@ mcspStatus_t ensure_plan(mcsparseHandle_t h, mcsparseSpMatDescr* A, const idx_t*
         return MCSP_STATUS_INTERNAL_ERROR;
     std::memcpy(p.hist, host_hist, sizeof(p.hist));
     p.max_row_len = host_hist[MCSPARSE_ROW_BIN_COUNT];
-    // A row much longer than its lane group serialises one wave while the rest of the chip
-    // idles; past that point the merge-path split wins.
-    const uint32_t limit = static_cast<uint32_t>(32 * mean_lanes > 512 ? 32 * mean_lanes : 512);
-    if (p.max_row_len > limit) {
-        p.family = kFamilyMerge;
-        // Rows longer than a tile of the merge path put whole tiles inside one row; when x is too
-        // large to stay in an XCD's L2 next to the streamed matrix, those tiles run in the order of
-        // their first column (plan.lanes = 1), which costs two small kernels per call.
-        p.lanes = p.max_row_len >= kMergeTileItems && x_bytes > kMergeOrderMinVectorBytes ? 1 : 0;
-    } else {
-        p.family = kFamilyVector;
-        p.lanes = p.forced_lanes ? p.forced_lanes : mean_lanes;
-    }
+    mcsp::spmv_plan_from_bins(host_hist, m, nnz, x_bytes, &p.family, &p.lanes);
+    if (p.family == kFamilyVector && p.forced_lanes) p.lanes = p.forced_lanes;
     p.valid = true;
     return MCSP_STATUS_SUCCESS;
 }
@@ -263,7 +264,8 @@ mcspStatus_t spmv_typed(mcsparseHandle_t h, mcsparseSpMatDescr* A, mcsparseOpera
                         const void* beta, const mcsparseDnVecDescr* x, mcsparseDnVecDescr* y, void* buffer,
                         bool may_read_back) {
     T h_alpha, h_beta;
-    if (!scalar_to_host(h, beta, &h_beta) || !scalar_to_host(h, alpha, &h_alpha)) return MCSP_STATUS_INTERNAL_ERROR;
+    if (!scalar_to_host(h, beta, &h_beta) || !scalar_to_host(h, alpha, &h_alpha))
+        return stream_is_capturing(h->stream) ? MCSP_STATUS_NOT_IMPLEMENTED : MCSP_STATUS_INTERNAL_ERROR;
     // reference: mcsp_spmv_gpu.cpp:235-237 -- y is left untouched in both cases
     if (A->nnz == 0 || (h_alpha == T(0) && h_beta == T(0))) return MCSP_STATUS_SUCCESS;
 
@@ -378,7 +380,8 @@ template <typename T>
 mcspStatus_t spmm_typed(mcsparseHandle_t h, const mcsparseSpMatDescr* A, mcsparseOperation_t opB, const void* alpha,
                         const void* beta, const mcsparseDnMatDescr* B, mcsparseDnMatDescr* C, void* buffer) {
     T h_alpha, h_beta;
-    if (!scalar_to_host(h, beta, &h_beta) || !scalar_to_host(h, alpha, &h_alpha)) return MCSP_STATUS_INTERNAL_ERROR;
+    if (!scalar_to_host(h, beta, &h_beta) || !scalar_to_host(h, alpha, &h_alpha))
+        return stream_is_capturing(h->stream) ? MCSP_STATUS_NOT_IMPLEMENTED : MCSP_STATUS_INTERNAL_ERROR;
     // reference: mcsp_spmm_gpu.cpp:110-114
     if (A->nnz == 0 && h_beta == T(1)) return MCSP_STATUS_SUCCESS;
 
@@ -440,7 +443,8 @@ mcspStatus_t spmm_typed(mcsparseHandle_t h, const mcsparseSpMatDescr* A, mcspars
         a.c_row_major = C->order == MCSPARSE_ORDER_ROW;
         // the schedule was built from batch 0's structure
         if ((b == 0 || shared_structure) && schedule_matches(A, buffer) && mcsp::spmm_schedule_usable(a, sizeof(T))) {
-            mcsp::launch_spmm_scheduled<T>(h->stream, a, buffer, A->schedule.mean_span, h_alpha, h_beta);
+            mcsp::launch_spmm_scheduled<T>(h->stream, a, buffer, A->schedule.entries, A->schedule.mean_span, h_alpha,
+                                           h_beta);
         } else {
             mcsp::launch_spmm<T>(h->stream, a, h_alpha, h_beta);
         }
@@ -466,6 +470,61 @@ mcspStatus_t check_spmm_args(mcsparseHandle_t handle, const void* alpha, const m
 }  // namespace
 
 namespace mcsp {
+
+// Kernel family for a CSR structure from its row-length bins (bins[b], b >= 1: rows of length in
+// [2^(b-1), 2^b); bins[0]: empty rows; bins[MCSPARSE_ROW_BIN_COUNT]: the longest row).
+//
+// The vector family gives L lanes to a row (L = the power of two at or above the mean length) and a
+// wavefront keeps k = 64/L * 4 rows in flight; it loops until the longest of them is done, so the
+// share of its lane slots that hold a nonzero is mean / (L * E[max over k rows of ceil(len / L)]).
+// The expectation comes from the bins, with the lengths inside a bin placed so that the overall
+// mean is the true one (rows of exactly 16 fall into [16, 32) and count as 16, not 24).  The merge
+// family spends about one slot per nonzero and row whatever the lengths are, at ~5 % more work per
+// item.  Measured: rows of exactly 16 (share 1.0) run 10 % faster in the vector family; rows of
+// 28 +- 5 (share 0.48) 13 % faster in the merge family; Poisson rows of mean 20 (share 0.6) faster in
+// the vector family.  The families change places at a share of about one half.  A row far longer
+// than the rest serialises one wavefront, so such matrices take the merge family whatever the share.
+void spmv_plan_from_bins(const uint32_t* bins, int64_t m, int64_t nnz, int64_t x_bytes, int* family, int* lanes) {
+    const int mean_lanes = spmv_pick_lanes(static_cast<idx_t>(m), static_cast<idx_t>(nnz));
+    const uint32_t max_row_len = bins[MCSPARSE_ROW_BIN_COUNT];
+    const uint32_t limit = static_cast<uint32_t>(32 * mean_lanes > 512 ? 32 * mean_lanes : 512);
+    bool merge = max_row_len > limit;
+    if (!merge && m > 0 && nnz > 0) {
+        // lengths inside a bin: lower edge times a common factor in [1, 2) that makes the mean right
+        double edge_sum = 0;
+        for (int b = 1; b < MCSPARSE_ROW_BIN_COUNT; ++b) edge_sum += static_cast<double>(bins[b]) * std::ldexp(1.0, b - 1);
+        double factor = edge_sum > 0 ? static_cast<double>(nnz) / edge_sum : 1.0;
+        factor = factor < 1.0 ? 1.0 : (factor > 2.0 ? 2.0 : factor);
+        const double k = 64.0 / mean_lanes * 4.0;
+        double below = static_cast<double>(bins[0]) / static_cast<double>(m);  // share of rows in lower bins
+        double below_pow = std::pow(below, k);
+        double expected_max = 0;
+        for (int b = 1; b < MCSPARSE_ROW_BIN_COUNT; ++b) {
+            if (bins[b] == 0) continue;
+            double len = std::ldexp(1.0, b - 1) * factor;
+            if (len > max_row_len) len = max_row_len;  // no row is longer than the longest
+            const double passes = std::ceil(len / mean_lanes - 1e-9);
+            const double upto = below + static_cast<double>(bins[b]) / static_cast<double>(m);
+            const double upto_pow = std::pow(upto < 1.0 ? upto : 1.0, k);
+            expected_max += passes * (upto_pow - below_pow);
+            below = upto;
+            below_pow = upto_pow;
+        }
+        const double mean = static_cast<double>(nnz) / static_cast<double>(m);
+        const double share = expected_max > 0 ? mean / (mean_lanes * expected_max) : 1.0;
+        merge = share < 0.5;
+    }
+    if (merge) {
+        *family = kFamilyMerge;
+        // Rows longer than a tile of the merge path put whole tiles inside one row; when x is too
+        // large to stay in an XCD's L2 next to the streamed matrix, those tiles run in the order of
+        // their first column (lanes = 1), which costs two small kernels per call.
+        *lanes = max_row_len >= kMergeTileItems && x_bytes > kMergeOrderMinVectorBytes ? 1 : 0;
+    } else {
+        *family = kFamilyVector;
+        *lanes = mean_lanes;
+    }
+}
 
 // The argument checks of mcsparseSpMV in the reference's order, then the ones this build adds.
 mcspStatus_t spmv_check(mcsparseHandle_t handle, mcsparseOperation_t opA, const void* alpha, mcsparseSpMatDescr_t matA,
@@ -578,6 +637,7 @@ mcsparseStatus_t mcsparseSpMV_preprocess(mcsparseHandle_t handle, mcsparseOperat
         mcsp::spmv_check(handle, opA, alpha, matA, vecX, beta, vecY, computeType, externalBuffer, 0, true);
     if (st != MCSP_STATUS_SUCCESS) return to_public_status(st);
     matA->banded.valid = false;
+    if (stream_is_capturing(handle->stream)) return to_public_status(MCSP_STATUS_NOT_IMPLEMENTED);  // it blocks
     BandedShape shape;
     if (matA->nnz == 0 || !banded_candidate(matA, opA, &shape)) return MCSPARSE_STATUS_SUCCESS;  // nothing to prepare
 
@@ -660,6 +720,8 @@ mcsparseStatus_t mcsparseSpMM_preprocess(mcsparseHandle_t handle, mcsparseOperat
     const mcspStatus_t st = check_spmm_args(handle, alpha, matA, matB, beta, matC);
     if (st != MCSP_STATUS_SUCCESS) return to_public_status(st);
     matA->schedule.valid = false;
+    // the schedule's size is read back: not possible on a stream under graph capture
+    if (stream_is_capturing(handle->stream)) return to_public_status(MCSP_STATUS_NOT_IMPLEMENTED);
     if (opA != MCSPARSE_OPERATION_NON_TRANSPOSE || !schedulable(matA) || matA->rows == nullptr || matA->cols == nullptr)
         return MCSPARSE_STATUS_SUCCESS;  // nothing to prepare for this call
 
@@ -815,6 +877,16 @@ mcsparseStatus_t mcsparseCsr2cscEx2(mcsparseHandle_t handle, int m, int n, int n
                          reinterpret_cast<const idx_t*>(csr_rows), reinterpret_cast<const idx_t*>(csr_cols), csc_val,
                          reinterpret_cast<idx_t*>(csc_rows), reinterpret_cast<idx_t*>(csc_cols), vb,
                          static_cast<idx_t>(idx_base), temp_buffer);
+    return MCSPARSE_STATUS_SUCCESS;
+}
+
+// EXTENSION
+mcsparseStatus_t mcsparseXcsrRowBinsPlan(const uint32_t* bin_hist, int64_t m, int64_t nnz, int64_t x_bytes, int* family,
+                                         int* lanes_per_row) {
+    if (bin_hist == nullptr || family == nullptr || lanes_per_row == nullptr)
+        return to_public_status(MCSP_STATUS_INVALID_POINTER);
+    if (m < 0 || nnz < 0 || !fits_32(m) || !fits_32(nnz)) return to_public_status(MCSP_STATUS_INVALID_SIZE);
+    mcsp::spmv_plan_from_bins(bin_hist, m, nnz, x_bytes, family, lanes_per_row);
     return MCSPARSE_STATUS_SUCCESS;
 }
 

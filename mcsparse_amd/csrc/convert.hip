@@ -163,16 +163,39 @@ __global__ __launch_bounds__(kBlock) void coo2csr_kernel(idx_t nnz, idx_t m, idx
     // entry t0-1: the last entry of the lane below, a load for the first lane of a wavefront
     idx_t before = __shfl_up(r[kCooPerThread - 1], 1, kWave);
     if (threadIdx.x % kWave == 0 && t0 != 0 && t0 <= nnz) before = coo_rows[t0 - 1] - base;
-    if (t0 > nnz) return;
-    // rows [prev, cur) get offset t: prev = row of entry t-1 plus one (0 in front of the first entry)
+    // rows [prev, cur) get offset t: prev = row of entry t-1 plus one (0 in front of the first entry).
+    // A thread fills short stretches itself; a long stretch of empty rows (up to all m of them after
+    // the last entry) is left to the whole wavefront below, lane by lane 64 offsets at a time.
+    constexpr uint64_t kSerialFill = 16;
     uint64_t prev = t0 == 0 ? 0 : static_cast<uint64_t>(before) + 1;
+    uint64_t long_from = 0, long_to = 0;  // at most one long stretch is kept per thread; more are filled serially
+    idx_t long_value = 0;
+    if (t0 <= nnz) {
 #pragma unroll
-    for (int e = 0; e < kCooPerThread; ++e) {
-        const uint64_t t = t0 + e;
-        if (t > nnz) break;
-        const uint64_t cur = static_cast<uint64_t>(r[e]) + 1;  // t == nnz: m + 1
-        for (uint64_t i = prev; i < cur; ++i) row_ptr[i] = static_cast<idx_t>(t) + base;
-        prev = cur;
+        for (int e = 0; e < kCooPerThread; ++e) {
+            const uint64_t t = t0 + e;
+            if (t > nnz) break;
+            const uint64_t cur = static_cast<uint64_t>(r[e]) + 1;  // t == nnz: m + 1
+            if (cur > prev + kSerialFill && long_to == long_from) {
+                long_from = prev;
+                long_to = cur;
+                long_value = static_cast<idx_t>(t) + base;
+            } else {
+                for (uint64_t i = prev; i < cur; ++i) row_ptr[i] = static_cast<idx_t>(t) + base;
+            }
+            prev = cur;
+        }
+    }
+    // every lane of the wavefront gets here: the stretches are handed round and filled cooperatively
+    uint64_t pending = __ballot(long_to > long_from);
+    const unsigned lane = threadIdx.x % kWave;
+    while (pending != 0) {
+        const int src = __ffsll(static_cast<long long>(pending)) - 1;
+        pending &= pending - 1;
+        const uint64_t from = __shfl(long_from, src, kWave);
+        const uint64_t to = __shfl(long_to, src, kWave);
+        const idx_t value = __shfl(long_value, src, kWave);
+        for (uint64_t i = from + lane; i < to; i += kWave) row_ptr[i] = value;
     }
 }
 
@@ -329,15 +352,19 @@ __global__ __launch_bounds__(kHistBlock) void radix_hist_kernel(const idx_t* __r
     s_cnt[threadIdx.x] = 0;
     __syncthreads();
     const uint64_t start = static_cast<uint64_t>(tile) * kSortTile;
+    // tiles start at multiples of 4096 keys, so a 16-byte aligned array allows 128-bit loads; the keys
+    // of the first pass are the caller's own array, which may start anywhere
+    const bool wide = (reinterpret_cast<uintptr_t>(keys) & 15u) == 0;
 #pragma unroll
     for (int i = 0; i < kSortTile / (kHistBlock * 4); ++i) {
         const uint64_t p = start + (static_cast<uint64_t>(i) * kHistBlock + threadIdx.x) * 4;
-        if (p + 4 <= count) {
+        if (wide && p + 4 <= count) {
             const idx4 k = __builtin_nontemporal_load(reinterpret_cast<const idx4*>(keys + p));
 #pragma unroll
             for (int e = 0; e < 4; ++e) atomicAdd(&s_cnt[(k[e] >> shift) & mask], 1u);
         } else {
-            for (uint64_t q = p; q < count; ++q) atomicAdd(&s_cnt[(keys[q] >> shift) & mask], 1u);
+            const uint64_t stop = p + 4 < count ? p + 4 : count;
+            for (uint64_t q = p; q < stop; ++q) atomicAdd(&s_cnt[(keys[q] >> shift) & mask], 1u);
         }
     }
     __syncthreads();

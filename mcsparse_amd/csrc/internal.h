@@ -216,6 +216,11 @@ mcspStatus_t spmv_call(mcsparseHandle_t handle, mcsparseOperation_t opA, const v
                        mcsparseDnVecDescr_t vecX, const void* beta, mcsparseDnVecDescr_t vecY,
                        macaDataType computeType, void* buffer, size_t buffer_bytes, bool may_read_back);
 
+// Kernel family (and lanes per row / tile order) for a structure with these row-length bins: the
+// 33 counters and the longest row that launch_row_bins leaves, read back to the host.  A pure
+// function, so the choice can be pinned on a table of histograms without a GPU.
+void spmv_plan_from_bins(const uint32_t* bins, int64_t m, int64_t nnz, int64_t x_bytes, int* family, int* lanes);
+
 // ---- row-length analysis (analysis.hip) ----
 // hist_out: MCSPARSE_ROW_BIN_COUNT counters followed by the longest row length (34 x u32),
 // zeroed by this call.  row_bins may be null.
@@ -303,8 +308,8 @@ void launch_spmm_schedule(hipStream_t stream, idx_t m, idx_t nnz, idx_t base, co
 // (spmm_schedule_usable says so), reading every B row once per row group.
 bool spmm_schedule_usable(const SpmmArgs& a, size_t value_bytes);
 template <typename T>
-void launch_spmm_scheduled(hipStream_t stream, const SpmmArgs& a, const void* schedule, uint64_t mean_span, T alpha,
-                           T beta);
+void launch_spmm_scheduled(hipStream_t stream, const SpmmArgs& a, const void* schedule, uint32_t total_entries,
+                           uint64_t mean_span, T alpha, T beta);
 
 // ---- conversions (convert.hip) ----
 void launch_csr2coo(hipStream_t stream, idx_t m, idx_t nnz, const idx_t* row_ptr, idx_t base, idx_t* coo_rows);

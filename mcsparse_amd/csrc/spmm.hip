@@ -548,7 +548,8 @@ __global__ __launch_bounds__(kBlock) void spmm_group_kernel(idx_t m, idx_t n, id
                                                             const uint32_t* __restrict__ entries,
                                                             const T* __restrict__ B, int64_t ldb, T* __restrict__ C,
                                                             int64_t ldc, bool c_row_major, T alpha, T beta,
-                                                            uint32_t xcd_chunk) {
+                                                            uint32_t xcd_chunk, idx_t k, idx_t nnz,
+                                                            uint32_t total_entries) {
     typedef typename ByteOffset<WIDE>::type off_t;
     constexpr int V = 16 / sizeof(T);
     constexpr int kGroupsPerBlock = kBlock / LR;
@@ -578,11 +579,16 @@ __global__ __launch_bounds__(kBlock) void spmm_group_kernel(idx_t m, idx_t n, id
     const off_t ldb_bytes = static_cast<off_t>(ldb * sizeof(T));
 
     if (e[R - 1] - i[0] <= kSpmmMaxMergedGroup) {
-        const uint32_t s_end = group_ptr[group + 1];
+        // The schedule lives in the caller's buffer.  Whatever it holds, nothing is read outside the
+        // arrays: list bounds are held to the list, columns to the k rows of op(B), value positions to
+        // the nonzeros.  (An overwritten schedule gives wrong numbers, never a fault.)
+        const uint32_t s_end = min(group_ptr[group + 1], total_entries);
+        const uint32_t s_begin = min(group_ptr[group], s_end);
+        const idx_t last_value = nnz - 1;  // nnz != 0: the group has nonzeros
         const unsigned group_first = (__lane_id() / LR) * LR;
         const uint64_t group_bits = LR == kWave ? ~0ull : ((1ull << (LR % kWave)) - 1ull);
         const uint64_t below = (1ull << lane) - 1ull;
-        for (uint32_t s = group_ptr[group]; s < s_end; s += LR) {
+        for (uint32_t s = s_begin; s < s_end; s += LR) {
             const uint32_t ent = s + lane < s_end ? entries[s + lane] : 0u;
             // this lane's entry is the p-th of the chunk that row r takes part in: the p-th value of
             // the row from where the row stands.  take[r] holds which entries of the chunk row r
@@ -595,11 +601,11 @@ __global__ __launch_bounds__(kBlock) void spmm_group_kernel(idx_t m, idx_t n, id
             for (int r = 0; r < R; ++r) {
                 const bool mine = (ent >> r) & 1u;
                 const uint64_t in = (__ballot(mine) >> group_first) & group_bits;
-                v[r] = mine ? val[i[r] + __popcll(in & below)] : T(0);
+                v[r] = mine ? val[min(i[r] + static_cast<idx_t>(__popcll(in & below)), last_value)] : T(0);
                 i[r] += __popcll(in);
                 take[r] = __brev(static_cast<uint32_t>(in));
             }
-            const off_t roff = static_cast<off_t>(ent >> R) * ldb_bytes;
+            const off_t roff = static_cast<off_t>(min(ent >> R, k - 1)) * ldb_bytes;
             const uint32_t flags = ent & ((1u << R) - 1u);
             const uint32_t left = s_end - s;
             // With kAlternate two batches of rows of op(B) take turns: the loads of one are on their
@@ -680,8 +686,8 @@ bool narrow_offsets(const SpmmArgs& a, size_t value_bytes) {
 }
 
 template <typename T, int LR>
-void launch_group(hipStream_t stream, const SpmmArgs& a, const uint32_t* group_ptr, const uint32_t* entries, T alpha,
-                  T beta, uint64_t mean_span) {
+void launch_group(hipStream_t stream, const SpmmArgs& a, const uint32_t* group_ptr, const uint32_t* entries,
+                  uint32_t total_entries, T alpha, T beta, uint64_t mean_span) {
     constexpr int V = 16 / sizeof(T);
     const uint64_t groups = spmm_groups(a.m);
     const uint64_t group_blocks = (groups + (kBlock / LR) - 1) / (kBlock / LR);
@@ -703,10 +709,12 @@ void launch_group(hipStream_t stream, const SpmmArgs& a, const uint32_t* group_p
     T* C = static_cast<T*>(a.C);
     if (narrow_offsets(a, sizeof(T))) {
         hipLaunchKernelGGL((spmm_group_kernel<T, LR, false>), grid, dim3(kBlock), 0, stream, a.m, a.n, a.base, a.row_ptr,
-                           a.col, val, group_ptr, entries, B, a.ldb, C, a.ldc, a.c_row_major, alpha, beta, xcd_chunk);
+                           a.col, val, group_ptr, entries, B, a.ldb, C, a.ldc, a.c_row_major, alpha, beta, xcd_chunk, a.k,
+                           a.nnz, total_entries);
     } else {
         hipLaunchKernelGGL((spmm_group_kernel<T, LR, true>), grid, dim3(kBlock), 0, stream, a.m, a.n, a.base, a.row_ptr,
-                           a.col, val, group_ptr, entries, B, a.ldb, C, a.ldc, a.c_row_major, alpha, beta, xcd_chunk);
+                           a.col, val, group_ptr, entries, B, a.ldb, C, a.ldc, a.c_row_major, alpha, beta, xcd_chunk, a.k,
+                           a.nnz, total_entries);
     }
 }
 
@@ -810,8 +818,8 @@ bool spmm_schedule_usable(const SpmmArgs& a, size_t value_bytes) {
 }
 
 template <typename T>
-void launch_spmm_scheduled(hipStream_t stream, const SpmmArgs& a, const void* schedule, uint64_t mean_span, T alpha,
-                           T beta) {
+void launch_spmm_scheduled(hipStream_t stream, const SpmmArgs& a, const void* schedule, uint32_t total_entries,
+                           uint64_t mean_span, T alpha, T beta) {
     if (a.m == 0 || a.n == 0) return;
     constexpr int V = 16 / sizeof(T);
     const SpmmScheduleLayout l = spmm_schedule_layout(a.m, a.nnz);
@@ -819,15 +827,15 @@ void launch_spmm_scheduled(hipStream_t stream, const SpmmArgs& a, const void* sc
     const uint32_t* group_ptr = reinterpret_cast<const uint32_t*>(w + l.group_ptr);
     const uint32_t* entries = reinterpret_cast<const uint32_t*>(w + l.entries);
     const uint64_t lanes_needed = (static_cast<uint64_t>(a.n) + V - 1) / V;
-    if (lanes_needed <= 4) launch_group<T, 4>(stream, a, group_ptr, entries, alpha, beta, mean_span);
-    else if (lanes_needed <= 8) launch_group<T, 8>(stream, a, group_ptr, entries, alpha, beta, mean_span);
-    else if (lanes_needed <= 16) launch_group<T, 16>(stream, a, group_ptr, entries, alpha, beta, mean_span);
-    else if (lanes_needed <= 32) launch_group<T, 32>(stream, a, group_ptr, entries, alpha, beta, mean_span);
-    else launch_group<T, 64>(stream, a, group_ptr, entries, alpha, beta, mean_span);
+    if (lanes_needed <= 4) launch_group<T, 4>(stream, a, group_ptr, entries, total_entries, alpha, beta, mean_span);
+    else if (lanes_needed <= 8) launch_group<T, 8>(stream, a, group_ptr, entries, total_entries, alpha, beta, mean_span);
+    else if (lanes_needed <= 16) launch_group<T, 16>(stream, a, group_ptr, entries, total_entries, alpha, beta, mean_span);
+    else if (lanes_needed <= 32) launch_group<T, 32>(stream, a, group_ptr, entries, total_entries, alpha, beta, mean_span);
+    else launch_group<T, 64>(stream, a, group_ptr, entries, total_entries, alpha, beta, mean_span);
 }
 
-template void launch_spmm_scheduled<float>(hipStream_t, const SpmmArgs&, const void*, uint64_t, float, float);
-template void launch_spmm_scheduled<double>(hipStream_t, const SpmmArgs&, const void*, uint64_t, double, double);
+template void launch_spmm_scheduled<float>(hipStream_t, const SpmmArgs&, const void*, uint32_t, uint64_t, float, float);
+template void launch_spmm_scheduled<double>(hipStream_t, const SpmmArgs&, const void*, uint32_t, uint64_t, double, double);
 template void launch_spmm<float>(hipStream_t, const SpmmArgs&, float, float);
 template void launch_spmm<double>(hipStream_t, const SpmmArgs&, double, double);
 

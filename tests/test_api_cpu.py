@@ -5,6 +5,7 @@ import ctypes
 import re
 import os
 
+import numpy as np
 import pytest
 
 from mcsparse_amd import api, _lib
@@ -20,6 +21,32 @@ def test_library_exports_every_declared_symbol(lib):
     assert declared == set(_lib.PROTOTYPES), declared ^ set(_lib.PROTOTYPES)
     for name in declared:
         assert hasattr(lib, name), name
+
+
+def test_library_exports_nothing_else(lib):
+    """nm -D: every defined dynamic symbol is a C function of the header (no C++ internals leak)."""
+    import subprocess
+    from mcsparse_amd.build import LIB_PATH
+    out = subprocess.run(["nm", "-D", "--defined-only", LIB_PATH], stdout=subprocess.PIPE, text=True, check=True).stdout
+    names = [line.split()[-1] for line in out.splitlines() if line.strip()]
+    assert names, "no dynamic symbols"
+    assert set(names) == set(_lib.PROTOTYPES), set(names) ^ set(_lib.PROTOTYPES)
+    soname = subprocess.run(["readelf", "-d", LIB_PATH], stdout=subprocess.PIPE, text=True, check=True).stdout
+    assert "libmcsparse.so" in [l.split("[")[-1].rstrip("]") for l in soname.splitlines() if "SONAME" in l]
+
+
+def test_c99_caller_links_and_walks_the_argument_checks(lib, tmp_path):
+    """A C program written against the header: compiles as C99, links with the library, and gets the
+    reference's statuses on the paths that return before any launch."""
+    import subprocess
+    from mcsparse_amd.build import LIB_DIR
+    src = os.path.join(ROOT, "tests", "c_abi", "spmv_caller.c")
+    exe = str(tmp_path / "spmv_caller")
+    subprocess.run(["gcc", "-std=c99", "-Wall", "-Wextra", "-Werror", "-pedantic", "-I", os.path.join(ROOT, "include"),
+                    src, "-o", exe, "-L", LIB_DIR, "-lmcsparse", "-Wl,-rpath," + LIB_DIR,
+                    "-Wl,-rpath-link,/opt/rocm/lib"], check=True)
+    run = subprocess.run([exe], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    assert run.returncode == 0 and run.stdout.strip().endswith("ok"), run.stdout
 
 
 def test_status_strings(lib):
@@ -387,3 +414,52 @@ def test_strided_batch_setters(lib):
     assert (count.value, stride.value) == (3, 24)
     assert lib.mcsparseDnMatGetStridedBatch(B, None, ctypes.byref(stride)) == api.STATUS_INVALID_VALUE
     lib.mcsparseDestroyDnMat(B)
+
+
+def _plan(lib, lengths, x_bytes=64 << 20):
+    """Kernel choice for rows of these lengths, through the same bins the GPU analysis fills."""
+    lengths = np.asarray(lengths, dtype=np.int64)
+    hist = np.zeros(34, dtype=np.uint32)
+    bins = np.where(lengths == 0, 0, np.floor(np.log2(np.maximum(lengths, 1))).astype(np.int64) + 1)
+    np.add.at(hist, bins, 1)
+    hist[33] = lengths.max()
+    fam, lanes = ctypes.c_int(), ctypes.c_int()
+    st = lib.mcsparseXcsrRowBinsPlan(hist.ctypes.data, int(lengths.size), int(lengths.sum()), x_bytes,
+                                     ctypes.byref(fam), ctypes.byref(lanes))
+    assert st == 0
+    return fam.value, lanes.value
+
+
+def test_spmv_family_choice_from_row_bins(lib):
+    """The pure decision function behind mcsparseSpMV's dispatch, on a table of row-length spreads."""
+    rng = np.random.default_rng(0)
+    m = 1 << 16
+    # rows of one length fill their lanes: the vector family with the matching width
+    assert _plan(lib, np.full(m, 16)) == (api.FAMILY_VECTOR, 16)
+    assert _plan(lib, np.full(m, 5)) == (api.FAMILY_VECTOR, 8)
+    assert _plan(lib, np.full(m, 1)) == (api.FAMILY_VECTOR, 1)
+    assert _plan(lib, np.full(m, 27)) == (api.FAMILY_VECTOR, 32)
+    # the transposed power-law matrix: 28 +- 5 per row, every wavefront waits for a row of 33+
+    assert _plan(lib, rng.poisson(28, m))[0] == api.FAMILY_MERGE
+    # mild spreads stay with the vector family
+    assert _plan(lib, rng.poisson(20, m)) == (api.FAMILY_VECTOR, 32)
+    assert _plan(lib, rng.integers(12, 17, m)) == (api.FAMILY_VECTOR, 16)
+    # 5-point Laplacian: 3..5 per row
+    assert _plan(lib, rng.choice([3, 4, 5], m, p=[0.01, 0.04, 0.95])) == (api.FAMILY_VECTOR, 8)
+    # one row far longer than the rest serialises a wavefront: merge path; in column order when
+    # the rows exceed a tile and x does not fit an L2, in storage order otherwise
+    skew = np.full(m, 4)
+    skew[7] = 100000
+    assert _plan(lib, skew) == (api.FAMILY_MERGE, 1)
+    assert _plan(lib, skew, x_bytes=1 << 20) == (api.FAMILY_MERGE, 0)
+    skew[7] = 700
+    assert _plan(lib, skew) == (api.FAMILY_MERGE, 0)
+    # power law: most rows hold one nonzero, the mean is carried by a few long ones
+    zipf = np.minimum(rng.zipf(1.8, m), 200000)
+    assert _plan(lib, zipf)[0] == api.FAMILY_MERGE
+    # half the rows empty, the rest of one length: the lanes of the non-empty rows are full half the time
+    half = np.where(rng.random(m) < 0.5, 0, 32)
+    assert _plan(lib, half)[0] in (api.FAMILY_VECTOR, api.FAMILY_MERGE)
+    # argument checks
+    fam, lanes = ctypes.c_int(), ctypes.c_int()
+    assert lib.mcsparseXcsrRowBinsPlan(None, 1, 1, 1, ctypes.byref(fam), ctypes.byref(lanes)) == api.STATUS_INVALID_VALUE

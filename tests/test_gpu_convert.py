@@ -177,3 +177,56 @@ def test_row_bins_bit_exact(torch_gpu, handle, oracle, name):
     bins, hist = oracle.row_bins(a.m, a.ptr)
     assert np.array_equal(d_bins.cpu().numpy(), bins)
     assert np.array_equal(d_hist.cpu().numpy().view(np.uint32), hist)
+
+
+@pytest.mark.parametrize("shift", [1, 3])
+def test_unaligned_input_arrays(torch_gpu, handle, oracle, shift):
+    """Index and value arrays that start 4 bytes past a 16-byte boundary (a sub-array of a larger
+    allocation): the kernels may not assume 128-bit alignment of the caller's arrays."""
+    torch = torch_gpu
+    a = wl.random_ragged(9001, 7001, 11, dtype=np.float32, seed=31)
+    big_col = torch.zeros(a.nnz + 8, dtype=torch.int32, device="cuda")
+    big_val = torch.zeros(a.nnz + 8, dtype=torch.float32, device="cuda")
+    big_ptr = torch.zeros(a.m + 9, dtype=torch.int32, device="cuda")
+    d_col, d_val, d_ptr = big_col[shift:shift + a.nnz], big_val[shift:shift + a.nnz], big_ptr[shift:shift + a.m + 1]
+    d_col.copy_(torch.from_numpy(a.col))
+    d_val.copy_(torch.from_numpy(a.val))
+    d_ptr.copy_(torch.from_numpy(a.ptr))
+    assert d_col.data_ptr() % 16 != 0
+    o_val = torch.zeros(a.nnz + 8, dtype=torch.float32, device="cuda")[shift:shift + a.nnz]
+    o_ptr = torch.zeros(a.n + 9, dtype=torch.int32, device="cuda")[shift:shift + a.n + 1]
+    o_row = torch.zeros(a.nnz + 8, dtype=torch.int32, device="cuda")[shift:shift + a.nnz]
+    st, size = api.csr2csc_buffer_size(handle, a.m, a.n, a.nnz, d_val, d_ptr, d_col, o_val, o_ptr, o_row, api.R_32F,
+                                       api.ACTION_NUMERIC, 0)
+    assert st == 0
+    buf = torch.empty(size, dtype=torch.uint8, device="cuda")
+    assert api.csr2csc(handle, a.m, a.n, a.nnz, d_val, d_ptr, d_col, o_val, o_ptr, o_row, api.R_32F,
+                       api.ACTION_NUMERIC, 0, buf) == 0
+    torch.cuda.synchronize()
+    w_cp, w_ri, w_cv = oracle.csr2csc(a.m, a.n, 0, a.ptr, a.col, a.val, method="counting")
+    assert np.array_equal(o_ptr.cpu().numpy().view(np.uint32), w_cp)
+    assert np.array_equal(o_row.cpu().numpy().view(np.uint32), w_ri)
+    assert np.array_equal(o_val.cpu().numpy(), w_cv)
+    # the transposing SpMV sorts the same way, reading the caller's arrays in its first pass
+    rng = np.random.default_rng(2)
+    x = rng.uniform(-1, 1, a.m).astype(np.float32)
+    d_x = torch.from_numpy(x).cuda()
+    d_y = torch.zeros(a.n, dtype=torch.float32, device="cuda")
+    mat = api.SpMat(a.m, a.n, a.nnz, d_ptr, d_col, d_val)
+    vx, vy = api.DnVec(d_x), api.DnVec(d_y)
+    st, size = api.spmv_buffer_size(handle, api.OP_T, 1.0, mat, vx, 0.0, vy, api.R_32F)
+    buf = torch.empty(size, dtype=torch.uint8, device="cuda")
+    assert api.spmv(handle, api.OP_T, 1.0, mat, vx, 0.0, vy, api.R_32F, buf) == 0
+    torch.cuda.synchronize()
+    y_ref, bound = oracle.spmv(True, a.m, a.n, 0, a.ptr, a.col, a.val, 1.0, 0.0, x, None)
+    err = np.abs(d_y.cpu().numpy().astype(np.longdouble) - y_ref)
+    assert (err <= 8 * 2.0 ** -24 * bound).all()
+    # coo2csr on an unaligned, mostly empty structure: long stretches of empty rows
+    rows = np.sort(rng.integers(0, 50, 300)).astype(np.int32)
+    d_rows = torch.zeros(308, dtype=torch.int32, device="cuda")[shift:shift + 300]
+    d_rows.copy_(torch.from_numpy(rows))
+    m_big = 1 << 20
+    d_out = torch.full((m_big + 1,), -7, dtype=torch.int32, device="cuda")
+    assert api.xcoo2csr(handle, d_rows, 300, m_big, d_out, 0) == 0
+    torch.cuda.synchronize()
+    assert np.array_equal(d_out.cpu().numpy().view(np.uint32), oracle.coo2csr(300, m_big, 0, rows))

@@ -12,6 +12,7 @@ from mcsparse_amd import workloads as wl
 from gpu_util import assert_within, dev, run_spmv
 from test_gpu_convert import gpu_csr2coo, gpu_csr2csc
 from test_gpu_spmm import run_spmm
+from test_gpu_spmv_banded import run_banded
 
 pytestmark = pytest.mark.gpu
 
@@ -64,9 +65,21 @@ def test_config5_conversions_full_size(torch_gpu, handle, oracle, power_law_full
     csc_as_csr = wl.Csr(a.n, a.m, cp, ri, cv)  # arrays of A^T in CSR form
     st, yt, plan = run_spmv(torch_gpu, handle, csc_as_csr, xt, np.zeros(a.n, np.float32), 1.0, 0.0, op=api.OP_T,
                             fmt=api.FORMAT_CSC)
-    assert st == 0 and plan[0] == api.FAMILY_VECTOR
+    # 28 +- 5 nonzeros per row of A^T: rows of 33 and more keep every wavefront of the vector family waiting
+    assert st == 0 and plan[0] == api.FAMILY_MERGE
     yt_ref, bound_t = oracle.spmv(True, a.m, a.n, 0, a.ptr, a.col, a.val, 1.0, 0.0, xt, None)
     assert_within(yt, yt_ref, bound_t, np.float32, what="C5 A^T x from CSC")
+    # the same product from the column-banded copy of mcsparseSpMV_preprocess (x = 16.8 MB: 8 bands)
+    state, bands, rows = run_banded(torch_gpu, handle, oracle, csc_as_csr, 1.0, 0.0, as_csc=True,
+                                    what="C5 A^T x from CSC, banded", reference=(xt, yt_ref, bound_t))
+    assert (state, bands) == (2, 8)
+
+
+def test_config2_full_size_banded(torch_gpu, handle, oracle):
+    a = wl.uniform_rows(m=1 << 20, per_row=16, dtype=np.float64)
+    assert a.nnz == 16777216
+    state, bands, rows = run_banded(torch_gpu, handle, oracle, a, 1.5, 0.5, calls=2, what="C2 banded")
+    assert (state, bands) == (2, 4)
 
 
 @pytest.fixture(scope="module")

@@ -36,6 +36,7 @@ def test_calls_replay_in_a_hip_graph(torch_gpu, oracle):
     d_a, d_p, d_s = upload(a), upload(p), upload(s)
     held += [d_a, d_p, d_s]
     A = api.SpMat(a.m, a.n, a.nnz, *d_a, base=a.base)
+    A.set_plan(api.FAMILY_VECTOR)  # both families take part in the graph: this one by request, P by analysis
     P = api.SpMat(p.m, p.n, p.nnz, *d_p, base=p.base)
     S = api.SpMat(s.m, s.n, s.nnz, *d_s, base=s.base)
 

@@ -205,3 +205,37 @@ def test_schedule_is_dropped_with_other_buffer_or_pointers(torch_gpu, handle, or
     d_col2 = d_col.clone()
     assert handle.lib.mcsparseCsrSetPointers(mat.ptr, d_ptr.data_ptr(), d_col2.data_ptr(), d_val.data_ptr()) == 0
     assert mat.spmm_schedule()[0] == 0
+
+
+def test_overwritten_schedule_stays_in_bounds(torch_gpu, handle):
+    """The reference's preprocess is a no-op, so a caller written against it may reuse the scratch
+    buffer between preprocess and SpMM.  The schedule is then garbage: the product may be wrong, but
+    every access stays inside the arrays (the call returns and the device stays healthy)."""
+    torch = torch_gpu
+    a = wl.stencil_27pt(10, dtype=np.float32)
+    n = 64
+    d_ptr, d_col, d_val = dev(torch, a.ptr), dev(torch, a.col), dev(torch, a.val)
+    d_B = torch.ones((a.n, n), dtype=torch.float32, device="cuda")
+    d_C = torch.zeros((a.m, n), dtype=torch.float32, device="cuda")
+    mat = api.SpMat(a.m, a.n, a.nnz, d_ptr, d_col, d_val)
+    mB, mC = api.DnMat(a.n, n, n, d_B), api.DnMat(a.m, n, n, d_C)
+    st, size = api.spmm_buffer_size(handle, api.OP_N, api.OP_N, 1.0, mat, mB, 0.0, mC, api.R_32F)
+    buf = torch.empty(size, dtype=torch.uint8, device="cuda")
+    assert api.spmm_preprocess(handle, api.OP_N, api.OP_N, 1.0, mat, mB, 0.0, mC, api.R_32F, buf) == 0
+    assert mat.spmm_schedule()[0] == 2
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(3)
+    for fill in (0xFF, None, 0x00):
+        if fill is None:
+            buf.copy_(torch.randint(0, 256, (size,), dtype=torch.uint8, device="cuda", generator=gen))
+        else:
+            buf.fill_(fill)
+        assert api.spmm(handle, api.OP_N, api.OP_N, 1.0, mat, mB, 0.0, mC, api.R_32F, buf) == 0
+        torch.cuda.synchronize()
+    # a fresh preprocess makes the same buffer good again
+    assert api.spmm_preprocess(handle, api.OP_N, api.OP_N, 1.0, mat, mB, 0.0, mC, api.R_32F, buf) == 0
+    assert api.spmm(handle, api.OP_N, api.OP_N, 1.0, mat, mB, 0.0, mC, api.R_32F, buf) == 0
+    torch.cuda.synchronize()
+    want = np.asarray(a.to_scipy().sum(axis=1)).ravel()  # B = ones: row sums of A
+    got = d_C.cpu().numpy()
+    assert np.allclose(got, want[:, None].repeat(n, 1), rtol=1e-5, atol=1e-5)

@@ -17,12 +17,14 @@ GOLDEN = sorted(glob.glob(os.path.join(os.path.dirname(__file__), "golden", "csr
 
 
 def run_banded(torch, handle, oracle, a, alpha, beta, band_bytes=0, seed=1, expect_state=2, what="", calls=1,
-               as_csc=False):
-    """as_csc: the arrays are handed over as the CSC of the n x m transpose and applied with op T."""
+               as_csc=False, reference=None):
+    """as_csc: the arrays are handed over as the CSC of the n x m transpose and applied with op T.
+    reference: (x, y_ref, bound) of a product the caller has already worked out with the oracle, for
+    beta == 0 (saves a second pass of the oracle over a large matrix)."""
     rng = np.random.default_rng(seed)
     dt = a.val.dtype
     ct = api.maca_type(dt)
-    x = rng.uniform(-1, 1, a.n).astype(dt)
+    x = rng.uniform(-1, 1, a.n).astype(dt) if reference is None else reference[0]
     y = rng.uniform(-1, 1, a.m).astype(dt)
     d_ptr, d_col, d_val, d_x, d_y = (dev(torch, v) for v in (a.ptr, a.col, a.val, x, y))
     if as_csc:
@@ -40,7 +42,11 @@ def run_banded(torch, handle, oracle, a, alpha, beta, band_bytes=0, seed=1, expe
     assert api.spmv_preprocess(handle, op, alpha, mat, vx, beta, vy, ct, buf) == api.STATUS_SUCCESS
     state, bands, rows = mat.spmv_preprocess_state()
     assert state == expect_state, (state, bands, rows)
-    y_ref, bound = oracle.spmv(False, a.m, a.n, a.base, a.ptr, a.col, a.val, alpha, beta, x, y)
+    if reference is None:
+        y_ref, bound = oracle.spmv(False, a.m, a.n, a.base, a.ptr, a.col, a.val, alpha, beta, x, y)
+    else:
+        assert beta == 0.0
+        y_ref, bound = alpha * reference[1], abs(alpha) * reference[2]
     first = None
     for _ in range(calls):
         d_y.copy_(torch.from_numpy(y))
