@@ -339,8 +339,16 @@ mcspStatus_t spmv_typed(mcsparseHandle_t h, mcsparseSpMatDescr* A, mcsparseOpera
 // CSC gets the transposed copy [row_ptr m+1 | col_ind nnz][values][csr2csc workspace]
 // (mcsp_spmm_gpu.cpp:818-849); 64-bit index arrays add their narrowed copies at the end.
 struct SpmmLayout {
-    size_t ptr, ind, vals, csr2csc_ws, narrow, total;
+    size_t ptr, ind, vals, csr2csc_ws, bt, ct, narrow, total;
+    int64_t n_padded;  // leading dimension of the row-major copies of op(B) and C
+    bool copy_b, copy_c;
 };
+
+// op(B)(kk, j) sits at kk*ldb + j for (N, row-major) and (T, column-major), else at j*ldb + kk.
+bool b_image_is_row_major(mcsparseOperation_t opB, const mcsparseDnMatDescr* B) {
+    const bool op_n = opB == MCSPARSE_OPERATION_NON_TRANSPOSE;
+    return (op_n && B->order == MCSPARSE_ORDER_ROW) || (!op_n && B->order == MCSPARSE_ORDER_COL);
+}
 
 bool schedulable(const mcsparseSpMatDescr* A) {
     return A->format == MCSPARSE_FORMAT_CSR && A->row_num > 0 && A->nnz > 0 &&
@@ -354,7 +362,12 @@ bool schedule_matches(const mcsparseSpMatDescr* A, const void* buffer) {
            s.nnz == A->nnz && s.base == static_cast<int>(A->idxBase);
 }
 
-SpmmLayout spmm_layout(const mcsparseSpMatDescr* A, size_t value_bytes) {
+// A column-major op(B) would be gathered element by element and a column-major C written element by
+// element; with room in the scratch buffer they are transposed instead (the reference copies the other
+// way round, into memory it allocates: mcsp_spmm_gpu.cpp:119-133): op(B) into a row-major copy before
+// the product, the product from a row-major C out into the caller's.
+SpmmLayout spmm_layout(const mcsparseSpMatDescr* A, const mcsparseDnMatDescr* B, const mcsparseDnMatDescr* C,
+                       mcsparseOperation_t opB, size_t value_bytes) {
     SpmmLayout l = {};
     size_t off = 0;
     if (A->format == MCSPARSE_FORMAT_CSR) {
@@ -370,6 +383,14 @@ SpmmLayout spmm_layout(const mcsparseSpMatDescr* A, size_t value_bytes) {
         off += align_up(mcsp::csr2csc_workspace_bytes(static_cast<idx_t>(A->col_num), static_cast<idx_t>(A->row_num),
                                                       static_cast<idx_t>(A->nnz), value_bytes));
     }
+    const int64_t n = C->col_num;
+    l.n_padded = (n + 3) / 4 * 4;
+    l.copy_b = !b_image_is_row_major(opB, B) && A->col_num > 0 && n > 0;
+    l.copy_c = C->order != MCSPARSE_ORDER_ROW && A->row_num > 0 && n > 0;
+    l.bt = off;
+    if (l.copy_b) off += align_up(static_cast<size_t>(A->col_num) * l.n_padded * value_bytes);
+    l.ct = off;
+    if (l.copy_c) off += align_up(static_cast<size_t>(A->row_num) * l.n_padded * value_bytes);
     l.narrow = off;
     off += narrow_bytes(A);
     l.total = off < kMinBuffer ? kMinBuffer : off;
@@ -386,7 +407,7 @@ mcspStatus_t spmm_typed(mcsparseHandle_t h, const mcsparseSpMatDescr* A, mcspars
     if (A->nnz == 0 && h_beta == T(1)) return MCSP_STATUS_SUCCESS;
 
     char* buf = static_cast<char*>(buffer);
-    const SpmmLayout l = spmm_layout(A, sizeof(T));
+    const SpmmLayout l = spmm_layout(A, B, C, opB, sizeof(T));
     // Strided batches (csr_spmm_device.hpp:102-108): batch b works on the arrays moved on by b
     // strides; the reference runs them as blockIdx.z of one launch, here they are launches in a
     // row on the stream, sharing the scratch buffer.
@@ -432,21 +453,44 @@ mcspStatus_t spmm_typed(mcsparseHandle_t h, const mcsparseSpMatDescr* A, mcspars
             mcsp::launch_coo2csr(h->stream, 0, a.m, built, a.base, built);
             a.row_ptr = built;
         }
-        a.B = static_cast<const char*>(B->values) + b * B->batchStride * static_cast<int64_t>(sizeof(T));
+        const T* b_user = reinterpret_cast<const T*>(static_cast<const char*>(B->values) +
+                                                     b * B->batchStride * static_cast<int64_t>(sizeof(T)));
+        T* c_user = reinterpret_cast<T*>(static_cast<char*>(C->values) +
+                                         b * C->batchStride * static_cast<int64_t>(sizeof(T)));
+        a.B = b_user;
         a.ldb = B->ld;
-        // op(B)(kk, j) sits at kk*ldb + j for (N, row-major) and (T, column-major), else at j*ldb + kk;
-        // the reference copies the first kind into the second (mcsp_spmm_gpu.cpp:119-133).
-        const bool op_n = opB == MCSPARSE_OPERATION_NON_TRANSPOSE;
-        a.b_row_major = (op_n && B->order == MCSPARSE_ORDER_ROW) || (!op_n && B->order == MCSPARSE_ORDER_COL);
-        a.C = static_cast<char*>(C->values) + b * C->batchStride * static_cast<int64_t>(sizeof(T));
+        a.b_row_major = b_image_is_row_major(opB, B);
+        a.C = c_user;
         a.ldc = C->ld;
         a.c_row_major = C->order == MCSPARSE_ORDER_ROW;
+        T beta_inner = h_beta;
+        if (l.copy_b && A->nnz != 0) {  // without nonzeros op(B) is never read (and may be NULL)
+            // the column-major image is a row-major n x k matrix: its transpose is op(B), row-major
+            T* bt = reinterpret_cast<T*>(buf + l.bt);
+            mcsp::launch_transpose<T>(h->stream, a.n, a.k, static_cast<idx_t>(l.n_padded), b_user, B->ld, bt, l.n_padded);
+            a.B = bt;
+            a.ldb = l.n_padded;
+            a.b_row_major = true;
+        }
+        if (l.copy_c) {
+            a.C = buf + l.ct;
+            a.ldc = l.n_padded;
+            a.c_row_major = true;
+            beta_inner = T(0);  // beta * C is added when the product is transposed out
+            // with both copies at hand the padded columns of op(B) are zeros: whole 128-bit vectors
+            if (l.copy_b && A->nnz != 0) a.n = static_cast<idx_t>(l.n_padded);
+        }
         // the schedule was built from batch 0's structure
         if ((b == 0 || shared_structure) && schedule_matches(A, buffer) && mcsp::spmm_schedule_usable(a, sizeof(T))) {
             mcsp::launch_spmm_scheduled<T>(h->stream, a, buffer, A->schedule.entries, A->schedule.mean_span, h_alpha,
-                                           h_beta);
+                                           beta_inner);
         } else {
-            mcsp::launch_spmm<T>(h->stream, a, h_alpha, h_beta);
+            mcsp::launch_spmm<T>(h->stream, a, h_alpha, beta_inner);
+        }
+        if (l.copy_c) {
+            mcsp::launch_transpose_accumulate<T>(h->stream, a.m, static_cast<idx_t>(C->col_num),
+                                                 reinterpret_cast<const T*>(buf + l.ct), l.n_padded, c_user, C->ld,
+                                                 h_beta);
         }
     }
     return MCSP_STATUS_SUCCESS;
@@ -685,7 +729,7 @@ mcsparseStatus_t mcsparseSpMV_preprocess(mcsparseHandle_t handle, mcsparseOperat
 
 // reference: src/kernels/level3/spmm/mcsp_spmm_gpu.cpp:309-342, :950-963
 mcsparseStatus_t mcsparseSpMM_bufferSize(mcsparseHandle_t handle, mcsparseOperation_t /*opA*/,
-                                         mcsparseOperation_t /*opB*/, const void* alpha, mcsparseSpMatDescr_t matA,
+                                         mcsparseOperation_t opB, const void* alpha, mcsparseSpMatDescr_t matA,
                                          mcsparseDnMatDescr_t matB, const void* beta, mcsparseDnMatDescr_t matC,
                                          macaDataType /*computeType*/, mcsparseSpMMAlg_t /*alg*/,
                                          size_t* bufferSize) {
@@ -697,7 +741,7 @@ mcsparseStatus_t mcsparseSpMM_bufferSize(mcsparseHandle_t handle, mcsparseOperat
     if (st != MCSP_STATUS_SUCCESS) return to_public_status(st);
     if (bufferSize == nullptr) return to_public_status(MCSP_STATUS_INVALID_POINTER);
     if (!format_is_built(matA->format)) return to_public_status(MCSP_STATUS_NOT_IMPLEMENTED);  // Blocked-ELL
-    *bufferSize = spmm_layout(matA, value_size(matA->valueType)).total;
+    *bufferSize = spmm_layout(matA, matB, matC, opB, value_size(matA->valueType)).total;
     if (matA->format == MCSPARSE_FORMAT_CSC) matA->is_buffersize_called = 1;
     return MCSPARSE_STATUS_SUCCESS;
 }
@@ -707,7 +751,7 @@ mcsparseStatus_t mcsparseSpMM_bufferSize(mcsparseHandle_t handle, mcsparseOperat
 // mcsparseSpMM uses it when it is handed the same buffer and the same CSR arrays, and falls back
 // to the schedule-free kernel otherwise.  Until then the caller must leave the buffer and the
 // structure of A alone; the values of A may change freely.
-mcsparseStatus_t mcsparseSpMM_preprocess(mcsparseHandle_t handle, mcsparseOperation_t opA, mcsparseOperation_t /*opB*/,
+mcsparseStatus_t mcsparseSpMM_preprocess(mcsparseHandle_t handle, mcsparseOperation_t opA, mcsparseOperation_t opB,
                                          const void* alpha, mcsparseSpMatDescr_t matA, mcsparseDnMatDescr_t matB,
                                          const void* beta, mcsparseDnMatDescr_t matC, macaDataType /*computeType*/,
                                          mcsparseSpMMAlg_t /*alg*/, void* externalBuffer) {
@@ -728,7 +772,7 @@ mcsparseStatus_t mcsparseSpMM_preprocess(mcsparseHandle_t handle, mcsparseOperat
     const idx_t m = static_cast<idx_t>(matA->row_num);
     const idx_t nnz = static_cast<idx_t>(matA->nnz);
     const IndexArrays ia = index_arrays(handle, matA, static_cast<char*>(externalBuffer) +
-                                                          spmm_layout(matA, value_size(matA->valueType)).narrow);
+                                                          spmm_layout(matA, matB, matC, opB, value_size(matA->valueType)).narrow);
     mcsp::launch_spmm_schedule(handle->stream, m, nnz, static_cast<idx_t>(matA->idxBase), ia.rows, ia.cols,
                                externalBuffer);
     const mcsp::SpmmScheduleLayout l = mcsp::spmm_schedule_layout(m, nnz);

@@ -311,6 +311,17 @@ template <typename T>
 void launch_spmm_scheduled(hipStream_t stream, const SpmmArgs& a, const void* schedule, uint32_t total_entries,
                            uint64_t mean_span, T alpha, T beta);
 
+// Dense transposes for column-major SpMM operands (spmm.hip).  src is rows x cols, row-major with
+// leading dimension lds.  launch_transpose: dst (cols x rows_padded, ldd) = transpose(src), the columns
+// [rows, rows_padded) of dst zero.  launch_transpose_accumulate: dst = beta * dst + transpose(src);
+// beta == 0 does not read dst.
+template <typename T>
+void launch_transpose(hipStream_t stream, idx_t rows, idx_t cols, idx_t rows_padded, const T* src, int64_t lds, T* dst,
+                      int64_t ldd);
+template <typename T>
+void launch_transpose_accumulate(hipStream_t stream, idx_t rows, idx_t cols, const T* src, int64_t lds, T* dst,
+                                 int64_t ldd, T beta);
+
 // ---- conversions (convert.hip) ----
 void launch_csr2coo(hipStream_t stream, idx_t m, idx_t nnz, const idx_t* row_ptr, idx_t base, idx_t* coo_rows);
 void launch_coo2csr(hipStream_t stream, idx_t nnz, idx_t m, const idx_t* coo_rows, idx_t base, idx_t* row_ptr);

@@ -388,6 +388,54 @@ __global__ __launch_bounds__(kBlock) void spmm_colb_kernel(idx_t m, idx_t n, idx
     }
 }
 
+// ---- dense transposes for column-major operands ---------------------------------------------
+// dst (cols x rows_padded, row-major, leading dimension ldd) <- transpose of src (rows x cols,
+// row-major, leading dimension lds), 64 x 64 elements per workgroup through LDS so that both sides
+// move whole cache lines.  Columns [rows, rows_padded) of dst are filled with zeros.  ACCUMULATE:
+// dst = beta * dst + transpose(src) (beta == 0 does not read dst) and nothing is padded.
+// Stands in for mcspDenseTransposeKernel (src/common/mcsp_dense_transpose_device.hpp:8-38).
+constexpr int kTransTile = 64;
+template <typename T, bool ACCUMULATE>
+__global__ __launch_bounds__(kBlock) void transpose_kernel(uint32_t rows, uint32_t cols, uint32_t rows_padded,
+                                                           const T* __restrict__ src, int64_t lds,
+                                                           T* __restrict__ dst, int64_t ldd, T beta) {
+    __shared__ T tile[kTransTile][kTransTile + 1];
+    const uint32_t tx = threadIdx.x % kTransTile;
+    const uint32_t ty = threadIdx.x / kTransTile;  // 0..3
+    const uint32_t r0 = blockIdx.x * kTransTile;   // along rows of src
+    const uint32_t c0 = blockIdx.y * kTransTile;   // along cols of src
+    T got[kTransTile / 4];
+#pragma unroll
+    for (int k = 0; k < kTransTile / 4; ++k) {
+        const uint32_t r = r0 + ty + 4 * k;
+        const uint32_t c = c0 + tx;
+        // clamped position, so that the sixteen loads are on their way together
+        const uint32_t rr = r < rows ? r : rows - 1;
+        const uint32_t cc = c < cols ? c : cols - 1;
+        got[k] = src[static_cast<int64_t>(rr) * lds + cc];
+    }
+#pragma unroll
+    for (int k = 0; k < kTransTile / 4; ++k) {
+        const uint32_t r = r0 + ty + 4 * k;
+        tile[ty + 4 * k][tx] = r < rows ? got[k] : T(0);
+    }
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < kTransTile / 4; ++k) {
+        const uint32_t c = c0 + ty + 4 * k;  // row of dst
+        const uint32_t r = r0 + tx;          // column of dst
+        if (c < cols && r < (ACCUMULATE ? rows : rows_padded)) {
+            T* out = dst + static_cast<int64_t>(c) * ldd + r;
+            const T v = tile[tx][ty + 4 * k];
+            if constexpr (ACCUMULATE) {
+                *out = beta == T(0) ? v : beta * *out + v;
+            } else {
+                *out = v;
+            }
+        }
+    }
+}
+
 // ---- row groups -------------------------------------------------------------------------
 // Neighbouring rows of a matrix from a mesh or a stencil share most of their columns.  A lane
 // group that owns kSpmmGroupRows consecutive rows walks the merged column list of the group
@@ -540,8 +588,13 @@ __device__ __forceinline__ bool shift_out_top(uint32_t& w) {
 // panels of LR*V columns.  The lanes of a group fetch LR entries of the merged list at once, one
 // each, work out from the flag bits which value of which row belongs to their entry, fetch
 // those, and pass row offsets, flags and values round in registers.
+// The register allocation of this kernel sits at the edge between six and four wavefronts per SIMD:
+// clamping the column of an entry (one instruction) made the compiler's scheduler settle on 118
+// registers instead of 79 and the kernel 13 % slower at 64 columns.  The occupancy the narrow groups
+// run best at is therefore asked for outright (six; the wider groups measured 6 % slower when held to
+// it and keep five).
 template <typename T, int LR, bool WIDE>
-__global__ __launch_bounds__(kBlock) void spmm_group_kernel(idx_t m, idx_t n, idx_t base,
+__global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(LR <= 16 ? 6 : 5))) void spmm_group_kernel(idx_t m, idx_t n, idx_t base,
                                                             const idx_t* __restrict__ row_ptr,
                                                             const idx_t* __restrict__ col, const T* __restrict__ val,
                                                             const uint32_t* __restrict__ group_ptr,
@@ -585,6 +638,7 @@ __global__ __launch_bounds__(kBlock) void spmm_group_kernel(idx_t m, idx_t n, id
         const uint32_t s_end = min(group_ptr[group + 1], total_entries);
         const uint32_t s_begin = min(group_ptr[group], s_end);
         const idx_t last_value = nnz - 1;  // nnz != 0: the group has nonzeros
+        const off_t roff_limit = static_cast<off_t>(k - 1) * ldb_bytes;
         const unsigned group_first = (__lane_id() / LR) * LR;
         const uint64_t group_bits = LR == kWave ? ~0ull : ((1ull << (LR % kWave)) - 1ull);
         const uint64_t below = (1ull << lane) - 1ull;
@@ -605,7 +659,7 @@ __global__ __launch_bounds__(kBlock) void spmm_group_kernel(idx_t m, idx_t n, id
                 i[r] += __popcll(in);
                 take[r] = __brev(static_cast<uint32_t>(in));
             }
-            const off_t roff = static_cast<off_t>(min(ent >> R, k - 1)) * ldb_bytes;
+            const off_t roff = min(static_cast<off_t>(ent >> R) * ldb_bytes, roff_limit);
             const uint32_t flags = ent & ((1u << R) - 1u);
             const uint32_t left = s_end - s;
             // With kAlternate two batches of rows of op(B) take turns: the loads of one are on their
@@ -834,6 +888,29 @@ void launch_spmm_scheduled(hipStream_t stream, const SpmmArgs& a, const void* sc
     else launch_group<T, 64>(stream, a, group_ptr, entries, total_entries, alpha, beta, mean_span);
 }
 
+template <typename T>
+void launch_transpose(hipStream_t stream, idx_t rows, idx_t cols, idx_t rows_padded, const T* src, int64_t lds, T* dst,
+                      int64_t ldd) {
+    if (rows == 0 || cols == 0) return;
+    const dim3 grid((rows_padded + kTransTile - 1) / kTransTile, (cols + kTransTile - 1) / kTransTile);
+    hipLaunchKernelGGL((transpose_kernel<T, false>), grid, dim3(kBlock), 0, stream, rows, cols, rows_padded, src, lds,
+                       dst, ldd, T(0));
+}
+
+template <typename T>
+void launch_transpose_accumulate(hipStream_t stream, idx_t rows, idx_t cols, const T* src, int64_t lds, T* dst,
+                                 int64_t ldd, T beta) {
+    if (rows == 0 || cols == 0) return;
+    const dim3 grid((rows + kTransTile - 1) / kTransTile, (cols + kTransTile - 1) / kTransTile);
+    hipLaunchKernelGGL((transpose_kernel<T, true>), grid, dim3(kBlock), 0, stream, rows, cols, rows, src, lds, dst, ldd,
+                       beta);
+}
+
+template void launch_transpose<float>(hipStream_t, idx_t, idx_t, idx_t, const float*, int64_t, float*, int64_t);
+template void launch_transpose<double>(hipStream_t, idx_t, idx_t, idx_t, const double*, int64_t, double*, int64_t);
+template void launch_transpose_accumulate<float>(hipStream_t, idx_t, idx_t, const float*, int64_t, float*, int64_t, float);
+template void launch_transpose_accumulate<double>(hipStream_t, idx_t, idx_t, const double*, int64_t, double*, int64_t,
+                                                  double);
 template void launch_spmm_scheduled<float>(hipStream_t, const SpmmArgs&, const void*, uint32_t, uint64_t, float, float);
 template void launch_spmm_scheduled<double>(hipStream_t, const SpmmArgs&, const void*, uint32_t, uint64_t, double, double);
 template void launch_spmm<float>(hipStream_t, const SpmmArgs&, float, float);
