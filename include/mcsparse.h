@@ -448,9 +448,10 @@ mcsparseStatus_t mcsparseSpMatGetSpMMSchedule(mcsparseSpMatDescr_t spMatDescr, i
  *     passed to both calls, and must be left alone in between, like the structure of A.
  *   - The copy includes the values.  After changing values in place call mcsparseSpMV_preprocess
  *     again; mcsparseSpMatSetValues and mcsparseCsrSetPointers drop the copy.
- *   - Matrices the layout cannot help (x fits in cache as it is, rows longer than a few hundred
- *     nonzeros, formats other than 32-bit CSR) are left to the ordinary kernels; the call still
- *     returns SUCCESS.  mcsparseSpMatGetSpMVPreprocess tells which case applies.
+ *   - Calls the layout cannot help (x fits in cache as it is, 64-bit indices, COO, the transposing
+ *     directions CSR op T and CSC op N) are left to the ordinary kernels; the call still returns
+ *     SUCCESS.  CSC with op T is prepared like CSR with op N.  mcsparseSpMatGetSpMVPreprocess tells
+ *     which case applies.
  *   - Results stay within the same bound as mcsparseSpMV's and are bit-reproducible from run to run.
  * The call blocks the host until the copy is built. */
 mcsparseStatus_t mcsparseSpMV_preprocess_bufferSize(mcsparseHandle_t handle, mcsparseOperation_t opA,

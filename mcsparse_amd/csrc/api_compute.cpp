@@ -685,7 +685,7 @@ mcsparseStatus_t mcsparseSpMV_preprocess(mcsparseHandle_t handle, mcsparseOperat
     BandedShape shape;
     if (matA->nnz == 0 || !banded_candidate(matA, opA, &shape)) return MCSPARSE_STATUS_SUCCESS;  // nothing to prepare
 
-    // the row-length analysis says whether the rows are short enough for the banded kernel
+    // the plan of the row kernels is worked out here as well, so that no later call has to block for it
     const CsrView v = make_view(matA, opA);
     const idx_t m = static_cast<idx_t>(v.m);
     const idx_t nnz = static_cast<idx_t>(matA->nnz);
@@ -708,11 +708,6 @@ mcsparseStatus_t mcsparseSpMV_preprocess(mcsparseHandle_t handle, mcsparseOperat
     b.shape = shape;
     b.region = banded_region_offset(matA, opA, vb);
     b.grid = 0;
-    if (matA->plan.forced_family == kFamilyAuto && matA->plan.max_row_len > mcsp::kBandedMaxRowLength) {
-        b.useful = false;
-        b.valid = true;
-        return MCSPARSE_STATUS_SUCCESS;
-    }
     char* region = static_cast<char*>(externalBuffer) + b.region;
     mcsp::launch_banded_build(handle->stream, shape, m, nnz, base, v.ptr, v.ind, matA->vals, vb, region);
     uint32_t xcd_start[9];

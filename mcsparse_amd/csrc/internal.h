@@ -107,7 +107,8 @@ struct BandedShape {
 };
 struct SpmvBanded {
     bool valid = false;
-    bool useful = false;     // false: preprocess looked at the matrix and left it to the row kernels
+    bool useful = false;     // false: preprocess looked at the matrix and left it to the row kernels (kept for
+                             // structures a later version may decline; every candidate is banded today)
     const void* buffer = nullptr;
     const void* rows = nullptr;
     const void* cols = nullptr;
@@ -250,11 +251,9 @@ void launch_row_sums_merge(hipStream_t stream, const SpmvArgs& a, T alpha, T bet
 int spmv_pick_lanes(idx_t m, idx_t nnz);
 
 // ---- column-banded SpMV (spmv_banded.hip) ----
-// Rows of a tile (one workgroup's share of a band), the width of a band of x in bytes, and the
-// longest row the banded kernel takes (it adds up a row's run inside a tile with one thread).
+// Rows of a tile (one workgroup's share of a band) and the width of a band of x in bytes.
 constexpr int kBandedMaxRowsPerTile = 1024;
 constexpr size_t kBandedBandBytes = size_t(2) << 20;
-constexpr uint32_t kBandedMaxRowLength = 256;
 struct BandedLayout {
     // kept between preprocess and SpMV: [0, keep); scratch of the build: [keep, total)
     size_t tile_ptr, xcd_start, entries, vals, partials, keep, tmp_keys, tmp_rows, sort_ws, total;

@@ -82,9 +82,13 @@ __global__ void banded_split_kernel(idx_t nnz, uint32_t tiles, const idx_t* __re
 // One tile per workgroup.  The tile's entries are staged a slab at a time: coalesced loads of the
 // packed entries and values, the gathers from the band of x, products and row numbers to LDS; the
 // ends of every row's run are found where neighbouring entries differ; then thread r adds up the run
-// of row r (and r + 256, ...) in storage order and keeps the sum in a register across slabs.
+// of row r (and r + 256, ...) in storage order into the row's accumulator in LDS.  A run longer than
+// kLongRun entries (a long row of a power-law matrix puts thousands into one band) is left to a whole
+// wavefront: lane l adds the entries l, l + 64, ... in order and the lane sums are added in a fixed
+// tree, so the result does not depend on which wavefront picks the run up.
 // Every index that comes out of the layout is clamped, so a layout the caller has overwritten gives
 // wrong numbers but never an access outside the arrays.
+constexpr uint32_t kLongRun = 48;
 template <typename T>
 __global__ __launch_bounds__(kBlock) void spmv_banded_kernel(idx_t m, idx_t n, idx_t nnz, idx_t base, uint32_t band_shift,
                                                              uint32_t rows_per_tile, uint32_t chunks, uint32_t tiles,
@@ -94,9 +98,12 @@ __global__ __launch_bounds__(kBlock) void spmv_banded_kernel(idx_t m, idx_t n, i
                                                              const T* __restrict__ vals, const T* __restrict__ x,
                                                              T* __restrict__ partials) {
     __shared__ T s_prod[kSlab];
+    __shared__ T s_acc[kBandedMaxRowsPerTile];
     __shared__ uint16_t s_row[kSlab];
     __shared__ uint16_t s_beg[kBandedMaxRowsPerTile];
     __shared__ uint16_t s_end[kBandedMaxRowsPerTile];
+    __shared__ uint16_t s_long[kSlab / kLongRun + 1];  // rows whose run in this slab is long
+    __shared__ uint32_t s_long_count;
 
     const uint32_t tid = threadIdx.x;
     const uint32_t xcd = blockIdx.x % kXcds;
@@ -119,10 +126,9 @@ __global__ __launch_bounds__(kBlock) void spmv_banded_kernel(idx_t m, idx_t n, i
     for (int q = 0; q < kRowsPerThread; ++q) {
         s_beg[q * kBlock + tid] = 0;
         s_end[q * kBlock + tid] = 0;
+        s_acc[q * kBlock + tid] = T(0);
     }
-    T acc[kRowsPerThread];
-#pragma unroll
-    for (int q = 0; q < kRowsPerThread; ++q) acc[q] = T(0);
+    if (tid == 0) s_long_count = 0;
 
     for (idx_t slab = e0; slab < e1; slab += kSlab) {
         const uint32_t cnt = e1 - slab < static_cast<idx_t>(kSlab) ? e1 - slab : kSlab;
@@ -174,21 +180,50 @@ __global__ __launch_bounds__(kBlock) void spmv_banded_kernel(idx_t m, idx_t n, i
                 uint32_t end = s_end[r];
                 uint32_t j = s_beg[r];
                 end = end < cnt ? end : cnt;
-                T sum = T(0);
-                for (; j < end; ++j) sum += s_prod[j];
-                acc[q] += sum;
-                s_beg[r] = 0;
-                s_end[r] = 0;
+                if (end > j + kLongRun) {
+                    // at most cnt / kLongRun such runs fit a slab, so the list cannot overflow; its
+                    // order does not matter, every run is summed on its own
+                    s_long[atomicAdd(&s_long_count, 1u) % (kSlab / kLongRun + 1)] = static_cast<uint16_t>(r);
+                } else {
+                    T sum = T(0);
+                    for (; j < end; ++j) sum += s_prod[j];
+                    s_acc[r] += sum;
+                    s_beg[r] = 0;
+                    s_end[r] = 0;
+                }
             }
         }
         __syncthreads();
+        const uint32_t long_runs = min(s_long_count, static_cast<uint32_t>(kSlab / kLongRun + 1));
+        if (long_runs != 0) {  // the same for the whole workgroup
+            const uint32_t lane = tid % kWave;
+            for (uint32_t w = tid / kWave; w < long_runs; w += kBlock / kWave) {
+                const uint32_t r = min(static_cast<uint32_t>(s_long[w]), tile_rows - 1);
+                uint32_t end = s_end[r];
+                const uint32_t beg = min(static_cast<uint32_t>(s_beg[r]), cnt);
+                end = end < cnt ? end : cnt;
+                T sum = T(0);
+                for (uint32_t j = beg + lane; j < end; j += kWave) sum += s_prod[j];
+                sum = group_sum<kWave>(sum);
+                if (lane == 0) {
+                    s_acc[r] += sum;
+                    s_beg[r] = 0;
+                    s_end[r] = 0;
+                }
+            }
+            __syncthreads();
+            if (tid == 0) s_long_count = 0;
+        }
+        // the next slab's products may only be written once every run of this one has been read: the
+        // barrier after the row sums (or the one after the long runs) stands between the two
     }
+    __syncthreads();
 
     T* out = partials + static_cast<uint64_t>(band) * m + row0;
 #pragma unroll
     for (int q = 0; q < kRowsPerThread; ++q) {
         const uint32_t r = q * kBlock + tid;
-        if (r < tile_rows) out[r] = acc[q];
+        if (r < tile_rows) out[r] = s_acc[r];
     }
 }
 

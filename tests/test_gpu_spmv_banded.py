@@ -139,11 +139,26 @@ def test_default_band_width_config2_reduced(torch_gpu, handle, oracle):
 
 
 def test_declined_structures_fall_back(torch_gpu, handle, oracle):
-    # x fits one band: nothing to do; long rows: left to the merge family.  SpMV still answers.
+    # x fits one band: nothing to do.  SpMV still answers.
     small = wl.random_ragged(2000, 3000, 9, dtype=np.float32, seed=3)
     run_banded(torch_gpu, handle, oracle, small, 1.0, 0.0, expect_state=0)
-    long_rows = wl.power_law(m=1 << 14, n=1 << 20, max_len=20000, dtype=np.float32)
-    run_banded(torch_gpu, handle, oracle, long_rows, 1.0, 0.0, expect_state=1)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_long_rows_in_a_band(torch_gpu, handle, oracle, dtype):
+    # power-law rows: runs of thousands of entries inside one band, over several slabs of a tile, next
+    # to rows of one entry; default bands (2 bands of fp32, 4 of fp64) and narrow ones
+    a = wl.power_law(m=1 << 14, n=1 << 20, max_len=20000, dtype=dtype)
+    assert a.row_lengths().max() > 5000
+    run_banded(torch_gpu, handle, oracle, a, 1.0, 0.0, calls=2)
+    run_banded(torch_gpu, handle, oracle, a, -1.5, 0.5, band_bytes=1 << 16)
+    b = wl.power_law(m=3000, n=3000, max_len=2500, dtype=dtype, config_id=8)
+    run_banded(torch_gpu, handle, oracle, b, 1.0, 0.0, band_bytes=2048)
+    # runs just around the length at which a wavefront takes over from a thread
+    for per_row in (47, 48, 49, 50, 97):
+        c = wl.uniform_rows(m=700, n=per_row + 3, per_row=per_row, dtype=dtype, config_id=60 + per_row)
+        c = wl.Csr(c.m, 4 * c.n, c.ptr, c.col, c.val)  # columns in the first of several bands
+        run_banded(torch_gpu, handle, oracle, c, 1.0, 0.0, band_bytes=128 * c.val.dtype.itemsize)
 
 
 def test_copy_is_dropped_with_the_arrays(torch_gpu, handle, oracle):
