@@ -183,8 +183,7 @@ def run_workload(name, args, ctx, steps=None, warmup=None, with_cpu=True):
 
     def spmv_buffer(st, the_op, fmt_is_csr):
         """Scratch of an SpMV set: with preprocessing, the larger buffer the banded copy lives in."""
-        direct = (the_op == api.OP_N) == fmt_is_csr  # CSR op N or CSC op T: the row kernels run as the arrays lie
-        use_pre = not args.no_preprocess and direct and not (args.family or args.lanes)
+        use_pre = not args.no_preprocess and not (args.family or args.lanes)
         if use_pre:
             rc, size = api.spmv_preprocess_buffer_size(handle, the_op, alpha, st["mat"], st["vx"], beta, st["vy"], ct)
         else:

@@ -444,14 +444,17 @@ mcsparseStatus_t mcsparseSpMatGetSpMMSchedule(mcsparseSpMatDescr_t spMatDescr, i
  * reference has no such step: include/interface/mcsp_generic.h:43-51).  It copies A into externalBuffer
  * in a column-banded layout in which the reads of x hit in cache; mcsparseSpMV then uses that copy
  * whenever it is called with the same externalBuffer, the same three CSR arrays and extents, op N.
- *   - externalBuffer needs mcsparseSpMV_preprocess_bufferSize bytes (about twice the matrix), is
+ *   - externalBuffer needs mcsparseSpMV_preprocess_bufferSize bytes (about three times the matrix), is
  *     passed to both calls, and must be left alone in between, like the structure of A.
  *   - The copy includes the values.  After changing values in place call mcsparseSpMV_preprocess
  *     again; mcsparseSpMatSetValues and mcsparseCsrSetPointers drop the copy.
- *   - Calls the layout cannot help (x fits in cache as it is, 64-bit indices, COO, the transposing
- *     directions CSR op T and CSC op N) are left to the ordinary kernels; the call still returns
- *     SUCCESS.  CSC with op T is prepared like CSR with op N.  mcsparseSpMatGetSpMVPreprocess tells
- *     which case applies.
+ *   - A copy serves the direction it was prepared for (the opA of the preprocess call).  For the
+ *     transposing directions (CSR with op T, CSC with op N) the copy is of the transpose, so that such
+ *     calls stop sorting the nonzeros by column on every call; externalBuffer then also needs room
+ *     for the conversion (about five times the matrix in all).
+ *   - Calls the layout cannot help (x fits in cache as it is, 64-bit indices, COO) are left to the
+ *     ordinary kernels; the call still returns SUCCESS.  mcsparseSpMatGetSpMVPreprocess tells which
+ *     case applies.
  *   - Results stay within the same bound as mcsparseSpMV's and are bit-reproducible from run to run.
  * The call blocks the host until the copy is built. */
 mcsparseStatus_t mcsparseSpMV_preprocess_bufferSize(mcsparseHandle_t handle, mcsparseOperation_t opA,

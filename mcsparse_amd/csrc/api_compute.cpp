@@ -239,24 +239,47 @@ size_t banded_region_offset(const mcsparseSpMatDescr* A, mcsparseOperation_t op,
     return align_up(spmv_layout(v, A->nnz, value_bytes, narrow_bytes(A)).total);
 }
 
-// What mcsparseSpMV_preprocess builds a banded copy for: calls that run the row kernels on the arrays
-// as they lie (CSR with op N, CSC with op T), 32-bit indices, fp32 / fp64.
+// What mcsparseSpMV_preprocess builds a banded copy for: CSR and CSC with 32-bit indices, fp32 / fp64.
+// The copy is of the matrix the row kernels would run on: the arrays as they lie (CSR with op N, CSC
+// with op T) or, for the transposing directions (CSR with op T, CSC with op N), their transpose, which
+// the preprocess call builds once with csr2csc.  `shape` is that matrix's; *rows its number of rows.
 bool banded_candidate(const mcsparseSpMatDescr* A, mcsparseOperation_t op, BandedShape* shape) {
     if ((A->format != MCSPARSE_FORMAT_CSR && A->format != MCSPARSE_FORMAT_CSC) || wide_indices(A)) return false;
     if (A->valueType != MACA_R_32F && A->valueType != MACA_R_64F) return false;
     const CsrView v = make_view(A, op);
-    if (v.transpose) return false;
-    return mcsp::banded_shape(static_cast<idx_t>(v.m), static_cast<idx_t>(v.n), static_cast<idx_t>(A->nnz),
+    const int64_t rows = v.transpose ? v.n : v.m;
+    const int64_t cols = v.transpose ? v.m : v.n;
+    return mcsp::banded_shape(static_cast<idx_t>(rows), static_cast<idx_t>(cols), static_cast<idx_t>(A->nnz),
                               static_cast<idx_t>(A->idxBase), value_size(A->valueType),
                               A->banded.band_bytes != 0 ? A->banded.band_bytes : mcsp::kBandedBandBytes, shape);
 }
 
-// The banded copy on the descriptor belongs to this call: same buffer, same arrays, same extents.
-bool banded_matches(const mcsparseSpMatDescr* A, const void* buffer, size_t value_bytes) {
+// Scratch of the preprocess call behind the banded copy of a transposing direction: the transpose in
+// CSR form and the workspace of the csr2csc that produces it.
+struct TransposeScratch {
+    size_t ptr, ind, vals, ws, total;
+};
+TransposeScratch transpose_scratch(const CsrView& v, int64_t nnz, size_t value_bytes) {
+    TransposeScratch t;
+    size_t off = 0;
+    t.ptr = off; off += align_up(static_cast<size_t>(v.n + 1) * sizeof(idx_t));
+    t.ind = off; off += align_up(static_cast<size_t>(nnz) * sizeof(idx_t));
+    t.vals = off; off += align_up(static_cast<size_t>(nnz) * value_bytes);
+    t.ws = off;
+    off += align_up(mcsp::csr2csc_workspace_bytes(static_cast<idx_t>(v.m), static_cast<idx_t>(v.n),
+                                                  static_cast<idx_t>(nnz), value_bytes));
+    t.total = off;
+    return t;
+}
+
+// The banded copy on the descriptor belongs to this call: same buffer, same arrays, same extents, same
+// direction.
+bool banded_matches(const mcsparseSpMatDescr* A, const void* buffer, size_t value_bytes, bool transposing) {
     const SpmvBanded& b = A->banded;
     return b.valid && b.useful && b.buffer == buffer && b.rows == A->rows && b.cols == A->cols && b.vals == A->vals &&
            b.m == A->row_num && b.n == A->col_num && b.nnz == A->nnz && b.base == static_cast<int>(A->idxBase) &&
-           b.type == A->valueType && value_size(b.type) == value_bytes && b.format == A->format;
+           b.type == A->valueType && value_size(b.type) == value_bytes && b.format == A->format &&
+           b.transposed == transposing;
 }
 
 template <typename T>
@@ -301,7 +324,7 @@ mcspStatus_t spmv_typed(mcsparseHandle_t h, mcsparseSpMatDescr* A, mcsparseOpera
             ensure_plan(h, A, v.ptr, signature, v.m, A->nnz, v.n * static_cast<int64_t>(sizeof(T)), buffer,
                         may_read_back);
         if (st != MCSP_STATUS_SUCCESS) return st;
-        if (A->plan.forced_family == kFamilyAuto && banded_matches(A, buffer, sizeof(T))) {
+        if (A->plan.forced_family == kFamilyAuto && banded_matches(A, buffer, sizeof(T), false)) {
             mcsp::launch_spmv_banded<T>(h->stream, A->banded.shape, A->banded.grid, a, h_alpha, h_beta,
                                         buf + A->banded.region);
             return MCSP_STATUS_SUCCESS;
@@ -320,6 +343,17 @@ mcspStatus_t spmv_typed(mcsparseHandle_t h, mcsparseSpMatDescr* A, mcsparseOpera
     // of csr2csc, which is a stable sort of one array less, and then sums the products of each column:
     // the sum of a column adds the same products in the same order (row order) as a row kernel on the
     // transpose would, without the gathers from x.
+    if (banded_matches(A, buffer, sizeof(T), true)) {
+        // mcsparseSpMV_preprocess has built the transpose, in the banded layout, once for all calls
+        a.m = static_cast<idx_t>(v.n);
+        a.n = static_cast<idx_t>(v.m);
+        a.row_ptr = nullptr;
+        a.col = nullptr;
+        a.val = nullptr;
+        mcsp::launch_spmv_banded<T>(h->stream, A->banded.shape, A->banded.grid, a, h_alpha, h_beta,
+                                    buf + A->banded.region);
+        return MCSP_STATUS_SUCCESS;
+    }
     idx_t* t_ptr = reinterpret_cast<idx_t*>(buf + l.col_ptr);
     void* t_val = buf + l.vals;
     mcsp::launch_transposed_products(h->stream, static_cast<idx_t>(v.m), static_cast<idx_t>(v.n), nnz, v.val, v.ptr, v.ind,
@@ -666,8 +700,10 @@ mcsparseStatus_t mcsparseSpMV_preprocess_bufferSize(mcsparseHandle_t handle, mcs
     if (banded_candidate(matA, opA, &shape)) {
         const size_t vb = value_size(matA->valueType);
         const CsrView v = make_view(matA, opA);
+        const idx_t rows = static_cast<idx_t>(v.transpose ? v.n : v.m);
         *bufferSize = banded_region_offset(matA, opA, vb) +
-                      mcsp::banded_layout(shape, static_cast<idx_t>(v.m), static_cast<idx_t>(matA->nnz), vb).total;
+                      align_up(mcsp::banded_layout(shape, rows, static_cast<idx_t>(matA->nnz), vb).total) +
+                      (v.transpose ? transpose_scratch(v, matA->nnz, vb).total : 0);
     }
     return MCSPARSE_STATUS_SUCCESS;
 }
@@ -685,15 +721,17 @@ mcsparseStatus_t mcsparseSpMV_preprocess(mcsparseHandle_t handle, mcsparseOperat
     BandedShape shape;
     if (matA->nnz == 0 || !banded_candidate(matA, opA, &shape)) return MCSPARSE_STATUS_SUCCESS;  // nothing to prepare
 
-    // the plan of the row kernels is worked out here as well, so that no later call has to block for it
     const CsrView v = make_view(matA, opA);
-    const idx_t m = static_cast<idx_t>(v.m);
+    const idx_t m = static_cast<idx_t>(v.transpose ? v.n : v.m);  // rows of the matrix that is banded
     const idx_t nnz = static_cast<idx_t>(matA->nnz);
     const idx_t base = static_cast<idx_t>(matA->idxBase);
     const size_t vb = value_size(matA->valueType);
-    const mcspStatus_t ps =
-        ensure_plan(handle, matA, v.ptr, v.ptr, v.m, matA->nnz, v.n * static_cast<int64_t>(vb), externalBuffer, true);
-    if (ps != MCSP_STATUS_SUCCESS) return to_public_status(ps);
+    if (!v.transpose) {
+        // the plan of the row kernels is worked out here as well, so that no later call has to block for it
+        const mcspStatus_t ps = ensure_plan(handle, matA, v.ptr, v.ptr, v.m, matA->nnz, v.n * static_cast<int64_t>(vb),
+                                            externalBuffer, true);
+        if (ps != MCSP_STATUS_SUCCESS) return to_public_status(ps);
+    }
     SpmvBanded& b = matA->banded;
     b.buffer = externalBuffer;
     b.rows = matA->rows;
@@ -705,11 +743,23 @@ mcsparseStatus_t mcsparseSpMV_preprocess(mcsparseHandle_t handle, mcsparseOperat
     b.base = static_cast<int>(matA->idxBase);
     b.type = matA->valueType;
     b.format = matA->format;
+    b.transposed = v.transpose;
     b.shape = shape;
     b.region = banded_region_offset(matA, opA, vb);
     b.grid = 0;
     char* region = static_cast<char*>(externalBuffer) + b.region;
-    mcsp::launch_banded_build(handle->stream, shape, m, nnz, base, v.ptr, v.ind, matA->vals, vb, region);
+    if (v.transpose) {
+        // the transpose in CSR form, behind the banded copy it is only the source of
+        char* scratch = region + align_up(mcsp::banded_layout(shape, m, nnz, vb).total);
+        const TransposeScratch t = transpose_scratch(v, matA->nnz, vb);
+        idx_t* t_ptr = reinterpret_cast<idx_t*>(scratch + t.ptr);
+        idx_t* t_ind = reinterpret_cast<idx_t*>(scratch + t.ind);
+        mcsp::launch_csr2csc(handle->stream, static_cast<idx_t>(v.m), static_cast<idx_t>(v.n), nnz, matA->vals, v.ptr,
+                             v.ind, scratch + t.vals, t_ind, t_ptr, vb, base, scratch + t.ws);
+        mcsp::launch_banded_build(handle->stream, shape, m, nnz, base, t_ptr, t_ind, scratch + t.vals, vb, region);
+    } else {
+        mcsp::launch_banded_build(handle->stream, shape, m, nnz, base, v.ptr, v.ind, matA->vals, vb, region);
+    }
     uint32_t xcd_start[9];
     const mcsp::BandedLayout l = mcsp::banded_layout(shape, m, nnz, vb);
     if (hipMemcpyAsync(xcd_start, region + l.xcd_start, sizeof(xcd_start), hipMemcpyDeviceToHost, handle->stream) !=

@@ -117,6 +117,7 @@ struct SpmvBanded {
     int base = 0;
     macaDataType type = MACA_R_32F;
     mcsparseFormat_t format = MCSPARSE_FORMAT_CSR;
+    bool transposed = false; // the copy is of the transpose of the arrays (CSR with op T, CSC with op N)
     size_t region = 0;       // offset of the banded copy inside the buffer
     BandedShape shape = {};
     uint32_t grid = 0;       // workgroups of the SpMV kernel

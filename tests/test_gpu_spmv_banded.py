@@ -110,26 +110,49 @@ def test_csc_applied_transposed(torch_gpu, handle, oracle):
     # CSC with op T runs the row kernels on the arrays as they lie, so it can be banded like CSR op N
     a = wl.random_ragged(4001, 20011, 17, dtype=np.float32, seed=21, base=1)
     run_banded(torch_gpu, handle, oracle, a, 1.25, -0.5, band_bytes=4096, as_csc=True, calls=2)
-    # the transposing directions are not banded: preprocess leaves them alone and SpMV still answers
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("fmt", [api.FORMAT_CSR, api.FORMAT_CSC])
+def test_transposing_directions_get_a_copy_of_the_transpose(torch_gpu, handle, oracle, dtype, fmt):
+    """CSR with op T and CSC with op N: the preprocess call transposes once, the calls run the banded kernel."""
     torch = torch_gpu
+    a = wl.random_ragged(6001, 20011, 13, dtype=dtype, seed=22, base=1)
+    ct = api.maca_type(dtype)
     rng = np.random.default_rng(2)
-    x = rng.uniform(-1, 1, a.m).astype(np.float32)
+    x = rng.uniform(-1, 1, a.m).astype(dtype)
+    y0 = rng.uniform(-1, 1, a.n).astype(dtype)
     d_ptr, d_col, d_val, d_x = (dev(torch, v) for v in (a.ptr, a.col, a.val, x))
-    d_y = torch.zeros(a.n, dtype=torch.float32, device="cuda")
-    mat = api.SpMat(a.m, a.n, a.nnz, d_ptr, d_col, d_val, base=1)
+    d_y = dev(torch, y0)
+    if fmt == api.FORMAT_CSR:  # the arrays are A (m x n): op T gives A^T x
+        mat, op = api.SpMat(a.m, a.n, a.nnz, d_ptr, d_col, d_val, base=1), api.OP_T
+    else:  # the same arrays read as the CSC of the n x m matrix A^T: op N gives A^T x
+        mat, op = api.SpMat(a.n, a.m, a.nnz, d_ptr, d_col, d_val, base=1, fmt=api.FORMAT_CSC), api.OP_N
     mat.set_band_bytes(4096)
     vx, vy = api.DnVec(d_x), api.DnVec(d_y)
-    st, size = api.spmv_preprocess_buffer_size(handle, api.OP_T, 1.0, mat, vx, 0.0, vy, api.R_32F)
+    st, size = api.spmv_preprocess_buffer_size(handle, op, 1.5, mat, vx, 0.5, vy, ct)
     assert st == api.STATUS_SUCCESS
-    st2, plain = api.spmv_buffer_size(handle, api.OP_T, 1.0, mat, vx, 0.0, vy, api.R_32F)
-    assert size == plain
+    st2, plain = api.spmv_buffer_size(handle, op, 1.5, mat, vx, 0.5, vy, ct)
+    assert size > plain
     buf = torch.empty(size, dtype=torch.uint8, device="cuda")
-    assert api.spmv_preprocess(handle, api.OP_T, 1.0, mat, vx, 0.0, vy, api.R_32F, buf) == api.STATUS_SUCCESS
-    assert mat.spmv_preprocess_state()[0] == 0
-    assert api.spmv(handle, api.OP_T, 1.0, mat, vx, 0.0, vy, api.R_32F, buf) == api.STATUS_SUCCESS
+    assert api.spmv_preprocess(handle, op, 1.5, mat, vx, 0.5, vy, ct, buf) == api.STATUS_SUCCESS
+    assert mat.spmv_preprocess_state()[0] == 2
+    y_ref, bound = oracle.spmv(True, a.m, a.n, 1, a.ptr, a.col, a.val, 1.5, 0.5, x, y0)
+    for _ in range(2):
+        d_y.copy_(torch.from_numpy(y0))
+        assert api.spmv(handle, op, 1.5, mat, vx, 0.5, vy, ct, buf) == api.STATUS_SUCCESS
+        torch.cuda.synchronize()
+        assert_within(d_y.cpu().numpy(), y_ref, bound, dtype, what="transposing direction, banded")
+    # the copy serves its own direction only: the other one runs the row kernels on the arrays as they lie
+    other = api.OP_N if op == api.OP_T else api.OP_T
+    x2 = rng.uniform(-1, 1, a.n).astype(dtype)
+    d_x2 = dev(torch, x2)
+    d_y2 = torch.zeros(a.m, dtype=d_x2.dtype, device="cuda")
+    vx2, vy2 = api.DnVec(d_x2), api.DnVec(d_y2)
+    assert api.spmv(handle, other, 1.0, mat, vx2, 0.0, vy2, ct, buf) == api.STATUS_SUCCESS
     torch.cuda.synchronize()
-    y_ref, bound = oracle.spmv(True, a.m, a.n, 1, a.ptr, a.col, a.val, 1.0, 0.0, x, None)
-    assert_within(d_y.cpu().numpy(), y_ref, bound, np.float32, what="op T after preprocess")
+    y_ref2, bound2 = oracle.spmv(False, a.m, a.n, 1, a.ptr, a.col, a.val, 1.0, 0.0, x2, None)
+    assert_within(d_y2.cpu().numpy(), y_ref2, bound2, dtype, what="the other direction")
 
 
 def test_default_band_width_config2_reduced(torch_gpu, handle, oracle):
