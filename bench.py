@@ -44,18 +44,27 @@ def _traffic(fetch_counts, write_counts):
 
 
 MEASURED_TRAFFIC = {
-    # spmv_banded_kernel<double> + banded_reduce_kernel<double>
-    "c2": (_traffic(111459.5 + 20554.1, 32768.0 + 8192.0), "profiles/spmv_banded_f64_c2_1Mx16.txt"),
-    # merge kernel (tiles in column order) + partition + tile order + fix-up
-    "c3": (_traffic(3305285.9 + 17229.2 + 251.2 + 3154.3, 25157.0 + 1391.2 + 1994.3 + 1375.1),
-           "profiles/spmv_merge_f32_c3_powerlaw.txt"),
-    "c4-64": (_traffic(613893.3, 524288.0), "profiles/spmm_group_f32_c4_stencil128.txt"),
-    "c4-256": (_traffic(3673719.8, 2097152.0), "profiles/spmm_group_f32_c4_stencil128.txt"),
+    # keys: (workload, the banded copy ran).  spmv_banded_kernel + banded_reduce_kernel
+    ("c2", True): (_traffic(108483.2 + 20567.1, 32768.0 + 8192.0), "profiles/spmv_banded_f64_c2_1Mx16.txt"),
+    ("c3", True): (_traffic(479341.2 + 65545.2, 133136.1 + 16384.0), "profiles/spmv_banded_f32_c3_powerlaw.txt"),
+    ("c3t", True): (_traffic(481300.5 + 65544.8, 131206.2 + 16384.0), "profiles/spmv_banded_f32_c3_powerlaw.txt"),
+    ("c5-spmv", True): (_traffic(481330.8 + 65544.6, 131202.3 + 16384.0),
+                        "profiles/spmv_banded_f32_c3_powerlaw.txt"),
+    # without the preprocess call: vector kernel; merge kernel (tiles in column order) + partition
+    # + tile order + fix-up
+    ("c2", False): (_traffic(653904.5, 10047.2), "profiles/spmv_vector_f64_c2_1Mx16.txt"),
+    ("c3", False): (_traffic(3305285.9 + 17229.2 + 251.2 + 3154.3, 25157.0 + 1391.2 + 1994.3 + 1375.1),
+                    "profiles/spmv_merge_f32_c3_powerlaw.txt"),
+    ("c4-64", False): (_traffic(613893.3, 524288.0), "profiles/spmm_group_f32_c4_stencil128.txt"),
+    ("c4-256", False): (_traffic(3673719.8, 2097152.0), "profiles/spmm_group_f32_c4_stencil128.txt"),
+    # group kernel + the transposes of B and of C
+    ("c4-64-col", False): (_traffic(596223.4 + 262180.7 + 262178.7, 3 * 524288.0),
+                           "profiles/spmm_colmajor_f32_c4_stencil128_n64.txt"),
     # csr2csc: 2 x scatter + the scatter that reads the CSR arrays in place + 3 x (histogram + scans)
     # + row starts per tile + coo2csr
-    "c5": (_traffic(2 * 701979.0 + 481119.4 + 3 * (229171.1 + 2 * 7206.6 + 14342.5) + 21136.0 + 237161.6,
-                    2 * 1387754.6 + 1421432.8 + 3 * (28789.0 + 2 * 14326.3 + 56.0) + 223.8 + 19514.6),
-           "profiles/csr2csc_radix_f32_c5_powerlaw.txt"),
+    ("c5", False): (_traffic(2 * 701979.0 + 481119.4 + 3 * (229171.1 + 2 * 7206.6 + 14342.5) + 21136.0 + 237161.6,
+                             2 * 1387754.6 + 1421432.8 + 3 * (28789.0 + 2 * 14326.3 + 56.0) + 223.8 + 19514.6),
+                    "profiles/csr2csc_radix_f32_c5_powerlaw.txt"),
 }
 
 
@@ -295,9 +304,7 @@ def run_workload(name, args, ctx, steps=None, warmup=None, with_cpu=True):
     mat0 = sets[0].get("mat")
     plan = mat0.plan() if mat0 is not None and kind in ("spmv", "spmv-csc") else None
     banded = mat0.spmv_preprocess_state() if mat0 is not None and kind in ("spmv", "spmv-csc") else None
-    traffic = MEASURED_TRAFFIC.get(name) if s == 1.0 else None
-    if traffic is not None and name == "c2" and not (banded and banded[0] == 2):
-        traffic = None  # the constant belongs to the banded kernels
+    traffic = MEASURED_TRAFFIC.get((name, bool(banded and banded[0] == 2))) if s == 1.0 else None
 
     out = {
         "metric": "CSR SpMV/SpMM achieved HBM GB/s (% of MI355X peak) + GFLOP/s at 1 GPU",

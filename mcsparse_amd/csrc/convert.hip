@@ -799,11 +799,28 @@ __global__ __launch_bounds__(kBlock) void identity_kernel(idx_t n, idx_t* __rest
     if (i < static_cast<uint64_t>(n)) p[i] = static_cast<idx_t>(i);
 }
 
+// Eight elements per thread, the indices first, then the eight gathers, then the stores: a thread has
+// eight gathers in flight, as the SpMV kernels have, so what this kernel takes is what the gathers cost.
+constexpr int kGatherPerThread = 8;
 template <typename T>
 __global__ __launch_bounds__(kBlock) void gather_kernel(idx_t nnz, const T* __restrict__ y, T* __restrict__ x_val,
                                                         const idx_t* __restrict__ x_ind, idx_t base) {
-    const uint64_t i = static_cast<uint64_t>(blockIdx.x) * kBlock + threadIdx.x;
-    if (i < static_cast<uint64_t>(nnz)) x_val[i] = y[load_stream(x_ind + i) - base];
+    const uint64_t first = static_cast<uint64_t>(blockIdx.x) * (kBlock * kGatherPerThread) + threadIdx.x;
+    const uint64_t last = static_cast<uint64_t>(nnz) - 1;  // nnz != 0: the grid has no workgroup otherwise
+    idx_t ind[kGatherPerThread];
+    T got[kGatherPerThread];
+#pragma unroll
+    for (int k = 0; k < kGatherPerThread; ++k) {
+        const uint64_t i = first + static_cast<uint64_t>(k) * kBlock;
+        ind[k] = load_stream(x_ind + (i < last ? i : last));
+    }
+#pragma unroll
+    for (int k = 0; k < kGatherPerThread; ++k) got[k] = y[ind[k] - base];
+#pragma unroll
+    for (int k = 0; k < kGatherPerThread; ++k) {
+        const uint64_t i = first + static_cast<uint64_t>(k) * kBlock;
+        if (i <= last) x_val[i] = got[k];
+    }
 }
 
 }  // namespace
@@ -961,8 +978,9 @@ void launch_identity(hipStream_t stream, idx_t n, idx_t* p) {
 template <typename T>
 void launch_gather(hipStream_t stream, idx_t nnz, const T* y, T* x_val, const idx_t* x_ind, idx_t base) {
     if (nnz == 0) return;
-    hipLaunchKernelGGL((gather_kernel<T>), dim3((static_cast<uint32_t>(nnz) + kBlock - 1) / kBlock), dim3(kBlock), 0,
-                       stream, nnz, y, x_val, x_ind, base);
+    constexpr uint32_t per_block = kBlock * kGatherPerThread;
+    hipLaunchKernelGGL((gather_kernel<T>), dim3((static_cast<uint32_t>(nnz) + per_block - 1) / per_block), dim3(kBlock),
+                       0, stream, nnz, y, x_val, x_ind, base);
 }
 
 namespace {
