@@ -280,7 +280,13 @@ mcsparseStatus_t mcsparseDnMatGetStridedBatch(mcsparseDnMatDescr_t dnMatDescr, i
 /* externalBuffer is caller-allocated device scratch of at least *bufferSize bytes and must be
  * non-NULL even for op N (src/kernels/level2/spmv/mcsp_spmv_gpu.cpp:703-705).  Work is
  * enqueued on the handle's stream.  With MCSPARSE_POINTER_MODE_DEVICE the scalars are read
- * with a blocking copy, as the reference does (src/include/mcsp_internal_host_utils.hpp:34-63). */
+ * with a blocking copy, as the reference does (src/include/mcsp_internal_host_utils.hpp:34-63).
+ *
+ * DIFFERENT FROM THE REFERENCE: the buffer is used, and is larger.  The reference returns 128
+ * bytes for CSR op N and never writes to the buffer (mcsp_spmv_gpu.cpp:1136-1147); here the
+ * buffer holds the row-length histogram and the workspace of the merge-path kernel even for op N
+ * (a few bytes per 1024 rows + nonzeros).  A caller that hard-codes the reference's 128 bytes
+ * would be written past: always allocate what mcsparseSpMV_bufferSize returns. */
 mcsparseStatus_t mcsparseSpMV(mcsparseHandle_t handle, mcsparseOperation_t opA, const void* alpha,
                               mcsparseSpMatDescr_t matA, mcsparseDnVecDescr_t vecX, const void* beta,
                               mcsparseDnVecDescr_t vecY, macaDataType computeType, mcsparseSpMVAlg_t alg,
@@ -309,8 +315,11 @@ mcsparseStatus_t mcsparseSpMM(mcsparseHandle_t handle, mcsparseOperation_t opA, 
 /* y = alpha*A*x + beta*y: include/interface/mcsp_level2.h:11-36.  transA is accepted and
  * ignored, exactly as in the reference (src/kernels/level2/spmv/mcsp_spmv_gpu.cpp:946-953 hands it
  * to a template that never reads it), so these always apply A itself.  The index base comes from
- * descrA.  csrmv has no scratch buffer and runs the sub-wavefront vector kernel; CsrmvEx gets a
- * buffer of *bufferSizeInBytes and runs the merge-path kernel. */
+ * descrA.  Neither call has a scratch buffer of known size (csrmv has none; CsrmvEx_bufferSize
+ * returns the reference's constant 128 and CsrmvEx never touches its buffer, as in the reference,
+ * mcsp_spmv_gpu.cpp:905-944,1149-1158), so both run the kernel that gives a group of lanes to each
+ * row.  The kernels that need scratch are reached through mcsparseSpMV, whose buffer size is NOT
+ * the reference's 128 bytes: see mcsparseSpMV_bufferSize. */
 mcsparseStatus_t mcsparseScsrmv(mcsparseHandle_t handle, mcsparseOperation_t transA, int m, int n, int nnz,
                                 const float* alpha, const mcsparseMatDescr_t descrA, const float* csrValA,
                                 const int* csrRowPtrA, const int* csrColIndA, const float* x, const float* beta,

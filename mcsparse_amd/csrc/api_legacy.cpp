@@ -29,8 +29,7 @@ bool descr_is_plain(const mcsparseMatDescr* d) {
 // `workspace` non-null selects the merge-path kernel.
 template <typename T>
 mcspStatus_t csrmv_impl(mcsparseHandle_t handle, int m, int n, int nnz, const T* alpha, const mcsparseMatDescr* descr,
-                        const T* val, const int* row_ptr, const int* col, const T* x, const T* beta, T* y,
-                        void* workspace) {
+                        const T* val, const int* row_ptr, const int* col, const T* x, const T* beta, T* y) {
     if (handle == nullptr) return MCSP_STATUS_INVALID_HANDLE;
     if (nnz < 0 || m < 0 || n < 0) return MCSP_STATUS_INVALID_SIZE;  // dead in the reference (uint32 casts)
     if (alpha == nullptr || beta == nullptr || row_ptr == nullptr || col == nullptr || val == nullptr ||
@@ -51,11 +50,9 @@ mcspStatus_t csrmv_impl(mcsparseHandle_t handle, int m, int n, int nnz, const T*
     a.val = val;
     a.x = x;
     a.y = y;
-    if (workspace != nullptr) {
-        mcsp::launch_spmv_merge<T>(handle->stream, a, h_alpha, h_beta, workspace, false);
-    } else {
-        mcsp::launch_spmv_vector<T>(handle->stream, a, h_alpha, h_beta, mcsp::spmv_pick_lanes(a.m, a.nnz));
-    }
+    // the typed entry points have no buffer whose size is known (csrmv has none, CsrmvEx's is the
+    // reference's constant 128 bytes and is never touched there, :905-944): row-per-lane-group kernel
+    mcsp::launch_spmv_vector<T>(handle->stream, a, h_alpha, h_beta, mcsp::spmv_pick_lanes(a.m, a.nnz));
     return MCSP_STATUS_SUCCESS;
 }
 
@@ -189,7 +186,7 @@ mcsparseStatus_t mcsparseScsrmv(mcsparseHandle_t handle, mcsparseOperation_t /*t
                                 const int* csrRowPtrA, const int* csrColIndA, const float* x, const float* beta,
                                 float* y) {
     return to_public_status(
-        csrmv_impl<float>(handle, m, n, nnz, alpha, descrA, csrValA, csrRowPtrA, csrColIndA, x, beta, y, nullptr));
+        csrmv_impl<float>(handle, m, n, nnz, alpha, descrA, csrValA, csrRowPtrA, csrColIndA, x, beta, y));
 }
 
 mcsparseStatus_t mcsparseDcsrmv(mcsparseHandle_t handle, mcsparseOperation_t /*transA*/, int m, int n, int nnz,
@@ -197,23 +194,20 @@ mcsparseStatus_t mcsparseDcsrmv(mcsparseHandle_t handle, mcsparseOperation_t /*t
                                 const int* csrRowPtrA, const int* csrColIndA, const double* x, const double* beta,
                                 double* y) {
     return to_public_status(
-        csrmv_impl<double>(handle, m, n, nnz, alpha, descrA, csrValA, csrRowPtrA, csrColIndA, x, beta, y, nullptr));
+        csrmv_impl<double>(handle, m, n, nnz, alpha, descrA, csrValA, csrRowPtrA, csrColIndA, x, beta, y));
 }
 
-// reference: :1149-1158 writes 128 without looking at any argument
+// reference: :1149-1158 writes 128 without looking at any argument; the same constant here, so
+// that a caller with the reference's size compiled in stays inside its buffer
 mcsparseStatus_t mcsparseCsrmvEx_bufferSize(mcsparseHandle_t handle, mcsparseAlgMode_t, mcsparseOperation_t, int m,
                                             int /*n*/, int nnz, const void*, macaDataType, const mcsparseMatDescr_t,
-                                            const void*, macaDataType csrValAtype, const int*, const int*, const void*,
+                                            const void*, macaDataType, const int*, const int*, const void*,
                                             macaDataType, const void*, macaDataType, void*, macaDataType, macaDataType,
                                             size_t* bufferSizeInBytes) {
     if (handle == nullptr) return to_public_status(MCSP_STATUS_INVALID_HANDLE);
     if (bufferSizeInBytes == nullptr) return to_public_status(MCSP_STATUS_INVALID_POINTER);
     if (m < 0 || nnz < 0) return to_public_status(MCSP_STATUS_INVALID_SIZE);
-    size_t vb = value_size(csrValAtype);
-    if (vb != 4 && vb != 8) vb = 8;
-    const size_t bytes = align_up(
-        mcsp::spmv_merge_workspace_bytes(static_cast<idx_t>(m), static_cast<idx_t>(nnz), vb));
-    *bufferSizeInBytes = bytes < kMinBuffer ? kMinBuffer : bytes;
+    *bufferSizeInBytes = kMinBuffer;
     return MCSPARSE_STATUS_SUCCESS;
 }
 
@@ -223,22 +217,22 @@ mcsparseStatus_t mcsparseCsrmvEx(mcsparseHandle_t handle, mcsparseAlgMode_t, mcs
                                  const mcsparseMatDescr_t descrA, const void* csrValA, macaDataType csrValAtype,
                                  const int* csrRowPtrA, const int* csrColIndA, const void* x, macaDataType xtype,
                                  const void* beta, macaDataType betatype, void* y, macaDataType ytype,
-                                 macaDataType executiontype, void* buffer) {
+                                 macaDataType executiontype, void* /*buffer*/) {
     if (!(alphatype == xtype && csrValAtype == xtype && betatype == xtype && ytype == xtype &&
           executiontype == xtype))
         return to_public_status(MCSP_STATUS_NOT_IMPLEMENTED);
-    // a missing buffer is not checked by the reference (it never uses it); here it selects the kernel
+    // the buffer is neither checked nor used, as in the reference
     switch (csrValAtype) {
         case MACA_R_32F:
             return to_public_status(csrmv_impl<float>(
                 handle, m, n, nnz, static_cast<const float*>(alpha), descrA, static_cast<const float*>(csrValA),
                 csrRowPtrA, csrColIndA, static_cast<const float*>(x), static_cast<const float*>(beta),
-                static_cast<float*>(y), buffer));
+                static_cast<float*>(y)));
         case MACA_R_64F:
             return to_public_status(csrmv_impl<double>(
                 handle, m, n, nnz, static_cast<const double*>(alpha), descrA, static_cast<const double*>(csrValA),
                 csrRowPtrA, csrColIndA, static_cast<const double*>(x), static_cast<const double*>(beta),
-                static_cast<double*>(y), buffer));
+                static_cast<double*>(y)));
         default:
             return to_public_status(MCSP_STATUS_NOT_IMPLEMENTED);  // complex types are not built
     }
