@@ -31,7 +31,8 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 
-OTHERS = ["c4-64", "c3", "c3t", "c5", "c5-spmv", "c5-coo", "c4-8", "c4-256", "c4-64-col", "c1"]
+OTHERS = ["c4-64", "c3", "c3t", "c5", "c5-spmv", "c5-coo", "c4-8", "c4-256", "c4-64-col", "c1",
+          "c2-alg1", "c3-alg1", "c3t-alg1"]
 OTHERS_BUDGET_S = 200.0  # wall-clock budget of the default invocation for the workloads above
 
 
@@ -83,6 +84,9 @@ def parse():
     p.add_argument("--family", type=int, default=0, help="force the SpMV kernel family (1 vector, 2 merge)")
     p.add_argument("--lanes", type=int, default=0, help="force lanes per row of the vector family")
     p.add_argument("--band-bytes", type=int, default=0, help="band width of mcsparseSpMV_preprocess (0 = default)")
+    p.add_argument("--alg1", action="store_true",
+                   help="MCSPARSE_SPMV_CSR_ALG1 for the SpMV workloads (a name ending in -alg1 says the same): "
+                        "preprocess builds the copy in column order, whose sums need not repeat bit for bit")
     p.add_argument("--cache", default=None, help="directory to keep generated matrices in between runs")
     return p.parse_args()
 
@@ -114,6 +118,9 @@ class Matrices:
 
 def describe(name):
     """(matrix key, kind, op is T, dense columns, alpha, beta, description) of a workload."""
+    if name.endswith("-alg1"):
+        d = describe(name[:-5])
+        return d[:6] + (d[6] + ", MCSPARSE_SPMV_CSR_ALG1",)
     if name == "c1":
         return "laplacian", "spmv", False, 0, 1.0, 0.0, "fp32 CSR SpMV, 5-pt Laplacian 256x256"
     if name == "c2":
@@ -144,6 +151,9 @@ def run_workload(name, args, ctx, steps=None, warmup=None, with_cpu=True):
     """Measures one workload; returns the JSON object of its line."""
     torch, api, wl, handle, stream = ctx["torch"], ctx["api"], ctx["wl"], ctx["handle"], ctx["stream"]
     key, kind, op_t, n_cols, alpha, beta, desc = describe(name)
+    alg = api.SPMV_CSR_ALG1 if (args.alg1 or name.endswith("-alg1")) else api.SPMV_ALG_DEFAULT
+    if args.alg1 and not name.endswith("-alg1") and kind in ("spmv", "spmv-csc"):
+        desc += ", MCSPARSE_SPMV_CSR_ALG1"
     a = ctx["matrices"].get(key)
     op = api.OP_T if op_t else api.OP_N
     s = args.scale
@@ -194,13 +204,15 @@ def run_workload(name, args, ctx, steps=None, warmup=None, with_cpu=True):
         """Scratch of an SpMV set: with preprocessing, the larger buffer the banded copy lives in."""
         use_pre = not args.no_preprocess and not (args.family or args.lanes)
         if use_pre:
-            rc, size = api.spmv_preprocess_buffer_size(handle, the_op, alpha, st["mat"], st["vx"], beta, st["vy"], ct)
+            rc, size = api.spmv_preprocess_buffer_size(handle, the_op, alpha, st["mat"], st["vx"], beta, st["vy"], ct,
+                                                       alg=alg)
         else:
             rc, size = api.spmv_buffer_size(handle, the_op, alpha, st["mat"], st["vx"], beta, st["vy"], ct)
         api.check(rc, "mcsparseSpMV_bufferSize")
         st["buf"] = torch.empty(size, dtype=torch.uint8, device="cuda")
         if use_pre:
-            timed(lambda: api.spmv_preprocess(handle, the_op, alpha, st["mat"], st["vx"], beta, st["vy"], ct, st["buf"]),
+            timed(lambda: api.spmv_preprocess(handle, the_op, alpha, st["mat"], st["vx"], beta, st["vy"], ct, st["buf"],
+                                              alg=alg),
                   "mcsparseSpMV_preprocess")
 
     for c in range(copies):
@@ -261,9 +273,9 @@ def run_workload(name, args, ctx, steps=None, warmup=None, with_cpu=True):
     def step(i):
         st = sets[i % copies]
         if kind == "spmv":
-            rc = api.spmv(handle, op, alpha, st["mat"], st["vx"], beta, st["vy"], ct, st["buf"])
+            rc = api.spmv(handle, op, alpha, st["mat"], st["vx"], beta, st["vy"], ct, st["buf"], alg=alg)
         elif kind == "spmv-csc":
-            rc = api.spmv(handle, api.OP_T, alpha, st["mat"], st["vx"], beta, st["vy"], ct, st["buf"])
+            rc = api.spmv(handle, api.OP_T, alpha, st["mat"], st["vx"], beta, st["vy"], ct, st["buf"], alg=alg)
         elif kind in ("spmm", "spmm-col"):
             rc = api.spmm(handle, api.OP_N, api.OP_N, alpha, st["mat"], st["mB"], beta, st["mC"], ct, st["buf"])
         elif kind == "csr2csc":

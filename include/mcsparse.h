@@ -476,7 +476,8 @@ mcsparseStatus_t mcsparseSpMV_preprocess(mcsparseHandle_t handle, mcsparseOperat
                                          mcsparseDnVecDescr_t vecY, macaDataType computeType, mcsparseSpMVAlg_t alg,
                                          void* externalBuffer);
 /* state 0 = not preprocessed, 1 = preprocessed and left to the ordinary kernels, 2 = banded copy in
- * use; bands and rows_per_tile describe the copy (0 unless state is 2). */
+ * use, 3 = the copy in column order (MCSPARSE_SPMV_CSR_ALG1) in use; bands and rows_per_tile describe
+ * the copy (0 unless state is 2 or 3). */
 mcsparseStatus_t mcsparseSpMatGetSpMVPreprocess(mcsparseSpMatDescr_t spMatDescr, int* state, int* bands,
                                                 int* rows_per_tile);
 

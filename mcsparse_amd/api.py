@@ -28,6 +28,8 @@ ORDER_COL, ORDER_ROW = 1, 2
 INDEX_16U, INDEX_32I, INDEX_64I = 1, 2, 3
 R_32F, R_64F, R_16F, C_32F, C_64F, R_32I = 0, 1, 2, 4, 5, 10
 SPMV_ALG_DEFAULT = 0
+SPMV_CSR_ALG1 = 2  # need not give the same bits on every run
+SPMV_CSR_ALG2 = 3  # the same bits on every run
 SPMM_ALG_DEFAULT = 0
 CSR2CSC_ALG1 = 1
 ROW_BIN_COUNT = 33
@@ -222,7 +224,7 @@ def spmv_buffer_size(handle, op, alpha, mat, x, beta, y, compute_type):
     return st, size.value
 
 
-def spmv(handle, op, alpha, mat, x, beta, y, compute_type, buffer):
+def spmv(handle, op, alpha, mat, x, beta, y, compute_type, buffer, alg=0):
     """alpha/beta are Python floats (host pointer mode) or device tensors (device pointer mode)."""
     if hasattr(alpha, "data_ptr"):
         pa, pb = alpha.data_ptr(), beta.data_ptr()
@@ -231,25 +233,24 @@ def spmv(handle, op, alpha, mat, x, beta, y, compute_type, buffer):
         a, b = _scalar(alpha, compute_type), _scalar(beta, compute_type)
         pa, pb = ctypes.addressof(a), ctypes.addressof(b)
         keep = (a, b)
-    st = handle.lib.mcsparseSpMV(handle.ptr, op, pa, mat.ptr, x.ptr, pb, y.ptr, compute_type, SPMV_ALG_DEFAULT,
-                                 _ptr(buffer))
+    st = handle.lib.mcsparseSpMV(handle.ptr, op, pa, mat.ptr, x.ptr, pb, y.ptr, compute_type, alg, _ptr(buffer))
     del keep
     return st
 
 
-def spmv_preprocess_buffer_size(handle, op, alpha, mat, x, beta, y, compute_type):
+def spmv_preprocess_buffer_size(handle, op, alpha, mat, x, beta, y, compute_type, alg=0):
     size = ctypes.c_size_t(0)
     a, b = _scalar(alpha, compute_type), _scalar(beta, compute_type)
     st = handle.lib.mcsparseSpMV_preprocess_bufferSize(handle.ptr, op, ctypes.addressof(a), mat.ptr, x.ptr,
-                                                       ctypes.addressof(b), y.ptr, compute_type, SPMV_ALG_DEFAULT,
+                                                       ctypes.addressof(b), y.ptr, compute_type, alg,
                                                        ctypes.byref(size))
     return st, size.value
 
 
-def spmv_preprocess(handle, op, alpha, mat, x, beta, y, compute_type, buffer):
+def spmv_preprocess(handle, op, alpha, mat, x, beta, y, compute_type, buffer, alg=0):
     a, b = _scalar(alpha, compute_type), _scalar(beta, compute_type)
     return handle.lib.mcsparseSpMV_preprocess(handle.ptr, op, ctypes.addressof(a), mat.ptr, x.ptr, ctypes.addressof(b),
-                                              y.ptr, compute_type, SPMV_ALG_DEFAULT, _ptr(buffer))
+                                              y.ptr, compute_type, alg, _ptr(buffer))
 
 
 def spmv_static_buffer(handle, op, alpha, mat, x, beta, y, compute_type):

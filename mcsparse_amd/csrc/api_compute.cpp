@@ -243,15 +243,22 @@ size_t banded_region_offset(const mcsparseSpMatDescr* A, mcsparseOperation_t op,
 // The copy is of the matrix the row kernels would run on: the arrays as they lie (CSR with op N, CSC
 // with op T) or, for the transposing directions (CSR with op T, CSC with op N), their transpose, which
 // the preprocess call builds once with csr2csc.  `shape` is that matrix's; *rows its number of rows.
-bool banded_candidate(const mcsparseSpMatDescr* A, mcsparseOperation_t op, BandedShape* shape) {
+bool banded_candidate(const mcsparseSpMatDescr* A, mcsparseOperation_t op, mcsparseSpMVAlg_t alg, BandedShape* shape) {
     if ((A->format != MCSPARSE_FORMAT_CSR && A->format != MCSPARSE_FORMAT_CSC) || wide_indices(A)) return false;
     if (A->valueType != MACA_R_32F && A->valueType != MACA_R_64F) return false;
     const CsrView v = make_view(A, op);
     const int64_t rows = v.transpose ? v.n : v.m;
     const int64_t cols = v.transpose ? v.m : v.n;
+    const size_t band_bytes = A->banded.band_bytes != 0 ? A->banded.band_bytes : mcsp::kBandedBandBytes;
+    shape->by_column = false;
+    // MCSPARSE_SPMV_CSR_ALG1 is the algorithm that need not give the same bits on every run: tiles in
+    // column order with sums formed in LDS as the products arrive, where the shape allows it
+    if (alg == MCSPARSE_SPMV_CSR_ALG1 &&
+        mcsp::column_order_shape(static_cast<idx_t>(rows), static_cast<idx_t>(cols), static_cast<idx_t>(A->nnz),
+                                 static_cast<idx_t>(A->idxBase), value_size(A->valueType), band_bytes, shape))
+        return true;
     return mcsp::banded_shape(static_cast<idx_t>(rows), static_cast<idx_t>(cols), static_cast<idx_t>(A->nnz),
-                              static_cast<idx_t>(A->idxBase), value_size(A->valueType),
-                              A->banded.band_bytes != 0 ? A->banded.band_bytes : mcsp::kBandedBandBytes, shape);
+                              static_cast<idx_t>(A->idxBase), value_size(A->valueType), band_bytes, shape);
 }
 
 // Scratch of the preprocess call behind the banded copy of a transposing direction: the transpose in
@@ -274,8 +281,11 @@ TransposeScratch transpose_scratch(const CsrView& v, int64_t nnz, size_t value_b
 
 // The banded copy on the descriptor belongs to this call: same buffer, same arrays, same extents, same
 // direction.
-bool banded_matches(const mcsparseSpMatDescr* A, const void* buffer, size_t value_bytes, bool transposing) {
+bool banded_matches(const mcsparseSpMatDescr* A, const void* buffer, size_t value_bytes, bool transposing,
+                    mcsparseSpMVAlg_t alg) {
     const SpmvBanded& b = A->banded;
+    // MCSPARSE_SPMV_CSR_ALG2 asks for the same bits on every run, which the copy in column order does not give
+    if (b.shape.by_column && alg == MCSPARSE_SPMV_CSR_ALG2) return false;
     return b.valid && b.useful && b.buffer == buffer && b.rows == A->rows && b.cols == A->cols && b.vals == A->vals &&
            b.m == A->row_num && b.n == A->col_num && b.nnz == A->nnz && b.base == static_cast<int>(A->idxBase) &&
            b.type == A->valueType && value_size(b.type) == value_bytes && b.format == A->format &&
@@ -285,7 +295,7 @@ bool banded_matches(const mcsparseSpMatDescr* A, const void* buffer, size_t valu
 template <typename T>
 mcspStatus_t spmv_typed(mcsparseHandle_t h, mcsparseSpMatDescr* A, mcsparseOperation_t op, const void* alpha,
                         const void* beta, const mcsparseDnVecDescr* x, mcsparseDnVecDescr* y, void* buffer,
-                        bool may_read_back) {
+                        bool may_read_back, mcsparseSpMVAlg_t alg) {
     T h_alpha, h_beta;
     if (!scalar_to_host(h, beta, &h_beta) || !scalar_to_host(h, alpha, &h_alpha))
         return stream_is_capturing(h->stream) ? MCSP_STATUS_NOT_IMPLEMENTED : MCSP_STATUS_INTERNAL_ERROR;
@@ -324,7 +334,7 @@ mcspStatus_t spmv_typed(mcsparseHandle_t h, mcsparseSpMatDescr* A, mcsparseOpera
             ensure_plan(h, A, v.ptr, signature, v.m, A->nnz, v.n * static_cast<int64_t>(sizeof(T)), buffer,
                         may_read_back);
         if (st != MCSP_STATUS_SUCCESS) return st;
-        if (A->plan.forced_family == kFamilyAuto && banded_matches(A, buffer, sizeof(T), false)) {
+        if (A->plan.forced_family == kFamilyAuto && banded_matches(A, buffer, sizeof(T), false, alg)) {
             mcsp::launch_spmv_banded<T>(h->stream, A->banded.shape, A->banded.grid, a, h_alpha, h_beta,
                                         buf + A->banded.region);
             return MCSP_STATUS_SUCCESS;
@@ -343,7 +353,7 @@ mcspStatus_t spmv_typed(mcsparseHandle_t h, mcsparseSpMatDescr* A, mcsparseOpera
     // of csr2csc, which is a stable sort of one array less, and then sums the products of each column:
     // the sum of a column adds the same products in the same order (row order) as a row kernel on the
     // transpose would, without the gathers from x.
-    if (banded_matches(A, buffer, sizeof(T), true)) {
+    if (banded_matches(A, buffer, sizeof(T), true, alg)) {
         // mcsparseSpMV_preprocess has built the transpose, in the banded layout, once for all calls
         a.m = static_cast<idx_t>(v.n);
         a.n = static_cast<idx_t>(v.m);
@@ -639,13 +649,14 @@ mcspStatus_t spmv_check(mcsparseHandle_t handle, mcsparseOperation_t opA, const 
 
 mcspStatus_t spmv_call(mcsparseHandle_t handle, mcsparseOperation_t opA, const void* alpha, mcsparseSpMatDescr_t matA,
                        mcsparseDnVecDescr_t vecX, const void* beta, mcsparseDnVecDescr_t vecY,
-                       macaDataType computeType, void* buffer, size_t buffer_bytes, bool may_read_back) {
+                       macaDataType computeType, void* buffer, size_t buffer_bytes, bool may_read_back,
+                       mcsparseSpMVAlg_t alg) {
     const mcspStatus_t st =
         spmv_check(handle, opA, alpha, matA, vecX, beta, vecY, computeType, buffer, buffer_bytes, may_read_back);
     if (st != MCSP_STATUS_SUCCESS) return st;
     if (computeType == MACA_R_32F)
-        return spmv_typed<float>(handle, matA, opA, alpha, beta, vecX, vecY, buffer, may_read_back);
-    return spmv_typed<double>(handle, matA, opA, alpha, beta, vecX, vecY, buffer, may_read_back);
+        return spmv_typed<float>(handle, matA, opA, alpha, beta, vecX, vecY, buffer, may_read_back, alg);
+    return spmv_typed<double>(handle, matA, opA, alpha, beta, vecX, vecY, buffer, may_read_back, alg);
 }
 
 }  // namespace mcsp
@@ -681,10 +692,10 @@ mcsparseStatus_t mcsparseSpMV_bufferSize(mcsparseHandle_t handle, mcsparseOperat
 // reference: src/kernels/level2/spmv/mcsp_spmv_gpu.cpp:686-903, :1123-1147
 mcsparseStatus_t mcsparseSpMV(mcsparseHandle_t handle, mcsparseOperation_t opA, const void* alpha,
                               mcsparseSpMatDescr_t matA, mcsparseDnVecDescr_t vecX, const void* beta,
-                              mcsparseDnVecDescr_t vecY, macaDataType computeType, mcsparseSpMVAlg_t /*alg*/,
+                              mcsparseDnVecDescr_t vecY, macaDataType computeType, mcsparseSpMVAlg_t alg,
                               void* externalBuffer) {
     return to_public_status(
-        mcsp::spmv_call(handle, opA, alpha, matA, vecX, beta, vecY, computeType, externalBuffer, 0, true));
+        mcsp::spmv_call(handle, opA, alpha, matA, vecX, beta, vecY, computeType, externalBuffer, 0, true, alg));
 }
 
 // EXTENSION
@@ -697,13 +708,14 @@ mcsparseStatus_t mcsparseSpMV_preprocess_bufferSize(mcsparseHandle_t handle, mcs
         mcsparseSpMV_bufferSize(handle, opA, alpha, matA, vecX, beta, vecY, computeType, alg, bufferSize);
     if (st != MCSPARSE_STATUS_SUCCESS) return st;
     BandedShape shape;
-    if (banded_candidate(matA, opA, &shape)) {
+    if (banded_candidate(matA, opA, alg, &shape)) {
         const size_t vb = value_size(matA->valueType);
         const CsrView v = make_view(matA, opA);
         const idx_t rows = static_cast<idx_t>(v.transpose ? v.n : v.m);
+        // the copy in column order carries its own scratch; the other builds a transpose behind itself
         *bufferSize = banded_region_offset(matA, opA, vb) +
                       align_up(mcsp::banded_layout(shape, rows, static_cast<idx_t>(matA->nnz), vb).total) +
-                      (v.transpose ? transpose_scratch(v, matA->nnz, vb).total : 0);
+                      (v.transpose && !shape.by_column ? transpose_scratch(v, matA->nnz, vb).total : 0);
     }
     return MCSPARSE_STATUS_SUCCESS;
 }
@@ -712,14 +724,14 @@ mcsparseStatus_t mcsparseSpMV_preprocess_bufferSize(mcsparseHandle_t handle, mcs
 mcsparseStatus_t mcsparseSpMV_preprocess(mcsparseHandle_t handle, mcsparseOperation_t opA, const void* alpha,
                                          mcsparseSpMatDescr_t matA, mcsparseDnVecDescr_t vecX, const void* beta,
                                          mcsparseDnVecDescr_t vecY, macaDataType computeType,
-                                         mcsparseSpMVAlg_t /*alg*/, void* externalBuffer) {
+                                         mcsparseSpMVAlg_t alg, void* externalBuffer) {
     const mcspStatus_t st =
         mcsp::spmv_check(handle, opA, alpha, matA, vecX, beta, vecY, computeType, externalBuffer, 0, true);
     if (st != MCSP_STATUS_SUCCESS) return to_public_status(st);
     matA->banded.valid = false;
     if (stream_is_capturing(handle->stream)) return to_public_status(MCSP_STATUS_NOT_IMPLEMENTED);  // it blocks
     BandedShape shape;
-    if (matA->nnz == 0 || !banded_candidate(matA, opA, &shape)) return MCSPARSE_STATUS_SUCCESS;  // nothing to prepare
+    if (matA->nnz == 0 || !banded_candidate(matA, opA, alg, &shape)) return MCSPARSE_STATUS_SUCCESS;  // nothing to prepare
 
     const CsrView v = make_view(matA, opA);
     const idx_t m = static_cast<idx_t>(v.transpose ? v.n : v.m);  // rows of the matrix that is banded
@@ -748,7 +760,23 @@ mcsparseStatus_t mcsparseSpMV_preprocess(mcsparseHandle_t handle, mcsparseOperat
     b.region = banded_region_offset(matA, opA, vb);
     b.grid = 0;
     char* region = static_cast<char*>(externalBuffer) + b.region;
-    if (v.transpose) {
+    if (shape.by_column) {
+        const mcsp::BandedLayout cl = mcsp::banded_layout(shape, m, nnz, vb);
+        idx_t* src_cols = reinterpret_cast<idx_t*>(region + cl.src_cols);
+        idx_t* src_rows = reinterpret_cast<idx_t*>(region + cl.src_rows);
+        if (v.transpose) {
+            // the nonzeros of the transpose sorted by its columns are the arrays as they lie: its
+            // columns are the rows of the view, its rows the column indices
+            mcsp::launch_csr2coo(handle->stream, static_cast<idx_t>(v.m), nnz, v.ptr, base, src_rows);
+            mcsp::launch_column_order_build(handle->stream, shape, m, nnz, base, v.ind, src_rows, matA->vals, vb, region);
+        } else {
+            mcsp::launch_sort_by_column(handle->stream, static_cast<idx_t>(v.m), static_cast<idx_t>(v.n), nnz, base, v.ptr,
+                                        v.ind, matA->vals, vb, src_cols, src_rows, region + cl.src_vals,
+                                        region + cl.sort_ws);
+            mcsp::launch_column_order_build(handle->stream, shape, m, nnz, base, src_rows, src_cols, region + cl.src_vals,
+                                            vb, region);
+        }
+    } else if (v.transpose) {
         // the transpose in CSR form, behind the banded copy it is only the source of
         char* scratch = region + align_up(mcsp::banded_layout(shape, m, nnz, vb).total);
         const TransposeScratch t = transpose_scratch(v, matA->nnz, vb);

@@ -371,7 +371,7 @@ mcsparseStatus_t mcsparseSpMatGetSpMMSchedule(mcsparseSpMatDescr_t d, int* state
 mcsparseStatus_t mcsparseSpMatGetSpMVPreprocess(mcsparseSpMatDescr_t d, int* state, int* bands, int* rows_per_tile) {
     if (d == nullptr || state == nullptr || bands == nullptr || rows_per_tile == nullptr)
         return to_public_status(MCSP_STATUS_INVALID_POINTER);
-    *state = !d->banded.valid ? 0 : (d->banded.useful ? 2 : 1);
+    *state = !d->banded.valid ? 0 : (!d->banded.useful ? 1 : (d->banded.shape.by_column ? 3 : 2));
     *bands = d->banded.valid && d->banded.useful ? static_cast<int>(d->banded.shape.bands) : 0;
     *rows_per_tile = d->banded.valid && d->banded.useful ? static_cast<int>(d->banded.shape.rows_per_tile) : 0;
     return MCSPARSE_STATUS_SUCCESS;

@@ -948,6 +948,48 @@ void launch_sort_by_column_band(hipStream_t stream, idx_t m, idx_t nnz, idx_t ba
                        value_bytes, t, csr);
 }
 
+namespace {
+// The two sets of arrays the passes of a sort alternate between, the counters and their scan, carved
+// out of a workspace of csr2csc_workspace_bytes.
+SortScratch sort_scratch_in(char* w, const Csr2CscLayout& l) {
+    SortScratch t;
+    t.keys[0] = reinterpret_cast<idx_t*>(w + l.keys_a);
+    t.keys[1] = reinterpret_cast<idx_t*>(w + l.keys_b);
+    t.aux[0] = reinterpret_cast<idx_t*>(w + l.rows_a);
+    t.aux[1] = reinterpret_cast<idx_t*>(w + l.rows_b);
+    t.vals[0] = w + l.vals_a;
+    t.vals[1] = w + l.vals_b;
+    t.counters = reinterpret_cast<uint32_t*>(w + l.counters);
+    t.scan_ws = reinterpret_cast<uint32_t*>(w + l.scan_ws);
+    t.tile_rows = reinterpret_cast<idx_t*>(w + l.tile_rows);
+    return t;
+}
+}  // namespace
+
+// The nonzeros of a CSR matrix in the order of a stable sort by column, as (column, row, value)
+// arrays with the index base left in: csr2csc without the offsets.  workspace: csr2csc_workspace_bytes.
+void launch_sort_by_column(hipStream_t stream, idx_t m, idx_t n, idx_t nnz, idx_t base, const idx_t* row_ptr,
+                           const idx_t* col, const void* val, size_t value_bytes, idx_t* cols_out, idx_t* rows_out,
+                           void* vals_out, void* workspace) {
+    if (m == 0 || n == 0 || nnz == 0) return;
+    const SortScratch t = sort_scratch_in(static_cast<char*>(workspace), csr2csc_layout(nnz, value_bytes));
+    CsrSource csr;
+    csr.rows = m;
+    csr.base = base;
+    radix_sort_triples(stream, nnz, bit_length(n - 1 + base), col, row_ptr, val, cols_out, rows_out, vals_out,
+                       value_bytes, t, csr);
+}
+
+// Stable sort of (key, aux, value) triples on the low key_bits (at most 16) of the keys.  The outputs
+// must not overlap the inputs or the workspace (csr2csc_workspace_bytes).
+void launch_sort_triples(hipStream_t stream, idx_t nnz, uint32_t key_bits, const idx_t* keys_in, const idx_t* aux_in,
+                         const void* vals_in, idx_t* keys_out, idx_t* aux_out, void* vals_out, size_t value_bytes,
+                         void* workspace) {
+    if (nnz == 0) return;
+    const SortScratch t = sort_scratch_in(static_cast<char*>(workspace), csr2csc_layout(nnz, value_bytes));
+    radix_sort_triples(stream, nnz, key_bits, keys_in, aux_in, vals_in, keys_out, aux_out, vals_out, value_bytes, t);
+}
+
 size_t index_sort_workspace_bytes(idx_t nnz) { return index_sort_layout(nnz).total; }
 
 void launch_coosort(hipStream_t stream, idx_t major_extent, idx_t minor_extent, idx_t nnz, idx_t* major, idx_t* minor,

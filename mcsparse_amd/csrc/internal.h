@@ -104,6 +104,10 @@ struct BandedShape {
     uint32_t rows_per_tile;
     uint32_t chunks;         // row chunks = tiles per band
     uint32_t tiles;
+    // false: entries of a tile in CSR order, row sums formed in a fixed order (bit-reproducible);
+    // true: entries of a tile in column order, products added to the row sums in LDS as they come
+    bool by_column = false;
+    uint32_t sub = 1;        // by_column: bands per group; `bands` then counts the groups (planes of partial sums)
 };
 struct SpmvBanded {
     bool valid = false;
@@ -216,7 +220,8 @@ mcspStatus_t spmv_check(mcsparseHandle_t handle, mcsparseOperation_t opA, const 
                         macaDataType computeType, const void* buffer, size_t buffer_bytes, bool may_read_back);
 mcspStatus_t spmv_call(mcsparseHandle_t handle, mcsparseOperation_t opA, const void* alpha, mcsparseSpMatDescr_t matA,
                        mcsparseDnVecDescr_t vecX, const void* beta, mcsparseDnVecDescr_t vecY,
-                       macaDataType computeType, void* buffer, size_t buffer_bytes, bool may_read_back);
+                       macaDataType computeType, void* buffer, size_t buffer_bytes, bool may_read_back,
+                       mcsparseSpMVAlg_t alg = MCSPARSE_SPMV_ALG_DEFAULT);
 
 // Kernel family (and lanes per row / tile order) for a structure with these row-length bins: the
 // 33 counters and the longest row that launch_row_bins leaves, read back to the host.  A pure
@@ -258,7 +263,19 @@ constexpr size_t kBandedBandBytes = size_t(2) << 20;
 struct BandedLayout {
     // kept between preprocess and SpMV: [0, keep); scratch of the build: [keep, total)
     size_t tile_ptr, xcd_start, entries, vals, partials, keep, tmp_keys, tmp_rows, sort_ws, total;
+    // by_column only: the nonzeros sorted by column (the source of the build) and the sorted tile numbers
+    size_t src_cols, src_rows, src_vals, tile_ids;
 };
+// The same decision for the copy whose tiles are in column order (BandedShape::by_column): tall tiles of
+// up to kColumnOrderRows rows, at most 64 bands and 65536 tiles.
+constexpr uint32_t kColumnOrderRows = 16384;
+bool column_order_shape(idx_t m, idx_t n, idx_t nnz, idx_t base, size_t value_bytes, size_t band_bytes,
+                        BandedShape* out);
+// r_keys / c_keys: row + base and column + base of every nonzero of the matrix to copy, in an order
+// sorted by column (any order among equal columns); vals in the same order.  Neither is written.
+void launch_column_order_build(hipStream_t stream, const BandedShape& s, idx_t m, idx_t nnz, idx_t base,
+                               const idx_t* r_keys, const idx_t* c_keys, const void* vals, size_t value_bytes,
+                               void* region);
 // False when the banded copy cannot help or cannot be built: x fits one band, more than 256 bands.
 bool banded_shape(idx_t m, idx_t n, idx_t nnz, idx_t base, size_t value_bytes, size_t band_bytes, BandedShape* out);
 BandedLayout banded_layout(const BandedShape& s, idx_t m, idx_t nnz, size_t value_bytes);
@@ -345,6 +362,17 @@ size_t band_sort_workspace_bytes(idx_t nnz);
 void launch_sort_by_column_band(hipStream_t stream, idx_t m, idx_t nnz, idx_t base, const idx_t* row_ptr, const idx_t* col,
                                 const void* val, size_t value_bytes, uint32_t band_shift, uint32_t band_bits,
                                 idx_t* cols_out, idx_t* rows_out, void* vals_out, void* workspace);
+
+// (column, row + base, value) arrays of the nonzeros in the order of a stable sort by column: csr2csc
+// without the offsets.  workspace: csr2csc_workspace_bytes.
+void launch_sort_by_column(hipStream_t stream, idx_t m, idx_t n, idx_t nnz, idx_t base, const idx_t* row_ptr,
+                           const idx_t* col, const void* val, size_t value_bytes, idx_t* cols_out, idx_t* rows_out,
+                           void* vals_out, void* workspace);
+// Stable sort of (key, aux, value) triples on the low key_bits (<= 16) of the keys; outputs apart from
+// the inputs and from the workspace (csr2csc_workspace_bytes).
+void launch_sort_triples(hipStream_t stream, idx_t nnz, uint32_t key_bits, const idx_t* keys_in, const idx_t* aux_in,
+                         const void* vals_in, idx_t* keys_out, idx_t* aux_out, void* vals_out, size_t value_bytes,
+                         void* workspace);
 
 // ---- index sorts (convert.hip) --------------------------------------------------------------
 size_t index_sort_workspace_bytes(idx_t nnz);

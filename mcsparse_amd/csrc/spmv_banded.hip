@@ -12,6 +12,12 @@
 // leaves one partial sum per row and band; a second kernel adds a row's partial sums in band order.
 // No atomics: every sum is formed in a fixed order, so results are bit-reproducible run to run.
 //
+// A second form of the copy (BandedShape::by_column) trades that reproducibility for fewer requests to
+// L2: tiles of up to 16384 rows whose entries are sorted by column, so that the lanes of a wavefront
+// gather neighbouring elements of x (several per 128-byte line), and products added to the tile's row
+// sums in LDS by ds_add_f64 in the order the wavefronts reach them.  Selected by
+// MCSPARSE_SPMV_CSR_ALG1 in mcsparseSpMV_preprocess.
+//
 // Stands in, like spmv.hip, for the gather loop of the reference's row kernel
 // (src/kernels/level2/spmv/csr_vector_device.hpp:40-57).
 #include "device_util.h"
@@ -257,6 +263,146 @@ __global__ __launch_bounds__(kBlock) void banded_reduce_kernel(idx_t m, uint32_t
     }
 }
 
+// ------------------------------------------------------------------------------------------
+// tiles in column order
+// ------------------------------------------------------------------------------------------
+// A packed word has room for 32 - log2(rows per tile) column bits, which for tiles of 16384 rows is a
+// band of 1 MiB of fp32: half of what an XCD's L2 holds comfortably.  `sub` consecutive bands therefore
+// form a group that shares one plane of partial sums: the tiles of a row chunk in the bands of a group
+// are neighbours in the tile list (tile = (group * chunks + chunk) * sub + band inside the group) and a
+// workgroup takes them in one go, keeping the row sums in LDS across them.
+//
+// Nonzero k (row key r, column key c, both with the index base in) gets its tile number and the same
+// packed word as above.  ids_out / packed_out may be the input arrays themselves (element k is read
+// before it is written).
+__global__ __launch_bounds__(kBlock) void column_order_pack_kernel(idx_t nnz, idx_t base, uint32_t band_shift,
+                                                                   uint32_t rows_per_tile, uint32_t chunks, uint32_t sub,
+                                                                   const idx_t* r_keys, const idx_t* c_keys,
+                                                                   idx_t* ids_out, idx_t* packed_out) {
+    const uint64_t k = static_cast<uint64_t>(blockIdx.x) * kBlock + threadIdx.x;
+    if (k >= nnz) return;
+    const idx_t band_mask = (1u << band_shift) - 1u;
+    const idx_t key = c_keys[k];
+    const idx_t row = r_keys[k] - base;
+    const uint32_t chunk = row / rows_per_tile;
+    const uint32_t band = key >> band_shift;
+    const uint32_t group = band / sub;
+    ids_out[k] = (group * chunks + chunk) * sub + (band - group * sub);
+    packed_out[k] = ((row - chunk * rows_per_tile) << band_shift) | (key & band_mask);
+}
+
+// One workgroup per compute unit: workgroup i belongs to XCD i % 8 and takes every 32nd unit (the tiles
+// of one row chunk in one band group) of that XCD's stretch.  The row sums of a unit live in LDS as
+// doubles (fp32 products are widened: ds_add_f32 runs at a quarter of the rate of ds_add_f64 on this
+// chip); a thread has kColumnIpt gathers in flight (4, 8, 16 measured: 16 is 1-4 % ahead).
+constexpr int kColumnBlock = 1024;
+constexpr int kColumnIpt = 16;
+constexpr uint32_t kColumnGroupsPerXcd = 32;
+
+// xcd_start for the kernel below, in units.  A stretch is dealt to the kColumnGroupsPerXcd workgroups of
+// its XCD in turns, so what counts is the largest number of nonzeros any one workgroup ends up with.
+// Two ways to cut the list of units are tried, equal nonzeros per XCD (good when units differ widely)
+// and equal counts (good when they are alike: one unit too many on an XCD doubles a workgroup's
+// share), and the better one is kept.
+__global__ __launch_bounds__(kBlock) void column_order_split_kernel(idx_t nnz, uint32_t units, uint32_t sub,
+                                                                    const idx_t* __restrict__ tile_ptr,
+                                                                    uint32_t* __restrict__ xcd_start) {
+    static_assert(kBlock == kXcds * kColumnGroupsPerXcd, "one thread per workgroup of the SpMV kernel");
+    __shared__ uint32_t s_start[2][kXcds + 1];
+    __shared__ unsigned long long s_worst[2];
+    const uint32_t tid = threadIdx.x;
+    if (tid <= kXcds) {
+        const uint64_t target = static_cast<uint64_t>(nnz) * tid / kXcds;
+        uint32_t lo = 0, hi = units;  // first unit whose offset is >= target
+        while (lo < hi) {
+            const uint32_t mid = (lo + hi) >> 1;
+            if (tile_ptr[static_cast<uint64_t>(mid) * sub] < target) lo = mid + 1; else hi = mid;
+        }
+        s_start[0][tid] = tid == 0 ? 0u : (tid == kXcds ? units : lo);
+        s_start[1][tid] = static_cast<uint32_t>(static_cast<uint64_t>(units) * tid / kXcds);
+    }
+    if (tid < 2) s_worst[tid] = 0;
+    __syncthreads();
+    const uint32_t xcd = tid / kColumnGroupsPerXcd, slot = tid % kColumnGroupsPerXcd;
+    for (int cut = 0; cut < 2; ++cut) {
+        unsigned long long share = 0;
+        for (uint32_t u = s_start[cut][xcd] + slot; u < s_start[cut][xcd + 1]; u += kColumnGroupsPerXcd)
+            share += tile_ptr[static_cast<uint64_t>(u + 1) * sub] - tile_ptr[static_cast<uint64_t>(u) * sub];
+        atomicMax(&s_worst[cut], share);
+    }
+    __syncthreads();
+    if (tid <= kXcds) xcd_start[tid] = s_start[s_worst[1] <= s_worst[0] ? 1 : 0][tid];
+}
+
+template <typename T>
+__global__ __launch_bounds__(kColumnBlock) void spmv_column_order_kernel(idx_t m, idx_t n, idx_t nnz, idx_t base,
+                                                                        uint32_t band_shift, uint32_t rows_per_tile,
+                                                                        uint32_t chunks, uint32_t units, uint32_t sub,
+                                                                        const uint32_t* __restrict__ xcd_start,
+                                                                        const idx_t* __restrict__ tile_ptr,
+                                                                        const idx_t* __restrict__ entries,
+                                                                        const T* __restrict__ vals,
+                                                                        const T* __restrict__ x,
+                                                                        T* __restrict__ partials) {
+    extern __shared__ __align__(16) unsigned char s_raw[];
+    double* s_acc = reinterpret_cast<double*>(s_raw);
+    const uint32_t tid = threadIdx.x;
+    const uint32_t xcd = blockIdx.x % kXcds;
+    const uint32_t stretch_end = min(xcd_start[xcd + 1], units);
+    const idx_t band_mask = (1u << band_shift) - 1u;
+    for (uint32_t r = tid; r < rows_per_tile; r += kColumnBlock) s_acc[r] = 0.0;
+    __syncthreads();
+    for (uint32_t unit = xcd_start[xcd] + blockIdx.x / kXcds; unit < stretch_end; unit += gridDim.x / kXcds) {
+        const uint32_t group = unit / chunks;
+        const uint32_t chunk = unit - group * chunks;
+        const uint64_t row0 = static_cast<uint64_t>(chunk) * rows_per_tile;
+        if (row0 >= m) continue;  // whole workgroup
+        const uint32_t tile_rows = static_cast<uint32_t>(m - row0 < rows_per_tile ? m - row0 : rows_per_tile);
+        for (uint32_t b = 0; b < sub; ++b) {
+            const uint64_t tile = static_cast<uint64_t>(unit) * sub + b;
+            idx_t e0 = tile_ptr[tile];
+            idx_t e1 = tile_ptr[tile + 1];
+            e0 = e0 < nnz ? e0 : nnz;
+            e1 = e1 < nnz ? e1 : nnz;
+            e1 = e1 > e0 ? e1 : e0;
+            const idx_t band_key = (group * sub + b) << band_shift;
+            for (idx_t slab = e0; slab < e1; slab += kColumnBlock * kColumnIpt) {
+                const uint32_t cnt = e1 - slab < static_cast<idx_t>(kColumnBlock * kColumnIpt)
+                                         ? e1 - slab
+                                         : kColumnBlock * kColumnIpt;
+                idx_t packed[kColumnIpt];
+                T v[kColumnIpt], xv[kColumnIpt];
+#pragma unroll
+                for (int i = 0; i < kColumnIpt; ++i) {
+                    const uint32_t k = min(static_cast<uint32_t>(i) * kColumnBlock + tid, cnt - 1);
+                    packed[i] = load_stream(entries + slab + k);
+                    v[i] = load_stream(vals + slab + k);
+                }
+#pragma unroll
+                for (int i = 0; i < kColumnIpt; ++i) {
+                    idx_t key = band_key | (packed[i] & band_mask);  // column + base
+                    key = key > base ? key : base;
+                    xv[i] = x[min(key - base, n - 1)];
+                }
+#pragma unroll
+                for (int i = 0; i < kColumnIpt; ++i) {
+                    const uint32_t k = static_cast<uint32_t>(i) * kColumnBlock + tid;
+                    // a row past the end of the tile (an overwritten layout) still lies inside the sums
+                    const uint32_t r = min(packed[i] >> band_shift, rows_per_tile - 1);
+                    if (k < cnt) unsafeAtomicAdd(&s_acc[r], static_cast<double>(v[i] * xv[i]));
+                }
+            }
+        }
+        __syncthreads();
+        T* out = partials + static_cast<uint64_t>(group) * m + row0;
+        for (uint32_t r = tid; r < rows_per_tile; r += kColumnBlock) {
+            if (r < tile_rows) out[r] = static_cast<T>(s_acc[r]);
+            s_acc[r] = 0.0;
+        }
+        __syncthreads();
+    }
+}
+
 }  // namespace
 
 bool banded_shape(idx_t m, idx_t n, idx_t nnz, idx_t base, size_t value_bytes, size_t band_bytes, BandedShape* out) {
@@ -285,6 +431,32 @@ bool banded_shape(idx_t m, idx_t n, idx_t nnz, idx_t base, size_t value_bytes, s
     return true;
 }
 
+bool column_order_shape(idx_t m, idx_t n, idx_t nnz, idx_t base, size_t value_bytes, size_t band_bytes,
+                        BandedShape* out) {
+    if (m == 0 || n == 0 || nnz == 0 || (value_bytes != 4 && value_bytes != 8)) return false;
+    uint32_t rows_per_tile = 64;
+    while (rows_per_tile < kColumnOrderRows && rows_per_tile < m) rows_per_tile *= 2;
+    const uint32_t row_bits = bit_length(rows_per_tile - 1);
+    uint32_t wanted = 0;  // log2 of the keys in band_bytes of x
+    while ((static_cast<size_t>(value_bytes) << (wanted + 1)) <= band_bytes) ++wanted;
+    const uint32_t shift = wanted > 32 - row_bits ? 32 - row_bits : wanted;
+    const uint32_t sub = 1u << (wanted - shift);  // bands that share a plane of partial sums
+    const uint64_t max_key = static_cast<uint64_t>(n) - 1 + base;
+    const uint64_t groups = (max_key >> wanted) + 1;
+    const uint64_t chunks = (static_cast<uint64_t>(m) + rows_per_tile - 1) / rows_per_tile;
+    // every group costs a partial sum per row; the tile numbers are sorted in at most two passes
+    if (groups > 64 || sub > 64 || groups * chunks * sub > 65536) return false;
+    out->band_shift = shift;
+    out->band_bits = bit_length(static_cast<uint32_t>(groups * sub - 1));
+    out->bands = static_cast<uint32_t>(groups);
+    out->rows_per_tile = rows_per_tile;
+    out->chunks = static_cast<uint32_t>(chunks);
+    out->tiles = static_cast<uint32_t>(groups * chunks * sub);
+    out->sub = sub;
+    out->by_column = true;
+    return true;
+}
+
 BandedLayout banded_layout(const BandedShape& s, idx_t m, idx_t nnz, size_t value_bytes) {
     BandedLayout l;
     const size_t idx_bytes = align_up(static_cast<size_t>(nnz) * sizeof(idx_t));
@@ -295,11 +467,41 @@ BandedLayout banded_layout(const BandedShape& s, idx_t m, idx_t nnz, size_t valu
     l.vals = off; off += align_up(static_cast<size_t>(nnz) * value_bytes);
     l.partials = off; off += align_up(static_cast<size_t>(s.bands) * m * value_bytes);
     l.keep = off;
+    l.src_cols = l.src_rows = l.src_vals = l.tile_ids = 0;
+    if (s.by_column) {
+        l.tmp_keys = l.tmp_rows = 0;
+        l.src_cols = off; off += idx_bytes;
+        l.src_rows = off; off += idx_bytes;
+        l.src_vals = off; off += align_up(static_cast<size_t>(nnz) * value_bytes);
+        l.tile_ids = off; off += idx_bytes;
+        l.sort_ws = off; off += align_up(csr2csc_workspace_bytes(m, 0, nnz, value_bytes));
+        l.total = off;
+        return l;
+    }
     l.tmp_keys = off; off += idx_bytes;
     l.tmp_rows = off; off += idx_bytes;
     l.sort_ws = off; off += align_up(band_sort_workspace_bytes(nnz));
     l.total = off;
     return l;
+}
+
+void launch_column_order_build(hipStream_t stream, const BandedShape& s, idx_t m, idx_t nnz, idx_t base,
+                               const idx_t* r_keys, const idx_t* c_keys, const void* vals, size_t value_bytes,
+                               void* region) {
+    const BandedLayout l = banded_layout(s, m, nnz, value_bytes);
+    char* w = static_cast<char*>(region);
+    // tile numbers and packed words take the place of the source arrays inside the region; a caller's
+    // own arrays (the transposing directions hand them in) are copied from, never written
+    idx_t* ids = reinterpret_cast<idx_t*>(w + l.src_cols);
+    idx_t* packed = reinterpret_cast<idx_t*>(w + l.src_rows);
+    hipLaunchKernelGGL(column_order_pack_kernel, dim3((nnz + kBlock - 1) / kBlock), dim3(kBlock), 0, stream, nnz, base,
+                       s.band_shift, s.rows_per_tile, s.chunks, s.sub, r_keys, c_keys, ids, packed);
+    idx_t* sorted_ids = reinterpret_cast<idx_t*>(w + l.tile_ids);
+    launch_sort_triples(stream, nnz, bit_length(s.tiles - 1), ids, packed, vals, sorted_ids,
+                        reinterpret_cast<idx_t*>(w + l.entries), w + l.vals, value_bytes, w + l.sort_ws);
+    launch_coo2csr(stream, nnz, s.tiles, sorted_ids, 0, reinterpret_cast<idx_t*>(w + l.tile_ptr));
+    hipLaunchKernelGGL(column_order_split_kernel, dim3(1), dim3(kBlock), 0, stream, nnz, s.tiles / s.sub, s.sub,
+                       reinterpret_cast<const idx_t*>(w + l.tile_ptr), reinterpret_cast<uint32_t*>(w + l.xcd_start));
 }
 
 void launch_banded_build(hipStream_t stream, const BandedShape& s, idx_t m, idx_t nnz, idx_t base, const idx_t* row_ptr,
@@ -335,7 +537,16 @@ void launch_spmv_banded(hipStream_t stream, const BandedShape& s, uint32_t grid,
     const BandedLayout l = banded_layout(s, a.m, a.nnz, sizeof(T));
     char* w = static_cast<char*>(region);
     T* partials = reinterpret_cast<T*>(w + l.partials);
-    if (grid != 0) {
+    if (s.by_column) {
+        const int lds = static_cast<int>(s.rows_per_tile * sizeof(double));
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(spmv_column_order_kernel<T>),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+        hipLaunchKernelGGL((spmv_column_order_kernel<T>), dim3(kColumnGroupsPerXcd * kXcds), dim3(kColumnBlock), lds,
+                           stream, a.m, a.n, a.nnz, a.base, s.band_shift, s.rows_per_tile, s.chunks, s.tiles / s.sub, s.sub,
+                           reinterpret_cast<const uint32_t*>(w + l.xcd_start),
+                           reinterpret_cast<const idx_t*>(w + l.tile_ptr), reinterpret_cast<const idx_t*>(w + l.entries),
+                           reinterpret_cast<const T*>(w + l.vals), static_cast<const T*>(a.x), partials);
+    } else if (grid != 0) {
         hipLaunchKernelGGL((spmv_banded_kernel<T>), dim3(grid), dim3(kBlock), 0, stream, a.m, a.n, a.nnz, a.base,
                            s.band_shift, s.rows_per_tile, s.chunks, s.tiles,
                            reinterpret_cast<const uint32_t*>(w + l.xcd_start),

@@ -46,7 +46,7 @@ extern "C" {
 mcsparseStatus_t mcsparseSpMV_staticBuffer(mcsparseHandle_t handle, mcsparseOperation_t opA, const void* alpha,
                                            mcsparseSpMatDescr_t matA, mcsparseDnVecDescr_t vecX, const void* beta,
                                            mcsparseDnVecDescr_t vecY, macaDataType computeType,
-                                           mcsparseSpMVAlg_t /*alg*/) {
+                                           mcsparseSpMVAlg_t alg) {
     // Every argument check, the size check included, comes before the device is touched; the checks
     // only need a buffer pointer that is not null.
     static unsigned char placeholder;
@@ -56,7 +56,7 @@ mcsparseStatus_t mcsparseSpMV_staticBuffer(mcsparseHandle_t handle, mcsparseOper
     void* buffer = nullptr;
     if (scratch_of_current_device(&buffer) != hipSuccess) return to_public_status(MCSP_STATUS_INTERNAL_ERROR);
     return to_public_status(
-        mcsp::spmv_call(handle, opA, alpha, matA, vecX, beta, vecY, computeType, buffer, kScratchBytes, false));
+        mcsp::spmv_call(handle, opA, alpha, matA, vecX, beta, vecY, computeType, buffer, kScratchBytes, false, alg));
 }
 
 }  // extern "C"

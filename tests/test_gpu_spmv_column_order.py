@@ -1,0 +1,144 @@
+"""GPU parity of the SpMV copy whose tiles are in column order (mcsparseSpMV_preprocess with
+MCSPARSE_SPMV_CSR_ALG1): products meet in LDS in the order the wavefronts reach them, so results are
+within the tolerance of every other family but not bitwise reproducible."""
+import glob
+import os
+
+import numpy as np
+import pytest
+
+from mcsparse_amd import api
+from mcsparse_amd import workloads as wl
+
+from gpu_util import assert_within, dev
+
+pytestmark = pytest.mark.gpu
+
+GOLDEN = sorted(glob.glob(os.path.join(os.path.dirname(__file__), "golden", "csr_*.npz")))
+
+
+def run(torch, handle, oracle, a, alpha, beta, op=api.OP_N, fmt=api.FORMAT_CSR, band_bytes=0, seed=1, expect_state=3,
+        calls=2, call_alg=api.SPMV_CSR_ALG1, what="column order"):
+    """a: the matrix whose arrays are handed over (m x n CSR).  fmt CSC reads the same arrays as the CSC of
+    the n x m transpose.  The product computed is A x for (CSR, N) and (CSC, T), A^T x otherwise."""
+    rng = np.random.default_rng(seed)
+    dt = a.val.dtype
+    ct = api.maca_type(dt)
+    transposed = (fmt == api.FORMAT_CSR) == (op == api.OP_T)
+    x = rng.uniform(-1, 1, a.m if transposed else a.n).astype(dt)
+    y = rng.uniform(-1, 1, a.n if transposed else a.m).astype(dt)
+    d_ptr, d_col, d_val, d_x, d_y = (dev(torch, v) for v in (a.ptr, a.col, a.val, x, y))
+    if fmt == api.FORMAT_CSR:
+        mat = api.SpMat(a.m, a.n, a.nnz, d_ptr, d_col, d_val, base=a.base)
+    else:
+        mat = api.SpMat(a.n, a.m, a.nnz, d_ptr, d_col, d_val, base=a.base, fmt=api.FORMAT_CSC)
+    if band_bytes:
+        mat.set_band_bytes(band_bytes)
+    vx, vy = api.DnVec(d_x), api.DnVec(d_y)
+    st, size = api.spmv_preprocess_buffer_size(handle, op, alpha, mat, vx, beta, vy, ct, alg=api.SPMV_CSR_ALG1)
+    assert st == api.STATUS_SUCCESS
+    buf = torch.empty(size, dtype=torch.uint8, device="cuda")
+    assert api.spmv_preprocess(handle, op, alpha, mat, vx, beta, vy, ct, buf, alg=api.SPMV_CSR_ALG1) == api.STATUS_SUCCESS
+    state, bands, rows = mat.spmv_preprocess_state()
+    assert state == expect_state, (state, bands, rows)
+    y_ref, bound = oracle.spmv(transposed, a.m, a.n, a.base, a.ptr, a.col, a.val, alpha, beta, x, y)
+    for _ in range(calls):
+        d_y.copy_(torch.from_numpy(y))
+        assert api.spmv(handle, op, alpha, mat, vx, beta, vy, ct, buf, alg=call_alg) == api.STATUS_SUCCESS
+        torch.cuda.synchronize()
+        assert_within(d_y.cpu().numpy(), y_ref, bound, dt, what=what)
+    return state, bands, rows, mat, buf
+
+
+@pytest.mark.parametrize("path", GOLDEN, ids=[os.path.basename(p)[:-4] for p in GOLDEN])
+@pytest.mark.parametrize("base", [0, 1])
+def test_golden_fixtures_column_order(torch_gpu, handle, path, base):
+    """Integer-valued fixtures: every summation order is exact, so the result must equal the fixture's."""
+    torch = torch_gpu
+    with np.load(path) as z:
+        g = {k: z[k] for k in z.files}
+    for dt in (np.float32, np.float64):
+        a = wl.Csr(int(g["m"]), int(g["n"]), g["ptr"], g["col"], g["val"].astype(dt)).with_base(base)
+        ct = api.maca_type(dt)
+        alpha, beta = float(g["alpha"]), float(g["beta"])
+        d_ptr, d_col, d_val, d_x, d_y = (dev(torch, v) for v in (a.ptr, a.col, a.val, g["x"].astype(dt),
+                                                                   g["y0"].astype(dt)))
+        mat = api.SpMat(a.m, a.n, a.nnz, d_ptr, d_col, d_val, base=base)
+        mat.set_band_bytes(64)
+        vx, vy = api.DnVec(d_x), api.DnVec(d_y)
+        st, size = api.spmv_preprocess_buffer_size(handle, api.OP_N, alpha, mat, vx, beta, vy, ct,
+                                                   alg=api.SPMV_CSR_ALG1)
+        assert st == api.STATUS_SUCCESS
+        buf = torch.empty(size, dtype=torch.uint8, device="cuda")
+        assert api.spmv_preprocess(handle, api.OP_N, alpha, mat, vx, beta, vy, ct, buf,
+                                   alg=api.SPMV_CSR_ALG1) == api.STATUS_SUCCESS
+        assert mat.spmv_preprocess_state()[0] in (2, 3)  # very wide fixtures need more than 64 such bands
+        assert api.spmv(handle, api.OP_N, alpha, mat, vx, beta, vy, ct, buf, alg=api.SPMV_CSR_ALG1) == api.STATUS_SUCCESS
+        torch.cuda.synchronize()
+        assert np.array_equal(d_y.cpu().numpy().astype(np.float64), g["y_n"])
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("base", [0, 1])
+def test_ragged_rows_several_chunks_and_bands(torch_gpu, handle, oracle, dtype, base):
+    # three row chunks of 16384, empty rows, several bands, tiles without entries
+    a = wl.random_ragged(40003, 30011, 9, dtype=dtype, seed=5, base=base)
+    state, bands, rows, _, _ = run(torch_gpu, handle, oracle, a, -0.75, 1.25, band_bytes=1 << 14)
+    assert rows == 16384 and bands >= 2
+    run(torch_gpu, handle, oracle, a, 2.0, 0.0)  # default band width
+
+
+@pytest.mark.parametrize("fmt,op", [(api.FORMAT_CSR, api.OP_T), (api.FORMAT_CSC, api.OP_N), (api.FORMAT_CSC, api.OP_T)])
+def test_other_directions(torch_gpu, handle, oracle, fmt, op):
+    a = wl.random_ragged(20001, 35011, 11, dtype=np.float64, seed=6, base=1)
+    run(torch_gpu, handle, oracle, a, 1.5, 0.5, op=op, fmt=fmt, band_bytes=1 << 15)
+
+
+def test_small_matrix_one_band(torch_gpu, handle, oracle):
+    a = wl.random_ragged(300, 200, 7, dtype=np.float32, seed=7)
+    state, bands, rows, _, _ = run(torch_gpu, handle, oracle, a, 1.0, 0.0)
+    assert bands == 1 and rows == 512
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_long_rows(torch_gpu, handle, oracle, dtype):
+    # thousands of products of one row meet in one accumulator
+    a = wl.power_law(m=1 << 15, n=1 << 20, max_len=20000, dtype=dtype)
+    run(torch_gpu, handle, oracle, a, 1.0, 0.0)
+    run(torch_gpu, handle, oracle, a, -1.5, 0.5, op=api.OP_T)
+
+
+def test_alg2_does_not_use_the_copy(torch_gpu, handle, oracle):
+    """MCSPARSE_SPMV_CSR_ALG2 promises the same bits on every run: the call runs the row kernels."""
+    a = wl.uniform_rows(m=20000, n=300000, per_row=8, dtype=np.float64, config_id=91)
+    run(torch_gpu, handle, oracle, a, 1.0, 0.0, call_alg=api.SPMV_CSR_ALG2)
+
+
+def test_wide_matrix_falls_back_to_the_banded_copy(torch_gpu, handle, oracle):
+    # more than 64 bands of this width: the reproducible banded copy is built instead
+    a = wl.random_ragged(5003, 30011, 23, dtype=np.float64, seed=3)
+    run(torch_gpu, handle, oracle, a, 1.0, 0.5, band_bytes=1024, expect_state=2)
+
+
+def test_overwritten_copy_stays_in_bounds(torch_gpu, handle, oracle):
+    torch = torch_gpu
+    a = wl.uniform_rows(m=40000, n=100000, per_row=8, dtype=np.float32, config_id=92)
+    state, bands, rows, mat, buf = run(torch, handle, oracle, a, 1.0, 0.0, band_bytes=1 << 16)
+    x = torch.rand(a.n, dtype=torch.float32, device="cuda")
+    y = torch.zeros(a.m, dtype=torch.float32, device="cuda")
+    # run() has dropped its descriptor's arrays; build a fresh one on live arrays and clobber its buffer
+    d_ptr, d_col, d_val = (dev(torch, v) for v in (a.ptr, a.col, a.val))
+    mat = api.SpMat(a.m, a.n, a.nnz, d_ptr, d_col, d_val)
+    mat.set_band_bytes(1 << 16)
+    vx, vy = api.DnVec(x), api.DnVec(y)
+    st, size = api.spmv_preprocess_buffer_size(handle, api.OP_N, 1.0, mat, vx, 0.0, vy, api.R_32F, alg=api.SPMV_CSR_ALG1)
+    buf = torch.empty(size, dtype=torch.uint8, device="cuda")
+    assert api.spmv_preprocess(handle, api.OP_N, 1.0, mat, vx, 0.0, vy, api.R_32F, buf, alg=api.SPMV_CSR_ALG1) == 0
+    assert mat.spmv_preprocess_state()[0] == 3
+    for fill in (0xFF, 0x00, None):
+        if fill is None:
+            buf.copy_(torch.randint(0, 256, (size,), dtype=torch.uint8, device="cuda"))
+        else:
+            buf.fill_(fill)
+        assert api.spmv(handle, api.OP_N, 1.0, mat, vx, 0.0, vy, api.R_32F, buf, alg=api.SPMV_CSR_ALG1) == 0
+        torch.cuda.synchronize()
