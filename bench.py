@@ -32,7 +32,7 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 
 OTHERS = ["c4-64", "c3", "c3t", "c5", "c5-spmv", "c5-coo", "c4-8", "c4-256", "c4-64-col", "c1",
-          "c2-alg1", "c3-alg1", "c3t-alg1"]
+          "c2-alg2", "c3-alg2", "c3t-alg2"]
 OTHERS_BUDGET_S = 200.0  # wall-clock budget of the default invocation for the workloads above
 
 
@@ -45,25 +45,26 @@ def _traffic(fetch_counts, write_counts):
 
 
 MEASURED_TRAFFIC = {
-    # keys: (workload, the banded copy ran).  spmv_banded_kernel + banded_reduce_kernel
-    ("c2", True): (_traffic(108483.2 + 20567.1, 32768.0 + 8192.0), "profiles/spmv_banded_f64_c2_1Mx16.txt"),
-    ("c3", True): (_traffic(479341.2 + 65545.2, 133136.1 + 16384.0), "profiles/spmv_banded_f32_c3_powerlaw.txt"),
-    ("c3t", True): (_traffic(481300.5 + 65544.8, 131206.2 + 16384.0), "profiles/spmv_banded_f32_c3_powerlaw.txt"),
-    ("c5-spmv", True): (_traffic(481330.8 + 65544.6, 131202.3 + 16384.0),
+    # keys: (workload, state of mcsparseSpMV_preprocess: 2 banded copy, 3 copy in column order, 0 neither).
+    # spmv_banded_kernel + banded_reduce_kernel
+    ("c2", 2): (_traffic(108483.2 + 20567.1, 32768.0 + 8192.0), "profiles/spmv_banded_f64_c2_1Mx16.txt"),
+    ("c3", 2): (_traffic(479341.2 + 65545.2, 133136.1 + 16384.0), "profiles/spmv_banded_f32_c3_powerlaw.txt"),
+    ("c3t", 2): (_traffic(481300.5 + 65544.8, 131206.2 + 16384.0), "profiles/spmv_banded_f32_c3_powerlaw.txt"),
+    ("c5-spmv", 2): (_traffic(481330.8 + 65544.6, 131202.3 + 16384.0),
                         "profiles/spmv_banded_f32_c3_powerlaw.txt"),
     # without the preprocess call: vector kernel; merge kernel (tiles in column order) + partition
     # + tile order + fix-up
-    ("c2", False): (_traffic(653904.5, 10047.2), "profiles/spmv_vector_f64_c2_1Mx16.txt"),
-    ("c3", False): (_traffic(3305285.9 + 17229.2 + 251.2 + 3154.3, 25157.0 + 1391.2 + 1994.3 + 1375.1),
+    ("c2", 0): (_traffic(653904.5, 10047.2), "profiles/spmv_vector_f64_c2_1Mx16.txt"),
+    ("c3", 0): (_traffic(3305285.9 + 17229.2 + 251.2 + 3154.3, 25157.0 + 1391.2 + 1994.3 + 1375.1),
                     "profiles/spmv_merge_f32_c3_powerlaw.txt"),
-    ("c4-64", False): (_traffic(613893.3, 524288.0), "profiles/spmm_group_f32_c4_stencil128.txt"),
-    ("c4-256", False): (_traffic(3673719.8, 2097152.0), "profiles/spmm_group_f32_c4_stencil128.txt"),
+    ("c4-64", 0): (_traffic(613893.3, 524288.0), "profiles/spmm_group_f32_c4_stencil128.txt"),
+    ("c4-256", 0): (_traffic(3673719.8, 2097152.0), "profiles/spmm_group_f32_c4_stencil128.txt"),
     # group kernel + the transposes of B and of C
-    ("c4-64-col", False): (_traffic(596223.4 + 262180.7 + 262178.7, 3 * 524288.0),
+    ("c4-64-col", 0): (_traffic(596223.4 + 262180.7 + 262178.7, 3 * 524288.0),
                            "profiles/spmm_colmajor_f32_c4_stencil128_n64.txt"),
     # csr2csc: 2 x scatter + the scatter that reads the CSR arrays in place + 3 x (histogram + scans)
     # + row starts per tile + coo2csr
-    ("c5", False): (_traffic(2 * 701979.0 + 481119.4 + 3 * (229171.1 + 2 * 7206.6 + 14342.5) + 21136.0 + 237161.6,
+    ("c5", 0): (_traffic(2 * 701979.0 + 481119.4 + 3 * (229171.1 + 2 * 7206.6 + 14342.5) + 21136.0 + 237161.6,
                              2 * 1387754.6 + 1421432.8 + 3 * (28789.0 + 2 * 14326.3 + 56.0) + 223.8 + 19514.6),
                     "profiles/csr2csc_radix_f32_c5_powerlaw.txt"),
 }
@@ -84,9 +85,10 @@ def parse():
     p.add_argument("--family", type=int, default=0, help="force the SpMV kernel family (1 vector, 2 merge)")
     p.add_argument("--lanes", type=int, default=0, help="force lanes per row of the vector family")
     p.add_argument("--band-bytes", type=int, default=0, help="band width of mcsparseSpMV_preprocess (0 = default)")
-    p.add_argument("--alg1", action="store_true",
-                   help="MCSPARSE_SPMV_CSR_ALG1 for the SpMV workloads (a name ending in -alg1 says the same): "
-                        "preprocess builds the copy in column order, whose sums need not repeat bit for bit")
+    p.add_argument("--alg2", action="store_true",
+                   help="MCSPARSE_SPMV_CSR_ALG2 for the SpMV workloads (a name ending in -alg2 says the same): "
+                        "preprocess builds the banded copy whose sums repeat bit for bit, instead of the "
+                        "faster copy in column order that the default algorithm gets")
     p.add_argument("--cache", default=None, help="directory to keep generated matrices in between runs")
     return p.parse_args()
 
@@ -118,9 +120,9 @@ class Matrices:
 
 def describe(name):
     """(matrix key, kind, op is T, dense columns, alpha, beta, description) of a workload."""
-    if name.endswith("-alg1"):
+    if name.endswith("-alg2"):
         d = describe(name[:-5])
-        return d[:6] + (d[6] + ", MCSPARSE_SPMV_CSR_ALG1",)
+        return d[:6] + (d[6] + ", MCSPARSE_SPMV_CSR_ALG2 (reproducible bits)",)
     if name == "c1":
         return "laplacian", "spmv", False, 0, 1.0, 0.0, "fp32 CSR SpMV, 5-pt Laplacian 256x256"
     if name == "c2":
@@ -151,9 +153,9 @@ def run_workload(name, args, ctx, steps=None, warmup=None, with_cpu=True):
     """Measures one workload; returns the JSON object of its line."""
     torch, api, wl, handle, stream = ctx["torch"], ctx["api"], ctx["wl"], ctx["handle"], ctx["stream"]
     key, kind, op_t, n_cols, alpha, beta, desc = describe(name)
-    alg = api.SPMV_CSR_ALG1 if (args.alg1 or name.endswith("-alg1")) else api.SPMV_ALG_DEFAULT
-    if args.alg1 and not name.endswith("-alg1") and kind in ("spmv", "spmv-csc"):
-        desc += ", MCSPARSE_SPMV_CSR_ALG1"
+    alg = api.SPMV_CSR_ALG2 if (args.alg2 or name.endswith("-alg2")) else api.SPMV_ALG_DEFAULT
+    if args.alg2 and not name.endswith("-alg2") and kind in ("spmv", "spmv-csc"):
+        desc += ", MCSPARSE_SPMV_CSR_ALG2 (reproducible bits)"
     a = ctx["matrices"].get(key)
     op = api.OP_T if op_t else api.OP_N
     s = args.scale
@@ -316,7 +318,9 @@ def run_workload(name, args, ctx, steps=None, warmup=None, with_cpu=True):
     mat0 = sets[0].get("mat")
     plan = mat0.plan() if mat0 is not None and kind in ("spmv", "spmv-csc") else None
     banded = mat0.spmv_preprocess_state() if mat0 is not None and kind in ("spmv", "spmv-csc") else None
-    traffic = MEASURED_TRAFFIC.get((name, bool(banded and banded[0] == 2))) if s == 1.0 else None
+    copy_state = banded[0] if banded and banded[0] in (2, 3) else 0
+    base_name = name[:-5] if name.endswith("-alg2") else name
+    traffic = MEASURED_TRAFFIC.get((base_name, copy_state)) if s == 1.0 else None
 
     out = {
         "metric": "CSR SpMV/SpMM achieved HBM GB/s (% of MI355X peak) + GFLOP/s at 1 GPU",

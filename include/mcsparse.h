@@ -464,7 +464,17 @@ mcsparseStatus_t mcsparseSpMatGetSpMMSchedule(mcsparseSpMatDescr_t spMatDescr, i
  *   - Calls the layout cannot help (x fits in cache as it is, 64-bit indices, COO) are left to the
  *     ordinary kernels; the call still returns SUCCESS.  mcsparseSpMatGetSpMVPreprocess tells which
  *     case applies.
- *   - Results stay within the same bound as mcsparseSpMV's and are bit-reproducible from run to run.
+ *   - alg chooses between two layouts (the reference ignores alg; the meanings are those APIs of this
+ *     family give the values).  MCSPARSE_SPMV_CSR_ALG2, the algorithm that promises the same bits on
+ *     every run, builds the banded copy described above: row sums are formed in a fixed order.  Every
+ *     other value builds the copy with its tiles in column order: the lanes of a wavefront then read
+ *     neighbouring elements of x, and the products are added to the row sums in LDS in the order the
+ *     wavefronts reach them.  That is faster by a quarter to a third on the benchmark matrices and stays
+ *     within the same error bound, but the last bits can differ between two calls.  Its buffer is larger
+ *     (about seven times the matrix: the build sorts the nonzeros by column first); shapes it does not
+ *     fit (more than 64 bands of x) get the banded copy.
+ *   - mcsparseSpMV called with MCSPARSE_SPMV_CSR_ALG2 never uses a copy in column order: it runs the
+ *     ordinary kernels, whose results are reproducible.
  * The call blocks the host until the copy is built. */
 mcsparseStatus_t mcsparseSpMV_preprocess_bufferSize(mcsparseHandle_t handle, mcsparseOperation_t opA,
                                                     const void* alpha, mcsparseSpMatDescr_t matA,

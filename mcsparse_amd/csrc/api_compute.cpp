@@ -251,9 +251,10 @@ bool banded_candidate(const mcsparseSpMatDescr* A, mcsparseOperation_t op, mcspa
     const int64_t cols = v.transpose ? v.m : v.n;
     const size_t band_bytes = A->banded.band_bytes != 0 ? A->banded.band_bytes : mcsp::kBandedBandBytes;
     shape->by_column = false;
-    // MCSPARSE_SPMV_CSR_ALG1 is the algorithm that need not give the same bits on every run: tiles in
-    // column order with sums formed in LDS as the products arrive, where the shape allows it
-    if (alg == MCSPARSE_SPMV_CSR_ALG1 &&
+    // Only MCSPARSE_SPMV_CSR_ALG2 promises the same bits on every run (the meaning APIs of this family
+    // give the values; the reference ignores alg).  Every other algorithm gets the faster copy, tiles in
+    // column order with sums formed in LDS as the products arrive, where the shape allows it.
+    if (alg != MCSPARSE_SPMV_CSR_ALG2 &&
         mcsp::column_order_shape(static_cast<idx_t>(rows), static_cast<idx_t>(cols), static_cast<idx_t>(A->nnz),
                                  static_cast<idx_t>(A->idxBase), value_size(A->valueType), band_bytes, shape))
         return true;

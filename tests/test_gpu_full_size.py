@@ -36,6 +36,10 @@ def test_config3_power_law_full_size(torch_gpu, handle, oracle, power_law_full):
     # call runs them in another order: that cannot change a single bit of the result.
     st, y_again, _ = run_spmv(torch_gpu, handle, a, x, np.zeros(a.m, np.float32), 1.0, 0.0)
     assert st == 0 and np.array_equal(y_again.view(np.uint32), y.view(np.uint32))
+    # the copy in column order (MCSPARSE_SPMV_CSR_ALG1): 8 planes of partial sums, two 1 MiB bands each
+    state, bands, rows = run_banded(torch_gpu, handle, oracle, a, 1.0, 0.0, what="C3 op N, column order",
+                                    reference=(x, y_ref, bound), alg=api.SPMV_CSR_ALG1, expect_state=3, calls=2)
+    assert (bands, rows) == (8, 16384)
     # tiles in storage order are twice as long, which moves the seams between partial sums
     st, y_plain, _ = run_spmv(torch_gpu, handle, a, x, np.zeros(a.m, np.float32), 1.0, 0.0, family=api.FAMILY_MERGE)
     assert st == 0
@@ -80,6 +84,13 @@ def test_config2_full_size_banded(torch_gpu, handle, oracle):
     assert a.nnz == 16777216
     state, bands, rows = run_banded(torch_gpu, handle, oracle, a, 1.5, 0.5, calls=2, what="C2 banded")
     assert (state, bands) == (2, 4)
+
+
+def test_config2_full_size_column_order(torch_gpu, handle, oracle):
+    a = wl.uniform_rows(m=1 << 20, per_row=16, dtype=np.float64)
+    state, bands, rows = run_banded(torch_gpu, handle, oracle, a, 1.5, 0.5, calls=2, what="C2 column order",
+                                    alg=api.SPMV_CSR_ALG1, expect_state=3)
+    assert (bands, rows) == (4, 16384)
 
 
 @pytest.fixture(scope="module")

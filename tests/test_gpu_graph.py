@@ -116,3 +116,45 @@ def test_calls_replay_in_a_hip_graph(torch_gpu, oracle):
     del graph
     torch.cuda.synchronize()
     handle.destroy()
+
+
+@pytest.mark.parametrize("alg,state", [(api.SPMV_ALG_DEFAULT, 3), (api.SPMV_CSR_ALG2, 2)])
+def test_preprocessed_spmv_replays_in_a_hip_graph(torch_gpu, oracle, alg, state):
+    """mcsparseSpMV on a copy built by mcsparseSpMV_preprocess (before the capture: it blocks) is two kernels."""
+    torch = torch_gpu
+    rng = np.random.default_rng(22)
+    side = torch.cuda.Stream()
+    handle = api.Handle(stream=side.cuda_stream)
+    a = wl.random_ragged(20000, 40000, 10, dtype=np.float64, seed=9)
+    d_ptr, d_col, d_val = dev(torch, a.ptr), dev(torch, a.col), dev(torch, a.val)
+    A = api.SpMat(a.m, a.n, a.nnz, d_ptr, d_col, d_val, base=a.base)
+    A.set_band_bytes(1 << 16)
+    x = torch.zeros(a.n, dtype=torch.float64, device="cuda")
+    y = torch.zeros(a.m, dtype=torch.float64, device="cuda")
+    vx, vy = api.DnVec(x), api.DnVec(y)
+    st, size = api.spmv_preprocess_buffer_size(handle, api.OP_N, 1.5, A, vx, 0.5, vy, api.R_64F, alg=alg)
+    assert st == 0
+    buf = torch.empty(size, dtype=torch.uint8, device="cuda")
+    with torch.cuda.stream(side):
+        assert api.spmv_preprocess(handle, api.OP_N, 1.5, A, vx, 0.5, vy, api.R_64F, buf, alg=alg) == 0
+        assert api.spmv(handle, api.OP_N, 1.5, A, vx, 0.5, vy, api.R_64F, buf, alg=alg) == 0
+    torch.cuda.synchronize()
+    assert A.spmv_preprocess_state()[0] == state
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        # a preprocess call would have to block: refused on a capturing stream, the copy stays as it is
+        assert api.spmv(handle, api.OP_N, 1.5, A, vx, 0.5, vy, api.R_64F, buf, alg=alg) == 0
+    torch.cuda.synchronize()
+    for replay in range(3):
+        hx = rng.uniform(-1, 1, a.n)
+        hy = rng.uniform(-1, 1, a.m)
+        x.copy_(torch.from_numpy(hx))
+        y.copy_(torch.from_numpy(hy))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        ref, bound = oracle.spmv(False, a.m, a.n, a.base, a.ptr, a.col, a.val, 1.5, 0.5, hx, hy)
+        assert_within(y.cpu().numpy(), ref, bound, np.float64, what="replay %d, state %d" % (replay, state))
+    del graph
+    torch.cuda.synchronize()
+    handle.destroy()

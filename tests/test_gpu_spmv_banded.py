@@ -17,10 +17,12 @@ GOLDEN = sorted(glob.glob(os.path.join(os.path.dirname(__file__), "golden", "csr
 
 
 def run_banded(torch, handle, oracle, a, alpha, beta, band_bytes=0, seed=1, expect_state=2, what="", calls=1,
-               as_csc=False, reference=None):
+               as_csc=False, reference=None, alg=api.SPMV_CSR_ALG2):
     """as_csc: the arrays are handed over as the CSC of the n x m transpose and applied with op T.
     reference: (x, y_ref, bound) of a product the caller has already worked out with the oracle, for
-    beta == 0 (saves a second pass of the oracle over a large matrix)."""
+    beta == 0 (saves a second pass of the oracle over a large matrix).
+    alg: MCSPARSE_SPMV_CSR_ALG2 asks for the reproducible banded copy (state 2); the default algorithm and
+    MCSPARSE_SPMV_CSR_ALG1 get the copy in column order (state 3), whose sums need not repeat bit for bit."""
     rng = np.random.default_rng(seed)
     dt = a.val.dtype
     ct = api.maca_type(dt)
@@ -36,10 +38,10 @@ def run_banded(torch, handle, oracle, a, alpha, beta, band_bytes=0, seed=1, expe
     if band_bytes:
         mat.set_band_bytes(band_bytes)
     vx, vy = api.DnVec(d_x), api.DnVec(d_y)
-    st, size = api.spmv_preprocess_buffer_size(handle, op, alpha, mat, vx, beta, vy, ct)
+    st, size = api.spmv_preprocess_buffer_size(handle, op, alpha, mat, vx, beta, vy, ct, alg=alg)
     assert st == api.STATUS_SUCCESS
     buf = torch.empty(size, dtype=torch.uint8, device="cuda")
-    assert api.spmv_preprocess(handle, op, alpha, mat, vx, beta, vy, ct, buf) == api.STATUS_SUCCESS
+    assert api.spmv_preprocess(handle, op, alpha, mat, vx, beta, vy, ct, buf, alg=alg) == api.STATUS_SUCCESS
     state, bands, rows = mat.spmv_preprocess_state()
     assert state == expect_state, (state, bands, rows)
     if reference is None:
@@ -50,13 +52,13 @@ def run_banded(torch, handle, oracle, a, alpha, beta, band_bytes=0, seed=1, expe
     first = None
     for _ in range(calls):
         d_y.copy_(torch.from_numpy(y))
-        assert api.spmv(handle, op, alpha, mat, vx, beta, vy, ct, buf) == api.STATUS_SUCCESS
+        assert api.spmv(handle, op, alpha, mat, vx, beta, vy, ct, buf, alg=alg) == api.STATUS_SUCCESS
         torch.cuda.synchronize()
         got = d_y.cpu().numpy()
         assert_within(got, y_ref, bound, dt, what=what or "banded spmv")
         if first is None:
             first = got
-        else:  # fixed summation order: the same bits every time
+        elif state == 2:  # fixed summation order: the same bits every time
             assert np.array_equal(first.view(np.uint8), got.view(np.uint8))
     return state, bands, rows
 
@@ -77,10 +79,10 @@ def test_golden_fixtures_banded(torch_gpu, handle, path, base):
         mat = api.SpMat(a.m, a.n, a.nnz, d_ptr, d_col, d_val, base=base)
         mat.set_band_bytes(64)  # 16 or 8 columns per band: even these small fixtures are cut into several
         vx, vy = api.DnVec(d_x), api.DnVec(d_y)
-        st, size = api.spmv_preprocess_buffer_size(handle, api.OP_N, alpha, mat, vx, beta, vy, ct)
+        st, size = api.spmv_preprocess_buffer_size(handle, api.OP_N, alpha, mat, vx, beta, vy, ct, alg=api.SPMV_CSR_ALG2)
         assert st == api.STATUS_SUCCESS
         buf = torch.empty(size, dtype=torch.uint8, device="cuda")
-        assert api.spmv_preprocess(handle, api.OP_N, alpha, mat, vx, beta, vy, ct, buf) == api.STATUS_SUCCESS
+        assert api.spmv_preprocess(handle, api.OP_N, alpha, mat, vx, beta, vy, ct, buf, alg=api.SPMV_CSR_ALG2) == api.STATUS_SUCCESS
         assert api.spmv(handle, api.OP_N, alpha, mat, vx, beta, vy, ct, buf) == api.STATUS_SUCCESS
         torch.cuda.synchronize()
         assert np.array_equal(d_y.cpu().numpy().astype(np.float64), g["y_n"])
@@ -130,12 +132,12 @@ def test_transposing_directions_get_a_copy_of_the_transpose(torch_gpu, handle, o
         mat, op = api.SpMat(a.n, a.m, a.nnz, d_ptr, d_col, d_val, base=1, fmt=api.FORMAT_CSC), api.OP_N
     mat.set_band_bytes(4096)
     vx, vy = api.DnVec(d_x), api.DnVec(d_y)
-    st, size = api.spmv_preprocess_buffer_size(handle, op, 1.5, mat, vx, 0.5, vy, ct)
+    st, size = api.spmv_preprocess_buffer_size(handle, op, 1.5, mat, vx, 0.5, vy, ct, alg=api.SPMV_CSR_ALG2)
     assert st == api.STATUS_SUCCESS
     st2, plain = api.spmv_buffer_size(handle, op, 1.5, mat, vx, 0.5, vy, ct)
     assert size > plain
     buf = torch.empty(size, dtype=torch.uint8, device="cuda")
-    assert api.spmv_preprocess(handle, op, 1.5, mat, vx, 0.5, vy, ct, buf) == api.STATUS_SUCCESS
+    assert api.spmv_preprocess(handle, op, 1.5, mat, vx, 0.5, vy, ct, buf, alg=api.SPMV_CSR_ALG2) == api.STATUS_SUCCESS
     assert mat.spmv_preprocess_state()[0] == 2
     y_ref, bound = oracle.spmv(True, a.m, a.n, 1, a.ptr, a.col, a.val, 1.5, 0.5, x, y0)
     for _ in range(2):
@@ -194,9 +196,9 @@ def test_copy_is_dropped_with_the_arrays(torch_gpu, handle, oracle):
     mat = api.SpMat(a.m, a.n, a.nnz, d_ptr, d_col, d_val)
     mat.set_band_bytes(8192)
     vx, vy = api.DnVec(d_x), api.DnVec(d_y)
-    st, size = api.spmv_preprocess_buffer_size(handle, api.OP_N, 1.0, mat, vx, 0.0, vy, api.R_32F)
+    st, size = api.spmv_preprocess_buffer_size(handle, api.OP_N, 1.0, mat, vx, 0.0, vy, api.R_32F, alg=api.SPMV_CSR_ALG2)
     buf = torch.empty(size, dtype=torch.uint8, device="cuda")
-    assert api.spmv_preprocess(handle, api.OP_N, 1.0, mat, vx, 0.0, vy, api.R_32F, buf) == api.STATUS_SUCCESS
+    assert api.spmv_preprocess(handle, api.OP_N, 1.0, mat, vx, 0.0, vy, api.R_32F, buf, alg=api.SPMV_CSR_ALG2) == api.STATUS_SUCCESS
     assert mat.spmv_preprocess_state()[0] == 2
     # new values through the descriptor: the copy (which holds the old ones) must not be used
     new_val = rng.uniform(-1, 1, a.nnz).astype(np.float32)
@@ -219,9 +221,9 @@ def test_overwritten_buffer_stays_in_bounds(torch_gpu, handle, oracle):
     mat = api.SpMat(a.m, a.n, a.nnz, d_ptr, d_col, d_val)
     mat.set_band_bytes(1 << 14)
     vx, vy = api.DnVec(d_x), api.DnVec(d_y)
-    st, size = api.spmv_preprocess_buffer_size(handle, api.OP_N, 1.0, mat, vx, 0.0, vy, api.R_64F)
+    st, size = api.spmv_preprocess_buffer_size(handle, api.OP_N, 1.0, mat, vx, 0.0, vy, api.R_64F, alg=api.SPMV_CSR_ALG2)
     buf = torch.empty(size, dtype=torch.uint8, device="cuda")
-    assert api.spmv_preprocess(handle, api.OP_N, 1.0, mat, vx, 0.0, vy, api.R_64F, buf) == api.STATUS_SUCCESS
+    assert api.spmv_preprocess(handle, api.OP_N, 1.0, mat, vx, 0.0, vy, api.R_64F, buf, alg=api.SPMV_CSR_ALG2) == api.STATUS_SUCCESS
     buf.fill_(0xFF)
     assert api.spmv(handle, api.OP_N, 1.0, mat, vx, 0.0, vy, api.R_64F, buf) == api.STATUS_SUCCESS
     torch.cuda.synchronize()

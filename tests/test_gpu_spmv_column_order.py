@@ -1,5 +1,5 @@
-"""GPU parity of the SpMV copy whose tiles are in column order (mcsparseSpMV_preprocess with
-MCSPARSE_SPMV_CSR_ALG1): products meet in LDS in the order the wavefronts reach them, so results are
+"""GPU parity of the SpMV copy whose tiles are in column order (mcsparseSpMV_preprocess with any algorithm
+but MCSPARSE_SPMV_CSR_ALG2): products meet in LDS in the order the wavefronts reach them, so results are
 within the tolerance of every other family but not bitwise reproducible."""
 import glob
 import os
@@ -112,6 +112,31 @@ def test_alg2_does_not_use_the_copy(torch_gpu, handle, oracle):
     """MCSPARSE_SPMV_CSR_ALG2 promises the same bits on every run: the call runs the row kernels."""
     a = wl.uniform_rows(m=20000, n=300000, per_row=8, dtype=np.float64, config_id=91)
     run(torch_gpu, handle, oracle, a, 1.0, 0.0, call_alg=api.SPMV_CSR_ALG2)
+
+
+def test_default_algorithm_gets_the_copy_in_column_order(torch_gpu, handle, oracle):
+    torch = torch_gpu
+    a = wl.uniform_rows(m=30000, n=400000, per_row=8, dtype=np.float64, config_id=93)
+    rng = np.random.default_rng(9)
+    x = rng.uniform(-1, 1, a.n)
+    d_ptr, d_col, d_val, d_x = (dev(torch, v) for v in (a.ptr, a.col, a.val, x))
+    d_y = torch.zeros(a.m, dtype=torch.float64, device="cuda")
+    mat = api.SpMat(a.m, a.n, a.nnz, d_ptr, d_col, d_val)
+    vx, vy = api.DnVec(d_x), api.DnVec(d_y)
+    sizes = {}
+    for alg in (api.SPMV_ALG_DEFAULT, api.SPMV_CSR_ALG1, api.SPMV_CSR_ALG2):
+        st, sizes[alg] = api.spmv_preprocess_buffer_size(handle, api.OP_N, 1.0, mat, vx, 0.0, vy, api.R_64F, alg=alg)
+        assert st == api.STATUS_SUCCESS
+    assert sizes[api.SPMV_ALG_DEFAULT] == sizes[api.SPMV_CSR_ALG1] > sizes[api.SPMV_CSR_ALG2]
+    buf = torch.empty(sizes[api.SPMV_ALG_DEFAULT], dtype=torch.uint8, device="cuda")
+    y_ref, bound = oracle.spmv(False, a.m, a.n, 0, a.ptr, a.col, a.val, 1.0, 0.0, x, None)
+    for alg, state in ((api.SPMV_ALG_DEFAULT, 3), (api.SPMV_CSR_ALG2, 2), (api.SPMV_CSR_ALG1, 3)):
+        assert api.spmv_preprocess(handle, api.OP_N, 1.0, mat, vx, 0.0, vy, api.R_64F, buf, alg=alg) == api.STATUS_SUCCESS
+        assert mat.spmv_preprocess_state()[0] == state
+        d_y.zero_()
+        assert api.spmv(handle, api.OP_N, 1.0, mat, vx, 0.0, vy, api.R_64F, buf) == api.STATUS_SUCCESS
+        torch.cuda.synchronize()
+        assert_within(d_y.cpu().numpy(), y_ref, bound, np.float64, what="alg %d" % alg)
 
 
 def test_wide_matrix_falls_back_to_the_banded_copy(torch_gpu, handle, oracle):
