@@ -52,6 +52,10 @@ MEASURED_TRAFFIC = {
     ("c3t", 2): (_traffic(481300.5 + 65544.8, 131206.2 + 16384.0), "profiles/spmv_banded_f32_c3_powerlaw.txt"),
     ("c5-spmv", 2): (_traffic(481330.8 + 65544.6, 131202.3 + 16384.0),
                         "profiles/spmv_banded_f32_c3_powerlaw.txt"),
+    # spmv_column_order_kernel + banded_reduce_kernel
+    ("c2", 3): (_traffic(120656.3 + 20579.5, 32768.0 + 8192.0), "profiles/spmv_column_order_f64_c2_1Mx16.txt"),
+    ("c3", 3): (_traffic(577677.6 + 65548.9, 131072.0 + 16384.0), "profiles/spmv_column_order_f32_c3_powerlaw.txt"),
+    ("c3t", 3): (_traffic(601553.7 + 65548.9, 131072.0 + 16384.0), "profiles/spmv_column_order_f32_c3_powerlaw.txt"),
     # without the preprocess call: vector kernel; merge kernel (tiles in column order) + partition
     # + tile order + fix-up
     ("c2", 0): (_traffic(653904.5, 10047.2), "profiles/spmv_vector_f64_c2_1Mx16.txt"),
