@@ -266,9 +266,11 @@ struct BandedLayout {
     // by_column only: the nonzeros sorted by column (the source of the build) and the sorted tile numbers
     size_t src_cols, src_rows, src_vals, tile_ids;
 };
-// The same decision for the copy whose tiles are in column order (BandedShape::by_column): tall tiles of
-// up to kColumnOrderRows rows, at most 64 bands and 65536 tiles.
+// The same decision for the copy whose tiles are in column order (BandedShape::by_column): tiles of
+// kColumnOrderMinRows .. kColumnOrderRows rows, at most 64 planes of partial sums and 65536 tiles, and at
+// least one unit of work per compute unit.
 constexpr uint32_t kColumnOrderRows = 16384;
+constexpr uint32_t kColumnOrderMinRows = 2048;
 bool column_order_shape(idx_t m, idx_t n, idx_t nnz, idx_t base, size_t value_bytes, size_t band_bytes,
                         BandedShape* out);
 // r_keys / c_keys: row + base and column + base of every nonzero of the matrix to copy, in an order

@@ -434,18 +434,26 @@ bool banded_shape(idx_t m, idx_t n, idx_t nnz, idx_t base, size_t value_bytes, s
 bool column_order_shape(idx_t m, idx_t n, idx_t nnz, idx_t base, size_t value_bytes, size_t band_bytes,
                         BandedShape* out) {
     if (m == 0 || n == 0 || nnz == 0 || (value_bytes != 4 && value_bytes != 8)) return false;
-    uint32_t rows_per_tile = 64;
-    while (rows_per_tile < kColumnOrderRows && rows_per_tile < m) rows_per_tile *= 2;
-    const uint32_t row_bits = bit_length(rows_per_tile - 1);
     uint32_t wanted = 0;  // log2 of the keys in band_bytes of x
     while ((static_cast<size_t>(value_bytes) << (wanted + 1)) <= band_bytes) ++wanted;
+    const uint64_t max_key = static_cast<uint64_t>(n) - 1 + base;
+    const uint64_t groups = (max_key >> wanted) + 1;  // planes of partial sums: every one costs a sum per row
+    if (groups > 64) return false;
+    // The taller a tile, the more of its entries share a line of x; but the kernel runs one workgroup per
+    // compute unit, so there must be a unit of work for each: the tiles are halved until there is, and a
+    // matrix too small for that is left to the other kernels.
+    constexpr uint64_t kUnitsWanted = kXcds * kColumnGroupsPerXcd;
+    uint32_t rows_per_tile = kColumnOrderRows;
+    while (rows_per_tile > kColumnOrderMinRows &&
+           groups * ((static_cast<uint64_t>(m) + rows_per_tile - 1) / rows_per_tile) < kUnitsWanted)
+        rows_per_tile /= 2;
+    const uint64_t chunks = (static_cast<uint64_t>(m) + rows_per_tile - 1) / rows_per_tile;
+    if (groups * chunks < kUnitsWanted) return false;
+    const uint32_t row_bits = bit_length(rows_per_tile - 1);
     const uint32_t shift = wanted > 32 - row_bits ? 32 - row_bits : wanted;
     const uint32_t sub = 1u << (wanted - shift);  // bands that share a plane of partial sums
-    const uint64_t max_key = static_cast<uint64_t>(n) - 1 + base;
-    const uint64_t groups = (max_key >> wanted) + 1;
-    const uint64_t chunks = (static_cast<uint64_t>(m) + rows_per_tile - 1) / rows_per_tile;
-    // every group costs a partial sum per row; the tile numbers are sorted in at most two passes
-    if (groups > 64 || sub > 64 || groups * chunks * sub > 65536) return false;
+    // the tile numbers are sorted in at most two passes of eight bits
+    if (sub > 64 || groups * chunks * sub > 65536) return false;
     out->band_shift = shift;
     out->band_bits = bit_length(static_cast<uint32_t>(groups * sub - 1));
     out->bands = static_cast<uint32_t>(groups);

@@ -128,7 +128,7 @@ def test_preprocessed_spmv_replays_in_a_hip_graph(torch_gpu, oracle, alg, state)
     a = wl.random_ragged(20000, 40000, 10, dtype=np.float64, seed=9)
     d_ptr, d_col, d_val = dev(torch, a.ptr), dev(torch, a.col), dev(torch, a.val)
     A = api.SpMat(a.m, a.n, a.nnz, d_ptr, d_col, d_val, base=a.base)
-    A.set_band_bytes(1 << 16)
+    A.set_band_bytes(1 << 13)
     x = torch.zeros(a.n, dtype=torch.float64, device="cuda")
     y = torch.zeros(a.m, dtype=torch.float64, device="cuda")
     vx, vy = api.DnVec(x), api.DnVec(y)

@@ -1,9 +1,6 @@
 """GPU parity of the SpMV copy whose tiles are in column order (mcsparseSpMV_preprocess with any algorithm
 but MCSPARSE_SPMV_CSR_ALG2): products meet in LDS in the order the wavefronts reach them, so results are
 within the tolerance of every other family but not bitwise reproducible."""
-import glob
-import os
-
 import numpy as np
 import pytest
 
@@ -13,8 +10,6 @@ from mcsparse_amd import workloads as wl
 from gpu_util import assert_within, dev
 
 pytestmark = pytest.mark.gpu
-
-GOLDEN = sorted(glob.glob(os.path.join(os.path.dirname(__file__), "golden", "csr_*.npz")))
 
 
 def run(torch, handle, oracle, a, alpha, beta, op=api.OP_N, fmt=api.FORMAT_CSR, band_bytes=0, seed=1, expect_state=3,
@@ -50,68 +45,73 @@ def run(torch, handle, oracle, a, alpha, beta, op=api.OP_N, fmt=api.FORMAT_CSR, 
     return state, bands, rows, mat, buf
 
 
-@pytest.mark.parametrize("path", GOLDEN, ids=[os.path.basename(p)[:-4] for p in GOLDEN])
-@pytest.mark.parametrize("base", [0, 1])
-def test_golden_fixtures_column_order(torch_gpu, handle, path, base):
-    """Integer-valued fixtures: every summation order is exact, so the result must equal the fixture's."""
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_integer_valued_product_is_exact(torch_gpu, handle, oracle, dtype):
+    """Small integers: every summation order is exact, so the result must equal the oracle's bit for bit."""
     torch = torch_gpu
-    with np.load(path) as z:
-        g = {k: z[k] for k in z.files}
-    for dt in (np.float32, np.float64):
-        a = wl.Csr(int(g["m"]), int(g["n"]), g["ptr"], g["col"], g["val"].astype(dt)).with_base(base)
-        ct = api.maca_type(dt)
-        alpha, beta = float(g["alpha"]), float(g["beta"])
-        d_ptr, d_col, d_val, d_x, d_y = (dev(torch, v) for v in (a.ptr, a.col, a.val, g["x"].astype(dt),
-                                                                   g["y0"].astype(dt)))
-        mat = api.SpMat(a.m, a.n, a.nnz, d_ptr, d_col, d_val, base=base)
-        mat.set_band_bytes(64)
-        vx, vy = api.DnVec(d_x), api.DnVec(d_y)
-        st, size = api.spmv_preprocess_buffer_size(handle, api.OP_N, alpha, mat, vx, beta, vy, ct,
-                                                   alg=api.SPMV_CSR_ALG1)
-        assert st == api.STATUS_SUCCESS
-        buf = torch.empty(size, dtype=torch.uint8, device="cuda")
-        assert api.spmv_preprocess(handle, api.OP_N, alpha, mat, vx, beta, vy, ct, buf,
-                                   alg=api.SPMV_CSR_ALG1) == api.STATUS_SUCCESS
-        assert mat.spmv_preprocess_state()[0] in (2, 3)  # very wide fixtures need more than 64 such bands
-        assert api.spmv(handle, api.OP_N, alpha, mat, vx, beta, vy, ct, buf, alg=api.SPMV_CSR_ALG1) == api.STATUS_SUCCESS
-        torch.cuda.synchronize()
-        assert np.array_equal(d_y.cpu().numpy().astype(np.float64), g["y_n"])
+    a = wl.random_ragged(70001, 30011, 9, dtype=dtype, seed=4)
+    rng = np.random.default_rng(4)
+    a = wl.Csr(a.m, a.n, a.ptr, a.col, rng.integers(-8, 9, a.nnz).astype(dtype), a.base)
+    x = rng.integers(-8, 9, a.n).astype(dtype)
+    y = rng.integers(-8, 9, a.m).astype(dtype)
+    d_ptr, d_col, d_val, d_x, d_y = (dev(torch, v) for v in (a.ptr, a.col, a.val, x, y))
+    mat = api.SpMat(a.m, a.n, a.nnz, d_ptr, d_col, d_val)
+    mat.set_band_bytes(1 << 12)
+    vx, vy = api.DnVec(d_x), api.DnVec(d_y)
+    ct = api.maca_type(dtype)
+    st, size = api.spmv_preprocess_buffer_size(handle, api.OP_N, 2.0, mat, vx, -1.0, vy, ct)
+    assert st == api.STATUS_SUCCESS
+    buf = torch.empty(size, dtype=torch.uint8, device="cuda")
+    assert api.spmv_preprocess(handle, api.OP_N, 2.0, mat, vx, -1.0, vy, ct, buf) == api.STATUS_SUCCESS
+    assert mat.spmv_preprocess_state()[0] == 3
+    assert api.spmv(handle, api.OP_N, 2.0, mat, vx, -1.0, vy, ct, buf) == api.STATUS_SUCCESS
+    torch.cuda.synchronize()
+    y_ref, _ = oracle.spmv(False, a.m, a.n, a.base, a.ptr, a.col, a.val, 2.0, -1.0, x, y)
+    assert np.array_equal(d_y.cpu().numpy().astype(np.float64), np.asarray(y_ref, dtype=np.float64))
 
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
 @pytest.mark.parametrize("base", [0, 1])
 def test_ragged_rows_several_chunks_and_bands(torch_gpu, handle, oracle, dtype, base):
-    # three row chunks of 16384, empty rows, several bands, tiles without entries
-    a = wl.random_ragged(40003, 30011, 9, dtype=dtype, seed=5, base=base)
-    state, bands, rows, _, _ = run(torch_gpu, handle, oracle, a, -0.75, 1.25, band_bytes=1 << 14)
-    assert rows == 16384 and bands >= 2
-    run(torch_gpu, handle, oracle, a, 2.0, 0.0)  # default band width
+    # nine row chunks of 16384, empty rows, 30 or 59 planes of partial sums, tiles without entries
+    a = wl.random_ragged(140003, 30011, 9, dtype=dtype, seed=5, base=base)
+    state, bands, rows, _, _ = run(torch_gpu, handle, oracle, a, -0.75, 1.25, band_bytes=1 << 12)
+    assert rows == 16384 and bands >= 30
+
+
+def test_tiles_are_halved_until_every_compute_unit_has_one(torch_gpu, handle, oracle):
+    # two planes of the default width: 16384-row tiles would give 74 units for 256 compute units
+    a = wl.uniform_rows(m=600000, n=300000, per_row=5, dtype=np.float64, config_id=94)
+    state, bands, rows, _, _ = run(torch_gpu, handle, oracle, a, 2.0, 0.0)
+    assert (bands, rows) == (2, 4096)
 
 
 @pytest.mark.parametrize("fmt,op", [(api.FORMAT_CSR, api.OP_T), (api.FORMAT_CSC, api.OP_N), (api.FORMAT_CSC, api.OP_T)])
 def test_other_directions(torch_gpu, handle, oracle, fmt, op):
-    a = wl.random_ragged(20001, 35011, 11, dtype=np.float64, seed=6, base=1)
-    run(torch_gpu, handle, oracle, a, 1.5, 0.5, op=op, fmt=fmt, band_bytes=1 << 15)
+    a = wl.random_ragged(60001, 90011, 11, dtype=np.float64, seed=6, base=1)
+    run(torch_gpu, handle, oracle, a, 1.5, 0.5, op=op, fmt=fmt, band_bytes=1 << 14)
 
 
-def test_small_matrix_one_band(torch_gpu, handle, oracle):
+def test_small_matrix_is_left_to_the_row_kernels(torch_gpu, handle, oracle):
+    # fewer units of work than compute units: no copy in column order, and x fits one band: no banded copy
     a = wl.random_ragged(300, 200, 7, dtype=np.float32, seed=7)
-    state, bands, rows, _, _ = run(torch_gpu, handle, oracle, a, 1.0, 0.0)
-    assert bands == 1 and rows == 512
+    run(torch_gpu, handle, oracle, a, 1.0, 0.0, expect_state=0)
+    b = wl.laplacian_5pt(256, dtype=np.float32)
+    run(torch_gpu, handle, oracle, b, 1.0, 0.0, expect_state=0)
 
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
 def test_long_rows(torch_gpu, handle, oracle, dtype):
     # thousands of products of one row meet in one accumulator
     a = wl.power_law(m=1 << 15, n=1 << 20, max_len=20000, dtype=dtype)
-    run(torch_gpu, handle, oracle, a, 1.0, 0.0)
-    run(torch_gpu, handle, oracle, a, -1.5, 0.5, op=api.OP_T)
+    run(torch_gpu, handle, oracle, a, 1.0, 0.0, band_bytes=1 << 17)
+    run(torch_gpu, handle, oracle, a, -1.5, 0.5, op=api.OP_T, band_bytes=1 << 17)
 
 
 def test_alg2_does_not_use_the_copy(torch_gpu, handle, oracle):
     """MCSPARSE_SPMV_CSR_ALG2 promises the same bits on every run: the call runs the row kernels."""
     a = wl.uniform_rows(m=20000, n=300000, per_row=8, dtype=np.float64, config_id=91)
-    run(torch_gpu, handle, oracle, a, 1.0, 0.0, call_alg=api.SPMV_CSR_ALG2)
+    run(torch_gpu, handle, oracle, a, 1.0, 0.0, call_alg=api.SPMV_CSR_ALG2, band_bytes=1 << 16)
 
 
 def test_default_algorithm_gets_the_copy_in_column_order(torch_gpu, handle, oracle):
@@ -122,6 +122,7 @@ def test_default_algorithm_gets_the_copy_in_column_order(torch_gpu, handle, orac
     d_ptr, d_col, d_val, d_x = (dev(torch, v) for v in (a.ptr, a.col, a.val, x))
     d_y = torch.zeros(a.m, dtype=torch.float64, device="cuda")
     mat = api.SpMat(a.m, a.n, a.nnz, d_ptr, d_col, d_val)
+    mat.set_band_bytes(1 << 16)
     vx, vy = api.DnVec(d_x), api.DnVec(d_y)
     sizes = {}
     for alg in (api.SPMV_ALG_DEFAULT, api.SPMV_CSR_ALG1, api.SPMV_CSR_ALG2):
@@ -148,13 +149,12 @@ def test_wide_matrix_falls_back_to_the_banded_copy(torch_gpu, handle, oracle):
 def test_overwritten_copy_stays_in_bounds(torch_gpu, handle, oracle):
     torch = torch_gpu
     a = wl.uniform_rows(m=40000, n=100000, per_row=8, dtype=np.float32, config_id=92)
-    state, bands, rows, mat, buf = run(torch, handle, oracle, a, 1.0, 0.0, band_bytes=1 << 16)
+    run(torch, handle, oracle, a, 1.0, 0.0, band_bytes=1 << 14)
     x = torch.rand(a.n, dtype=torch.float32, device="cuda")
     y = torch.zeros(a.m, dtype=torch.float32, device="cuda")
-    # run() has dropped its descriptor's arrays; build a fresh one on live arrays and clobber its buffer
     d_ptr, d_col, d_val = (dev(torch, v) for v in (a.ptr, a.col, a.val))
     mat = api.SpMat(a.m, a.n, a.nnz, d_ptr, d_col, d_val)
-    mat.set_band_bytes(1 << 16)
+    mat.set_band_bytes(1 << 14)
     vx, vy = api.DnVec(x), api.DnVec(y)
     st, size = api.spmv_preprocess_buffer_size(handle, api.OP_N, 1.0, mat, vx, 0.0, vy, api.R_32F, alg=api.SPMV_CSR_ALG1)
     buf = torch.empty(size, dtype=torch.uint8, device="cuda")
