@@ -167,3 +167,46 @@ def test_overwritten_copy_stays_in_bounds(torch_gpu, handle, oracle):
             buf.fill_(fill)
         assert api.spmv(handle, api.OP_N, 1.0, mat, vx, 0.0, vy, api.R_32F, buf, alg=api.SPMV_CSR_ALG1) == 0
         torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("seed", [31, 32, 33, 34])
+def test_random_shapes(torch_gpu, handle, oracle, seed):
+    """Shapes drawn around the cuts the layout makes: tile heights 2048..16384, one to 64 planes, band groups of
+    one and two bands, all four (format, op) pairs; whatever copy the library decides on, the product is right."""
+    r = np.random.default_rng(seed)
+    seen = set()
+    for case in range(6):
+        dtype = [np.float32, np.float64][int(r.integers(0, 2))]
+        m = int(r.choice([9000, 20000, 33000, 70000, 150000]))
+        n = int(r.choice([5000, 40000, 262144, 300001]))
+        mean = int(r.choice([3, 9, 20]))
+        band_bytes = int(r.choice([1 << 12, 1 << 14, 1 << 16, 1 << 20, 0]))
+        a = wl.random_ragged(m, n, mean, dtype=dtype, seed=seed * 100 + case, base=int(r.integers(0, 2)))
+        fmt, op = [(api.FORMAT_CSR, api.OP_N), (api.FORMAT_CSR, api.OP_T), (api.FORMAT_CSC, api.OP_N),
+                   (api.FORMAT_CSC, api.OP_T)][int(r.integers(0, 4))]
+        alpha, beta = [(1.0, 0.0), (-1.5, 0.75), (2.0, 1.0)][int(r.integers(0, 3))]
+        what = "seed %d case %d: %d x %d, mean %d, %s, band %d, fmt %d op %d" % (
+            seed, case, m, n, mean, np.dtype(dtype).name, band_bytes, fmt, op)
+        rng = np.random.default_rng(seed)
+        transposed = (fmt == api.FORMAT_CSR) == (op == api.OP_T)
+        x = rng.uniform(-1, 1, a.m if transposed else a.n).astype(dtype)
+        y = rng.uniform(-1, 1, a.n if transposed else a.m).astype(dtype)
+        d_ptr, d_col, d_val, d_x, d_y = (dev(torch_gpu, v) for v in (a.ptr, a.col, a.val, x, y))
+        if fmt == api.FORMAT_CSR:
+            mat = api.SpMat(a.m, a.n, a.nnz, d_ptr, d_col, d_val, base=a.base)
+        else:
+            mat = api.SpMat(a.n, a.m, a.nnz, d_ptr, d_col, d_val, base=a.base, fmt=api.FORMAT_CSC)
+        if band_bytes:
+            mat.set_band_bytes(band_bytes)
+        vx, vy = api.DnVec(d_x), api.DnVec(d_y)
+        ct = api.maca_type(dtype)
+        st, size = api.spmv_preprocess_buffer_size(handle, op, alpha, mat, vx, beta, vy, ct)
+        assert st == api.STATUS_SUCCESS, what
+        buf = torch_gpu.empty(size, dtype=torch_gpu.uint8, device="cuda")
+        assert api.spmv_preprocess(handle, op, alpha, mat, vx, beta, vy, ct, buf) == api.STATUS_SUCCESS, what
+        seen.add(mat.spmv_preprocess_state()[0])
+        assert api.spmv(handle, op, alpha, mat, vx, beta, vy, ct, buf) == api.STATUS_SUCCESS, what
+        torch_gpu.cuda.synchronize()
+        y_ref, bound = oracle.spmv(transposed, a.m, a.n, a.base, a.ptr, a.col, a.val, alpha, beta, x, y)
+        assert_within(d_y.cpu().numpy(), y_ref, bound, dtype, what=what)
+    assert 3 in seen, seen
