@@ -56,6 +56,8 @@ MEASURED_TRAFFIC = {
     ("c2", 3): (_traffic(120656.3 + 20579.5, 32768.0 + 8192.0), "profiles/spmv_column_order_f64_c2_1Mx16.txt"),
     ("c3", 3): (_traffic(577677.6 + 65548.9, 131072.0 + 16384.0), "profiles/spmv_column_order_f32_c3_powerlaw.txt"),
     ("c3t", 3): (_traffic(601553.7 + 65548.9, 131072.0 + 16384.0), "profiles/spmv_column_order_f32_c3_powerlaw.txt"),
+    ("c5-spmv", 3): (_traffic(601424.1 + 65548.9, 131072.0 + 16384.0),
+                     "profiles/spmv_column_order_f32_c3_powerlaw.txt"),
     # without the preprocess call: vector kernel; merge kernel (tiles in column order) + partition
     # + tile order + fix-up
     ("c2", 0): (_traffic(653904.5, 10047.2), "profiles/spmv_vector_f64_c2_1Mx16.txt"),
@@ -443,14 +445,18 @@ def gather_probe(torch, api, handle, args):
     """x_val[i] = y[x_ind[i]] for as many uniformly random indices as c2 has nonzeros, from a table
     the size of c2's x, from one band of the banded layout (2 MiB) and from one that fits every L2:
     the cost of the gathers of a random-column SpMV with everything else (row offsets, values, sums)
-    taken away.  mcsparseDgthr runs eight independent gathers per thread, like the SpMV kernels."""
+    taken away.  mcsparseDgthr runs eight independent gathers per thread, like the SpMV kernels.
+    Second part: the same gathers from the 2 MiB table with the indices sorted inside blocks, so that
+    a block holds 1, 4, 16 indices per 128-byte line (what sorting a tile by column does to an SpMV)."""
     count = 1 << 24
     steps = args.steps or 20
     rng = np.random.default_rng(7)
-    out = {"workload": "gather-probe", "gathers": count, "element_bytes": 8, "steps": steps, "tables": []}
+    out = {"workload": "gather-probe", "gathers": count, "element_bytes": 8, "steps": steps, "tables": [],
+           "sorted_blocks": []}
     stream = torch.cuda.current_stream()
-    for table_elems in (1 << 17, 1 << 18, 1 << 20):
-        ind = torch.from_numpy(rng.integers(0, table_elems, count, dtype=np.int32)).cuda()
+
+    def measure(ind_host, table_elems):
+        ind = torch.from_numpy(ind_host).cuda()
         table = torch.rand(table_elems, dtype=torch.float64, device="cuda")
         dst = torch.zeros(count, dtype=torch.float64, device="cuda")
         for _ in range(3):
@@ -461,10 +467,19 @@ def gather_probe(torch, api, handle, args):
             api.check(api.gthr(handle, count, table, dst, ind, 0))
         e1.record(stream)
         torch.cuda.synchronize()
-        us = e0.elapsed_time(e1) * 1e3 / steps
+        return e0.elapsed_time(e1) * 1e3 / steps
+
+    for table_elems in (1 << 17, 1 << 18, 1 << 20):
+        us = measure(rng.integers(0, table_elems, count, dtype=np.int32), table_elems)
         out["tables"].append({"table_MB": table_elems * 8 / 1e6, "us_per_call": round(us, 1),
                               "gathers_per_us": round(count / us, 1),
                               "streamed_bytes_per_call": count * (4 + 8)})
+    table_elems = 1 << 18
+    ind = rng.integers(0, table_elems, count, dtype=np.int32)
+    for block in (1 << 14, 1 << 16, 1 << 18, count):
+        us = measure(np.sort(ind.reshape(-1, block), axis=1).reshape(-1), table_elems)
+        out["sorted_blocks"].append({"table_MB": table_elems * 8 / 1e6, "block": block,
+                                     "indices_per_line": block * 16 / table_elems, "us_per_call": round(us, 1)})
     print(json.dumps(out))
     return 0
 
