@@ -265,6 +265,7 @@ struct BandedLayout {
     size_t tile_ptr, xcd_start, entries, vals, partials, keep, tmp_keys, tmp_rows, sort_ws, total;
     // by_column only: the nonzeros sorted by column (the source of the build) and the sorted tile numbers
     size_t src_cols, src_rows, src_vals, tile_ids;
+    size_t next_unit;  // by_column: one work counter per XCD
 };
 // The same decision for the copy whose tiles are in column order (BandedShape::by_column): tiles of
 // kColumnOrderMinRows .. kColumnOrderRows rows, at most 64 planes of partial sums and 65536 tiles, and at

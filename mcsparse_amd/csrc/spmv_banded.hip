@@ -35,6 +35,7 @@ constexpr int kIpt = 16;
 constexpr int kSlab = kBlock * kIpt;  // entries a workgroup stages at a time
 constexpr int kRowsPerThread = kBandedMaxRowsPerTile / kBlock;
 constexpr uint32_t kXcds = 8;  // accelerator complex dies of an MI355X; workgroup i runs on XCD i % 8
+constexpr uint32_t kColumnGroupsPerXcd = 32;  // workgroups per XCD of the kernel on tiles in column order: one per CU
 static_assert(kBandedMaxRowsPerTile % kBlock == 0, "rows of a tile are dealt to the threads in rounds");
 static_assert(kSlab <= 65536 && kBandedMaxRowsPerTile <= 65536, "16-bit positions in LDS");
 
@@ -237,9 +238,12 @@ __global__ __launch_bounds__(kBlock) void spmv_banded_kernel(idx_t m, idx_t n, i
 }
 
 // y[r] = beta*y[r] + alpha * (partials[0][r] + partials[1][r] + ...), the bands in order.
+// next_unit (may be null): the work counters of spmv_column_order_kernel, put back to their start for the next call.
 template <typename T, bool BETA0>
 __global__ __launch_bounds__(kBlock) void banded_reduce_kernel(idx_t m, uint32_t bands, const T* __restrict__ partials,
-                                                               T* __restrict__ y, T alpha, T beta) {
+                                                               T* __restrict__ y, T alpha, T beta,
+                                                               uint32_t* __restrict__ next_unit) {
+    if (next_unit != nullptr && blockIdx.x == 0 && threadIdx.x < kXcds) next_unit[threadIdx.x] = kColumnGroupsPerXcd;
     const uint64_t r = static_cast<uint64_t>(blockIdx.x) * kBlock + threadIdx.x;
     if (r >= m) return;
     constexpr uint32_t kAhead = 8;
@@ -297,7 +301,6 @@ __global__ __launch_bounds__(kBlock) void column_order_pack_kernel(idx_t nnz, id
 // chip); a thread has kColumnIpt gathers in flight (4, 8, 16 measured: 16 is 1-4 % ahead).
 constexpr int kColumnBlock = 1024;
 constexpr int kColumnIpt = 16;
-constexpr uint32_t kColumnGroupsPerXcd = 32;
 
 // xcd_start for the kernel below, in units.  A stretch is dealt to the kColumnGroupsPerXcd workgroups of
 // its XCD in turns, so what counts is the largest number of nonzeros any one workgroup ends up with.
@@ -306,11 +309,13 @@ constexpr uint32_t kColumnGroupsPerXcd = 32;
 // share), and the better one is kept.
 __global__ __launch_bounds__(kBlock) void column_order_split_kernel(idx_t nnz, uint32_t units, uint32_t sub,
                                                                     const idx_t* __restrict__ tile_ptr,
-                                                                    uint32_t* __restrict__ xcd_start) {
+                                                                    uint32_t* __restrict__ xcd_start,
+                                                                    uint32_t* __restrict__ next_unit) {
     static_assert(kBlock == kXcds * kColumnGroupsPerXcd, "one thread per workgroup of the SpMV kernel");
     __shared__ uint32_t s_start[2][kXcds + 1];
     __shared__ unsigned long long s_worst[2];
     const uint32_t tid = threadIdx.x;
+    if (tid < kXcds) next_unit[tid] = kColumnGroupsPerXcd;  // the work counters of the SpMV kernel: see there
     if (tid <= kXcds) {
         const uint64_t target = static_cast<uint64_t>(nnz) * tid / kXcds;
         uint32_t lo = 0, hi = units;  // first unit whose offset is >= target
@@ -339,12 +344,14 @@ __global__ __launch_bounds__(kColumnBlock) void spmv_column_order_kernel(idx_t m
                                                                         uint32_t band_shift, uint32_t rows_per_tile,
                                                                         uint32_t chunks, uint32_t units, uint32_t sub,
                                                                         const uint32_t* __restrict__ xcd_start,
+                                                                        uint32_t* __restrict__ next_unit,
                                                                         const idx_t* __restrict__ tile_ptr,
                                                                         const idx_t* __restrict__ entries,
                                                                         const T* __restrict__ vals,
                                                                         const T* __restrict__ x,
                                                                         T* __restrict__ partials) {
     extern __shared__ __align__(16) unsigned char s_raw[];
+    __shared__ uint32_t s_unit;
     double* s_acc = reinterpret_cast<double*>(s_raw);
     const uint32_t tid = threadIdx.x;
     const uint32_t xcd = blockIdx.x % kXcds;
@@ -352,7 +359,19 @@ __global__ __launch_bounds__(kColumnBlock) void spmv_column_order_kernel(idx_t m
     const idx_t band_mask = (1u << band_shift) - 1u;
     for (uint32_t r = tid; r < rows_per_tile; r += kColumnBlock) s_acc[r] = 0.0;
     __syncthreads();
-    for (uint32_t unit = xcd_start[xcd] + blockIdx.x / kXcds; unit < stretch_end; unit += gridDim.x / kXcds) {
+    // The units of an XCD's stretch differ in size (power-law rows): a workgroup starts with the unit of
+    // its own number and takes the next off a counter whenever it gets free.  The counter starts at the
+    // number of workgroups per XCD: the reduce kernel of the call before, or the build, has left it so.
+    // Every workgroup ends when the counter has passed the stretch.
+    bool first = true;
+    while (true) {
+        if (tid == 0)
+            s_unit = xcd_start[xcd] + (first ? blockIdx.x / kXcds : atomicAdd(&next_unit[xcd], 1u));
+        first = false;
+        __syncthreads();
+        const uint32_t unit = s_unit;
+        __syncthreads();  // read by all before it is written again
+        if (unit >= stretch_end) break;  // whole workgroup; also where an overwritten counter ends up
         const uint32_t group = unit / chunks;
         const uint32_t chunk = unit - group * chunks;
         const uint64_t row0 = static_cast<uint64_t>(chunk) * rows_per_tile;
@@ -471,6 +490,7 @@ BandedLayout banded_layout(const BandedShape& s, idx_t m, idx_t nnz, size_t valu
     size_t off = 0;
     l.tile_ptr = off; off += align_up((static_cast<size_t>(s.tiles) + 1) * sizeof(idx_t));
     l.xcd_start = off; off += align_up((kXcds + 1) * sizeof(uint32_t));
+    l.next_unit = off; off += align_up(kXcds * sizeof(uint32_t));
     l.entries = off; off += idx_bytes;
     l.vals = off; off += align_up(static_cast<size_t>(nnz) * value_bytes);
     l.partials = off; off += align_up(static_cast<size_t>(s.bands) * m * value_bytes);
@@ -509,7 +529,8 @@ void launch_column_order_build(hipStream_t stream, const BandedShape& s, idx_t m
                         reinterpret_cast<idx_t*>(w + l.entries), w + l.vals, value_bytes, w + l.sort_ws);
     launch_coo2csr(stream, nnz, s.tiles, sorted_ids, 0, reinterpret_cast<idx_t*>(w + l.tile_ptr));
     hipLaunchKernelGGL(column_order_split_kernel, dim3(1), dim3(kBlock), 0, stream, nnz, s.tiles / s.sub, s.sub,
-                       reinterpret_cast<const idx_t*>(w + l.tile_ptr), reinterpret_cast<uint32_t*>(w + l.xcd_start));
+                       reinterpret_cast<const idx_t*>(w + l.tile_ptr), reinterpret_cast<uint32_t*>(w + l.xcd_start),
+                       reinterpret_cast<uint32_t*>(w + l.next_unit));
 }
 
 void launch_banded_build(hipStream_t stream, const BandedShape& s, idx_t m, idx_t nnz, idx_t base, const idx_t* row_ptr,
@@ -551,7 +572,7 @@ void launch_spmv_banded(hipStream_t stream, const BandedShape& s, uint32_t grid,
                                   hipFuncAttributeMaxDynamicSharedMemorySize, lds);
         hipLaunchKernelGGL((spmv_column_order_kernel<T>), dim3(kColumnGroupsPerXcd * kXcds), dim3(kColumnBlock), lds,
                            stream, a.m, a.n, a.nnz, a.base, s.band_shift, s.rows_per_tile, s.chunks, s.tiles / s.sub, s.sub,
-                           reinterpret_cast<const uint32_t*>(w + l.xcd_start),
+                           reinterpret_cast<const uint32_t*>(w + l.xcd_start), reinterpret_cast<uint32_t*>(w + l.next_unit),
                            reinterpret_cast<const idx_t*>(w + l.tile_ptr), reinterpret_cast<const idx_t*>(w + l.entries),
                            reinterpret_cast<const T*>(w + l.vals), static_cast<const T*>(a.x), partials);
     } else if (grid != 0) {
@@ -562,12 +583,13 @@ void launch_spmv_banded(hipStream_t stream, const BandedShape& s, uint32_t grid,
                            reinterpret_cast<const T*>(w + l.vals), static_cast<const T*>(a.x), partials);
     }
     const dim3 rows_grid((a.m + kBlock - 1) / kBlock);
+    uint32_t* next_unit = s.by_column ? reinterpret_cast<uint32_t*>(w + l.next_unit) : nullptr;
     if (beta == T(0)) {
         hipLaunchKernelGGL((banded_reduce_kernel<T, true>), rows_grid, dim3(kBlock), 0, stream, a.m, s.bands,
-                           static_cast<const T*>(partials), static_cast<T*>(a.y), alpha, beta);
+                           static_cast<const T*>(partials), static_cast<T*>(a.y), alpha, beta, next_unit);
     } else {
         hipLaunchKernelGGL((banded_reduce_kernel<T, false>), rows_grid, dim3(kBlock), 0, stream, a.m, s.bands,
-                           static_cast<const T*>(partials), static_cast<T*>(a.y), alpha, beta);
+                           static_cast<const T*>(partials), static_cast<T*>(a.y), alpha, beta, next_unit);
     }
 }
 
