@@ -449,10 +449,10 @@ mcsparseStatus_t mcsparseSpMatSetSpMVPlan(mcsparseSpMatDescr_t spMatDescr, int f
  * merged_entries = total length of the merged column lists of all row groups (compare with nnz). */
 mcsparseStatus_t mcsparseSpMatGetSpMMSchedule(mcsparseSpMatDescr_t spMatDescr, int* state, int64_t* merged_entries);
 
-/* Optional preparation of y = alpha*A*x + beta*y for a CSR matrix that is multiplied many times (the
+/* Optional preparation of y = alpha*op(A)*x + beta*y for a matrix that is multiplied many times (the
  * reference has no such step: include/interface/mcsp_generic.h:43-51).  It copies A into externalBuffer
  * in a column-banded layout in which the reads of x hit in cache; mcsparseSpMV then uses that copy
- * whenever it is called with the same externalBuffer, the same three CSR arrays and extents, op N.
+ * whenever it is called with the same externalBuffer, the same three arrays and extents and the same opA.
  *   - externalBuffer needs mcsparseSpMV_preprocess_bufferSize bytes (about three times the matrix), is
  *     passed to both calls, and must be left alone in between, like the structure of A.
  *   - The copy includes the values.  After changing values in place call mcsparseSpMV_preprocess
@@ -461,7 +461,9 @@ mcsparseStatus_t mcsparseSpMatGetSpMMSchedule(mcsparseSpMatDescr_t spMatDescr, i
  *     transposing directions (CSR with op T, CSC with op N) the copy is of the transpose, so that such
  *     calls stop sorting the nonzeros by column on every call; externalBuffer then also needs room
  *     for the conversion (about five times the matrix in all).
- *   - Calls the layout cannot help (x fits in cache as it is, 64-bit indices, COO) are left to the
+ *   - CSR, CSC and COO descriptors with 32- or 64-bit indices can be prepared (64-bit indices are
+ *     narrowed and COO row indices turned into offsets once, inside externalBuffer).  Calls the layout
+ *     cannot help (x fits in cache as it is, a matrix too small to fill the GPU) are left to the
  *     ordinary kernels; the call still returns SUCCESS.  mcsparseSpMatGetSpMVPreprocess tells which
  *     case applies.
  *   - alg chooses between two layouts (the reference ignores alg; the meanings are those APIs of this

@@ -239,12 +239,12 @@ size_t banded_region_offset(const mcsparseSpMatDescr* A, mcsparseOperation_t op,
     return align_up(spmv_layout(v, A->nnz, value_bytes, narrow_bytes(A)).total);
 }
 
-// What mcsparseSpMV_preprocess builds a banded copy for: CSR and CSC with 32-bit indices, fp32 / fp64.
+// What mcsparseSpMV_preprocess builds a copy for: CSR, CSC and COO, 32- or 64-bit indices, fp32 / fp64.
 // The copy is of the matrix the row kernels would run on: the arrays as they lie (CSR with op N, CSC
 // with op T) or, for the transposing directions (CSR with op T, CSC with op N), their transpose, which
 // the preprocess call builds once with csr2csc.  `shape` is that matrix's; *rows its number of rows.
 bool banded_candidate(const mcsparseSpMatDescr* A, mcsparseOperation_t op, mcsparseSpMVAlg_t alg, BandedShape* shape) {
-    if ((A->format != MCSPARSE_FORMAT_CSR && A->format != MCSPARSE_FORMAT_CSC) || wide_indices(A)) return false;
+    if (!format_is_built(A->format)) return false;
     if (A->valueType != MACA_R_32F && A->valueType != MACA_R_64F) return false;
     const CsrView v = make_view(A, op);
     const int64_t rows = v.transpose ? v.n : v.m;
@@ -310,6 +310,23 @@ mcspStatus_t spmv_typed(mcsparseHandle_t h, mcsparseSpMatDescr* A, mcsparseOpera
     const SpmvLayout l = spmv_layout(v, A->nnz, sizeof(T), narrow_bytes(A));
     // what identifies the structure to the plan cache: the caller's own array
     const void* signature = v.coo_rows != nullptr ? static_cast<const void*>(v.coo_rows) : v.ptr;
+    if ((v.transpose || A->plan.forced_family == kFamilyAuto) && banded_matches(A, buffer, sizeof(T), v.transpose, alg)) {
+        // mcsparseSpMV_preprocess has copied the matrix of this direction (for a transposing one, its
+        // transpose) into the buffer: the caller's arrays are not read at all
+        mcsp::SpmvArgs a;
+        a.nnz = nnz;
+        a.base = base;
+        a.x = x->values;
+        a.y = y->values;
+        a.m = static_cast<idx_t>(v.transpose ? v.n : v.m);
+        a.n = static_cast<idx_t>(v.transpose ? v.m : v.n);
+        a.row_ptr = nullptr;
+        a.col = nullptr;
+        a.val = nullptr;
+        mcsp::launch_spmv_banded<T>(h->stream, A->banded.shape, A->banded.grid, a, h_alpha, h_beta,
+                                    buf + A->banded.region);
+        return MCSP_STATUS_SUCCESS;
+    }
     if (wide_indices(A)) {
         const IndexArrays ia = index_arrays(h, A, buf + l.narrow);
         v = make_view(A, op, ia.rows, ia.cols);
@@ -335,11 +352,6 @@ mcspStatus_t spmv_typed(mcsparseHandle_t h, mcsparseSpMatDescr* A, mcsparseOpera
             ensure_plan(h, A, v.ptr, signature, v.m, A->nnz, v.n * static_cast<int64_t>(sizeof(T)), buffer,
                         may_read_back);
         if (st != MCSP_STATUS_SUCCESS) return st;
-        if (A->plan.forced_family == kFamilyAuto && banded_matches(A, buffer, sizeof(T), false, alg)) {
-            mcsp::launch_spmv_banded<T>(h->stream, A->banded.shape, A->banded.grid, a, h_alpha, h_beta,
-                                        buf + A->banded.region);
-            return MCSP_STATUS_SUCCESS;
-        }
         if (A->plan.family == kFamilyMerge) {
             mcsp::launch_spmv_merge<T>(h->stream, a, h_alpha, h_beta, buf + l.merge_ws, A->plan.lanes != 0);
         } else {
@@ -354,17 +366,6 @@ mcspStatus_t spmv_typed(mcsparseHandle_t h, mcsparseSpMatDescr* A, mcsparseOpera
     // of csr2csc, which is a stable sort of one array less, and then sums the products of each column:
     // the sum of a column adds the same products in the same order (row order) as a row kernel on the
     // transpose would, without the gathers from x.
-    if (banded_matches(A, buffer, sizeof(T), true, alg)) {
-        // mcsparseSpMV_preprocess has built the transpose, in the banded layout, once for all calls
-        a.m = static_cast<idx_t>(v.n);
-        a.n = static_cast<idx_t>(v.m);
-        a.row_ptr = nullptr;
-        a.col = nullptr;
-        a.val = nullptr;
-        mcsp::launch_spmv_banded<T>(h->stream, A->banded.shape, A->banded.grid, a, h_alpha, h_beta,
-                                    buf + A->banded.region);
-        return MCSP_STATUS_SUCCESS;
-    }
     idx_t* t_ptr = reinterpret_cast<idx_t*>(buf + l.col_ptr);
     void* t_val = buf + l.vals;
     mcsp::launch_transposed_products(h->stream, static_cast<idx_t>(v.m), static_cast<idx_t>(v.n), nnz, v.val, v.ptr, v.ind,
@@ -734,15 +735,31 @@ mcsparseStatus_t mcsparseSpMV_preprocess(mcsparseHandle_t handle, mcsparseOperat
     BandedShape shape;
     if (matA->nnz == 0 || !banded_candidate(matA, opA, alg, &shape)) return MCSPARSE_STATUS_SUCCESS;  // nothing to prepare
 
-    const CsrView v = make_view(matA, opA);
+    CsrView v = make_view(matA, opA);
     const idx_t m = static_cast<idx_t>(v.transpose ? v.n : v.m);  // rows of the matrix that is banded
     const idx_t nnz = static_cast<idx_t>(matA->nnz);
     const idx_t base = static_cast<idx_t>(matA->idxBase);
     const size_t vb = value_size(matA->valueType);
+    // 64-bit indices are narrowed and COO rows turned into offsets in the part of the buffer a plain call
+    // uses for the same purpose; the copy does not refer to them afterwards
+    const void* signature = v.coo_rows != nullptr ? static_cast<const void*>(v.coo_rows) : v.ptr;
+    {
+        char* buf = static_cast<char*>(externalBuffer);
+        const SpmvLayout sl = spmv_layout(v, matA->nnz, vb, narrow_bytes(matA));
+        if (wide_indices(matA)) {
+            const IndexArrays ia = index_arrays(handle, matA, buf + sl.narrow);
+            v = make_view(matA, opA, ia.rows, ia.cols);
+        }
+        if (v.coo_rows != nullptr) {
+            idx_t* built = reinterpret_cast<idx_t*>(buf + sl.coo_ptr);
+            mcsp::launch_coo2csr(handle->stream, nnz, static_cast<idx_t>(v.m), v.coo_rows, base, built);
+            v.ptr = built;
+        }
+    }
     if (!v.transpose) {
         // the plan of the row kernels is worked out here as well, so that no later call has to block for it
-        const mcspStatus_t ps = ensure_plan(handle, matA, v.ptr, v.ptr, v.m, matA->nnz, v.n * static_cast<int64_t>(vb),
-                                            externalBuffer, true);
+        const mcspStatus_t ps = ensure_plan(handle, matA, v.ptr, signature, v.m, matA->nnz,
+                                            v.n * static_cast<int64_t>(vb), externalBuffer, true);
         if (ps != MCSP_STATUS_SUCCESS) return to_public_status(ps);
     }
     SpmvBanded& b = matA->banded;

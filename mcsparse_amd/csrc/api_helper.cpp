@@ -266,6 +266,7 @@ mcsparseStatus_t mcsparseCooSetPointers(mcsparseSpMatDescr_t d, void* cooRows, v
     d->cols = cooColumns;
     d->vals = cooValues;
     d->plan.valid = false;
+    d->banded.valid = false;
     return MCSPARSE_STATUS_SUCCESS;
 }
 

@@ -210,3 +210,40 @@ def test_random_shapes(torch_gpu, handle, oracle, seed):
         y_ref, bound = oracle.spmv(transposed, a.m, a.n, a.base, a.ptr, a.col, a.val, alpha, beta, x, y)
         assert_within(d_y.cpu().numpy(), y_ref, bound, dtype, what=what)
     assert 3 in seen, seen
+
+
+@pytest.mark.parametrize("alg,state", [(api.SPMV_ALG_DEFAULT, 3), (api.SPMV_CSR_ALG2, 2)])
+@pytest.mark.parametrize("fmt", [api.FORMAT_CSR, api.FORMAT_CSC, api.FORMAT_COO])
+@pytest.mark.parametrize("index_type", [api.INDEX_32I, api.INDEX_64I])
+def test_copies_of_coo_and_64_bit_inputs(torch_gpu, handle, oracle, alg, state, fmt, index_type):
+    """mcsparseSpMV_preprocess narrows 64-bit indices and turns COO rows into offsets once; the calls then read
+    nothing but the copy.  Both directions of every format."""
+    torch = torch_gpu
+    a = wl.random_ragged(60001, 50021, 8, dtype=np.float64, seed=40 + fmt, base=1)
+    if fmt == api.FORMAT_CSR and index_type == api.INDEX_32I:
+        pytest.skip("covered by the tests above")
+    itype = np.int64 if index_type == api.INDEX_64I else np.int32
+    first = a.ptr if fmt != api.FORMAT_COO else np.repeat(np.arange(a.m) + a.base, np.diff(a.ptr.astype(np.int64)))
+    d_first, d_col, d_val = dev(torch, first.astype(itype)), dev(torch, a.col.astype(itype)), dev(torch, a.val)
+    shape = (a.n, a.m) if fmt == api.FORMAT_CSC else (a.m, a.n)
+    rng = np.random.default_rng(8)
+    for op in (api.OP_N, api.OP_T):
+        # the arrays are A's CSR (or COO); read as CSC they are the n x m transpose
+        transposed = (fmt != api.FORMAT_CSC) == (op == api.OP_T)
+        x = rng.uniform(-1, 1, a.m if transposed else a.n)
+        y = rng.uniform(-1, 1, a.n if transposed else a.m)
+        d_x, d_y = dev(torch, x), dev(torch, y)
+        mat = api.SpMat(shape[0], shape[1], a.nnz, d_first, d_col, d_val, base=1, fmt=fmt, index_type=index_type)
+        mat.set_band_bytes(1 << 14)
+        vx, vy = api.DnVec(d_x), api.DnVec(d_y)
+        st, size = api.spmv_preprocess_buffer_size(handle, op, 1.5, mat, vx, -0.5, vy, api.R_64F, alg=alg)
+        assert st == api.STATUS_SUCCESS
+        buf = torch.empty(size, dtype=torch.uint8, device="cuda")
+        assert api.spmv_preprocess(handle, op, 1.5, mat, vx, -0.5, vy, api.R_64F, buf, alg=alg) == api.STATUS_SUCCESS
+        assert mat.spmv_preprocess_state()[0] == state
+        y_ref, bound = oracle.spmv(transposed, a.m, a.n, 1, a.ptr, a.col, a.val, 1.5, -0.5, x, y)
+        for _ in range(2):
+            d_y.copy_(torch.from_numpy(y))
+            assert api.spmv(handle, op, 1.5, mat, vx, -0.5, vy, api.R_64F, buf, alg=alg) == api.STATUS_SUCCESS
+            torch.cuda.synchronize()
+            assert_within(d_y.cpu().numpy(), y_ref, bound, np.float64, what="fmt %d index %d op %d" % (fmt, index_type, op))
