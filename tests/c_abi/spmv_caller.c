@@ -73,6 +73,52 @@ int main(void) {
            MCSPARSE_STATUS_INVALID_VALUE);
     EXPECT(mcsparseCsrSetPointers(A, fake, fake, fake), MCSPARSE_STATUS_SUCCESS);
 
+    /* the preparation step (an extension): sizes depend on the algorithm, arguments are checked like SpMV's */
+    {
+        const int64_t big = 1 << 20;
+        size_t plain = 0, banded = 0, by_column = 0;
+        int state = -1, bands = -1, rows_per_tile = -1;
+        mcsparseSpMatDescr_t W = NULL;
+        mcsparseDnVecDescr_t WX = NULL, WY = NULL;
+        EXPECT(mcsparseCreateCsr(&W, big, big, 16 * big, fake, fake, fake, MCSPARSE_INDEX_32I, MCSPARSE_INDEX_32I,
+                                 MCSPARSE_INDEX_BASE_ZERO, MACA_R_64F),
+               MCSPARSE_STATUS_SUCCESS);
+        EXPECT(mcsparseCreateDnVec(&WX, big, fake, MACA_R_64F), MCSPARSE_STATUS_SUCCESS);
+        EXPECT(mcsparseCreateDnVec(&WY, big, fake, MACA_R_64F), MCSPARSE_STATUS_SUCCESS);
+        EXPECT(mcsparseSpMV_bufferSize(h, MCSPARSE_OPERATION_NON_TRANSPOSE, &alpha, W, WX, &beta, WY, MACA_R_64F,
+                                       MCSPARSE_SPMV_ALG_DEFAULT, &plain),
+               MCSPARSE_STATUS_SUCCESS);
+        EXPECT(mcsparseSpMV_preprocess_bufferSize(h, MCSPARSE_OPERATION_NON_TRANSPOSE, &alpha, W, WX, &beta, WY,
+                                                  MACA_R_64F, MCSPARSE_SPMV_CSR_ALG2, &banded),
+               MCSPARSE_STATUS_SUCCESS);
+        EXPECT(mcsparseSpMV_preprocess_bufferSize(h, MCSPARSE_OPERATION_NON_TRANSPOSE, &alpha, W, WX, &beta, WY,
+                                                  MACA_R_64F, MCSPARSE_SPMV_ALG_DEFAULT, &by_column),
+               MCSPARSE_STATUS_SUCCESS);
+        if (!(plain < banded && banded < by_column)) {
+            printf("unexpected preprocess buffer sizes %zu %zu %zu\n", plain, banded, by_column);
+            return 1;
+        }
+        EXPECT(mcsparseSpMV_preprocess(h, MCSPARSE_OPERATION_NON_TRANSPOSE, &alpha, W, WX, &beta, WY, MACA_R_64F,
+                                       MCSPARSE_SPMV_ALG_DEFAULT, NULL),
+               MCSPARSE_STATUS_INVALID_VALUE);
+        EXPECT(mcsparseSpMV_preprocess(NULL, MCSPARSE_OPERATION_NON_TRANSPOSE, &alpha, W, WX, &beta, WY, MACA_R_64F,
+                                       MCSPARSE_SPMV_ALG_DEFAULT, fake),
+               MCSPARSE_STATUS_NOT_INITIALIZED);
+        EXPECT(mcsparseSpMatGetSpMVPreprocess(W, &state, &bands, &rows_per_tile), MCSPARSE_STATUS_SUCCESS);
+        if (state != 0 || bands != 0 || rows_per_tile != 0) {
+            printf("a descriptor that was never prepared reports state %d\n", state);
+            return 1;
+        }
+        EXPECT(mcsparseSpMatSetSpMVBandBytes(W, 8), MCSPARSE_STATUS_INVALID_VALUE);
+        EXPECT(mcsparseSpMatSetSpMVBandBytes(W, 1 << 20), MCSPARSE_STATUS_SUCCESS);
+        EXPECT(mcsparseSpMV_staticBuffer(h, MCSPARSE_OPERATION_NON_TRANSPOSE, NULL, W, WX, &beta, WY, MACA_R_64F,
+                                         MCSPARSE_SPMV_ALG_DEFAULT),
+               MCSPARSE_STATUS_INVALID_VALUE);
+        EXPECT(mcsparseDestroyDnVec(WX), MCSPARSE_STATUS_SUCCESS);
+        EXPECT(mcsparseDestroyDnVec(WY), MCSPARSE_STATUS_SUCCESS);
+        EXPECT(mcsparseDestroySpMat(W), MCSPARSE_STATUS_SUCCESS);
+    }
+
     /* SpMM: op(A) = T is not supported for CSR; shapes are checked */
     {
         mcsparseDnMatDescr_t B = NULL, C = NULL;
