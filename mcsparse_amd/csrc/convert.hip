@@ -75,66 +75,88 @@ __device__ __forceinline__ idx_t wave_count_row_starts(const idx_t* __restrict__
     return static_cast<idx_t>(lo);
 }
 
-// coo_rows[j] = row of nonzero j (+ base).  One tile of the merged path per workgroup, so empty
-// rows, 1-nonzero rows and 200k-nonzero rows all cost one item each.
+// coo_rows[j] = row of nonzero j (+ base).  Tiles of the merged path of (row ends, nonzeros), so empty
+// rows, 1-nonzero rows and 200k-nonzero rows all cost one item each.  A workgroup takes kExpandTiles
+// tiles in a row: only where its first tile begins has to be searched for in row_ptr (a chain of
+// dependent loads); every tile ends where the row ends loaded for it say, and the next begins there.
 // Reference semantics: src/kernels/conversion/coo2csr_device.hpp:26-41.
+constexpr int kExpandTiles = 8;
 __global__ __launch_bounds__(kBlock) void csr2coo_kernel(idx_t m, idx_t nnz, idx_t base,
                                                          const idx_t* __restrict__ row_ptr,
                                                          idx_t* __restrict__ coo_rows) {
     __shared__ idx_t s_row_end[kExpandTile + 1];
     __shared__ idx_t s_ids[kExpandTile];
-    __shared__ idx_t s_x[2];
+    __shared__ idx_t s_x;
 
     const uint32_t tid = threadIdx.x;
     const uint64_t total = static_cast<uint64_t>(m) + nnz;
-    const uint64_t d0 = static_cast<uint64_t>(blockIdx.x) * kExpandTile;
-    const uint64_t d1 = d0 + kExpandTile < total ? d0 + kExpandTile : total;
-    const unsigned wave = tid / kWave;
-    if (wave < 2) {
-        const idx_t x = wave_merge_search(wave == 0 ? d0 : d1, m, nnz, base, row_ptr);
-        if (tid % kWave == 0) s_x[wave] = x;
+    const uint64_t d_begin = static_cast<uint64_t>(blockIdx.x) * kExpandTiles * kExpandTile;
+    if (tid / kWave == 0) {
+        const idx_t x = wave_merge_search(d_begin, m, nnz, base, row_ptr);
+        if (tid == 0) s_x = x;
     }
     __syncthreads();
-    const idx_t x0 = s_x[0];
-    const idx_t x1 = s_x[1];
-    const idx_t y0 = static_cast<idx_t>(d0 - x0);
-    const idx_t y1 = static_cast<idx_t>(d1 - x1);
-    const idx_t tile_rows = x1 - x0;
-    const idx_t tile_nnz = y1 - y0;
-    const idx_t tile_items = tile_rows + tile_nnz;
-
-    for (idx_t i = tid; i <= tile_rows; i += kBlock) {
-        const idx_t r = x0 + i;
-        s_row_end[i] = r < m ? row_ptr[r + 1] - base : 0xFFFFFFFFu;
-    }
-    __syncthreads();
-
-    const idx_t dt = min(static_cast<idx_t>(tid * kExpandIpt), tile_items);
-    idx_t lo = dt > tile_nnz ? dt - tile_nnz : 0;
-    idx_t hi = dt < tile_rows ? dt : tile_rows;
-    while (lo < hi) {
-        const idx_t mid = (lo + hi) >> 1;
-        if (s_row_end[mid] <= y0 + (dt - mid - 1)) {
-            lo = mid + 1;
-        } else {
-            hi = mid;
+    idx_t x0 = s_x;
+    for (int t = 0; t < kExpandTiles; ++t) {
+        const uint64_t d0 = d_begin + static_cast<uint64_t>(t) * kExpandTile;
+        if (d0 >= total) break;  // whole workgroup
+        const uint64_t d1 = d0 + kExpandTile < total ? d0 + kExpandTile : total;
+        const idx_t y0 = static_cast<idx_t>(d0 - x0);
+        // Row ends from row x0 on, a workgroup's width at a time, until the row is in at which the tile
+        // ends: row x0 + i with its nonzeros and its end lies before d1 when x0 + i + end + 1 <= d1.
+        // Rows past the matrix end nowhere.
+        uint32_t last = 0;
+        for (uint32_t loaded = 0;; loaded += kBlock) {
+            const uint32_t i = loaded + tid;
+            if (i <= kExpandTile) {
+                const uint64_t r = static_cast<uint64_t>(x0) + i;
+                s_row_end[i] = r < m ? row_ptr[r + 1] - base : 0xFFFFFFFFu;
+            }
+            __syncthreads();
+            last = min(loaded + kBlock - 1, static_cast<uint32_t>(kExpandTile));
+            if (last == kExpandTile || static_cast<uint64_t>(x0) + last + s_row_end[last] + 1 > d1) break;
         }
-    }
-    idx_t row_l = lo;
-    idx_t nz = y0 + (dt - lo);
-#pragma unroll
-    for (int i = 0; i < kExpandIpt; ++i) {
-        if (dt + i < tile_items) {
-            if (nz < s_row_end[row_l]) {
-                s_ids[nz - y0] = x0 + row_l + base;
-                ++nz;
+        // rows that lie in the tile with their ends: the first `tile_rows` of them
+        uint32_t lo = 0, hi = last + 1;
+        while (lo < hi) {
+            const uint32_t mid = (lo + hi) >> 1;
+            if (static_cast<uint64_t>(x0) + mid + s_row_end[mid] + 1 <= d1) lo = mid + 1; else hi = mid;
+        }
+        const idx_t tile_rows = lo;
+        const idx_t x1 = x0 + tile_rows;
+        const idx_t y1 = static_cast<idx_t>(d1 - x1);
+        const idx_t tile_nnz = y1 - y0;
+        const idx_t tile_items = tile_rows + tile_nnz;
+
+        const idx_t dt = min(static_cast<idx_t>(tid * kExpandIpt), tile_items);
+        lo = dt > tile_nnz ? dt - tile_nnz : 0;
+        hi = dt < tile_rows ? dt : tile_rows;
+        while (lo < hi) {
+            const idx_t mid = (lo + hi) >> 1;
+            if (s_row_end[mid] <= y0 + (dt - mid - 1)) {
+                lo = mid + 1;
             } else {
-                ++row_l;
+                hi = mid;
             }
         }
+        idx_t row_l = lo;
+        idx_t nz = y0 + (dt - lo);
+#pragma unroll
+        for (int i = 0; i < kExpandIpt; ++i) {
+            if (dt + i < tile_items) {
+                if (nz < s_row_end[row_l]) {
+                    s_ids[nz - y0] = x0 + row_l + base;
+                    ++nz;
+                } else {
+                    ++row_l;
+                }
+            }
+        }
+        __syncthreads();
+        for (idx_t k = tid; k < tile_nnz; k += kBlock) coo_rows[y0 + k] = s_ids[k];
+        __syncthreads();  // the next tile writes both arrays again
+        x0 = x1;
     }
-    __syncthreads();
-    for (idx_t k = tid; k < tile_nnz; k += kBlock) coo_rows[y0 + k] = s_ids[k];
 }
 
 // Offsets from sorted row indices: boundary t (between entry t-1 and entry t, 0 <= t <= nnz) fills
@@ -828,8 +850,9 @@ __global__ __launch_bounds__(kBlock) void gather_kernel(idx_t nnz, const T* __re
 void launch_csr2coo(hipStream_t stream, idx_t m, idx_t nnz, const idx_t* row_ptr, idx_t base, idx_t* coo_rows) {
     if (nnz == 0) return;
     const uint64_t total = static_cast<uint64_t>(m) + nnz;
-    const uint32_t tiles = static_cast<uint32_t>((total + kExpandTile - 1) / kExpandTile);
-    hipLaunchKernelGGL(csr2coo_kernel, dim3(tiles), dim3(kBlock), 0, stream, m, nnz, base, row_ptr, coo_rows);
+    const uint64_t per_group = static_cast<uint64_t>(kExpandTiles) * kExpandTile;
+    const uint32_t groups = static_cast<uint32_t>((total + per_group - 1) / per_group);
+    hipLaunchKernelGGL(csr2coo_kernel, dim3(groups), dim3(kBlock), 0, stream, m, nnz, base, row_ptr, coo_rows);
 }
 
 void launch_coo2csr(hipStream_t stream, idx_t nnz, idx_t m, const idx_t* coo_rows, idx_t base, idx_t* row_ptr) {
