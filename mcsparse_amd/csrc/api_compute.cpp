@@ -518,7 +518,14 @@ mcspStatus_t spmm_typed(mcsparseHandle_t h, const mcsparseSpMatDescr* A, mcspars
             a.ldb = l.n_padded;
             a.b_row_major = true;
         }
-        if (l.copy_c) {
+        // The kernel that works from the schedule owns four consecutive rows per lane group and writes them
+        // into a column-major C as they lie there, 16 bytes per column: no row-major copy of C then.
+        const bool scheduled_here = (b == 0 || shared_structure) && schedule_matches(A, buffer);
+        const bool direct_c = l.copy_c && scheduled_here && mcsp::spmm_schedule_usable(a, sizeof(T)) &&
+                              reinterpret_cast<uintptr_t>(c_user) % 16 == 0 &&
+                              (static_cast<uint64_t>(C->ld) * sizeof(T)) % 16 == 0;
+        const bool copy_c = l.copy_c && !direct_c;
+        if (copy_c) {
             a.C = buf + l.ct;
             a.ldc = l.n_padded;
             a.c_row_major = true;
@@ -527,13 +534,13 @@ mcspStatus_t spmm_typed(mcsparseHandle_t h, const mcsparseSpMatDescr* A, mcspars
             if (l.copy_b && A->nnz != 0) a.n = static_cast<idx_t>(l.n_padded);
         }
         // the schedule was built from batch 0's structure
-        if ((b == 0 || shared_structure) && schedule_matches(A, buffer) && mcsp::spmm_schedule_usable(a, sizeof(T))) {
+        if (scheduled_here && mcsp::spmm_schedule_usable(a, sizeof(T))) {
             mcsp::launch_spmm_scheduled<T>(h->stream, a, buffer, A->schedule.entries, A->schedule.mean_span, h_alpha,
                                            beta_inner);
         } else {
             mcsp::launch_spmm<T>(h->stream, a, h_alpha, beta_inner);
         }
-        if (l.copy_c) {
+        if (copy_c) {
             mcsp::launch_transpose_accumulate<T>(h->stream, a.m, static_cast<idx_t>(C->col_num),
                                                  reinterpret_cast<const T*>(buf + l.ct), l.n_padded, c_user, C->ld,
                                                  h_beta);

@@ -156,6 +156,28 @@ __device__ __forceinline__ void store_c(T* __restrict__ C, int64_t ldc, bool c_r
     }
 }
 
+// Four consecutive rows of one column of a column-major C (16-byte aligned): beta*C + alpha*acc with
+// 128-bit accesses, C untouched by reads if beta == 0.
+template <typename T>
+__device__ __forceinline__ void store_c_four_rows(T* __restrict__ Cp, T a0, T a1, T a2, T a3, T alpha, T beta) {
+    constexpr int W = 16 / sizeof(T);  // elements per 128-bit access: 4 floats, 2 doubles
+    const T acc[4] = {a0, a1, a2, a3};
+    const bool beta0 = beta == T(0);
+#pragma unroll
+    for (int h = 0; h < 4 / W; ++h) {
+        Vec<T, W> out;
+        if (beta0) {
+#pragma unroll
+            for (int i = 0; i < W; ++i) out.v[i] = alpha * acc[h * W + i];
+        } else {
+            const Vec<T, W> old = load_vec<T, W>(Cp + h * W);
+#pragma unroll
+            for (int i = 0; i < W; ++i) out.v[i] = beta * old.v[i] + alpha * acc[h * W + i];
+        }
+        store_vec<T, W>(Cp + h * W, out);
+    }
+}
+
 // op(B) row-major.  LR lanes per row of A, V adjacent columns per lane; blockIdx.y walks the
 // column panels of LR*V columns.  V > 1 requires n, ldb (and ldc when C is row-major) to be
 // multiples of V and 16-byte aligned base pointers, which the launcher checks.
@@ -727,6 +749,19 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(LR <= 16
     }
 
     if (!stores) return;
+    // A column-major C holds the four rows of the group next to each other in every column: 16 or 32
+    // bytes per column and lane, which the lane groups of a workgroup (64 consecutive rows) complete to
+    // whole lines.
+    static_assert(R == 4, "four rows per 128-bit (fp32) or two 128-bit (fp64) accesses");
+    const bool whole_columns = !c_row_major && r0 + R <= static_cast<uint64_t>(m) &&
+                               ((reinterpret_cast<uintptr_t>(C) | static_cast<uintptr_t>(ldc * sizeof(T))) & 15u) == 0;
+    if (whole_columns) {
+#pragma unroll
+        for (int c = 0; c < V; ++c)
+            store_c_four_rows<T>(C + static_cast<int64_t>(c0 + c) * ldc + r0, acc[0][c], acc[1][c], acc[2][c], acc[3][c], alpha,
+                                 beta);
+        return;
+    }
 #pragma unroll
     for (int r = 0; r < R; ++r) {
         if (r0 + r < static_cast<uint64_t>(m)) store_c<T, V>(C, ldc, c_row_major, r0 + r, c0, acc[r], alpha, beta);
