@@ -65,8 +65,8 @@ MEASURED_TRAFFIC = {
                     "profiles/spmv_merge_f32_c3_powerlaw.txt"),
     ("c4-64", 0): (_traffic(613893.3, 524288.0), "profiles/spmm_group_f32_c4_stencil128.txt"),
     ("c4-256", 0): (_traffic(3673719.8, 2097152.0), "profiles/spmm_group_f32_c4_stencil128.txt"),
-    # group kernel + the transposes of B and of C
-    ("c4-64-col", 0): (_traffic(596223.4 + 262180.7 + 262178.7, 3 * 524288.0),
+    # group kernel (writes the column-major C itself) + the transpose of B
+    ("c4-64-col", 0): (_traffic(589819.9 + 262180.0, 537321.5 + 524288.0),
                            "profiles/spmm_colmajor_f32_c4_stencil128_n64.txt"),
     # csr2csc: 2 x scatter + the scatter that reads the CSR arrays in place + 3 x (histogram + scans)
     # + row starts per tile + coo2csr
