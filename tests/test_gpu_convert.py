@@ -230,3 +230,31 @@ def test_unaligned_input_arrays(torch_gpu, handle, oracle, shift):
     assert api.xcoo2csr(handle, d_rows, 300, m_big, d_out, 0) == 0
     torch.cuda.synchronize()
     assert np.array_equal(d_out.cpu().numpy().view(np.uint32), oracle.coo2csr(300, m_big, 0, rows))
+
+
+@pytest.mark.parametrize("items", [2048, 2049, 8 * 2048 - 1, 8 * 2048, 8 * 2048 + 1, 3 * 8 * 2048 + 5])
+@pytest.mark.parametrize("shape", ["even", "empty_head", "empty_tail", "one_long_row"])
+def test_csr2coo_around_the_tile_and_group_sizes(torch_gpu, handle, oracle, items, shape):
+    """csr2coo cuts rows + nonzeros into tiles of 2048 items and walks 8 tiles per workgroup."""
+    rng = np.random.default_rng(items)
+    m = items // 3
+    nnz = items - m
+    if shape == "even":
+        lens = np.full(m, nnz // m, np.int64)
+        lens[: nnz - lens.sum()] += 1
+    elif shape == "empty_head":   # every row ends inside the first tiles, the nonzeros come last
+        lens = np.zeros(m, np.int64)
+        lens[m - 3:] = [nnz - 2, 1, 1]
+    elif shape == "empty_tail":
+        lens = np.zeros(m, np.int64)
+        lens[:2] = [1, nnz - 1]
+    else:
+        lens = np.zeros(m, np.int64)
+        lens[int(rng.integers(0, m))] = nnz
+    assert lens.sum() == nnz
+    ptr = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    for base in (0, 1):
+        a = wl.Csr(m, nnz + 1, ptr + base, np.zeros(nnz, np.int32) + base, np.zeros(nnz, np.float32), base)
+        st, coo = gpu_csr2coo(torch_gpu, handle, a)
+        assert st == 0
+        assert np.array_equal(coo.view(np.uint32), oracle.csr2coo(m, base, a.ptr, nnz)), (items, shape, base)
