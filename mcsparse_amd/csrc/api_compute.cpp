@@ -795,8 +795,11 @@ mcsparseStatus_t mcsparseSpMV_preprocess(mcsparseHandle_t handle, mcsparseOperat
             mcsp::launch_csr2coo(handle->stream, static_cast<idx_t>(v.m), nnz, v.ptr, base, src_rows);
             mcsp::launch_column_order_build(handle->stream, shape, m, nnz, base, v.ind, src_rows, matA->vals, vb, region);
         } else {
+            // what the kernel gains from is lanes that share a 128-byte line of x: the order of the columns
+            // inside a line does not matter, so the sort leaves the bits that tell them apart alone
+            const uint32_t line_bits = vb == 8 ? 4 : 5;
             mcsp::launch_sort_by_column(handle->stream, static_cast<idx_t>(v.m), static_cast<idx_t>(v.n), nnz, base, v.ptr,
-                                        v.ind, matA->vals, vb, src_cols, src_rows, region + cl.src_vals,
+                                        v.ind, matA->vals, vb, line_bits, src_cols, src_rows, region + cl.src_vals,
                                         region + cl.sort_ws);
             mcsp::launch_column_order_build(handle->stream, shape, m, nnz, base, src_rows, src_cols, region + cl.src_vals,
                                             vb, region);

@@ -990,17 +990,21 @@ SortScratch sort_scratch_in(char* w, const Csr2CscLayout& l) {
 }  // namespace
 
 // The nonzeros of a CSR matrix in the order of a stable sort by column, as (column, row, value)
-// arrays with the index base left in: csr2csc without the offsets.  workspace: csr2csc_workspace_bytes.
+// arrays with the index base left in: csr2csc without the offsets.  low_bits > 0 leaves that many low
+// bits of the column keys out of the sort: columns that differ only there stay in CSR order.
+// workspace: csr2csc_workspace_bytes.
 void launch_sort_by_column(hipStream_t stream, idx_t m, idx_t n, idx_t nnz, idx_t base, const idx_t* row_ptr,
-                           const idx_t* col, const void* val, size_t value_bytes, idx_t* cols_out, idx_t* rows_out,
-                           void* vals_out, void* workspace) {
+                           const idx_t* col, const void* val, size_t value_bytes, uint32_t low_bits, idx_t* cols_out,
+                           idx_t* rows_out, void* vals_out, void* workspace) {
     if (m == 0 || n == 0 || nnz == 0) return;
     const SortScratch t = sort_scratch_in(static_cast<char*>(workspace), csr2csc_layout(nnz, value_bytes));
     CsrSource csr;
     csr.rows = m;
     csr.base = base;
-    radix_sort_triples(stream, nnz, bit_length(n - 1 + base), col, row_ptr, val, cols_out, rows_out, vals_out,
-                       value_bytes, t, csr);
+    csr.first_bit = low_bits;
+    const uint32_t bits = bit_length(n - 1 + base);
+    radix_sort_triples(stream, nnz, bits > low_bits ? bits - low_bits : 0, col, row_ptr, val, cols_out, rows_out,
+                       vals_out, value_bytes, t, csr);
 }
 
 // Stable sort of (key, aux, value) triples on the low key_bits (at most 16) of the keys.  The outputs

@@ -275,7 +275,8 @@ constexpr uint32_t kColumnOrderMinRows = 2048;
 bool column_order_shape(idx_t m, idx_t n, idx_t nnz, idx_t base, size_t value_bytes, size_t band_bytes,
                         BandedShape* out);
 // r_keys / c_keys: row + base and column + base of every nonzero of the matrix to copy, in an order
-// sorted by column (any order among equal columns); vals in the same order.  Neither is written.
+// sorted by the 128-byte line of x the column lies in (any order inside a line); vals in the same
+// order.  Neither is written.
 void launch_column_order_build(hipStream_t stream, const BandedShape& s, idx_t m, idx_t nnz, idx_t base,
                                const idx_t* r_keys, const idx_t* c_keys, const void* vals, size_t value_bytes,
                                void* region);
@@ -367,10 +368,11 @@ void launch_sort_by_column_band(hipStream_t stream, idx_t m, idx_t nnz, idx_t ba
                                 idx_t* cols_out, idx_t* rows_out, void* vals_out, void* workspace);
 
 // (column, row + base, value) arrays of the nonzeros in the order of a stable sort by column: csr2csc
-// without the offsets.  workspace: csr2csc_workspace_bytes.
+// without the offsets; the low_bits lowest bits of the column keys are left out of the sort.
+// workspace: csr2csc_workspace_bytes.
 void launch_sort_by_column(hipStream_t stream, idx_t m, idx_t n, idx_t nnz, idx_t base, const idx_t* row_ptr,
-                           const idx_t* col, const void* val, size_t value_bytes, idx_t* cols_out, idx_t* rows_out,
-                           void* vals_out, void* workspace);
+                           const idx_t* col, const void* val, size_t value_bytes, uint32_t low_bits, idx_t* cols_out,
+                           idx_t* rows_out, void* vals_out, void* workspace);
 // Stable sort of (key, aux, value) triples on the low key_bits (<= 16) of the keys; outputs apart from
 // the inputs and from the workspace (csr2csc_workspace_bytes).
 void launch_sort_triples(hipStream_t stream, idx_t nnz, uint32_t key_bits, const idx_t* keys_in, const idx_t* aux_in,
