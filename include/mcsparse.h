@@ -454,7 +454,9 @@ mcsparseStatus_t mcsparseSpMatGetSpMMSchedule(mcsparseSpMatDescr_t spMatDescr, i
  * in a column-banded layout in which the reads of x hit in cache; mcsparseSpMV then uses that copy
  * whenever it is called with the same externalBuffer, the same three arrays and extents and the same opA.
  *   - externalBuffer needs mcsparseSpMV_preprocess_bufferSize bytes (about three times the matrix), is
- *     passed to both calls, and must be left alone in between, like the structure of A.
+ *     passed to both calls, and must be left alone in between, like the structure of A.  It also holds
+ *     the partial sums of the call in flight: two mcsparseSpMV calls that use the same copy must not
+ *     overlap in time (one stream, or an event between them).
  *   - The copy includes the values.  After changing values in place call mcsparseSpMV_preprocess
  *     again; mcsparseSpMatSetValues and mcsparseCsrSetPointers drop the copy.
  *   - A copy serves the direction it was prepared for (the opA of the preprocess call).  For the
