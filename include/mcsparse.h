@@ -286,7 +286,14 @@ mcsparseStatus_t mcsparseDnMatGetStridedBatch(mcsparseDnMatDescr_t dnMatDescr, i
  * bytes for CSR op N and never writes to the buffer (mcsp_spmv_gpu.cpp:1136-1147); here the
  * buffer holds the row-length histogram and the workspace of the merge-path kernel even for op N
  * (a few bytes per 1024 rows + nonzeros).  A caller that hard-codes the reference's 128 bytes
- * would be written past: always allocate what mcsparseSpMV_bufferSize returns. */
+ * would be written past: always allocate what mcsparseSpMV_bufferSize returns.
+ *
+ * alg (ignored by the reference): the direct kernels of the non-transposing directions give the same
+ * bits on every run whatever alg is.  A transposing call (CSR or COO with op T, CSC with op N) orders the
+ * products value * x[row] by column in the buffer: completely under MCSPARSE_SPMV_CSR_ALG2, whose sums
+ * then add in row order and repeat their bits; with any other value, for 2^14 to 2^22 columns, only into
+ * buckets of neighbouring columns whose sums are formed in the order the products arrive, which is more
+ * than twice as fast and stays within the same error bound, but the last bits can differ between runs. */
 mcsparseStatus_t mcsparseSpMV(mcsparseHandle_t handle, mcsparseOperation_t opA, const void* alpha,
                               mcsparseSpMatDescr_t matA, mcsparseDnVecDescr_t vecX, const void* beta,
                               mcsparseDnVecDescr_t vecY, macaDataType computeType, mcsparseSpMVAlg_t alg,

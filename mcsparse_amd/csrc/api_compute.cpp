@@ -368,6 +368,19 @@ mcspStatus_t spmv_typed(mcsparseHandle_t h, mcsparseSpMatDescr* A, mcsparseOpera
     // transpose would, without the gathers from x.
     idx_t* t_ptr = reinterpret_cast<idx_t*>(buf + l.col_ptr);
     void* t_val = buf + l.vals;
+    // Unless the caller asked for the algorithm whose bits repeat (MCSPARSE_SPMV_CSR_ALG2): one pass of
+    // that sort, into buckets of neighbouring columns, and the sums of a bucket's columns formed in LDS
+    // in whatever order the products arrive.
+    uint32_t bucket_shift = 0;
+    if (alg != MCSPARSE_SPMV_CSR_ALG2 &&
+        mcsp::bucketed_products_shape(static_cast<idx_t>(v.n), base, &bucket_shift)) {
+        mcsp::BucketedProducts b;
+        mcsp::launch_bucketed_products(h->stream, static_cast<idx_t>(v.m), static_cast<idx_t>(v.n), nnz, v.val, v.ptr,
+                                       v.ind, x->values, t_val, sizeof(T), base, buf + l.csr2csc_ws, &b);
+        mcsp::launch_bucket_sums<T>(h->stream, static_cast<idx_t>(v.n), nnz, base, b, static_cast<const T*>(t_val),
+                                    static_cast<T*>(y->values), h_alpha, h_beta);
+        return MCSP_STATUS_SUCCESS;
+    }
     mcsp::launch_transposed_products(h->stream, static_cast<idx_t>(v.m), static_cast<idx_t>(v.n), nnz, v.val, v.ptr, v.ind,
                                      x->values, t_val, t_ptr, sizeof(T), base, buf + l.csr2csc_ws);
     a.m = static_cast<idx_t>(v.n);

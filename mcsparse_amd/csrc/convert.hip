@@ -377,16 +377,37 @@ __global__ __launch_bounds__(kHistBlock) void radix_hist_kernel(const idx_t* __r
     // tiles start at multiples of 4096 keys, so a 16-byte aligned array allows 128-bit loads; the keys
     // of the first pass are the caller's own array, which may start anywhere
     const bool wide = (reinterpret_cast<uintptr_t>(keys) & 15u) == 0;
+    const uint32_t lane = lane_id();
 #pragma unroll
     for (int i = 0; i < kSortTile / (kHistBlock * 4); ++i) {
         const uint64_t p = start + (static_cast<uint64_t>(i) * kHistBlock + threadIdx.x) * 4;
-        if (wide && p + 4 <= count) {
-            const idx4 k = __builtin_nontemporal_load(reinterpret_cast<const idx4*>(keys + p));
+        const bool full = wide && p + 4 <= count;
+        idx4 k = {0, 0, 0, 0};
+        if (full) k = __builtin_nontemporal_load(reinterpret_cast<const idx4*>(keys + p));
+        uint32_t d[4];
 #pragma unroll
-            for (int e = 0; e < 4; ++e) atomicAdd(&s_cnt[(k[e] >> shift) & mask], 1u);
-        } else {
-            const uint64_t stop = p + 4 < count ? p + 4 : count;
-            for (uint64_t q = p; q < stop; ++q) atomicAdd(&s_cnt[(keys[q] >> shift) & mask], 1u);
+        for (int e = 0; e < 4; ++e) d[e] = (k[e] >> shift) & mask;
+        // Keys that are sorted inside long rows carry the same high digit many times in a row, and LDS
+        // takes the adds of a wavefront to one counter one after the other.  A lane whose four keys
+        // share a digit joins the lanes before it that hold the same one: the first lane of such a run
+        // adds for all of them.
+        const bool uni = full && d[0] == d[1] && d[1] == d[2] && d[2] == d[3];
+        const uint32_t before = __shfl_up(uni ? d[0] : ~0u, 1, kWave);  // ~0u is no digit
+        const bool head = lane == 0 || !uni || before != d[0];
+        const uint64_t heads = __ballot(head);
+        if (head) {
+            if (uni) {
+                const uint64_t later = lane == kWave - 1 ? 0 : heads >> (lane + 1);
+                const uint32_t run = later != 0 ? static_cast<uint32_t>(__ffsll(static_cast<unsigned long long>(later)))
+                                                : kWave - lane;
+                atomicAdd(&s_cnt[d[0]], 4u * run);
+            } else if (full) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) atomicAdd(&s_cnt[d[e]], 1u);
+            } else {
+                const uint64_t stop = p + 4 < count ? p + 4 : count;
+                for (uint64_t q = p; q < stop; ++q) atomicAdd(&s_cnt[(keys[q] >> shift) & mask], 1u);
+            }
         }
     }
     __syncthreads();
@@ -929,6 +950,46 @@ void launch_transposed_products(hipStream_t stream, idx_t m, idx_t n, idx_t nnz,
     radix_sort_triples(stream, nnz, bit_length(n - 1 + base), col, row_ptr, csr_val, sorted_keys, nullptr, products,
                        value_bytes, t, csr);
     launch_coo2csr(stream, nnz, n, sorted_keys, base, col_ptr);
+}
+
+bool bucketed_products_shape(idx_t n, idx_t base, uint32_t* shift) {
+    const uint32_t bits = bit_length(n - 1 + base);
+    // fewer keys than that: the full sort is two short passes; more: a bucket's sums no longer fit in LDS
+    if (bits < kBucketMinKeyBits || bits > 8 + kBucketMaxShift) return false;
+    *shift = bits - 8;
+    return true;
+}
+
+// One pass of the same sort, for a transposing SpMV that may add the products of a column in any order:
+// (column, value * x[row]) pairs ordered by the top eight bits of the column keys only, that is in up to
+// 256 buckets of 2^shift neighbouring columns, inside a bucket in CSR order.  The sums over a bucket's
+// columns then fit in LDS.  workspace as for launch_transposed_products.
+void launch_bucketed_products(hipStream_t stream, idx_t m, idx_t n, idx_t nnz, const void* csr_val, const idx_t* row_ptr,
+                              const idx_t* col, const void* x, void* products, size_t value_bytes, idx_t base,
+                              void* workspace, BucketedProducts* out) {
+    uint32_t shift = 0;
+    if (m == 0 || nnz == 0 || !bucketed_products_shape(n, base, &shift)) return;
+    const Csr2CscLayout l = csr2csc_layout(nnz, value_bytes, true);
+    char* w = static_cast<char*>(workspace);
+    idx_t* keys = reinterpret_cast<idx_t*>(w + l.sorted_keys);
+    SortScratch t;  // one pass writes the outputs directly: no alternating sets
+    t.keys[0] = t.keys[1] = nullptr;
+    t.aux[0] = t.aux[1] = nullptr;
+    t.vals[0] = t.vals[1] = nullptr;
+    t.counters = reinterpret_cast<uint32_t*>(w + l.counters);
+    t.scan_ws = reinterpret_cast<uint32_t*>(w + l.scan_ws);
+    t.tile_rows = reinterpret_cast<idx_t*>(w + l.tile_rows);
+    CsrSource csr;
+    csr.rows = m;
+    csr.base = base;
+    csr.times_x = x;
+    csr.first_bit = shift;
+    radix_sort_triples(stream, nnz, 8, col, row_ptr, csr_val, keys, nullptr, products, value_bytes, t, csr);
+    out->keys = keys;
+    out->starts = t.counters;  // after the scan, counters[digit * tiles] is where the digit's keys begin
+    out->stride = sort_tiles(nnz);
+    out->shift = shift;
+    out->buckets = static_cast<uint32_t>((static_cast<uint64_t>(n) - 1 + base) >> shift) + 1;
 }
 
 // Scratch of launch_sort_by_column_band: the counters of one pass, their scan, the row starts per tile.

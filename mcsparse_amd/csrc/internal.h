@@ -359,6 +359,28 @@ void launch_transposed_products(hipStream_t stream, idx_t m, idx_t n, idx_t nnz,
                                 const idx_t* col, const void* x, void* products, idx_t* col_ptr, size_t value_bytes,
                                 idx_t base, void* workspace);
 
+// The same products in up to 256 buckets of 2^shift neighbouring column keys (index base included),
+// bucket b starting at starts[b * stride] and ending where the next begins (the last at nnz); inside a
+// bucket the pairs are in CSR order, not sorted.  One pass over the nonzeros instead of the three of a
+// full sort: for callers that then add the products of a column in any order.  The shape function says
+// whether the keys allow it (between 2^14 and 2^22 of them: a bucket's sums must fit in LDS as doubles).
+constexpr uint32_t kBucketMinKeyBits = 15;
+constexpr uint32_t kBucketMaxShift = 14;
+struct BucketedProducts {
+    const idx_t* keys = nullptr;
+    const uint32_t* starts = nullptr;
+    uint32_t stride = 0, shift = 0, buckets = 0;
+};
+bool bucketed_products_shape(idx_t n, idx_t base, uint32_t* shift);
+void launch_bucketed_products(hipStream_t stream, idx_t m, idx_t n, idx_t nnz, const void* csr_val, const idx_t* row_ptr,
+                              const idx_t* col, const void* x, void* products, size_t value_bytes, idx_t base,
+                              void* workspace, BucketedProducts* out);
+// y[c] = alpha * (sum of the products of column c) + beta * y[c] for all n columns, from such buckets;
+// the sums are formed in LDS in the order the wavefronts reach the products.
+template <typename T>
+void launch_bucket_sums(hipStream_t stream, idx_t n, idx_t nnz, idx_t base, const BucketedProducts& b, const T* products,
+                        T* y, T alpha, T beta);
+
 // One stable radix pass over the nonzeros of a CSR matrix where they lie, on band_bits (<= 8) bits
 // of the keys from bit band_shift on (key = column index, index base included): cols_out / rows_out
 // (row + base) / vals_out hold the nonzeros band by band, inside a band in CSR order.

@@ -565,6 +565,78 @@ void launch_row_sums_merge(hipStream_t stream, const SpmvArgs& a, T alpha, T bet
     launch_spmv_merge_tiles<T, kItemsInOrder, true>(stream, a, alpha, beta, workspace, false);
 }
 
+// ---- sums over the columns of bucketed products ----
+// One workgroup per bucket of 2^shift neighbouring column keys: the sums of the bucket's columns live in
+// LDS as doubles (fp32 products are widened: ds_add_f64 runs at four times the rate of ds_add_f32 on this
+// chip), the bucket's (key, product) pairs stream past once, kBucketIpt of them in flight per thread, and
+// every column of the bucket is written at the end, with or without products.
+constexpr int kBucketBlock = 1024;
+constexpr int kBucketIpt = 16;
+constexpr uint32_t kBucketDigits = 256;  // rows of the sort's counter table: one per value of a digit
+
+template <typename T>
+__global__ __launch_bounds__(kBucketBlock) void bucket_sums_kernel(idx_t n, idx_t nnz, idx_t base, uint32_t shift,
+                                                                  uint32_t stride,
+                                                                  const uint32_t* __restrict__ starts,
+                                                                  const idx_t* __restrict__ keys,
+                                                                  const T* __restrict__ products, T* __restrict__ y,
+                                                                  T alpha, T beta) {
+    extern __shared__ __align__(16) unsigned char s_raw[];
+    double* s_acc = reinterpret_cast<double*>(s_raw);
+    const uint32_t tid = threadIdx.x;
+    const uint32_t bucket = blockIdx.x;
+    const uint32_t width = 1u << shift;
+    for (uint32_t r = tid; r < width; r += kBucketBlock) s_acc[r] = 0.0;
+    idx_t e0 = starts[static_cast<uint64_t>(bucket) * stride];
+    idx_t e1 = bucket + 1 < kBucketDigits ? starts[static_cast<uint64_t>(bucket + 1) * stride] : nnz;
+    e0 = e0 < nnz ? e0 : nnz;
+    e1 = e1 < nnz ? e1 : nnz;
+    e1 = e1 > e0 ? e1 : e0;
+    __syncthreads();
+    for (idx_t slab = e0; slab < e1; slab += kBucketBlock * kBucketIpt) {
+        const uint32_t cnt = e1 - slab < static_cast<idx_t>(kBucketBlock * kBucketIpt) ? e1 - slab
+                                                                                       : kBucketBlock * kBucketIpt;
+        idx_t key[kBucketIpt];
+        T p[kBucketIpt];
+#pragma unroll
+        for (int i = 0; i < kBucketIpt; ++i) {
+            const uint32_t k = min(static_cast<uint32_t>(i) * kBucketBlock + tid, cnt - 1);
+            key[i] = load_stream(keys + slab + k);
+            p[i] = load_stream(products + slab + k);
+        }
+#pragma unroll
+        for (int i = 0; i < kBucketIpt; ++i) {
+            const uint32_t k = static_cast<uint32_t>(i) * kBucketBlock + tid;
+            // the low bits of a key are its place in the bucket, whatever the key holds
+            if (k < cnt) unsafeAtomicAdd(&s_acc[key[i] & (width - 1)], static_cast<double>(p[i]));
+        }
+    }
+    __syncthreads();
+    const uint64_t key0 = static_cast<uint64_t>(bucket) << shift;
+    for (uint32_t r = tid; r < width; r += kBucketBlock) {
+        const uint64_t k = key0 + r;
+        if (k < base || k - base >= n) continue;  // keys below the index base and past the last column
+        const uint64_t c = k - base;
+        const T s = alpha * static_cast<T>(s_acc[r]);
+        y[c] = beta == T(0) ? s : s + beta * y[c];
+    }
+}
+
+template <typename T>
+void launch_bucket_sums(hipStream_t stream, idx_t n, idx_t nnz, idx_t base, const BucketedProducts& b, const T* products,
+                        T* y, T alpha, T beta) {
+    if (b.buckets == 0 || b.buckets > kBucketDigits || b.shift > kBucketMaxShift) return;
+    const size_t lds = sizeof(double) << b.shift;
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(bucket_sums_kernel<T>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
+    hipLaunchKernelGGL((bucket_sums_kernel<T>), dim3(b.buckets), dim3(kBucketBlock), lds, stream, n, nnz, base, b.shift,
+                       b.stride, b.starts, b.keys, products, y, alpha, beta);
+}
+
+template void launch_bucket_sums<float>(hipStream_t, idx_t, idx_t, idx_t, const BucketedProducts&, const float*, float*,
+                                        float, float);
+template void launch_bucket_sums<double>(hipStream_t, idx_t, idx_t, idx_t, const BucketedProducts&, const double*,
+                                         double*, double, double);
 template void launch_row_sums_merge<float>(hipStream_t, const SpmvArgs&, float, float, void*);
 template void launch_row_sums_merge<double>(hipStream_t, const SpmvArgs&, double, double, void*);
 template void launch_spmv_vector<float>(hipStream_t, const SpmvArgs&, float, float, int);

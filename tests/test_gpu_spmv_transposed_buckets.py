@@ -1,0 +1,119 @@
+"""GPU parity of the transposing mcsparseSpMV without a preprocess call (CSR op T, CSC op N, COO op T).
+
+With 2^14 .. 2^22 column keys and any algorithm but MCSPARSE_SPMV_CSR_ALG2 the call orders the products
+value * x[row] by the top eight bits of their column only and forms the sums of each bucket of columns in LDS,
+in the order the products arrive; outside that range, and under ALG2, it sorts them completely and adds them in
+row order.  Integer-valued operands make every order of summation exact, so those cases are compared bit for
+bit; the rest within 8*u*(|alpha| (|A|^T |x|)_i + |beta y_i|)."""
+import numpy as np
+import pytest
+
+from mcsparse_amd import api
+from mcsparse_amd import workloads as wl
+
+from gpu_util import assert_within, dev
+
+pytestmark = pytest.mark.gpu
+
+
+def run(torch, handle, a, x, y, alpha, beta, fmt=api.FORMAT_CSR, index_type=api.INDEX_32I, alg=api.SPMV_ALG_DEFAULT,
+        repeats=1):
+    """alpha * A^T x + beta * y for the m x n matrix `a`, asked for in the way the format transposes: CSR and COO
+    arrays with op T, the same arrays read as the CSC of the n x m transpose with op N."""
+    itype = np.int64 if index_type == api.INDEX_64I else np.int32
+    first = a.ptr if fmt != api.FORMAT_COO else np.repeat(np.arange(a.m) + a.base, a.row_lengths())
+    d_first, d_col, d_val = dev(torch, first.astype(itype)), dev(torch, a.col.astype(itype)), dev(torch, a.val)
+    shape = (a.n, a.m) if fmt == api.FORMAT_CSC else (a.m, a.n)
+    op = api.OP_N if fmt == api.FORMAT_CSC else api.OP_T
+    mat = api.SpMat(shape[0], shape[1], a.nnz, d_first, d_col, d_val, base=a.base, fmt=fmt, index_type=index_type)
+    d_x, d_y = dev(torch, x), dev(torch, y)
+    vx, vy = api.DnVec(d_x), api.DnVec(d_y)
+    ct = api.maca_type(a.val.dtype)
+    st, size = api.spmv_buffer_size(handle, op, alpha, mat, vx, beta, vy, ct)
+    assert st == api.STATUS_SUCCESS
+    buf = torch.empty(size, dtype=torch.uint8, device="cuda")
+    out = []
+    for _ in range(repeats):
+        d_y.copy_(torch.from_numpy(y))
+        assert api.spmv(handle, op, alpha, mat, vx, beta, vy, ct, buf, alg=alg) == api.STATUS_SUCCESS
+        torch.cuda.synchronize()
+        out.append(d_y.cpu().numpy())
+    return out if repeats > 1 else out[0]
+
+
+def integer_valued(a, seed):
+    rng = np.random.default_rng(seed)
+    a.val[:] = rng.integers(-3, 4, a.nnz)
+    x = rng.integers(-4, 5, a.m).astype(a.val.dtype)
+    y = rng.integers(-8, 9, a.n).astype(a.val.dtype)
+    return x, y
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("base", [0, 1])
+@pytest.mark.parametrize("n", [16384, 16385, 100003, 1 << 20, 1 << 22])
+def test_exact_on_integers_across_the_key_range(torch_gpu, handle, dtype, base, n):
+    # 16384 columns from base 0 are 14 key bits (the full sort), 16385 are 15 (the first bucketed shape); 2^22
+    # columns from base 1 are 23 (the full sort again)
+    a = wl.random_ragged(3001, n, 40, dtype=dtype, seed=n % 97 + base, base=base)
+    x, y = integer_valued(a, n)
+    want = 2 * (a.to_scipy().T.astype(np.float64) @ x.astype(np.float64)) - 3 * y
+    got = run(torch_gpu, handle, a, x, y, 2.0, -3.0)
+    assert np.array_equal(got.astype(np.float64), want), "n=%d base=%d" % (n, base)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_within_the_bound_and_columns_without_entries(torch_gpu, handle, oracle, dtype):
+    # 200 rows of 30 entries over 70001 columns: most columns have no entry and must still get beta * y
+    a = wl.random_ragged(200, 70001, 30, dtype=dtype, seed=5, empty_fraction=0.5)
+    rng = np.random.default_rng(6)
+    x = rng.uniform(-1, 1, a.m).astype(dtype)
+    y = rng.uniform(-1, 1, a.n).astype(dtype)
+    for alpha, beta in ((1.0, 0.0), (-0.75, 1.25), (0.0, 2.0)):
+        got = run(torch_gpu, handle, a, x, y, alpha, beta)
+        y_ref, bound = oracle.spmv(True, a.m, a.n, a.base, a.ptr, a.col, a.val, alpha, beta, x, y)
+        assert_within(got, y_ref, bound, dtype, what="alpha %g beta %g" % (alpha, beta))
+    # beta = 0 never reads y: what was there does not matter, in any column
+    got = run(torch_gpu, handle, a, x, np.full(a.n, np.nan, dtype), 1.0, 0.0)
+    y_ref, bound = oracle.spmv(True, a.m, a.n, a.base, a.ptr, a.col, a.val, 1.0, 0.0, x, np.zeros(a.n, dtype))
+    assert_within(got, y_ref, bound, dtype, what="y of NaN under beta 0")
+
+
+def test_one_column_with_most_of_the_entries(torch_gpu, handle):
+    # every row has an entry in column 40000: one LDS sum takes 50000 products, one bucket most of the matrix
+    m, n = 50000, 300000
+    rng = np.random.default_rng(11)
+    others = np.sort(rng.integers(0, n - 1, (m, 3)), axis=1)
+    others[others >= 40000] += 1  # keep column 40000 for the common entry
+    col = np.sort(np.concatenate([others, np.full((m, 1), 40000)], axis=1), axis=1)
+    keep = np.ones(col.shape, bool)
+    keep[:, 1:] = col[:, 1:] != col[:, :-1]  # no duplicates inside a row
+    lens = keep.sum(axis=1)
+    a = wl.Csr(m, n, np.concatenate([[0], np.cumsum(lens)]), col[keep], np.zeros(int(lens.sum()), np.float64))
+    x, y = integer_valued(a, 12)
+    want = a.to_scipy().T @ x + y
+    got = run(torch_gpu, handle, a, x, y, 1.0, 1.0)
+    assert np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("fmt", [api.FORMAT_CSR, api.FORMAT_CSC, api.FORMAT_COO])
+@pytest.mark.parametrize("index_type", [api.INDEX_32I, api.INDEX_64I])
+def test_every_format_that_transposes(torch_gpu, handle, fmt, index_type):
+    a = wl.random_ragged(20011, 50021, 9, dtype=np.float32, seed=20 + fmt, base=1)
+    x, y = integer_valued(a, 21)
+    want = (a.to_scipy().T.astype(np.float64) @ x.astype(np.float64)) + 2 * y
+    got = run(torch_gpu, handle, a, x, y, 1.0, 2.0, fmt=fmt, index_type=index_type)
+    assert np.array_equal(got.astype(np.float64), want)
+
+
+def test_alg2_repeats_its_bits_and_both_agree(torch_gpu, handle, oracle):
+    a = wl.power_law(m=60000, n=90001, max_len=20000, dtype=np.float32)
+    rng = np.random.default_rng(31)
+    x = rng.uniform(-1, 1, a.m).astype(np.float32)
+    y = rng.uniform(-1, 1, a.n).astype(np.float32)
+    y_ref, bound = oracle.spmv(True, a.m, a.n, a.base, a.ptr, a.col, a.val, 1.5, 0.5, x, y)
+    first, second = run(torch_gpu, handle, a, x, y, 1.5, 0.5, alg=api.SPMV_CSR_ALG2, repeats=2)
+    assert np.array_equal(first, second)
+    assert_within(first, y_ref, bound, np.float32, what="sorted products")
+    for got in run(torch_gpu, handle, a, x, y, 1.5, 0.5, repeats=2):
+        assert_within(got, y_ref, bound, np.float32, what="bucketed products")
