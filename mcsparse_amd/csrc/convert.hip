@@ -459,6 +459,7 @@ struct ValueOf<8> { typedef uint64_t type; };
 
 // AUX = false: (key, value) pairs, rows_out is not written.  TIMES_X (with FROM_CSR, without AUX): the
 // value that travels is value * x[row of the nonzero], in the floating-point type of VB bytes.
+// short_keys (TIMES_X only, shift <= 16): keys_out is an array of uint16_t that receives the key bits below `shift`.
 template <int VB>
 struct RealOf { typedef float type; };
 template <>
@@ -469,7 +470,7 @@ __global__ __launch_bounds__(kSortBlock) void radix_scatter_kernel(
     const idx_t* __restrict__ keys_in, const idx_t* __restrict__ rows_in, const void* __restrict__ vals_in_v,
     idx_t* __restrict__ keys_out, idx_t* __restrict__ rows_out, void* __restrict__ vals_out_v, idx_t count,
     uint32_t shift, uint32_t bits, uint32_t tiles, const uint32_t* __restrict__ counters,
-    const idx_t* __restrict__ tile_rows, idx_t base, const void* __restrict__ x_v) {
+    const idx_t* __restrict__ tile_rows, idx_t base, const void* __restrict__ x_v, bool short_keys) {
     static_assert(AUX || VB != 0, "pairs carry a value");
     static_assert(!TIMES_X || (FROM_CSR && !AUX), "products are formed where the rows are worked out");
     typedef typename ValueOf<VB>::type val_t;
@@ -652,7 +653,13 @@ __global__ __launch_bounds__(kSortBlock) void radix_scatter_kernel(
             const idx_t k = s_keys[slot];
             const uint32_t d = (k >> shift) & mask;
             const uint64_t out = static_cast<uint64_t>(s_dest[d]) + (slot - s_start[d]);
-            keys_out[out] = k;
+            if constexpr (TIMES_X) {
+                // short_keys: the last pass of a sort on the top bits keeps only what lies below them, in 16 bits
+                if (short_keys) reinterpret_cast<uint16_t*>(keys_out)[out] = static_cast<uint16_t>(k & ((1u << shift) - 1u));
+                else keys_out[out] = k;
+            } else {
+                keys_out[out] = k;
+            }
             if constexpr (AUX) rows_out[out] = s_rows[slot];
             if constexpr (VB != 0) vals_out[out] = s_vals[slot];
         }
@@ -689,30 +696,30 @@ template <int VB>
 void launch_scatter(hipStream_t stream, bool from_csr, uint32_t grid, const idx_t* keys_in, const idx_t* aux_in,
                     const void* vals_in, idx_t* keys_out, idx_t* aux_out, void* vals_out, idx_t count, uint32_t shift,
                     uint32_t bits, uint32_t tiles, const uint32_t* counters, const idx_t* tile_rows, idx_t base,
-                    bool pairs, const void* x) {
+                    bool pairs, const void* x, bool short_keys) {
     const void* none = nullptr;
     if constexpr (VB != 0) {
         if (pairs && from_csr) {
             hipLaunchKernelGGL((radix_scatter_kernel<VB, true, false, true>), dim3(grid), dim3(kSortBlock), 0, stream, keys_in,
                                aux_in, vals_in, keys_out, aux_out, vals_out, count, shift, bits, tiles, counters, tile_rows,
-                               base, x);
+                               base, x, short_keys);
             return;
         }
         if (pairs) {
             hipLaunchKernelGGL((radix_scatter_kernel<VB, false, false, false>), dim3(grid), dim3(kSortBlock), 0, stream, keys_in,
                                aux_in, vals_in, keys_out, aux_out, vals_out, count, shift, bits, tiles, counters, tile_rows,
-                               base, none);
+                               base, none, false);
             return;
         }
     }
     if (from_csr) {
         hipLaunchKernelGGL((radix_scatter_kernel<VB, true, true, false>), dim3(grid), dim3(kSortBlock), 0, stream, keys_in,
                            aux_in, vals_in, keys_out, aux_out, vals_out, count, shift, bits, tiles, counters, tile_rows, base,
-                           none);
+                           none, false);
     } else {
         hipLaunchKernelGGL((radix_scatter_kernel<VB, false, true, false>), dim3(grid), dim3(kSortBlock), 0, stream, keys_in,
                            aux_in, vals_in, keys_out, aux_out, vals_out, count, shift, bits, tiles, counters, tile_rows, base,
-                           none);
+                           none, false);
     }
 }
 
@@ -726,6 +733,9 @@ struct CsrSource {
     const void* times_x = nullptr;
     // lowest key bit the sort looks at: the keys are ordered by bits [first_bit, first_bit + key_bits)
     uint32_t first_bit = 0;
+    // with times_x, in a sort of one pass: keys_out is an array of uint16_t that receives the key bits below
+    // first_bit (<= 16 of them), which is all that tells the keys of one digit apart
+    bool short_keys = false;
 };
 
 // Stable LSD radix sort of (key, aux, value) triples on the low key_bits of the keys, in
@@ -756,7 +766,8 @@ void radix_sort_triples(hipStream_t stream, idx_t count, uint32_t key_bits, cons
         launch_exclusive_scan(stream, t.counters, static_cast<uint64_t>(radix) * tiles, t.scan_ws);
         auto* launch = value_bytes == 0 ? launch_scatter<0> : value_bytes == 4 ? launch_scatter<4> : launch_scatter<8>;
         launch(stream, from_csr, scatter_grid, keys_in, aux_in, vals_in, k_out, a_out, v_out, count, shift, bits, tiles,
-               t.counters, t.tile_rows, csr.base, csr.times_x != nullptr, csr.times_x);
+               t.counters, t.tile_rows, csr.base, csr.times_x != nullptr, csr.times_x,
+               csr.short_keys && last && from_csr);
         keys_in = k_out;
         aux_in = a_out;
         vals_in = v_out;
@@ -963,7 +974,8 @@ bool bucketed_products_shape(idx_t n, idx_t base, uint32_t* shift) {
 // One pass of the same sort, for a transposing SpMV that may add the products of a column in any order:
 // (column, value * x[row]) pairs ordered by the top eight bits of the column keys only, that is in up to
 // 256 buckets of 2^shift neighbouring columns, inside a bucket in CSR order.  The sums over a bucket's
-// columns then fit in LDS.  workspace as for launch_transposed_products.
+// columns then fit in LDS.  Of a key only its place in the bucket is written, as 16 bits: a quarter fewer
+// bytes for this pass to write and the sums to read.  workspace as for launch_transposed_products.
 void launch_bucketed_products(hipStream_t stream, idx_t m, idx_t n, idx_t nnz, const void* csr_val, const idx_t* row_ptr,
                               const idx_t* col, const void* x, void* products, size_t value_bytes, idx_t base,
                               void* workspace, BucketedProducts* out) {
@@ -971,7 +983,7 @@ void launch_bucketed_products(hipStream_t stream, idx_t m, idx_t n, idx_t nnz, c
     if (m == 0 || nnz == 0 || !bucketed_products_shape(n, base, &shift)) return;
     const Csr2CscLayout l = csr2csc_layout(nnz, value_bytes, true);
     char* w = static_cast<char*>(workspace);
-    idx_t* keys = reinterpret_cast<idx_t*>(w + l.sorted_keys);
+    idx_t* keys = reinterpret_cast<idx_t*>(w + l.sorted_keys);  // room for 32-bit keys, used for 16-bit ones
     SortScratch t;  // one pass writes the outputs directly: no alternating sets
     t.keys[0] = t.keys[1] = nullptr;
     t.aux[0] = t.aux[1] = nullptr;
@@ -984,8 +996,9 @@ void launch_bucketed_products(hipStream_t stream, idx_t m, idx_t n, idx_t nnz, c
     csr.base = base;
     csr.times_x = x;
     csr.first_bit = shift;
+    csr.short_keys = true;
     radix_sort_triples(stream, nnz, 8, col, row_ptr, csr_val, keys, nullptr, products, value_bytes, t, csr);
-    out->keys = keys;
+    out->keys = reinterpret_cast<const uint16_t*>(keys);
     out->starts = t.counters;  // after the scan, counters[digit * tiles] is where the digit's keys begin
     out->stride = sort_tiles(nnz);
     out->shift = shift;

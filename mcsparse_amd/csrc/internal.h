@@ -361,13 +361,14 @@ void launch_transposed_products(hipStream_t stream, idx_t m, idx_t n, idx_t nnz,
 
 // The same products in up to 256 buckets of 2^shift neighbouring column keys (index base included),
 // bucket b starting at starts[b * stride] and ending where the next begins (the last at nnz); inside a
-// bucket the pairs are in CSR order, not sorted.  One pass over the nonzeros instead of the three of a
+// bucket the pairs are in CSR order, not sorted, and keys[] holds a key's low `shift` bits, its place in
+// the bucket.  Both arrays may be read up to the next even index past nnz.  One pass over the nonzeros instead of the three of a
 // full sort: for callers that then add the products of a column in any order.  The shape function says
 // whether the keys allow it (between 2^14 and 2^22 of them: a bucket's sums must fit in LDS as doubles).
 constexpr uint32_t kBucketMinKeyBits = 15;
 constexpr uint32_t kBucketMaxShift = 14;
 struct BucketedProducts {
-    const idx_t* keys = nullptr;
+    const uint16_t* keys = nullptr;
     const uint32_t* starts = nullptr;
     uint32_t stride = 0, shift = 0, buckets = 0;
 };

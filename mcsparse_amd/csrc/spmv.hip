@@ -568,19 +568,25 @@ void launch_row_sums_merge(hipStream_t stream, const SpmvArgs& a, T alpha, T bet
 // ---- sums over the columns of bucketed products ----
 // One workgroup per bucket of 2^shift neighbouring column keys: the sums of the bucket's columns live in
 // LDS as doubles (fp32 products are widened: ds_add_f64 runs at four times the rate of ds_add_f32 on this
-// chip), the bucket's (key, product) pairs stream past once, kBucketIpt of them in flight per thread, and
+// chip), the bucket's (key, product) pairs stream past once, 2 * kBucketIpt of them in flight per thread, and
 // every column of the bucket is written at the end, with or without products.
 constexpr int kBucketBlock = 1024;
-constexpr int kBucketIpt = 16;
+constexpr int kBucketIpt = 8;  // loads of two pairs each
 constexpr uint32_t kBucketDigits = 256;  // rows of the sort's counter table: one per value of a digit
+
+template <typename T>
+struct PairOf { typedef float type __attribute__((ext_vector_type(2))); };
+template <>
+struct PairOf<double> { typedef double type __attribute__((ext_vector_type(2))); };
 
 template <typename T>
 __global__ __launch_bounds__(kBucketBlock) void bucket_sums_kernel(idx_t n, idx_t nnz, idx_t base, uint32_t shift,
                                                                   uint32_t stride,
                                                                   const uint32_t* __restrict__ starts,
-                                                                  const idx_t* __restrict__ keys,
+                                                                  const uint16_t* __restrict__ keys,
                                                                   const T* __restrict__ products, T* __restrict__ y,
                                                                   T alpha, T beta) {
+    typedef typename PairOf<T>::type pair_t;
     extern __shared__ __align__(16) unsigned char s_raw[];
     double* s_acc = reinterpret_cast<double*>(s_raw);
     const uint32_t tid = threadIdx.x;
@@ -593,22 +599,31 @@ __global__ __launch_bounds__(kBucketBlock) void bucket_sums_kernel(idx_t n, idx_
     e1 = e1 < nnz ? e1 : nnz;
     e1 = e1 > e0 ? e1 : e0;
     __syncthreads();
-    for (idx_t slab = e0; slab < e1; slab += kBucketBlock * kBucketIpt) {
-        const uint32_t cnt = e1 - slab < static_cast<idx_t>(kBucketBlock * kBucketIpt) ? e1 - slab
+    // Two neighbouring pairs per load (the vector memory unit takes a load instruction of a wavefront in
+    // the same time whatever its width): entries 2q and 2q + 1, of which the first of the bucket's first
+    // load and the second of its last may belong to a neighbour.
+    const uint32_t* keys2 = reinterpret_cast<const uint32_t*>(keys);
+    const pair_t* products2 = reinterpret_cast<const pair_t*>(products);
+    const idx_t q0 = e0 / 2;
+    const idx_t q1 = e1 / 2 + (e1 & 1u);  // e1 <= nnz < 2^32: no overflow
+    for (idx_t slab = q0; slab < q1; slab += kBucketBlock * kBucketIpt) {
+        const uint32_t cnt = q1 - slab < static_cast<idx_t>(kBucketBlock * kBucketIpt) ? q1 - slab
                                                                                        : kBucketBlock * kBucketIpt;
-        idx_t key[kBucketIpt];
-        T p[kBucketIpt];
+        uint32_t key[kBucketIpt];
+        pair_t p[kBucketIpt];
 #pragma unroll
         for (int i = 0; i < kBucketIpt; ++i) {
             const uint32_t k = min(static_cast<uint32_t>(i) * kBucketBlock + tid, cnt - 1);
-            key[i] = load_stream(keys + slab + k);
-            p[i] = load_stream(products + slab + k);
+            key[i] = load_stream(keys2 + slab + k);
+            p[i] = load_stream(products2 + slab + k);
         }
 #pragma unroll
         for (int i = 0; i < kBucketIpt; ++i) {
             const uint32_t k = static_cast<uint32_t>(i) * kBucketBlock + tid;
+            const uint64_t e = (static_cast<uint64_t>(slab) + k) * 2;
             // the low bits of a key are its place in the bucket, whatever the key holds
-            if (k < cnt) unsafeAtomicAdd(&s_acc[key[i] & (width - 1)], static_cast<double>(p[i]));
+            if (k < cnt && e >= e0) unsafeAtomicAdd(&s_acc[key[i] & (width - 1)], static_cast<double>(p[i].x));
+            if (k < cnt && e + 1 < e1) unsafeAtomicAdd(&s_acc[(key[i] >> 16) & (width - 1)], static_cast<double>(p[i].y));
         }
     }
     __syncthreads();
