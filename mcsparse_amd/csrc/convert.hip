@@ -484,6 +484,11 @@ __global__ __launch_bounds__(kSortBlock) void radix_scatter_kernel(
     __shared__ idx_t s_keys[kSortTile];
     __shared__ idx_t s_rows[(AUX || FROM_CSR) ? kSortTile : 1];
     __shared__ val_t s_vals[VB ? kSortTile : 1];
+    // FROM_CSR: one bit per nonzero of the tile that begins a row, how many rows begin before each 64 of
+    // them, and whether two rows begin at the same nonzero (an empty row)
+    __shared__ unsigned long long s_begins[FROM_CSR ? kSortTile / kWave : 1];
+    __shared__ uint32_t s_begins_before[FROM_CSR ? kSortTile / kWave : 1];
+    __shared__ uint32_t s_empty_rows;
 
     const uint32_t tid = threadIdx.x;
     const unsigned lane = tid % kWave;
@@ -501,6 +506,10 @@ __global__ __launch_bounds__(kSortBlock) void radix_scatter_kernel(
         static_cast<uint32_t>(count - tile_start < kSortTile ? count - tile_start : kSortTile);
 
     for (uint32_t i = tid; i < kSortWaves * kMaxRadix; i += kSortBlock) (&s_cnt[0][0])[i] = 0;
+    if constexpr (FROM_CSR) {
+        if (tid < kSortTile / kWave) s_begins[tid] = 0;
+        if (tid == 0) s_empty_rows = 0;
+    }
     __syncthreads();
 
     // FROM_CSR: the row starts that fall inside the tile, relative to it, go to LDS (s_rows is
@@ -575,14 +584,40 @@ __global__ __launch_bounds__(kSortBlock) void radix_scatter_kernel(
 #pragma unroll
         for (int i = 0; i < kSortIpt; ++i) {
             const idx_t j = i * kSortBlock + tid;
-            if (staged && j < inside) s_rows[j] = start_of[i] - tile_first;
+            if (staged && j < inside) {
+                const idx_t at = start_of[i] - tile_first;
+                s_rows[j] = at;
+                if (at < static_cast<idx_t>(kSortTile)) {  // the tile's last row may end where the next tile begins
+                    const unsigned long long bit = 1ull << (at % kWave);
+                    if ((atomicOr(&s_begins[at / kWave], bit) & bit) != 0) s_empty_rows = 1;
+                }
+            }
         }
     }
     __syncthreads();
 
     if constexpr (FROM_CSR) {
+        // The row of a nonzero is the first row of the tile plus the rows that begin at or before it.  Without
+        // empty rows that is a count of bits: the lanes of a wavefront hold 64 neighbouring nonzeros, one word
+        // of s_begins, in every round.  Otherwise, a search per nonzero.
+        const bool by_bits = staged && s_empty_rows == 0;  // the same for the whole workgroup
+        if (by_bits) {
+            static_assert(kSortWaveItems / kWave == kSortIpt && kSortTile / kWave == kWave, "a word per wavefront and round");
+            if (wave == 0) {
+                const uint32_t c = __popcll(s_begins[lane]);
+                s_begins_before[lane] = wave_inclusive_sum(c) - c;
+            }
+            __syncthreads();
+            const unsigned long long up_to_lane = (2ull << lane) - 1ull;  // lane 63: all ones
+#pragma unroll
+            for (int i = 0; i < kSortIpt; ++i) {
+                const uint32_t word = wave * kSortIpt + i;
+                row[i] = first_row + s_begins_before[word] + __popcll(s_begins[word] & up_to_lane) + base;
+            }
+        }
 #pragma unroll
         for (int i = 0; i < kSortIpt; ++i) {
+            if (by_bits) break;
             const uint32_t p = wave * kSortWaveItems + i * kWave + lane;
             idx_t lo = 0;
             idx_t hi = inside;
