@@ -32,7 +32,7 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 
 OTHERS = ["c4-64", "c3", "c3t", "c5", "c5-spmv", "c5-coo", "c4-8", "c4-256", "c4-64-col", "c1",
-          "c2-alg2", "c3-alg2", "c3t-alg2"]
+          "c2-alg2", "c3-alg2", "c3t-alg2", "c2-direct", "c3-direct", "c3t-direct"]
 OTHERS_BUDGET_S = 200.0  # wall-clock budget of the default invocation for the workloads above
 
 
@@ -63,6 +63,10 @@ MEASURED_TRAFFIC = {
     ("c2", 0): (_traffic(653904.5, 10047.2), "profiles/spmv_vector_f64_c2_1Mx16.txt"),
     ("c3", 0): (_traffic(3305285.9 + 17229.2 + 251.2 + 3154.3, 25157.0 + 1391.2 + 1994.3 + 1375.1),
                     "profiles/spmv_merge_f32_c3_powerlaw.txt"),
+    # op T without the preprocess call: key histogram + scans + row starts per tile + one scatter pass + bucket sums
+    ("c3t", 0): (_traffic(229180.3 + 14342.5 + 2 * 7207.2 + 21132.3 + 489308.2 + 421987.3,
+                          28832.0 + 56.0 + 2 * 14325.6 + 223.8 + 692310.6 + 16384.0),
+                 "profiles/spmv_transposed_buckets_f32_c3_powerlaw.txt"),
     ("c4-64", 0): (_traffic(613893.3, 524288.0), "profiles/spmm_group_f32_c4_stencil128.txt"),
     ("c4-256", 0): (_traffic(3673719.8, 2097152.0), "profiles/spmm_group_f32_c4_stencil128.txt"),
     # group kernel (writes the column-major C itself) + the transpose of B
@@ -129,6 +133,9 @@ def describe(name):
     if name.endswith("-alg2"):
         d = describe(name[:-5])
         return d[:6] + (d[6] + ", MCSPARSE_SPMV_CSR_ALG2 (reproducible bits)",)
+    if name.endswith("-direct"):
+        d = describe(name[:-7])
+        return d[:6] + (d[6] + ", no preprocess call (the two calls the reference's API has)",)
     if name == "c1":
         return "laplacian", "spmv", False, 0, 1.0, 0.0, "fp32 CSR SpMV, 5-pt Laplacian 256x256"
     if name == "c2":
@@ -210,7 +217,7 @@ def run_workload(name, args, ctx, steps=None, warmup=None, with_cpu=True):
 
     def spmv_buffer(st, the_op, fmt_is_csr):
         """Scratch of an SpMV set: with preprocessing, the larger buffer the banded copy lives in."""
-        use_pre = not args.no_preprocess and not (args.family or args.lanes)
+        use_pre = not args.no_preprocess and not name.endswith("-direct") and not (args.family or args.lanes)
         if use_pre:
             rc, size = api.spmv_preprocess_buffer_size(handle, the_op, alpha, st["mat"], st["vx"], beta, st["vy"], ct,
                                                        alg=alg)
@@ -325,7 +332,7 @@ def run_workload(name, args, ctx, steps=None, warmup=None, with_cpu=True):
     plan = mat0.plan() if mat0 is not None and kind in ("spmv", "spmv-csc") else None
     banded = mat0.spmv_preprocess_state() if mat0 is not None and kind in ("spmv", "spmv-csc") else None
     copy_state = banded[0] if banded and banded[0] in (2, 3) else 0
-    base_name = name[:-5] if name.endswith("-alg2") else name
+    base_name = name[:-5] if name.endswith("-alg2") else name[:-7] if name.endswith("-direct") else name
     traffic = MEASURED_TRAFFIC.get((base_name, copy_state)) if s == 1.0 else None
 
     out = {
