@@ -158,3 +158,42 @@ def test_preprocessed_spmv_replays_in_a_hip_graph(torch_gpu, oracle, alg, state)
     del graph
     torch.cuda.synchronize()
     handle.destroy()
+
+
+@pytest.mark.parametrize("alg", [api.SPMV_ALG_DEFAULT, api.SPMV_CSR_ALG2])
+def test_transposing_spmv_replays_in_a_hip_graph(torch_gpu, oracle, alg):
+    """op T without a preprocess call: the sort passes and the column sums (in LDS by default, in row order under
+    MCSPARSE_SPMV_CSR_ALG2) are kernels only, whatever the algorithm."""
+    torch = torch_gpu
+    rng = np.random.default_rng(23)
+    side = torch.cuda.Stream()
+    handle = api.Handle(stream=side.cuda_stream)
+    a = wl.random_ragged(9000, 70001, 14, dtype=np.float32, seed=10, base=1)
+    d_ptr, d_col, d_val = dev(torch, a.ptr), dev(torch, a.col), dev(torch, a.val)
+    A = api.SpMat(a.m, a.n, a.nnz, d_ptr, d_col, d_val, base=a.base)
+    x = torch.zeros(a.m, dtype=torch.float32, device="cuda")
+    y = torch.zeros(a.n, dtype=torch.float32, device="cuda")
+    vx, vy = api.DnVec(x), api.DnVec(y)
+    st, size = api.spmv_buffer_size(handle, api.OP_T, -0.5, A, vx, 2.0, vy, api.R_32F)
+    assert st == 0
+    buf = torch.empty(size, dtype=torch.uint8, device="cuda")
+    with torch.cuda.stream(side):
+        assert api.spmv(handle, api.OP_T, -0.5, A, vx, 2.0, vy, api.R_32F, buf, alg=alg) == 0
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        assert api.spmv(handle, api.OP_T, -0.5, A, vx, 2.0, vy, api.R_32F, buf, alg=alg) == 0
+    torch.cuda.synchronize()
+    for replay in range(3):
+        hx = rng.uniform(-1, 1, a.m).astype(np.float32)
+        hy = rng.uniform(-1, 1, a.n).astype(np.float32)
+        x.copy_(torch.from_numpy(hx))
+        y.copy_(torch.from_numpy(hy))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        ref, bound = oracle.spmv(True, a.m, a.n, a.base, a.ptr, a.col, a.val, -0.5, 2.0, hx, hy)
+        assert_within(y.cpu().numpy(), ref, bound, np.float32, what="replay %d, alg %d" % (replay, alg))
+    del graph
+    torch.cuda.synchronize()
+    handle.destroy()
