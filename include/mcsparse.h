@@ -292,7 +292,8 @@ mcsparseStatus_t mcsparseDnMatGetStridedBatch(mcsparseDnMatDescr_t dnMatDescr, i
  * bits on every run whatever alg is.  A transposing call (CSR or COO with op T, CSC with op N) orders the
  * products value * x[row] by column in the buffer: completely under MCSPARSE_SPMV_CSR_ALG2, whose sums
  * then add in row order and repeat their bits; with any other value, for 2^14 to 2^22 columns, only into
- * buckets of neighbouring columns whose sums are formed in the order the products arrive, which is more
+ * buckets of neighbouring columns whose sums are formed in the order the products arrive (and for fewer
+ * columns with many nonzeros each, not at all: the sums are formed as the nonzeros lie), which is more
  * than twice as fast and stays within the same error bound, but the last bits can differ between runs. */
 mcsparseStatus_t mcsparseSpMV(mcsparseHandle_t handle, mcsparseOperation_t opA, const void* alpha,
                               mcsparseSpMatDescr_t matA, mcsparseDnVecDescr_t vecX, const void* beta,

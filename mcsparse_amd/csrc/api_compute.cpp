@@ -371,6 +371,22 @@ mcspStatus_t spmv_typed(mcsparseHandle_t h, mcsparseSpMatDescr* A, mcsparseOpera
     // Unless the caller asked for the algorithm whose bits repeat (MCSPARSE_SPMV_CSR_ALG2): one pass of
     // that sort, into buckets of neighbouring columns, and the sums of a bucket's columns formed in LDS
     // in whatever order the products arrive.
+    if (alg != MCSPARSE_SPMV_CSR_ALG2 && mcsp::skinny_transpose_shape(static_cast<idx_t>(v.n), nnz, base)) {
+        // few columns, many nonzeros in each: nothing is ordered at all.  The scratch of the sort holds the
+        // rows of the nonzeros (for CSR offsets) and the partial sums.
+        char* ws = buf + l.csr2csc_ws;
+        const idx_t* rows = v.coo_rows;
+        if (rows == nullptr) {
+            idx_t* expanded = reinterpret_cast<idx_t*>(ws);
+            mcsp::launch_csr2coo(h->stream, static_cast<idx_t>(v.m), nnz, v.ptr, base, expanded);
+            rows = expanded;
+        }
+        mcsp::launch_skinny_transpose<T>(h->stream, static_cast<idx_t>(v.m), static_cast<idx_t>(v.n), nnz, base, rows,
+                                         v.ind, static_cast<const T*>(v.val), static_cast<const T*>(x->values),
+                                         static_cast<T*>(y->values), h_alpha, h_beta,
+                                         ws + align_up(static_cast<size_t>(nnz) * sizeof(idx_t)));
+        return MCSP_STATUS_SUCCESS;
+    }
     uint32_t bucket_shift = 0;
     if (alg != MCSPARSE_SPMV_CSR_ALG2 &&
         mcsp::bucketed_products_shape(static_cast<idx_t>(v.n), base, &bucket_shift)) {

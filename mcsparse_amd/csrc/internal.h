@@ -382,6 +382,17 @@ template <typename T>
 void launch_bucket_sums(hipStream_t stream, idx_t n, idx_t nnz, idx_t base, const BucketedProducts& b, const T* products,
                         T* y, T alpha, T beta);
 
+// y = alpha * A^T x + beta * y for an m x n matrix with fewer than 2^14 column keys and many nonzeros per
+// column, without sorting anything: shares of the nonzeros are summed into copies of y in LDS, the copies
+// into y.  rows[nnz] = row + base of every nonzero (COO rows, or csr2coo of the offsets); workspace of
+// skinny_transpose_workspace_bytes(n) bytes, which the shape function keeps below 16 bytes per nonzero.
+constexpr uint32_t kSkinnyMinNonzerosPerColumn = 128;
+bool skinny_transpose_shape(idx_t n, idx_t nnz, idx_t base);
+size_t skinny_transpose_workspace_bytes(idx_t n);
+template <typename T>
+void launch_skinny_transpose(hipStream_t stream, idx_t m, idx_t n, idx_t nnz, idx_t base, const idx_t* rows,
+                             const idx_t* col, const T* val, const T* x, T* y, T alpha, T beta, void* workspace);
+
 // One stable radix pass over the nonzeros of a CSR matrix where they lie, on band_bits (<= 8) bits
 // of the keys from bit band_shift on (key = column index, index base included): cols_out / rows_out
 // (row + base) / vals_out hold the nonzeros band by band, inside a band in CSR order.

@@ -652,6 +652,101 @@ template void launch_bucket_sums<float>(hipStream_t, idx_t, idx_t, idx_t, const 
                                         float, float);
 template void launch_bucket_sums<double>(hipStream_t, idx_t, idx_t, idx_t, const BucketedProducts&, const double*,
                                          double*, double, double);
+// ---- A^T x for a matrix with few columns ----
+// With fewer than 2^14 column keys all of y fits in the LDS of one workgroup, so nothing is sorted: each
+// of kSkinnyGroups workgroups takes an equal share of the nonzeros as they lie, adds value * x[row] to
+// its own copy of y in LDS (doubles), and writes the copy out as a plane of partial sums; a second
+// kernel adds the planes up.  rows[] holds the row (+ base) of every nonzero: the COO row array, or
+// what csr2coo makes of the offsets.
+constexpr int kSkinnyGroups = 256;  // one per compute unit
+constexpr int kSkinnyBlock = 1024;
+constexpr int kSkinnyIpt = 8;
+
+template <typename T>
+__global__ __launch_bounds__(kSkinnyBlock) void skinny_products_kernel(idx_t m, idx_t n, idx_t nnz, idx_t base,
+                                                                      const idx_t* __restrict__ rows,
+                                                                      const idx_t* __restrict__ col,
+                                                                      const T* __restrict__ val,
+                                                                      const T* __restrict__ x,
+                                                                      double* __restrict__ planes) {
+    extern __shared__ __align__(16) unsigned char s_raw[];
+    double* s_acc = reinterpret_cast<double*>(s_raw);
+    const uint32_t tid = threadIdx.x;
+    for (uint32_t c = tid; c < n; c += kSkinnyBlock) s_acc[c] = 0.0;
+    __syncthreads();
+    const idx_t e0 = static_cast<idx_t>(static_cast<uint64_t>(nnz) * blockIdx.x / kSkinnyGroups);
+    const idx_t e1 = static_cast<idx_t>(static_cast<uint64_t>(nnz) * (blockIdx.x + 1) / kSkinnyGroups);
+    for (idx_t slab = e0; slab < e1; slab += kSkinnyBlock * kSkinnyIpt) {
+        const uint32_t cnt = e1 - slab < static_cast<idx_t>(kSkinnyBlock * kSkinnyIpt) ? e1 - slab
+                                                                                       : kSkinnyBlock * kSkinnyIpt;
+        idx_t c[kSkinnyIpt], r[kSkinnyIpt];
+        T v[kSkinnyIpt], xr[kSkinnyIpt];
+#pragma unroll
+        for (int i = 0; i < kSkinnyIpt; ++i) {
+            const uint32_t k = min(static_cast<uint32_t>(i) * kSkinnyBlock + tid, cnt - 1);
+            c[i] = load_stream(col + slab + k);
+            r[i] = load_stream(rows + slab + k);
+            v[i] = load_stream(val + slab + k);
+        }
+#pragma unroll
+        for (int i = 0; i < kSkinnyIpt; ++i) {
+            const idx_t row = r[i] > base ? r[i] - base : 0;
+            xr[i] = x[min(row, m - 1)];
+        }
+#pragma unroll
+        for (int i = 0; i < kSkinnyIpt; ++i) {
+            const uint32_t k = static_cast<uint32_t>(i) * kSkinnyBlock + tid;
+            const idx_t column = c[i] > base ? c[i] - base : 0;
+            if (k < cnt) unsafeAtomicAdd(&s_acc[min(column, n - 1)], static_cast<double>(v[i] * xr[i]));
+        }
+    }
+    __syncthreads();
+    double* out = planes + static_cast<uint64_t>(blockIdx.x) * n;
+    for (uint32_t c = tid; c < n; c += kSkinnyBlock) out[c] = s_acc[c];
+}
+
+template <typename T>
+__global__ __launch_bounds__(kBlock) void skinny_reduce_kernel(idx_t n, const double* __restrict__ planes,
+                                                               T* __restrict__ y, T alpha, T beta) {
+    const uint64_t c = static_cast<uint64_t>(blockIdx.x) * kBlock + threadIdx.x;
+    if (c >= n) return;
+    double sum = 0.0;
+#pragma unroll 8
+    for (int g = 0; g < kSkinnyGroups; ++g) sum += planes[static_cast<uint64_t>(g) * n + c];
+    const T s = alpha * static_cast<T>(sum);
+    y[c] = beta == T(0) ? s : s + beta * y[c];
+}
+
+bool skinny_transpose_shape(idx_t n, idx_t nnz, idx_t base) {
+    // all keys below 2^14: a copy of y fits in LDS as doubles; enough columns that the lanes of a wavefront
+    // seldom meet on one sum; enough nonzeros that the planes are small beside them (and fit the scratch)
+    return static_cast<uint64_t>(n) + base <= (1u << kBucketMaxShift) && n >= 256 &&
+           static_cast<uint64_t>(nnz) >= static_cast<uint64_t>(kSkinnyMinNonzerosPerColumn) * n;
+}
+
+size_t skinny_transpose_workspace_bytes(idx_t n) {
+    return static_cast<size_t>(kSkinnyGroups) * n * sizeof(double);
+}
+
+template <typename T>
+void launch_skinny_transpose(hipStream_t stream, idx_t m, idx_t n, idx_t nnz, idx_t base, const idx_t* rows,
+                             const idx_t* col, const T* val, const T* x, T* y, T alpha, T beta, void* workspace) {
+    if (m == 0 || n == 0 || nnz == 0) return;
+    double* planes = static_cast<double*>(workspace);
+    const size_t lds = static_cast<size_t>(n) * sizeof(double);
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(skinny_products_kernel<T>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
+    hipLaunchKernelGGL((skinny_products_kernel<T>), dim3(kSkinnyGroups), dim3(kSkinnyBlock), lds, stream, m, n, nnz, base,
+                       rows, col, val, x, planes);
+    hipLaunchKernelGGL((skinny_reduce_kernel<T>), dim3((n + kBlock - 1) / kBlock), dim3(kBlock), 0, stream, n,
+                       static_cast<const double*>(planes), y, alpha, beta);
+}
+
+template void launch_skinny_transpose<float>(hipStream_t, idx_t, idx_t, idx_t, idx_t, const idx_t*, const idx_t*,
+                                             const float*, const float*, float*, float, float, void*);
+template void launch_skinny_transpose<double>(hipStream_t, idx_t, idx_t, idx_t, idx_t, const idx_t*, const idx_t*,
+                                              const double*, const double*, double*, double, double, void*);
+
 template void launch_row_sums_merge<float>(hipStream_t, const SpmvArgs&, float, float, void*);
 template void launch_row_sums_merge<double>(hipStream_t, const SpmvArgs&, double, double, void*);
 template void launch_spmv_vector<float>(hipStream_t, const SpmvArgs&, float, float, int);

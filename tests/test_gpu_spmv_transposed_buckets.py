@@ -117,3 +117,47 @@ def test_alg2_repeats_its_bits_and_both_agree(torch_gpu, handle, oracle):
     assert_within(first, y_ref, bound, np.float32, what="sorted products")
     for got in run(torch_gpu, handle, a, x, y, 1.5, 0.5, repeats=2):
         assert_within(got, y_ref, bound, np.float32, what="bucketed products")
+
+
+# ---- few columns, many nonzeros in each: no sort at all, copies of y in LDS ----
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("n,base", [(256, 0), (1000, 1), (16383, 1), (16384, 0), (16384, 1), (255, 0)])
+def test_few_columns_exact_on_integers(torch_gpu, handle, dtype, n, base):
+    # 16384 columns from base 1 are one key too many for a copy of y in LDS, 255 columns too few: both take
+    # other paths and must agree all the same
+    m = 340000
+    a = wl.random_ragged(m, n, 8, dtype=dtype, seed=n % 89 + base, base=base)  # a fifth of the rows empty
+    assert a.nnz >= 128 * n
+    x, y = integer_valued(a, n + 1)
+    want = 3 * (a.to_scipy().T.astype(np.float64) @ x.astype(np.float64)) - y
+    got = run(torch_gpu, handle, a, x, y, 3.0, -1.0)
+    assert np.array_equal(got.astype(np.float64), want), "n=%d base=%d" % (n, base)
+
+
+@pytest.mark.parametrize("fmt", [api.FORMAT_CSR, api.FORMAT_CSC, api.FORMAT_COO])
+@pytest.mark.parametrize("index_type", [api.INDEX_32I, api.INDEX_64I])
+def test_few_columns_every_format_within_the_bound(torch_gpu, handle, oracle, fmt, index_type):
+    a = wl.random_ragged(150001, 3001, 5, dtype=np.float32, seed=60 + fmt, base=1, empty_fraction=0.3)
+    assert a.nnz >= 128 * a.n
+    rng = np.random.default_rng(61)
+    x = rng.uniform(-1, 1, a.m).astype(np.float32)
+    y = rng.uniform(-1, 1, a.n).astype(np.float32)
+    y_ref, bound = oracle.spmv(True, a.m, a.n, a.base, a.ptr, a.col, a.val, -1.5, 0.75, x, y)
+    got = run(torch_gpu, handle, a, x, y, -1.5, 0.75, fmt=fmt, index_type=index_type)
+    assert_within(got, y_ref, bound, np.float32, what="fmt %d index %d" % (fmt, index_type))
+    # beta = 0 never reads y
+    got = run(torch_gpu, handle, a, x, np.full(a.n, np.nan, np.float32), 2.0, 0.0, fmt=fmt, index_type=index_type)
+    y_ref, bound = oracle.spmv(True, a.m, a.n, a.base, a.ptr, a.col, a.val, 2.0, 0.0, x, np.zeros(a.n, np.float32))
+    assert_within(got, y_ref, bound, np.float32, what="NaN in y, fmt %d index %d" % (fmt, index_type))
+
+
+def test_few_columns_alg2_repeats_its_bits(torch_gpu, handle, oracle):
+    a = wl.random_ragged(200000, 2048, 6, dtype=np.float64, seed=70)
+    rng = np.random.default_rng(71)
+    x, y = rng.uniform(-1, 1, a.m), rng.uniform(-1, 1, a.n)
+    y_ref, bound = oracle.spmv(True, a.m, a.n, a.base, a.ptr, a.col, a.val, 1.0, 1.0, x, y)
+    first, second = run(torch_gpu, handle, a, x, y, 1.0, 1.0, alg=api.SPMV_CSR_ALG2, repeats=2)
+    assert np.array_equal(first, second)
+    assert_within(first, y_ref, bound, np.float64, what="sorted products")
+    assert_within(run(torch_gpu, handle, a, x, y, 1.0, 1.0), y_ref, bound, np.float64, what="copies of y in LDS")
