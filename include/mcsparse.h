@@ -131,7 +131,9 @@ typedef enum { MCSPARSE_ORDER_COL = 1, MCSPARSE_ORDER_ROW = 2 } mcsparseOrder_t;
 /* :112-116 -- 32I arrays are processed as unsigned 32-bit (src/include/mcsp_internal_types.h:4) */
 typedef enum { MCSPARSE_INDEX_16U = 1, MCSPARSE_INDEX_32I = 2, MCSPARSE_INDEX_64I = 3 } mcsparseIndexType_t;
 
-/* :124-134 -- accepted and ignored on this path, as in the reference */
+/* :124-134 -- the reference accepts and ignores them on this path.  Here MCSPARSE_SPMV_CSR_ALG2 (= CSRMV_ALG2)
+ * selects the variants whose sums are added in a fixed order, so that two runs give the same bits; every other
+ * value the faster ones (see mcsparseSpMV and mcsparseSpMV_preprocess).  The error bound is the same. */
 typedef enum {
     MCSPARSE_MV_ALG_DEFAULT = 0,
     MCSPARSE_COOMV_ALG = 1,
