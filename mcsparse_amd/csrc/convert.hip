@@ -17,42 +17,11 @@ namespace {
 constexpr int kBlock = 256;
 
 // ------------------------------------------------------------------------------------------
-// merge-path tiles over (row ends, nonzero indices), shared by csr2coo
+// row lookups in row_ptr, shared by csr2coo and the sorts that read a CSR matrix in place
 // ------------------------------------------------------------------------------------------
-constexpr int kExpandIpt = 8;
-constexpr int kExpandTile = kBlock * kExpandIpt;
-
-// Wavefront-cooperative merge-path search: number of row ends that precede diagonal d.
-// 64 probes per round shrink the interval 64-fold, so 4M rows need 4 dependent loads instead
-// of 22.  Every lane of the wave must call this; all lanes return the same value.
-__device__ __forceinline__ idx_t wave_merge_search(uint64_t d, idx_t m, idx_t nnz, idx_t base,
-                                                   const idx_t* __restrict__ row_ptr) {
-    uint64_t lo = d > nnz ? d - nnz : 0;
-    uint64_t hi = d < m ? d : m;
-    const unsigned lane = lane_id();
-    while (lo < hi) {
-        const uint64_t span = hi - lo;
-        const uint64_t step = (span + kWave - 1) / kWave;
-        const uint64_t probe = lo + lane * step;
-        bool pred = false;
-        if (probe < hi) {
-            const uint64_t row_end = row_ptr[probe + 1] - base;
-            pred = row_end <= d - probe - 1;
-        }
-        const unsigned count = __popcll(__ballot(pred));
-        if (count == 0) {
-            hi = lo;
-        } else {
-            const uint64_t new_hi = lo + static_cast<uint64_t>(count) * step;
-            lo = lo + static_cast<uint64_t>(count - 1) * step + 1;
-            hi = new_hi < hi ? new_hi : hi;
-        }
-    }
-    return static_cast<idx_t>(lo);
-}
-
-// Number of rows r in [0, m] whose first nonzero index row_ptr[r] - base is <= g, found like the
-// merge-path search above; with g a nonzero index the answer minus one is the row that holds g.
+// Number of rows r in [0, m] whose first nonzero index row_ptr[r] - base is <= g, found with
+// 64 probes per round, which shrink the interval 64-fold (4M rows: 4 dependent loads instead of 22);
+// with g a nonzero index the answer minus one is the row that holds g.
 // Every lane of the wave must call this; all lanes return the same value.
 __device__ __forceinline__ idx_t wave_count_row_starts(const idx_t* __restrict__ row_ptr, idx_t m, idx_t base, idx_t g) {
     uint64_t lo = 0;
@@ -75,87 +44,144 @@ __device__ __forceinline__ idx_t wave_count_row_starts(const idx_t* __restrict__
     return static_cast<idx_t>(lo);
 }
 
-// coo_rows[j] = row of nonzero j (+ base).  Tiles of the merged path of (row ends, nonzeros), so empty
-// rows, 1-nonzero rows and 200k-nonzero rows all cost one item each.  A workgroup takes kExpandTiles
-// tiles in a row: only where its first tile begins has to be searched for in row_ptr (a chain of
-// dependent loads); every tile ends where the row ends loaded for it say, and the next begins there.
-// Reference semantics: src/kernels/conversion/coo2csr_device.hpp:26-41.
+// Inclusive sum over the 64 lanes of a wavefront: four shifted adds inside each row of 16 lanes,
+// then the last lane of rows 0 and 2 is added to rows 1 and 3, then lane 31 to rows 2 and 3.
+__device__ __forceinline__ uint32_t wave_inclusive_sum(uint32_t v) {
+    constexpr int kRowShr = 0x110, kRowBcast15 = 0x142, kRowBcast31 = 0x143;
+    int x = static_cast<int>(v);
+    x += __builtin_amdgcn_update_dpp(0, x, kRowShr + 1, 0xF, 0xF, false);
+    x += __builtin_amdgcn_update_dpp(0, x, kRowShr + 2, 0xF, 0xF, false);
+    x += __builtin_amdgcn_update_dpp(0, x, kRowShr + 4, 0xF, 0xF, false);
+    x += __builtin_amdgcn_update_dpp(0, x, kRowShr + 8, 0xF, 0xF, false);
+    x += __builtin_amdgcn_update_dpp(0, x, kRowBcast15, 0xA, 0xF, false);
+    x += __builtin_amdgcn_update_dpp(0, x, kRowBcast31, 0xC, 0xF, false);
+    return static_cast<uint32_t>(x);
+}
+
+// coo_rows[j] = row of nonzero j (+ base) = the number of rows that begin at or before j, minus one.
+// A tile is 4096 nonzeros.  The rows that begin inside it are read from row_ptr (the first of them is
+// known from the tile before; only where a workgroup's first tile begins is searched for, a chain of
+// dependent loads) and set bits in a 4096-bit map in LDS; a thread then writes four neighbouring rows at a
+// time, each a count of bits, as one 16-byte store.  A tile in which two rows begin at the same nonzero
+// (an empty row) cannot be told from the map: its threads search the staged row starts instead, or
+// row_ptr itself when more rows begin in the tile than LDS holds.  A workgroup takes kExpandTiles tiles in
+// a row.  Reference semantics: src/kernels/conversion/coo2csr_device.hpp:26-41.
 constexpr int kExpandTiles = 8;
+constexpr int kCooTile = 4096;
+constexpr int kCooWords = kCooTile / kWave;
+constexpr int kCooLoads = 4;  // row starts per thread and round
 __global__ __launch_bounds__(kBlock) void csr2coo_kernel(idx_t m, idx_t nnz, idx_t base,
                                                          const idx_t* __restrict__ row_ptr,
                                                          idx_t* __restrict__ coo_rows) {
-    __shared__ idx_t s_row_end[kExpandTile + 1];
-    __shared__ idx_t s_ids[kExpandTile];
-    __shared__ idx_t s_x;
+    typedef idx_t idx4 __attribute__((ext_vector_type(4)));
+    static_assert(kCooWords == kWave && kCooTile == kBlock * 16, "a word per lane; four stores of four rows per thread");
+    __shared__ idx_t s_start[kCooTile];
+    __shared__ unsigned long long s_begins[kCooWords];
+    __shared__ uint32_t s_begins_before[kCooWords];
+    __shared__ idx_t s_first;
+    __shared__ uint32_t s_empty_rows;
+    __shared__ uint32_t s_inside;
 
     const uint32_t tid = threadIdx.x;
-    const uint64_t total = static_cast<uint64_t>(m) + nnz;
-    const uint64_t d_begin = static_cast<uint64_t>(blockIdx.x) * kExpandTiles * kExpandTile;
+    const unsigned lane = tid % kWave;
+    const uint64_t group_first = static_cast<uint64_t>(blockIdx.x) * kExpandTiles * kCooTile;
+    if (group_first >= nnz) return;  // whole workgroup
     if (tid / kWave == 0) {
-        const idx_t x = wave_merge_search(d_begin, m, nnz, base, row_ptr);
-        if (tid == 0) s_x = x;
+        const idx_t c = wave_count_row_starts(row_ptr, m, base, static_cast<idx_t>(group_first));
+        if (tid == 0) s_first = c;
     }
     __syncthreads();
-    idx_t x0 = s_x;
+    uint64_t before = s_first;  // rows (of the m + 1 offsets) that begin at or before the tile's first nonzero
+    const bool wide = (reinterpret_cast<uintptr_t>(coo_rows) & 15u) == 0;
     for (int t = 0; t < kExpandTiles; ++t) {
-        const uint64_t d0 = d_begin + static_cast<uint64_t>(t) * kExpandTile;
-        if (d0 >= total) break;  // whole workgroup
-        const uint64_t d1 = d0 + kExpandTile < total ? d0 + kExpandTile : total;
-        const idx_t y0 = static_cast<idx_t>(d0 - x0);
-        // Row ends from row x0 on, a workgroup's width at a time, until the row is in at which the tile
-        // ends: row x0 + i with its nonzeros and its end lies before d1 when x0 + i + end + 1 <= d1.
-        // Rows past the matrix end nowhere.
-        uint32_t last = 0;
-        for (uint32_t loaded = 0;; loaded += kBlock) {
-            const uint32_t i = loaded + tid;
-            if (i <= kExpandTile) {
-                const uint64_t r = static_cast<uint64_t>(x0) + i;
-                s_row_end[i] = r < m ? row_ptr[r + 1] - base : 0xFFFFFFFFu;
-            }
-            __syncthreads();
-            last = min(loaded + kBlock - 1, static_cast<uint32_t>(kExpandTile));
-            if (last == kExpandTile || static_cast<uint64_t>(x0) + last + s_row_end[last] + 1 > d1) break;
-        }
-        // rows that lie in the tile with their ends: the first `tile_rows` of them
-        uint32_t lo = 0, hi = last + 1;
-        while (lo < hi) {
-            const uint32_t mid = (lo + hi) >> 1;
-            if (static_cast<uint64_t>(x0) + mid + s_row_end[mid] + 1 <= d1) lo = mid + 1; else hi = mid;
-        }
-        const idx_t tile_rows = lo;
-        const idx_t x1 = x0 + tile_rows;
-        const idx_t y1 = static_cast<idx_t>(d1 - x1);
-        const idx_t tile_nnz = y1 - y0;
-        const idx_t tile_items = tile_rows + tile_nnz;
-
-        const idx_t dt = min(static_cast<idx_t>(tid * kExpandIpt), tile_items);
-        lo = dt > tile_nnz ? dt - tile_nnz : 0;
-        hi = dt < tile_rows ? dt : tile_rows;
-        while (lo < hi) {
-            const idx_t mid = (lo + hi) >> 1;
-            if (s_row_end[mid] <= y0 + (dt - mid - 1)) {
-                lo = mid + 1;
-            } else {
-                hi = mid;
-            }
-        }
-        idx_t row_l = lo;
-        idx_t nz = y0 + (dt - lo);
-#pragma unroll
-        for (int i = 0; i < kExpandIpt; ++i) {
-            if (dt + i < tile_items) {
-                if (nz < s_row_end[row_l]) {
-                    s_ids[nz - y0] = x0 + row_l + base;
-                    ++nz;
-                } else {
-                    ++row_l;
-                }
-            }
+        const uint64_t j0 = group_first + static_cast<uint64_t>(t) * kCooTile;
+        if (j0 >= nnz) break;  // whole workgroup
+        const uint32_t count = static_cast<uint32_t>(nnz - j0 < kCooTile ? nnz - j0 : kCooTile);
+        if (tid < kCooWords) s_begins[tid] = 0;
+        if (tid == 0) {
+            s_empty_rows = 0;
+            s_inside = 0;
         }
         __syncthreads();
-        for (idx_t k = tid; k < tile_nnz; k += kBlock) coo_rows[y0 + k] = s_ids[k];
-        __syncthreads();  // the next tile writes both arrays again
-        x0 = x1;
+        // the offsets from `before` on, until one lies past the tile: those up to j0 + 4096 begin a row of this
+        // tile (or, at j0 + 4096 itself, are counted for the next one)
+        uint32_t inside = 0;
+        for (uint32_t loaded = 0;; loaded += kBlock * kCooLoads) {
+            uint64_t at[kCooLoads];
+#pragma unroll
+            for (int k = 0; k < kCooLoads; ++k) {
+                const uint64_t r = before + loaded + static_cast<uint32_t>(k) * kBlock + tid;
+                const uint64_t r_read = r <= m ? r : m;
+                const idx_t v = row_ptr[r_read];
+                at[k] = r <= m ? static_cast<uint64_t>(v - base) - j0 : ~0ull;  // > 0: row `before` begins after j0
+            }
+            uint32_t mine = 0;  // one past the last offset of this thread that lies inside
+#pragma unroll
+            for (int k = 0; k < kCooLoads; ++k) {
+                if (at[k] > static_cast<uint64_t>(kCooTile)) continue;
+                const uint32_t i = loaded + static_cast<uint32_t>(k) * kBlock + tid;
+                mine = i + 1;
+                if (i < static_cast<uint32_t>(kCooTile)) s_start[i] = static_cast<idx_t>(at[k]);
+                if (at[k] < static_cast<uint64_t>(kCooTile)) {
+                    const unsigned long long bit = 1ull << (at[k] % kWave);
+                    if ((atomicOr(&s_begins[at[k] / kWave], bit) & bit) != 0) s_empty_rows = 1;
+                }
+            }
+            // the offsets ascend, so those inside come first: their number is where the last one stands
+            if (mine != 0) atomicMax(&s_inside, mine);
+            __syncthreads();
+            inside = s_inside;
+            if (inside < loaded + kBlock * kCooLoads) break;  // whole workgroup: the round held one past the tile
+        }
+        const bool by_bits = s_empty_rows == 0;  // the same for the whole workgroup
+        if (by_bits) {
+            if (tid < kWave) {
+                const uint32_t c = __popcll(s_begins[lane]);
+                s_begins_before[lane] = wave_inclusive_sum(c) - c;
+            }
+            __syncthreads();
+        }
+        const bool staged = inside <= static_cast<uint32_t>(kCooTile);
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const uint32_t p = (static_cast<uint32_t>(k) * kBlock + tid) * 4;  // four neighbouring nonzeros of the tile
+            if (p >= count) continue;
+            idx_t rows[4];
+            if (by_bits) {
+                const uint32_t word = p / kWave, bit = p % kWave;
+                const unsigned long long w = s_begins[word];
+                // rows that begin before nonzero p, then one more for every bit of the four at p .. p + 3
+                idx_t row = static_cast<idx_t>(before + s_begins_before[word] + __popcll(w & ((1ull << bit) - 1ull)) - 1 + base);
+                const uint32_t four = static_cast<uint32_t>(w >> bit) & 0xFu;  // bit <= 60
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    row += (four >> e) & 1u;
+                    rows[e] = row;
+                }
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    uint32_t lo = 0, hi = inside;  // row starts of the tile at or before nonzero p + e
+                    while (lo < hi) {
+                        const uint32_t mid = (lo + hi) >> 1;
+                        const uint64_t begins = staged ? s_start[mid] : static_cast<uint64_t>(row_ptr[before + mid] - base) - j0;
+                        if (begins <= p + e) lo = mid + 1; else hi = mid;
+                    }
+                    rows[e] = static_cast<idx_t>(before + lo - 1 + base);
+                }
+            }
+            idx_t* out = coo_rows + j0 + p;
+            if (wide && p + 4 <= count) {
+                idx4 v = {rows[0], rows[1], rows[2], rows[3]};
+                __builtin_nontemporal_store(v, reinterpret_cast<idx4*>(out));
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    if (p + e < count) out[e] = rows[e];
+            }
+        }
+        before += inside;
+        __syncthreads();  // the next tile clears the map
     }
 }
 
@@ -412,20 +438,6 @@ __global__ __launch_bounds__(kHistBlock) void radix_hist_kernel(const idx_t* __r
     }
     __syncthreads();
     if (threadIdx.x < radix) counters[static_cast<uint64_t>(threadIdx.x) * tiles + tile] = s_cnt[threadIdx.x];
-}
-
-// Inclusive sum over the 64 lanes of a wavefront: four shifted adds inside each row of 16 lanes,
-// then the last lane of rows 0 and 2 is added to rows 1 and 3, then lane 31 to rows 2 and 3.
-__device__ __forceinline__ uint32_t wave_inclusive_sum(uint32_t v) {
-    constexpr int kRowShr = 0x110, kRowBcast15 = 0x142, kRowBcast31 = 0x143;
-    int x = static_cast<int>(v);
-    x += __builtin_amdgcn_update_dpp(0, x, kRowShr + 1, 0xF, 0xF, false);
-    x += __builtin_amdgcn_update_dpp(0, x, kRowShr + 2, 0xF, 0xF, false);
-    x += __builtin_amdgcn_update_dpp(0, x, kRowShr + 4, 0xF, 0xF, false);
-    x += __builtin_amdgcn_update_dpp(0, x, kRowShr + 8, 0xF, 0xF, false);
-    x += __builtin_amdgcn_update_dpp(0, x, kRowBcast15, 0xA, 0xF, false);
-    x += __builtin_amdgcn_update_dpp(0, x, kRowBcast31, 0xC, 0xF, false);
-    return static_cast<uint32_t>(x);
 }
 
 // Exclusive scan of one value per digit, held by the first kMaxRadix threads of the scatter
@@ -916,9 +928,8 @@ __global__ __launch_bounds__(kBlock) void gather_kernel(idx_t nnz, const T* __re
 
 void launch_csr2coo(hipStream_t stream, idx_t m, idx_t nnz, const idx_t* row_ptr, idx_t base, idx_t* coo_rows) {
     if (nnz == 0) return;
-    const uint64_t total = static_cast<uint64_t>(m) + nnz;
-    const uint64_t per_group = static_cast<uint64_t>(kExpandTiles) * kExpandTile;
-    const uint32_t groups = static_cast<uint32_t>((total + per_group - 1) / per_group);
+    const uint64_t per_group = static_cast<uint64_t>(kExpandTiles) * kCooTile;
+    const uint32_t groups = static_cast<uint32_t>((static_cast<uint64_t>(nnz) + per_group - 1) / per_group);
     hipLaunchKernelGGL(csr2coo_kernel, dim3(groups), dim3(kBlock), 0, stream, m, nnz, base, row_ptr, coo_rows);
 }
 
