@@ -232,29 +232,44 @@ def test_unaligned_input_arrays(torch_gpu, handle, oracle, shift):
     assert np.array_equal(d_out.cpu().numpy().view(np.uint32), oracle.coo2csr(300, m_big, 0, rows))
 
 
-@pytest.mark.parametrize("items", [2048, 2049, 8 * 2048 - 1, 8 * 2048, 8 * 2048 + 1, 3 * 8 * 2048 + 5])
-@pytest.mark.parametrize("shape", ["even", "empty_head", "empty_tail", "one_long_row"])
-def test_csr2coo_around_the_tile_and_group_sizes(torch_gpu, handle, oracle, items, shape):
-    """csr2coo cuts rows + nonzeros into tiles of 2048 items and walks 8 tiles per workgroup."""
-    rng = np.random.default_rng(items)
-    m = items // 3
-    nnz = items - m
-    if shape == "even":
+@pytest.mark.parametrize("nnz", [4095, 4096, 4097, 8 * 4096 - 1, 8 * 4096, 8 * 4096 + 1, 3 * 8 * 4096 + 5])
+@pytest.mark.parametrize("shape", ["ones", "even", "empty_head", "empty_tail", "one_long_row", "every_other_empty"])
+def test_csr2coo_around_the_tile_and_group_sizes(torch_gpu, handle, oracle, nnz, shape):
+    """csr2coo cuts the nonzeros into tiles of 4096 and walks 8 tiles per workgroup; the rows of a tile come from a
+    map of the 4096 places a row can begin at (rows of one nonzero fill it), from the staged offsets when a row is
+    empty, and from row_ptr itself when more than 4096 rows begin in a tile."""
+    rng = np.random.default_rng(nnz)
+    if shape == "ones":
+        lens = np.ones(nnz, np.int64)
+    elif shape == "even":
+        m = nnz // 3
         lens = np.full(m, nnz // m, np.int64)
         lens[: nnz - lens.sum()] += 1
-    elif shape == "empty_head":   # every row ends inside the first tiles, the nonzeros come last
-        lens = np.zeros(m, np.int64)
-        lens[m - 3:] = [nnz - 2, 1, 1]
+    elif shape == "empty_head":   # every row begins at the first nonzero, the nonzeros come last
+        lens = np.zeros(nnz // 2, np.int64)
+        lens[-3:] = [nnz - 2, 1, 1]
     elif shape == "empty_tail":
-        lens = np.zeros(m, np.int64)
+        lens = np.zeros(nnz // 2, np.int64)
         lens[:2] = [1, nnz - 1]
-    else:
-        lens = np.zeros(m, np.int64)
-        lens[int(rng.integers(0, m))] = nnz
+    elif shape == "one_long_row":
+        lens = np.zeros(nnz // 2, np.int64)
+        lens[int(rng.integers(0, lens.size))] = nnz
+    else:                         # two rows begin at every nonzero: 8192 in a tile
+        lens = np.zeros(2 * nnz, np.int64)
+        lens[1::2] = 1
+    m = lens.size
     assert lens.sum() == nnz
     ptr = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
     for base in (0, 1):
         a = wl.Csr(m, nnz + 1, ptr + base, np.zeros(nnz, np.int32) + base, np.zeros(nnz, np.float32), base)
         st, coo = gpu_csr2coo(torch_gpu, handle, a)
         assert st == 0
-        assert np.array_equal(coo.view(np.uint32), oracle.csr2coo(m, base, a.ptr, nnz)), (items, shape, base)
+        assert np.array_equal(coo.view(np.uint32), oracle.csr2coo(m, base, a.ptr, nnz)), (nnz, shape, base)
+    # an output array that is not 16-byte aligned is written one element at a time
+    d_ptr = dev(torch_gpu, ptr)
+    d_out = torch_gpu.full((nnz + 3,), -7, dtype=torch_gpu.int32, device="cuda")
+    assert api.xcsr2coo(handle, d_ptr, nnz, m, d_out[1:nnz + 1], 0) == 0
+    torch_gpu.cuda.synchronize()
+    got = d_out.cpu().numpy()
+    assert got[0] == -7 and (got[nnz + 1:] == -7).all()
+    assert np.array_equal(got[1:nnz + 1].view(np.uint32), oracle.csr2coo(m, 0, ptr, nnz)), (nnz, shape, "unaligned")
