@@ -67,17 +67,21 @@ __device__ __forceinline__ uint32_t wave_inclusive_sum(uint32_t v) {
 // row_ptr itself when more rows begin in the tile than LDS holds.  A workgroup takes kExpandTiles tiles in
 // a row.  Reference semantics: src/kernels/conversion/coo2csr_device.hpp:26-41.
 constexpr int kExpandTiles = 8;
-constexpr int kCooTile = 4096;
+constexpr int kCooBlock = 256;
+constexpr int kCooTile = kCooBlock * 16;  // four stores of four rows per thread
 constexpr int kCooWords = kCooTile / kWave;
 constexpr int kCooLoads = 4;  // row starts per thread and round
-__global__ __launch_bounds__(kBlock) void csr2coo_kernel(idx_t m, idx_t nnz, idx_t base,
+__global__ __launch_bounds__(kCooBlock) void csr2coo_kernel(idx_t m, idx_t nnz, idx_t base,
                                                          const idx_t* __restrict__ row_ptr,
                                                          idx_t* __restrict__ coo_rows) {
     typedef idx_t idx4 __attribute__((ext_vector_type(4)));
-    static_assert(kCooWords == kWave && kCooTile == kBlock * 16, "a word per lane; four stores of four rows per thread");
+    static_assert((kCooWords % kWave == 0 || kCooWords < kWave) && kCooWords <= kCooBlock && kCooBlock % kWave == 0,
+                  "the words of the map are counted a wavefront at a time");
+    constexpr int kScanLanes = (kCooWords + kWave - 1) / kWave * kWave;
     __shared__ idx_t s_start[kCooTile];
     __shared__ unsigned long long s_begins[kCooWords];
     __shared__ uint32_t s_begins_before[kCooWords];
+    __shared__ uint32_t s_wave_begins[(kCooWords + kWave - 1) / kWave];
     __shared__ idx_t s_first;
     __shared__ uint32_t s_empty_rows;
     __shared__ uint32_t s_inside;
@@ -106,11 +110,11 @@ __global__ __launch_bounds__(kBlock) void csr2coo_kernel(idx_t m, idx_t nnz, idx
         // the offsets from `before` on, until one lies past the tile: those up to j0 + 4096 begin a row of this
         // tile (or, at j0 + 4096 itself, are counted for the next one)
         uint32_t inside = 0;
-        for (uint32_t loaded = 0;; loaded += kBlock * kCooLoads) {
+        for (uint32_t loaded = 0;; loaded += kCooBlock * kCooLoads) {
             uint64_t at[kCooLoads];
 #pragma unroll
             for (int k = 0; k < kCooLoads; ++k) {
-                const uint64_t r = before + loaded + static_cast<uint32_t>(k) * kBlock + tid;
+                const uint64_t r = before + loaded + static_cast<uint32_t>(k) * kCooBlock + tid;
                 const uint64_t r_read = r <= m ? r : m;
                 const idx_t v = row_ptr[r_read];
                 at[k] = r <= m ? static_cast<uint64_t>(v - base) - j0 : ~0ull;  // > 0: row `before` begins after j0
@@ -119,7 +123,7 @@ __global__ __launch_bounds__(kBlock) void csr2coo_kernel(idx_t m, idx_t nnz, idx
 #pragma unroll
             for (int k = 0; k < kCooLoads; ++k) {
                 if (at[k] > static_cast<uint64_t>(kCooTile)) continue;
-                const uint32_t i = loaded + static_cast<uint32_t>(k) * kBlock + tid;
+                const uint32_t i = loaded + static_cast<uint32_t>(k) * kCooBlock + tid;
                 mine = i + 1;
                 if (i < static_cast<uint32_t>(kCooTile)) s_start[i] = static_cast<idx_t>(at[k]);
                 if (at[k] < static_cast<uint64_t>(kCooTile)) {
@@ -131,27 +135,31 @@ __global__ __launch_bounds__(kBlock) void csr2coo_kernel(idx_t m, idx_t nnz, idx
             if (mine != 0) atomicMax(&s_inside, mine);
             __syncthreads();
             inside = s_inside;
-            if (inside < loaded + kBlock * kCooLoads) break;  // whole workgroup: the round held one past the tile
+            if (inside < loaded + kCooBlock * kCooLoads) break;  // whole workgroup: the round held one past the tile
         }
         const bool by_bits = s_empty_rows == 0;  // the same for the whole workgroup
         if (by_bits) {
-            if (tid < kWave) {
-                const uint32_t c = __popcll(s_begins[lane]);
-                s_begins_before[lane] = wave_inclusive_sum(c) - c;
+            if (tid < kScanLanes) {  // whole wavefronts
+                const uint32_t c = tid < kCooWords ? __popcll(s_begins[tid]) : 0;
+                const uint32_t upto = wave_inclusive_sum(c);
+                if (tid < kCooWords) s_begins_before[tid] = upto - c;
+                if (lane == kWave - 1) s_wave_begins[tid / kWave] = upto;
             }
             __syncthreads();
         }
         const bool staged = inside <= static_cast<uint32_t>(kCooTile);
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
-            const uint32_t p = (static_cast<uint32_t>(k) * kBlock + tid) * 4;  // four neighbouring nonzeros of the tile
+            const uint32_t p = (static_cast<uint32_t>(k) * kCooBlock + tid) * 4;  // four neighbouring nonzeros of the tile
             if (p >= count) continue;
             idx_t rows[4];
             if (by_bits) {
                 const uint32_t word = p / kWave, bit = p % kWave;
                 const unsigned long long w = s_begins[word];
                 // rows that begin before nonzero p, then one more for every bit of the four at p .. p + 3
-                idx_t row = static_cast<idx_t>(before + s_begins_before[word] + __popcll(w & ((1ull << bit) - 1ull)) - 1 + base);
+                uint64_t upto = before + s_begins_before[word];
+                for (uint32_t v = 0; v < word / kWave; ++v) upto += s_wave_begins[v];  // wavefronts of words before this one
+                idx_t row = static_cast<idx_t>(upto + __popcll(w & ((1ull << bit) - 1ull)) - 1 + base);
                 const uint32_t four = static_cast<uint32_t>(w >> bit) & 0xFu;  // bit <= 60
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
@@ -930,7 +938,7 @@ void launch_csr2coo(hipStream_t stream, idx_t m, idx_t nnz, const idx_t* row_ptr
     if (nnz == 0) return;
     const uint64_t per_group = static_cast<uint64_t>(kExpandTiles) * kCooTile;
     const uint32_t groups = static_cast<uint32_t>((static_cast<uint64_t>(nnz) + per_group - 1) / per_group);
-    hipLaunchKernelGGL(csr2coo_kernel, dim3(groups), dim3(kBlock), 0, stream, m, nnz, base, row_ptr, coo_rows);
+    hipLaunchKernelGGL(csr2coo_kernel, dim3(groups), dim3(kCooBlock), 0, stream, m, nnz, base, row_ptr, coo_rows);
 }
 
 void launch_coo2csr(hipStream_t stream, idx_t nnz, idx_t m, const idx_t* coo_rows, idx_t base, idx_t* row_ptr) {
