@@ -371,7 +371,7 @@ mcspStatus_t spmv_typed(mcsparseHandle_t h, mcsparseSpMatDescr* A, mcsparseOpera
     // Unless the caller asked for the algorithm whose bits repeat (MCSPARSE_SPMV_CSR_ALG2): one pass of
     // that sort, into buckets of neighbouring columns, and the sums of a bucket's columns formed in LDS
     // in whatever order the products arrive.
-    if (alg != MCSPARSE_SPMV_CSR_ALG2 && mcsp::skinny_transpose_shape(static_cast<idx_t>(v.n), nnz, base)) {
+    if (alg != MCSPARSE_SPMV_CSR_ALG2 && mcsp::skinny_transpose_shape(static_cast<idx_t>(v.n), nnz)) {
         // few columns, many nonzeros in each: nothing is ordered at all.  The scratch of the sort holds the
         // rows of the nonzeros (for CSR offsets) and the partial sums.
         char* ws = buf + l.csr2csc_ws;
@@ -389,11 +389,11 @@ mcspStatus_t spmv_typed(mcsparseHandle_t h, mcsparseSpMatDescr* A, mcsparseOpera
     }
     uint32_t bucket_shift = 0;
     if (alg != MCSPARSE_SPMV_CSR_ALG2 &&
-        mcsp::bucketed_products_shape(static_cast<idx_t>(v.n), base, &bucket_shift)) {
+        mcsp::bucketed_products_shape(static_cast<idx_t>(v.n), &bucket_shift)) {
         mcsp::BucketedProducts b;
         mcsp::launch_bucketed_products(h->stream, static_cast<idx_t>(v.m), static_cast<idx_t>(v.n), nnz, v.val, v.ptr,
                                        v.ind, x->values, t_val, sizeof(T), base, buf + l.csr2csc_ws, &b);
-        mcsp::launch_bucket_sums<T>(h->stream, static_cast<idx_t>(v.n), nnz, base, b, static_cast<const T*>(t_val),
+        mcsp::launch_bucket_sums<T>(h->stream, static_cast<idx_t>(v.n), nnz, b, static_cast<const T*>(t_val),
                                     static_cast<T*>(y->values), h_alpha, h_beta);
         return MCSP_STATUS_SUCCESS;
     }

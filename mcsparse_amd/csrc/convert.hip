@@ -390,12 +390,12 @@ constexpr int kMaxRadix = 256;
 constexpr uint32_t kXcds = 8;                          // accelerator complex dies of an MI355X
 static_assert(kSortBlock >= kMaxRadix, "one thread per digit");
 
-// counters[digit * tiles + tile] = how many keys of `tile` carry `digit`.  256 threads, 16 keys
+// counters[digit * tiles + tile] = how many keys of `tile` carry `digit` (the digit of key - bias).  256 threads, 16 keys
 // each, read as four 128-bit loads (tiles start at multiples of 4096 keys, so they are aligned).
 constexpr int kHistBlock = 256;
 __global__ __launch_bounds__(kHistBlock) void radix_hist_kernel(const idx_t* __restrict__ keys, idx_t count,
                                                                 uint32_t shift, uint32_t bits, uint32_t tiles,
-                                                                uint32_t* __restrict__ counters) {
+                                                                uint32_t* __restrict__ counters, idx_t bias) {
     typedef idx_t idx4 __attribute__((ext_vector_type(4)));
     __shared__ uint32_t s_cnt[kMaxRadix];
     const uint32_t radix = 1u << bits;
@@ -420,7 +420,7 @@ __global__ __launch_bounds__(kHistBlock) void radix_hist_kernel(const idx_t* __r
         if (full) k = __builtin_nontemporal_load(reinterpret_cast<const idx4*>(keys + p));
         uint32_t d[4];
 #pragma unroll
-        for (int e = 0; e < 4; ++e) d[e] = (k[e] >> shift) & mask;
+        for (int e = 0; e < 4; ++e) d[e] = ((k[e] - bias) >> shift) & mask;
         // Keys that are sorted inside long rows carry the same high digit many times in a row, and LDS
         // takes the adds of a wavefront to one counter one after the other.  A lane whose four keys
         // share a digit joins the lanes before it that hold the same one: the first lane of such a run
@@ -440,7 +440,7 @@ __global__ __launch_bounds__(kHistBlock) void radix_hist_kernel(const idx_t* __r
                 for (int e = 0; e < 4; ++e) atomicAdd(&s_cnt[d[e]], 1u);
             } else {
                 const uint64_t stop = p + 4 < count ? p + 4 : count;
-                for (uint64_t q = p; q < stop; ++q) atomicAdd(&s_cnt[(keys[q] >> shift) & mask], 1u);
+                for (uint64_t q = p; q < stop; ++q) atomicAdd(&s_cnt[((keys[q] - bias) >> shift) & mask], 1u);
             }
         }
     }
@@ -479,7 +479,8 @@ struct ValueOf<8> { typedef uint64_t type; };
 
 // AUX = false: (key, value) pairs, rows_out is not written.  TIMES_X (with FROM_CSR, without AUX): the
 // value that travels is value * x[row of the nonzero], in the floating-point type of VB bytes.
-// short_keys (TIMES_X only, shift <= 16): keys_out is an array of uint16_t that receives the key bits below `shift`.
+// short_keys (TIMES_X only, shift <= 16): keys_out is an array of uint16_t that receives the bits of key - bias below
+// `shift`.  bias is subtracted from a key wherever a digit is taken from it (the index base, where that saves a bit).
 template <int VB>
 struct RealOf { typedef float type; };
 template <>
@@ -490,7 +491,7 @@ __global__ __launch_bounds__(kSortBlock) void radix_scatter_kernel(
     const idx_t* __restrict__ keys_in, const idx_t* __restrict__ rows_in, const void* __restrict__ vals_in_v,
     idx_t* __restrict__ keys_out, idx_t* __restrict__ rows_out, void* __restrict__ vals_out_v, idx_t count,
     uint32_t shift, uint32_t bits, uint32_t tiles, const uint32_t* __restrict__ counters,
-    const idx_t* __restrict__ tile_rows, idx_t base, const void* __restrict__ x_v, bool short_keys) {
+    const idx_t* __restrict__ tile_rows, idx_t base, const void* __restrict__ x_v, bool short_keys, idx_t bias) {
     static_assert(AUX || VB != 0, "pairs carry a value");
     static_assert(!TIMES_X || (FROM_CSR && !AUX), "products are formed where the rows are worked out");
     typedef typename ValueOf<VB>::type val_t;
@@ -574,7 +575,7 @@ __global__ __launch_bounds__(kSortBlock) void radix_scatter_kernel(
     for (int i = 0; i < kSortIpt; ++i) {
         const uint32_t p = wave * kSortWaveItems + i * kWave + lane;
         const bool live = p < tile_count;
-        const uint32_t d = (key[i] >> shift) & mask;
+        const uint32_t d = ((key[i] - bias) >> shift) & mask;
         // lanes of this wave holding the same digit in this round: per bit of the digit, keep the
         // lanes that voted as this lane did (vote xor own bit, spread over the word, is 0 there)
         uint64_t peers = __ballot(live);
@@ -691,7 +692,7 @@ __global__ __launch_bounds__(kSortBlock) void radix_scatter_kernel(
     for (int i = 0; i < kSortIpt; ++i) {
         const uint32_t p = wave * kSortWaveItems + i * kWave + lane;
         if (p < tile_count) {
-            const uint32_t d = (key[i] >> shift) & mask;
+            const uint32_t d = ((key[i] - bias) >> shift) & mask;
             const uint32_t slot = s_start[d] + s_cnt[wave][d] + rank[i];
             s_keys[slot] = key[i];
             if constexpr (AUX) s_rows[slot] = row[i];
@@ -706,11 +707,11 @@ __global__ __launch_bounds__(kSortBlock) void radix_scatter_kernel(
         const uint32_t slot = i * kSortBlock + tid;
         if (slot < tile_count) {
             const idx_t k = s_keys[slot];
-            const uint32_t d = (k >> shift) & mask;
+            const uint32_t d = ((k - bias) >> shift) & mask;
             const uint64_t out = static_cast<uint64_t>(s_dest[d]) + (slot - s_start[d]);
             if constexpr (TIMES_X) {
                 // short_keys: the last pass of a sort on the top bits keeps only what lies below them, in 16 bits
-                if (short_keys) reinterpret_cast<uint16_t*>(keys_out)[out] = static_cast<uint16_t>(k & ((1u << shift) - 1u));
+                if (short_keys) reinterpret_cast<uint16_t*>(keys_out)[out] = static_cast<uint16_t>((k - bias) & ((1u << shift) - 1u));
                 else keys_out[out] = k;
             } else {
                 keys_out[out] = k;
@@ -751,30 +752,30 @@ template <int VB>
 void launch_scatter(hipStream_t stream, bool from_csr, uint32_t grid, const idx_t* keys_in, const idx_t* aux_in,
                     const void* vals_in, idx_t* keys_out, idx_t* aux_out, void* vals_out, idx_t count, uint32_t shift,
                     uint32_t bits, uint32_t tiles, const uint32_t* counters, const idx_t* tile_rows, idx_t base,
-                    bool pairs, const void* x, bool short_keys) {
+                    bool pairs, const void* x, bool short_keys, idx_t bias) {
     const void* none = nullptr;
     if constexpr (VB != 0) {
         if (pairs && from_csr) {
             hipLaunchKernelGGL((radix_scatter_kernel<VB, true, false, true>), dim3(grid), dim3(kSortBlock), 0, stream, keys_in,
                                aux_in, vals_in, keys_out, aux_out, vals_out, count, shift, bits, tiles, counters, tile_rows,
-                               base, x, short_keys);
+                               base, x, short_keys, bias);
             return;
         }
         if (pairs) {
             hipLaunchKernelGGL((radix_scatter_kernel<VB, false, false, false>), dim3(grid), dim3(kSortBlock), 0, stream, keys_in,
                                aux_in, vals_in, keys_out, aux_out, vals_out, count, shift, bits, tiles, counters, tile_rows,
-                               base, none, false);
+                               base, none, false, bias);
             return;
         }
     }
     if (from_csr) {
         hipLaunchKernelGGL((radix_scatter_kernel<VB, true, true, false>), dim3(grid), dim3(kSortBlock), 0, stream, keys_in,
                            aux_in, vals_in, keys_out, aux_out, vals_out, count, shift, bits, tiles, counters, tile_rows, base,
-                           none, false);
+                           none, false, bias);
     } else {
         hipLaunchKernelGGL((radix_scatter_kernel<VB, false, true, false>), dim3(grid), dim3(kSortBlock), 0, stream, keys_in,
                            aux_in, vals_in, keys_out, aux_out, vals_out, count, shift, bits, tiles, counters, tile_rows, base,
-                           none, false);
+                           none, false, bias);
     }
 }
 
@@ -791,6 +792,8 @@ struct CsrSource {
     // with times_x, in a sort of one pass: keys_out is an array of uint16_t that receives the key bits below
     // first_bit (<= 16 of them), which is all that tells the keys of one digit apart
     bool short_keys = false;
+    // subtracted from every key before its digits are taken (the keys themselves travel unchanged)
+    idx_t bias = 0;
 };
 
 // Stable LSD radix sort of (key, aux, value) triples on the low key_bits of the keys, in
@@ -817,12 +820,12 @@ void radix_sort_triples(hipStream_t stream, idx_t count, uint32_t key_bits, cons
         idx_t* a_out = last ? aux_out : t.aux[p & 1];
         void* v_out = last ? vals_out : t.vals[p & 1];
         hipLaunchKernelGGL(radix_hist_kernel, dim3(scatter_grid), dim3(kHistBlock), 0, stream, keys_in, count, shift, bits,
-                           tiles, t.counters);
+                           tiles, t.counters, csr.bias);
         launch_exclusive_scan(stream, t.counters, static_cast<uint64_t>(radix) * tiles, t.scan_ws);
         auto* launch = value_bytes == 0 ? launch_scatter<0> : value_bytes == 4 ? launch_scatter<4> : launch_scatter<8>;
         launch(stream, from_csr, scatter_grid, keys_in, aux_in, vals_in, k_out, a_out, v_out, count, shift, bits, tiles,
                t.counters, t.tile_rows, csr.base, csr.times_x != nullptr, csr.times_x,
-               csr.short_keys && last && from_csr);
+               csr.short_keys && last && from_csr, csr.bias);
         keys_in = k_out;
         aux_in = a_out;
         vals_in = v_out;
@@ -1017,8 +1020,8 @@ void launch_transposed_products(hipStream_t stream, idx_t m, idx_t n, idx_t nnz,
     launch_coo2csr(stream, nnz, n, sorted_keys, base, col_ptr);
 }
 
-bool bucketed_products_shape(idx_t n, idx_t base, uint32_t* shift) {
-    const uint32_t bits = bit_length(n - 1 + base);
+bool bucketed_products_shape(idx_t n, uint32_t* shift) {
+    const uint32_t bits = bit_length(n - 1);  // of the columns without their index base
     // fewer keys than that: the full sort is two short passes; more: a bucket's sums no longer fit in LDS
     if (bits < kBucketMinKeyBits || bits > 8 + kBucketMaxShift) return false;
     *shift = bits - 8;
@@ -1026,15 +1029,15 @@ bool bucketed_products_shape(idx_t n, idx_t base, uint32_t* shift) {
 }
 
 // One pass of the same sort, for a transposing SpMV that may add the products of a column in any order:
-// (column, value * x[row]) pairs ordered by the top eight bits of the column keys only, that is in up to
-// 256 buckets of 2^shift neighbouring columns, inside a bucket in CSR order.  The sums over a bucket's
+// (column, value * x[row]) pairs ordered by the top eight bits of the columns (index base taken off) only, that is
+// in up to 256 buckets of 2^shift neighbouring columns, inside a bucket in CSR order.  The sums over a bucket's
 // columns then fit in LDS.  Of a key only its place in the bucket is written, as 16 bits: a quarter fewer
 // bytes for this pass to write and the sums to read.  workspace as for launch_transposed_products.
 void launch_bucketed_products(hipStream_t stream, idx_t m, idx_t n, idx_t nnz, const void* csr_val, const idx_t* row_ptr,
                               const idx_t* col, const void* x, void* products, size_t value_bytes, idx_t base,
                               void* workspace, BucketedProducts* out) {
     uint32_t shift = 0;
-    if (m == 0 || nnz == 0 || !bucketed_products_shape(n, base, &shift)) return;
+    if (m == 0 || nnz == 0 || !bucketed_products_shape(n, &shift)) return;
     const Csr2CscLayout l = csr2csc_layout(nnz, value_bytes, true);
     char* w = static_cast<char*>(workspace);
     idx_t* keys = reinterpret_cast<idx_t*>(w + l.sorted_keys);  // room for 32-bit keys, used for 16-bit ones
@@ -1051,12 +1054,13 @@ void launch_bucketed_products(hipStream_t stream, idx_t m, idx_t n, idx_t nnz, c
     csr.times_x = x;
     csr.first_bit = shift;
     csr.short_keys = true;
+    csr.bias = base;
     radix_sort_triples(stream, nnz, 8, col, row_ptr, csr_val, keys, nullptr, products, value_bytes, t, csr);
     out->keys = reinterpret_cast<const uint16_t*>(keys);
     out->starts = t.counters;  // after the scan, counters[digit * tiles] is where the digit's keys begin
     out->stride = sort_tiles(nnz);
     out->shift = shift;
-    out->buckets = static_cast<uint32_t>((static_cast<uint64_t>(n) - 1 + base) >> shift) + 1;
+    out->buckets = static_cast<uint32_t>((n - 1) >> shift) + 1;
 }
 
 // Scratch of launch_sort_by_column_band: the counters of one pass, their scan, the row starts per tile.

@@ -359,12 +359,13 @@ void launch_transposed_products(hipStream_t stream, idx_t m, idx_t n, idx_t nnz,
                                 const idx_t* col, const void* x, void* products, idx_t* col_ptr, size_t value_bytes,
                                 idx_t base, void* workspace);
 
-// The same products in up to 256 buckets of 2^shift neighbouring column keys (index base included),
-// bucket b starting at starts[b * stride] and ending where the next begins (the last at nnz); inside a
-// bucket the pairs are in CSR order, not sorted, and keys[] holds a key's low `shift` bits, its place in
-// the bucket.  Both arrays may be read up to the next even index past nnz.  One pass over the nonzeros instead of the three of a
+// The same products in up to 256 buckets of 2^shift neighbouring columns (index base taken off: bucket b
+// holds columns [b << shift, (b + 1) << shift)), bucket b starting at starts[b * stride] and ending where
+// the next begins (the last at nnz); inside a bucket the pairs are in CSR order, not sorted, and keys[]
+// holds a column's low `shift` bits, its place in the bucket.  Both arrays may be read up to the next even index past nnz.  One pass over the nonzeros instead of the three of a
 // full sort: for callers that then add the products of a column in any order.  The shape function says
-// whether the keys allow it (between 2^14 and 2^22 of them: a bucket's sums must fit in LDS as doubles).
+// whether the shape allows it (more than 2^14 and at most 2^22 columns: a bucket's sums must fit in LDS as
+// doubles).
 constexpr uint32_t kBucketMinKeyBits = 15;
 constexpr uint32_t kBucketMaxShift = 14;
 struct BucketedProducts {
@@ -372,22 +373,22 @@ struct BucketedProducts {
     const uint32_t* starts = nullptr;
     uint32_t stride = 0, shift = 0, buckets = 0;
 };
-bool bucketed_products_shape(idx_t n, idx_t base, uint32_t* shift);
+bool bucketed_products_shape(idx_t n, uint32_t* shift);
 void launch_bucketed_products(hipStream_t stream, idx_t m, idx_t n, idx_t nnz, const void* csr_val, const idx_t* row_ptr,
                               const idx_t* col, const void* x, void* products, size_t value_bytes, idx_t base,
                               void* workspace, BucketedProducts* out);
 // y[c] = alpha * (sum of the products of column c) + beta * y[c] for all n columns, from such buckets;
 // the sums are formed in LDS in the order the wavefronts reach the products.
 template <typename T>
-void launch_bucket_sums(hipStream_t stream, idx_t n, idx_t nnz, idx_t base, const BucketedProducts& b, const T* products,
-                        T* y, T alpha, T beta);
+void launch_bucket_sums(hipStream_t stream, idx_t n, idx_t nnz, const BucketedProducts& b, const T* products, T* y,
+                        T alpha, T beta);
 
-// y = alpha * A^T x + beta * y for an m x n matrix with fewer than 2^14 column keys and many nonzeros per
+// y = alpha * A^T x + beta * y for an m x n matrix with at most 2^14 columns and many nonzeros per
 // column, without sorting anything: shares of the nonzeros are summed into copies of y in LDS, the copies
 // into y.  rows[nnz] = row + base of every nonzero (COO rows, or csr2coo of the offsets); workspace of
 // skinny_transpose_workspace_bytes(n) bytes, which the shape function keeps below 16 bytes per nonzero.
 constexpr uint32_t kSkinnyMinNonzerosPerColumn = 128;
-bool skinny_transpose_shape(idx_t n, idx_t nnz, idx_t base);
+bool skinny_transpose_shape(idx_t n, idx_t nnz);
 size_t skinny_transpose_workspace_bytes(idx_t n);
 template <typename T>
 void launch_skinny_transpose(hipStream_t stream, idx_t m, idx_t n, idx_t nnz, idx_t base, const idx_t* rows,

@@ -580,7 +580,7 @@ template <>
 struct PairOf<double> { typedef double type __attribute__((ext_vector_type(2))); };
 
 template <typename T>
-__global__ __launch_bounds__(kBucketBlock) void bucket_sums_kernel(idx_t n, idx_t nnz, idx_t base, uint32_t shift,
+__global__ __launch_bounds__(kBucketBlock) void bucket_sums_kernel(idx_t n, idx_t nnz, uint32_t shift,
                                                                   uint32_t stride,
                                                                   const uint32_t* __restrict__ starts,
                                                                   const uint16_t* __restrict__ keys,
@@ -627,33 +627,32 @@ __global__ __launch_bounds__(kBucketBlock) void bucket_sums_kernel(idx_t n, idx_
         }
     }
     __syncthreads();
-    const uint64_t key0 = static_cast<uint64_t>(bucket) << shift;
+    const uint64_t first = static_cast<uint64_t>(bucket) << shift;
     for (uint32_t r = tid; r < width; r += kBucketBlock) {
-        const uint64_t k = key0 + r;
-        if (k < base || k - base >= n) continue;  // keys below the index base and past the last column
-        const uint64_t c = k - base;
+        const uint64_t c = first + r;
+        if (c >= n) continue;  // the last bucket may reach past the last column
         const T s = alpha * static_cast<T>(s_acc[r]);
         y[c] = beta == T(0) ? s : s + beta * y[c];
     }
 }
 
 template <typename T>
-void launch_bucket_sums(hipStream_t stream, idx_t n, idx_t nnz, idx_t base, const BucketedProducts& b, const T* products,
-                        T* y, T alpha, T beta) {
+void launch_bucket_sums(hipStream_t stream, idx_t n, idx_t nnz, const BucketedProducts& b, const T* products, T* y,
+                        T alpha, T beta) {
     if (b.buckets == 0 || b.buckets > kBucketDigits || b.shift > kBucketMaxShift) return;
     const size_t lds = sizeof(double) << b.shift;
     (void)hipFuncSetAttribute(reinterpret_cast<const void*>(bucket_sums_kernel<T>),
                               hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
-    hipLaunchKernelGGL((bucket_sums_kernel<T>), dim3(b.buckets), dim3(kBucketBlock), lds, stream, n, nnz, base, b.shift,
+    hipLaunchKernelGGL((bucket_sums_kernel<T>), dim3(b.buckets), dim3(kBucketBlock), lds, stream, n, nnz, b.shift,
                        b.stride, b.starts, b.keys, products, y, alpha, beta);
 }
 
-template void launch_bucket_sums<float>(hipStream_t, idx_t, idx_t, idx_t, const BucketedProducts&, const float*, float*,
-                                        float, float);
-template void launch_bucket_sums<double>(hipStream_t, idx_t, idx_t, idx_t, const BucketedProducts&, const double*,
-                                         double*, double, double);
+template void launch_bucket_sums<float>(hipStream_t, idx_t, idx_t, const BucketedProducts&, const float*, float*, float,
+                                        float);
+template void launch_bucket_sums<double>(hipStream_t, idx_t, idx_t, const BucketedProducts&, const double*, double*,
+                                         double, double);
 // ---- A^T x for a matrix with few columns ----
-// With fewer than 2^14 column keys all of y fits in the LDS of one workgroup, so nothing is sorted: each
+// With at most 2^14 columns all of y fits in the LDS of one workgroup, so nothing is sorted: each
 // of kSkinnyGroups workgroups takes an equal share of the nonzeros as they lie, adds value * x[row] to
 // its own copy of y in LDS (doubles), and writes the copy out as a plane of partial sums; a second
 // kernel adds the planes up.  rows[] holds the row (+ base) of every nonzero: the COO row array, or
@@ -717,10 +716,10 @@ __global__ __launch_bounds__(kBlock) void skinny_reduce_kernel(idx_t n, const do
     y[c] = beta == T(0) ? s : s + beta * y[c];
 }
 
-bool skinny_transpose_shape(idx_t n, idx_t nnz, idx_t base) {
-    // all keys below 2^14: a copy of y fits in LDS as doubles; enough columns that the lanes of a wavefront
+bool skinny_transpose_shape(idx_t n, idx_t nnz) {
+    // at most 2^14 columns: a copy of y fits in LDS as doubles; enough columns that the lanes of a wavefront
     // seldom meet on one sum; enough nonzeros that the planes are small beside them (and fit the scratch)
-    return static_cast<uint64_t>(n) + base <= (1u << kBucketMaxShift) && n >= 256 &&
+    return n <= (1u << kBucketMaxShift) && n >= 256 &&
            static_cast<uint64_t>(nnz) >= static_cast<uint64_t>(kSkinnyMinNonzerosPerColumn) * n;
 }
 

@@ -1,9 +1,10 @@
 """GPU parity of the transposing mcsparseSpMV without a preprocess call (CSR op T, CSC op N, COO op T).
 
-With 2^14 .. 2^22 column keys and any algorithm but MCSPARSE_SPMV_CSR_ALG2 the call orders the products
-value * x[row] by the top eight bits of their column only and forms the sums of each bucket of columns in LDS,
-in the order the products arrive; outside that range, and under ALG2, it sorts them completely and adds them in
-row order.  Integer-valued operands make every order of summation exact, so those cases are compared bit for
+With more than 2^14 and at most 2^22 columns and any algorithm but MCSPARSE_SPMV_CSR_ALG2 the call orders the
+products value * x[row] by the top eight bits of their column only and forms the sums of each bucket of columns in
+LDS, in the order the products arrive; with at most 2^14 columns and many nonzeros in each it orders nothing and
+sums into copies of y in LDS; otherwise, and under ALG2, it sorts the products completely and adds them in row
+order.  Integer-valued operands make every order of summation exact, so those cases are compared bit for
 bit; the rest within 8*u*(|alpha| (|A|^T |x|)_i + |beta y_i|)."""
 import numpy as np
 import pytest
@@ -51,10 +52,10 @@ def integer_valued(a, seed):
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
 @pytest.mark.parametrize("base", [0, 1])
-@pytest.mark.parametrize("n", [16384, 16385, 100003, 1 << 20, 1 << 22])
+@pytest.mark.parametrize("n", [16384, 16385, 100003, 1 << 20, 1 << 22, (1 << 22) + 1])
 def test_exact_on_integers_across_the_key_range(torch_gpu, handle, dtype, base, n):
-    # 16384 columns from base 0 are 14 key bits (the full sort), 16385 are 15 (the first bucketed shape); 2^22
-    # columns from base 1 are 23 (the full sort again)
+    # 16384 columns with few nonzeros each take the full sort, 16385 are the first bucketed shape, 2^22 the last one;
+    # the index base does not count
     a = wl.random_ragged(3001, n, 40, dtype=dtype, seed=n % 97 + base, base=base)
     x, y = integer_valued(a, n)
     want = 2 * (a.to_scipy().T.astype(np.float64) @ x.astype(np.float64)) - 3 * y
@@ -124,8 +125,8 @@ def test_alg2_repeats_its_bits_and_both_agree(torch_gpu, handle, oracle):
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
 @pytest.mark.parametrize("n,base", [(256, 0), (1000, 1), (16383, 1), (16384, 0), (16384, 1), (255, 0)])
 def test_few_columns_exact_on_integers(torch_gpu, handle, dtype, n, base):
-    # 16384 columns from base 1 are one key too many for a copy of y in LDS, 255 columns too few: both take
-    # other paths and must agree all the same
+    # 16384 columns are the most a copy of y in LDS holds, whatever the index base; 255 columns are too few and
+    # take the full sort
     m = 340000
     a = wl.random_ragged(m, n, 8, dtype=dtype, seed=n % 89 + base, base=base)  # a fifth of the rows empty
     assert a.nnz >= 128 * n
