@@ -984,9 +984,11 @@ void launch_csr2csc(hipStream_t stream, idx_t m, idx_t n, idx_t nnz, const void*
     CsrSource csr;
     csr.rows = m;
     csr.base = base;
-    // keys are the raw column indices (index base included), so the largest key is n - 1 + base
-    radix_sort_triples(stream, nnz, bit_length(n - 1 + base), col, row_ptr, csr_val, sorted_keys, row_ind, csc_val,
-                       value_bytes, t, csr);
+    // keys are the raw column indices (index base included); the digits are taken from key - base, so that a
+    // one-based matrix with 2^16 or 2^24 columns does not pay a pass for the one key that needs another bit
+    csr.bias = base;
+    radix_sort_triples(stream, nnz, bit_length(n - 1), col, row_ptr, csr_val, sorted_keys, row_ind, csc_val, value_bytes,
+                       t, csr);
     launch_coo2csr(stream, nnz, n, sorted_keys, base, col_ptr);
 }
 
@@ -1015,8 +1017,9 @@ void launch_transposed_products(hipStream_t stream, idx_t m, idx_t n, idx_t nnz,
     csr.rows = m;
     csr.base = base;
     csr.times_x = x;
-    radix_sort_triples(stream, nnz, bit_length(n - 1 + base), col, row_ptr, csr_val, sorted_keys, nullptr, products,
-                       value_bytes, t, csr);
+    csr.bias = base;  // as in launch_csr2csc
+    radix_sort_triples(stream, nnz, bit_length(n - 1), col, row_ptr, csr_val, sorted_keys, nullptr, products, value_bytes,
+                       t, csr);
     launch_coo2csr(stream, nnz, n, sorted_keys, base, col_ptr);
 }
 
