@@ -273,3 +273,15 @@ def test_csr2coo_around_the_tile_and_group_sizes(torch_gpu, handle, oracle, nnz,
     got = d_out.cpu().numpy()
     assert got[0] == -7 and (got[nnz + 1:] == -7).all()
     assert np.array_equal(got[1:nnz + 1].view(np.uint32), oracle.csr2coo(m, 0, ptr, nnz)), (nnz, shape, "unaligned")
+
+
+@pytest.mark.parametrize("base", [0, 1])
+@pytest.mark.parametrize("n", [256, 257, 65536, 65537, 1 << 24])
+def test_csr2csc_where_the_column_count_fills_whole_digits(torch_gpu, handle, oracle, n, base):
+    """The passes of the sort are counted from the columns without their index base: a one-based matrix whose last
+    column is 2^8, 2^16 or 2^24 sorts in as many passes as the zero-based one, and in the same order."""
+    a = wl.random_ragged(3000, n, 12, dtype=np.float32, seed=n % 101 + base, base=base)
+    # the first and the last column are there, so the smallest and the largest key are
+    a.col[0] = base
+    a.col[-1] = n - 1 + base
+    check_csr2csc(torch_gpu, handle, oracle, a, "n %d base %d" % (n, base))
