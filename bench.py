@@ -54,8 +54,8 @@ MEASURED_TRAFFIC = {
                         "profiles/spmv_banded_f32_c3_powerlaw.txt"),
     # spmv_column_order_kernel + banded_reduce_kernel
     ("c2", 3): (_traffic(120550.0 + 20579.5, 32776.0 + 8192.0), "profiles/spmv_column_order_f64_c2_1Mx16.txt"),
-    ("c3", 3): (_traffic(580586.2 + 65548.9, 131136.0 + 16384.0), "profiles/spmv_column_order_f32_c3_powerlaw.txt"),
-    ("c3t", 3): (_traffic(602349.7 + 65548.9, 131136.0 + 16384.0), "profiles/spmv_column_order_f32_c3_powerlaw.txt"),
+    ("c3", 3): (_traffic(573723.6 + 65552.8, 133184.0 + 16384.0), "profiles/spmv_column_order_f32_c3_powerlaw.txt"),
+    ("c3t", 3): (_traffic(602847.9 + 65552.8, 133184.0 + 16384.0), "profiles/spmv_column_order_f32_c3_powerlaw.txt"),
     ("c5-spmv", 3): (_traffic(601424.1 + 65548.9, 131072.0 + 16384.0),
                      "profiles/spmv_column_order_f32_c3_powerlaw.txt"),
     # without the preprocess call: vector kernel; merge kernel (tiles in column order) + partition
