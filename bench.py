@@ -410,9 +410,11 @@ def main():
     t_start = time.perf_counter()
     out = run_workload(name, args, ctx)
 
-    # The default invocation also measures the other configurations, each with fewer steps, while the
-    # wall-clock budget lasts; what does not fit is named under "others_skipped".
-    default_run = (name == "c2" and args.steps is None and args.warmup is None and not args.no_others and
+    # A run of the headline workload (with or without --steps / --warmup, which apply to it alone) also measures
+    # the other configurations, each with fewer steps, while the wall-clock budget lasts; what does not fit is named
+    # under "others_skipped".  --no-others, or any flag that changes how the headline runs, leaves them out.
+    default_run = (name == "c2" and not args.no_others and not args.no_preprocess and not args.alg2 and
+                   not args.no_cpu_baseline and args.scale == 1.0 and
                    not (args.family or args.lanes or args.band_bytes or args.copies))
     if default_run:
         others, skipped = {}, []
