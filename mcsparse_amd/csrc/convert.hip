@@ -201,6 +201,8 @@ __global__ __launch_bounds__(kCooBlock) void csr2coo_kernel(idx_t m, idx_t nnz, 
 // Reference semantics: src/kernels/conversion/coo2csr_device.hpp:8-24.
 constexpr int kCooPerThread = 4;
 constexpr int kCooVectors = 2;
+constexpr uint32_t kCooFillRows = 4096;        // offsets a workgroup of the fill kernel looks after
+constexpr uint64_t kCooDeferredFill = 8192;    // stretches of more offsets than this are its work (>= kCooFillRows)
 template <bool VEC>
 __global__ __launch_bounds__(kBlock) void coo2csr_kernel(idx_t nnz, idx_t m, idx_t base,
                                                          const idx_t* __restrict__ coo_rows,
@@ -233,8 +235,9 @@ __global__ __launch_bounds__(kBlock) void coo2csr_kernel(idx_t nnz, idx_t m, idx
         idx_t before = __shfl_up(r[j][kCooPerThread - 1], 1, kWave);
         if (lane == 0) before = lead[j];
         // rows [prev, cur) get offset t: prev = row of entry t-1 plus one (0 in front of the first entry).
-        // A thread fills short stretches itself; a long stretch of empty rows (up to all m of them after
-        // the last entry) is left to the whole wavefront below, lane by lane 64 offsets at a time.
+        // A thread fills short stretches itself; a longer stretch of empty rows is left to the whole
+        // wavefront below, lane by lane 64 offsets at a time; one of more than kCooDeferredFill offsets (up to
+        // all m of them after the last entry) to the kernel after this one.
         constexpr uint64_t kSerialFill = 16;
         uint64_t prev = t0 == 0 ? 0 : static_cast<uint64_t>(before) + 1;
         uint64_t long_from = 0, long_to = 0;  // at most one long stretch is kept per thread; more are filled serially
@@ -245,7 +248,10 @@ __global__ __launch_bounds__(kBlock) void coo2csr_kernel(idx_t nnz, idx_t m, idx
                 const uint64_t t = t0 + e;
                 if (t > nnz) break;
                 const uint64_t cur = static_cast<uint64_t>(r[j][e]) + 1;  // t == nnz: m + 1
-                if (cur > prev + kSerialFill && long_to == long_from) {
+                if (cur > prev + kCooDeferredFill) {
+                    // left to coo2csr_fill_kernel: the rows of a matrix with few entries, or all those after the
+                    // last entry, would keep one wavefront busy for as long as the rest of the launch takes
+                } else if (cur > prev + kSerialFill && long_to == long_from) {
                     long_from = prev;
                     long_to = cur;
                     long_value = static_cast<idx_t>(t) + base;
@@ -265,6 +271,65 @@ __global__ __launch_bounds__(kBlock) void coo2csr_kernel(idx_t nnz, idx_t m, idx
             const idx_t value = __shfl(long_value, src, kWave);
             for (uint64_t i = from + lane; i < to; i += kWave) row_ptr[i] = value;
         }
+    }
+}
+
+// Number of entries whose row (index base taken off) is below p, in sorted rows, found with 64 probes per
+// round.  Every lane of the wave must call this; all lanes return the same value.
+__device__ __forceinline__ idx_t wave_count_rows_below(const idx_t* __restrict__ coo_rows, idx_t nnz, idx_t base, uint64_t p) {
+    uint64_t lo = 0;
+    uint64_t hi = nnz;
+    const unsigned lane = lane_id();
+    while (lo < hi) {
+        const uint64_t span = hi - lo;
+        const uint64_t step = (span + kWave - 1) / kWave;
+        const uint64_t probe = lo + lane * step;
+        const bool pred = probe < hi && static_cast<uint64_t>(coo_rows[probe] - base) < p;
+        const unsigned count = __popcll(__ballot(pred));
+        if (count == 0) {
+            hi = lo;
+        } else {
+            const uint64_t new_hi = lo + static_cast<uint64_t>(count) * step;
+            lo = lo + static_cast<uint64_t>(count - 1) * step + 1;
+            hi = new_hi < hi ? new_hi : hi;
+        }
+    }
+    return static_cast<idx_t>(lo);
+}
+
+// The stretches of more than kCooDeferredFill equal offsets that coo2csr_kernel leaves out: a workgroup looks
+// after kCooFillRows offsets.  Such a stretch is longer than that, so if it touches the workgroup's offsets it holds
+// the first or the last of them: for both, the number t of entries in rows below says which stretch they lie in
+// (from the row of entry t-1, exclusive, to the row of entry t, inclusive) and what it holds (t + base).
+__global__ __launch_bounds__(kBlock) void coo2csr_fill_kernel(idx_t nnz, idx_t m, idx_t base,
+                                                              const idx_t* __restrict__ coo_rows,
+                                                              idx_t* __restrict__ row_ptr) {
+    __shared__ uint64_t s_from[2], s_to[2];
+    __shared__ idx_t s_value[2];
+    const uint32_t tid = threadIdx.x;
+    const uint64_t i0 = static_cast<uint64_t>(blockIdx.x) * kCooFillRows;
+    const uint64_t total = static_cast<uint64_t>(m) + 1;  // offsets 0 .. m
+    if (i0 >= total) return;  // whole workgroup
+    const uint64_t i1 = i0 + kCooFillRows < total ? i0 + kCooFillRows : total;
+    const uint32_t which = tid / kWave;
+    if (which < 2) {  // whole wavefronts
+        const uint64_t p = which == 0 ? i0 : i1 - 1;
+        const idx_t t = wave_count_rows_below(coo_rows, nnz, base, p);
+        // offsets (row of entry t-1, row of entry t] hold t + base; before the first entry from 0, after the last to m
+        const uint64_t from = t == 0 ? 0 : static_cast<uint64_t>(coo_rows[t - 1] - base) + 1;
+        const uint64_t to = t == nnz ? total : static_cast<uint64_t>(coo_rows[t] - base) + 1;
+        if (tid % kWave == 0) {
+            const bool deferred = to > from + kCooDeferredFill;
+            s_from[which] = deferred ? (from > i0 ? from : i0) : 0;
+            s_to[which] = deferred ? (to < i1 ? to : i1) : 0;
+            s_value[which] = t + base;
+        }
+    }
+    __syncthreads();
+    const int stretches = s_from[1] == s_from[0] && s_to[1] == s_to[0] ? 1 : 2;  // one stretch may hold both ends
+    for (int k = 0; k < stretches; ++k) {
+        const idx_t value = s_value[k];
+        for (uint64_t i = s_from[k] + tid; i < s_to[k]; i += kBlock) row_ptr[i] = value;
     }
 }
 
@@ -965,6 +1030,11 @@ void launch_coo2csr(hipStream_t stream, idx_t nnz, idx_t m, const idx_t* coo_row
         hipLaunchKernelGGL(coo2csr_kernel<true>, grid, dim3(kBlock), 0, stream, nnz, m, base, coo_rows, row_ptr);
     } else {
         hipLaunchKernelGGL(coo2csr_kernel<false>, grid, dim3(kBlock), 0, stream, nnz, m, base, coo_rows, row_ptr);
+    }
+    if (static_cast<uint64_t>(m) + 1 > kCooDeferredFill) {  // else no stretch is long enough to have been left out
+        const uint64_t blocks = (static_cast<uint64_t>(m) + 1 + kCooFillRows - 1) / kCooFillRows;
+        hipLaunchKernelGGL(coo2csr_fill_kernel, dim3(static_cast<uint32_t>(blocks)), dim3(kBlock), 0, stream, nnz, m, base,
+                           coo_rows, row_ptr);
     }
 }
 

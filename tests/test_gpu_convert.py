@@ -285,3 +285,30 @@ def test_csr2csc_where_the_column_count_fills_whole_digits(torch_gpu, handle, or
     a.col[0] = base
     a.col[-1] = n - 1 + base
     check_csr2csc(torch_gpu, handle, oracle, a, "n %d base %d" % (n, base))
+
+
+@pytest.mark.parametrize("m", [8191, 8192, 8193, 12289, 1 << 20, 3000001])
+@pytest.mark.parametrize("shape", ["few", "clump", "both_ends", "one_row", "gaps_8192", "gaps_8193", "none_after_half"])
+def test_coo2csr_long_stretches_of_empty_rows(torch_gpu, handle, oracle, m, shape):
+    """Stretches of more than 8192 equal offsets (rows without entries) are left to a second kernel, a workgroup per
+    4096 offsets; shorter ones are filled where they are found."""
+    rng = np.random.default_rng(m % 1000 + len(shape))
+    if shape == "few":
+        rows = rng.integers(0, m, 7)
+    elif shape == "clump":
+        rows = rng.integers(m // 2, min(m, m // 2 + 40), 5000)
+    elif shape == "both_ends":
+        rows = np.concatenate([rng.integers(0, 10, 100), rng.integers(m - 10, m, 100)])
+    elif shape == "one_row":
+        rows = np.full(3000, m // 3)
+    elif shape == "gaps_8192":
+        rows = np.arange(0, m, 8192)   # stretches of exactly 8192 offsets: filled in place
+    elif shape == "gaps_8193":
+        rows = np.arange(0, m, 8193)   # one more: left to the second kernel
+    else:
+        rows = rng.integers(0, m // 2, 20000)
+    rows = np.sort(rows).astype(np.int32)
+    for base in (0, 1):
+        st, ptr = gpu_coo2csr(torch_gpu, handle, rows + base, rows.size, m, base)
+        assert st == 0
+        assert np.array_equal(ptr.view(np.uint32), oracle.coo2csr(rows.size, m, base, rows + base)), (m, shape, base)
