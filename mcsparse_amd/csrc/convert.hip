@@ -1148,6 +1148,8 @@ void launch_bucketed_products(hipStream_t stream, idx_t m, idx_t n, idx_t nnz, c
     out->stride = sort_tiles(nnz);
     out->shift = shift;
     out->buckets = static_cast<uint32_t>((n - 1) >> shift) + 1;
+    out->spare = w + l.keys_a;  // the sets the passes of a full sort alternate between
+    out->spare_bytes = l.counters - l.keys_a;
 }
 
 // Scratch of launch_sort_by_column_band: the counters of one pass, their scan, the row starts per tile.

@@ -372,6 +372,8 @@ struct BucketedProducts {
     const uint16_t* keys = nullptr;
     const uint32_t* starts = nullptr;
     uint32_t stride = 0, shift = 0, buckets = 0;
+    void* spare = nullptr;  // part of the workspace the pass did not use, for the sums of buckets that are split
+    size_t spare_bytes = 0;
 };
 bool bucketed_products_shape(idx_t n, uint32_t* shift);
 void launch_bucketed_products(hipStream_t stream, idx_t m, idx_t n, idx_t nnz, const void* csr_val, const idx_t* row_ptr,

@@ -579,28 +579,99 @@ struct PairOf { typedef float type __attribute__((ext_vector_type(2))); };
 template <>
 struct PairOf<double> { typedef double type __attribute__((ext_vector_type(2))); };
 
-template <typename T>
-__global__ __launch_bounds__(kBucketBlock) void bucket_sums_kernel(idx_t n, idx_t nnz, uint32_t shift,
-                                                                  uint32_t stride,
-                                                                  const uint32_t* __restrict__ starts,
-                                                                  const uint16_t* __restrict__ keys,
-                                                                  const T* __restrict__ products, T* __restrict__ y,
-                                                                  T alpha, T beta) {
-    typedef typename PairOf<T>::type pair_t;
-    extern __shared__ __align__(16) unsigned char s_raw[];
-    double* s_acc = reinterpret_cast<double*>(s_raw);
-    const uint32_t tid = threadIdx.x;
-    const uint32_t bucket = blockIdx.x;
-    const uint32_t width = 1u << shift;
-    for (uint32_t r = tid; r < width; r += kBucketBlock) s_acc[r] = 0.0;
-    idx_t e0 = starts[static_cast<uint64_t>(bucket) * stride];
-    idx_t e1 = bucket + 1 < kBucketDigits ? starts[static_cast<uint64_t>(bucket + 1) * stride] : nnz;
+// Which part of which bucket a workgroup takes.  A bucket whose pairs number more than twice `share` (the mean of
+// a bucket, rounded up) is dealt to several workgroups, ceil(count / share) of them, so that columns that crowd
+// into a few buckets (a matrix sorted by degree) do not leave the work to a few CUs: workgroup b < 256 takes the
+// first part of bucket b, the workgroups from 256 on the further parts, bucket by bucket.  The parts of a split
+// bucket leave their sums as planes in `planes`, numbered in the same order, for bucket_merge_kernel.
+struct BucketPart {
+    uint32_t bucket;  // kBucketDigits: none
+    uint32_t part, parts;
+    uint32_t plane;   // of part 0 of this bucket, when parts > 1
+};
+__device__ __forceinline__ uint32_t bucket_count(const uint32_t* __restrict__ starts, uint32_t stride, idx_t nnz, uint32_t b,
+                                                 idx_t* first) {
+    idx_t e0 = starts[static_cast<uint64_t>(b) * stride];
+    idx_t e1 = b + 1 < kBucketDigits ? starts[static_cast<uint64_t>(b + 1) * stride] : nnz;
     e0 = e0 < nnz ? e0 : nnz;
     e1 = e1 < nnz ? e1 : nnz;
     e1 = e1 > e0 ? e1 : e0;
+    *first = e0;
+    return e1 - e0;
+}
+// every thread of the workgroup must call this (it holds barriers); s_parts: kBucketDigits words of LDS
+__device__ __forceinline__ BucketPart bucket_part(uint32_t group, bool merge, const uint32_t* __restrict__ starts,
+                                                  uint32_t stride, idx_t nnz, uint32_t share, uint32_t* s_parts,
+                                                  uint32_t* s_out) {
+    for (uint32_t b = threadIdx.x; b < kBucketDigits; b += blockDim.x) {
+        idx_t first;
+        const uint32_t count = bucket_count(starts, stride, nnz, b, &first);
+        s_parts[b] = count / 2 > share ? (count + share - 1) / share : 1u;  // more than twice the share: split
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        uint32_t bucket = kBucketDigits, part = 0;
+        if (merge || group < kBucketDigits) {
+            bucket = group;
+        } else {
+            uint32_t further = group - kBucketDigits;
+            for (uint32_t b = 0; b < kBucketDigits; ++b) {
+                const uint32_t extra = s_parts[b] - 1;
+                if (further < extra) {
+                    bucket = b;
+                    part = further + 1;
+                    break;
+                }
+                further -= extra;
+            }
+        }
+        uint32_t plane = 0;
+        for (uint32_t b = 0; b < bucket && b < kBucketDigits; ++b) plane += s_parts[b] > 1 ? s_parts[b] : 0;
+        s_out[0] = bucket;
+        s_out[1] = part;
+        s_out[2] = plane;
+    }
+    __syncthreads();
+    BucketPart p;
+    p.bucket = s_out[0];
+    p.part = s_out[1];
+    p.plane = s_out[2];
+    p.parts = p.bucket < kBucketDigits ? s_parts[p.bucket] : 0;
+    return p;
+}
+
+template <typename T>
+__global__ __launch_bounds__(kBucketBlock) void bucket_sums_kernel(idx_t n, idx_t nnz, uint32_t shift,
+                                                                  uint32_t stride, uint32_t buckets, uint32_t share,
+                                                                  const uint32_t* __restrict__ starts,
+                                                                  const uint16_t* __restrict__ keys,
+                                                                  const T* __restrict__ products, T* __restrict__ y,
+                                                                  double* __restrict__ planes, T alpha, T beta) {
+    typedef typename PairOf<T>::type pair_t;
+    extern __shared__ __align__(16) unsigned char s_raw[];
+    __shared__ uint32_t s_parts[kBucketDigits];
+    __shared__ uint32_t s_mine[3];
+    double* s_acc = reinterpret_cast<double*>(s_raw);
+    const uint32_t tid = threadIdx.x;
+    // a workgroup whose own bucket is in one piece (the common case) need not look at the others
+    BucketPart mine = {blockIdx.x, 0, 1, 0};
+    bool look = blockIdx.x >= kBucketDigits;
+    if (!look) {
+        idx_t at;
+        look = bucket_count(starts, stride, nnz, blockIdx.x, &at) / 2 > share;  // the same for the whole workgroup
+    }
+    if (look) mine = bucket_part(blockIdx.x, false, starts, stride, nnz, share, s_parts, s_mine);
+    const uint32_t bucket = mine.bucket;
+    if (bucket >= buckets) return;  // whole workgroup: no further part left for it, or no such bucket
+    const uint32_t width = 1u << shift;
+    for (uint32_t r = tid; r < width; r += kBucketBlock) s_acc[r] = 0.0;
+    idx_t b0;
+    const uint32_t count = bucket_count(starts, stride, nnz, bucket, &b0);
+    const idx_t e0 = b0 + static_cast<idx_t>(static_cast<uint64_t>(count) * mine.part / mine.parts);
+    const idx_t e1 = b0 + static_cast<idx_t>(static_cast<uint64_t>(count) * (mine.part + 1) / mine.parts);
     __syncthreads();
     // Two neighbouring pairs per load (the vector memory unit takes a load instruction of a wavefront in
-    // the same time whatever its width): entries 2q and 2q + 1, of which the first of the bucket's first
+    // the same time whatever its width): entries 2q and 2q + 1, of which the first of the part's first
     // load and the second of its last may belong to a neighbour.
     const uint32_t* keys2 = reinterpret_cast<const uint32_t*>(keys);
     const pair_t* products2 = reinterpret_cast<const pair_t*>(products);
@@ -622,11 +693,17 @@ __global__ __launch_bounds__(kBucketBlock) void bucket_sums_kernel(idx_t n, idx_
             const uint32_t k = static_cast<uint32_t>(i) * kBucketBlock + tid;
             const uint64_t e = (static_cast<uint64_t>(slab) + k) * 2;
             // the low bits of a key are its place in the bucket, whatever the key holds
-            if (k < cnt && e >= e0) unsafeAtomicAdd(&s_acc[key[i] & (width - 1)], static_cast<double>(p[i].x));
-            if (k < cnt && e + 1 < e1) unsafeAtomicAdd(&s_acc[(key[i] >> 16) & (width - 1)], static_cast<double>(p[i].y));
+            if (k < cnt && e >= e0 && e < e1) unsafeAtomicAdd(&s_acc[key[i] & (width - 1)], static_cast<double>(p[i].x));
+            if (k < cnt && e + 1 >= e0 && e + 1 < e1)
+                unsafeAtomicAdd(&s_acc[(key[i] >> 16) & (width - 1)], static_cast<double>(p[i].y));
         }
     }
     __syncthreads();
+    if (mine.parts > 1) {  // whole workgroup
+        double* out = planes + (static_cast<uint64_t>(mine.plane) + mine.part) * width;
+        for (uint32_t r = tid; r < width; r += kBucketBlock) out[r] = s_acc[r];
+        return;
+    }
     const uint64_t first = static_cast<uint64_t>(bucket) << shift;
     for (uint32_t r = tid; r < width; r += kBucketBlock) {
         const uint64_t c = first + r;
@@ -636,15 +713,69 @@ __global__ __launch_bounds__(kBucketBlock) void bucket_sums_kernel(idx_t n, idx_
     }
 }
 
+// The columns of the buckets that were dealt to several workgroups: their planes added up.  kBucketMergeParts
+// workgroups per bucket, each with its share of the bucket's columns; those of a bucket in one piece have nothing
+// to do.
+constexpr uint32_t kBucketMergeParts = 16;
+template <typename T>
+__global__ __launch_bounds__(kBlock) void bucket_merge_kernel(idx_t n, idx_t nnz, uint32_t shift, uint32_t stride,
+                                                              uint32_t buckets, uint32_t share,
+                                                              const uint32_t* __restrict__ starts,
+                                                              const double* __restrict__ planes, T* __restrict__ y,
+                                                              T alpha, T beta) {
+    __shared__ uint32_t s_parts[kBucketDigits];
+    __shared__ uint32_t s_mine[3];
+    {
+        idx_t at;
+        if (bucket_count(starts, stride, nnz, blockIdx.x / kBucketMergeParts, &at) / 2 <= share) return;  // whole workgroup
+    }
+    const BucketPart mine = bucket_part(blockIdx.x / kBucketMergeParts, true, starts, stride, nnz, share, s_parts, s_mine);
+    if (mine.bucket >= buckets || mine.parts < 2) return;  // whole workgroup
+    const uint32_t width = 1u << shift;
+    const uint32_t slice = (width + kBucketMergeParts - 1) / kBucketMergeParts;
+    const uint32_t r0 = (blockIdx.x % kBucketMergeParts) * slice;
+    const uint32_t r1 = r0 + slice < width ? r0 + slice : width;
+    const uint64_t first = static_cast<uint64_t>(mine.bucket) << shift;
+    const double* in = planes + static_cast<uint64_t>(mine.plane) * width;
+    for (uint32_t r = r0 + threadIdx.x; r < r1; r += kBlock) {
+        const uint64_t c = first + r;
+        if (c >= n) continue;
+        double sum = 0.0;
+        for (uint32_t part = 0; part < mine.parts; ++part) sum += in[static_cast<uint64_t>(part) * width + r];
+        const T s = alpha * static_cast<T>(sum);
+        y[c] = beta == T(0) ? s : s + beta * y[c];
+    }
+}
+
 template <typename T>
 void launch_bucket_sums(hipStream_t stream, idx_t n, idx_t nnz, const BucketedProducts& b, const T* products, T* y,
                         T alpha, T beta) {
     if (b.buckets == 0 || b.buckets > kBucketDigits || b.shift > kBucketMaxShift) return;
     const size_t lds = sizeof(double) << b.shift;
+    // A bucket with more than twice `share` pairs is dealt to several workgroups, ceil(count / share) of them.  share
+    // is the mean of a bucket, so that at most 256 further workgroups are needed, or more where the spare scratch is
+    // short: the split buckets leave fewer than 2 * nnz / share planes (one per `share` pairs, and one more for each
+    // of the fewer than nnz / share buckets that are split at all).
+    const uint64_t max_planes = b.spare != nullptr ? b.spare_bytes / lds : 0;
+    const bool split = max_planes >= 4;
+    uint64_t share = (static_cast<uint64_t>(nnz) + kBucketDigits - 1) / kBucketDigits;
+    if (split) {
+        const uint64_t fits = (2 * static_cast<uint64_t>(nnz) + max_planes - 1) / max_planes + 1;
+        share = share > fits ? share : fits;
+    } else {
+        share = nnz;  // no bucket holds more
+    }
+    double* planes = static_cast<double*>(b.spare);
     (void)hipFuncSetAttribute(reinterpret_cast<const void*>(bucket_sums_kernel<T>),
                               hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
-    hipLaunchKernelGGL((bucket_sums_kernel<T>), dim3(b.buckets), dim3(kBucketBlock), lds, stream, n, nnz, b.shift,
-                       b.stride, b.starts, b.keys, products, y, alpha, beta);
+    hipLaunchKernelGGL((bucket_sums_kernel<T>), dim3(split ? 2 * kBucketDigits : b.buckets), dim3(kBucketBlock), lds, stream,
+                       n, nnz, b.shift, b.stride, b.buckets, static_cast<uint32_t>(share), b.starts, b.keys, products, y,
+                       planes, alpha, beta);
+    if (split) {
+        hipLaunchKernelGGL((bucket_merge_kernel<T>), dim3(kBucketDigits * kBucketMergeParts), dim3(kBlock), 0, stream, n,
+                           nnz, b.shift, b.stride, b.buckets, static_cast<uint32_t>(share), b.starts,
+                           static_cast<const double*>(planes), y, alpha, beta);
+    }
 }
 
 template void launch_bucket_sums<float>(hipStream_t, idx_t, idx_t, const BucketedProducts&, const float*, float*, float,

@@ -162,3 +162,33 @@ def test_few_columns_alg2_repeats_its_bits(torch_gpu, handle, oracle):
     assert np.array_equal(first, second)
     assert_within(first, y_ref, bound, np.float64, what="sorted products")
     assert_within(run(torch_gpu, handle, a, x, y, 1.0, 1.0), y_ref, bound, np.float64, what="copies of y in LDS")
+
+
+# ---- columns that crowd into a few buckets: a crowded bucket is dealt to several workgroups ----
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("rows,per_row", [(300, 3), (40000, 5), (400000, 12)])
+@pytest.mark.parametrize("shape", ["one_bucket", "third_in_one", "two_buckets", "last_bucket"])
+def test_crowded_buckets_exact_on_integers(torch_gpu, handle, dtype, rows, per_row, shape):
+    """2^22 columns are 256 buckets of 16384.  With 900 nonzeros nothing is split (no room for planes of partial
+    sums), with 200 000 the parts are as many as the spare scratch holds planes, with 4.8 M the crowded bucket is
+    dealt out in shares of a 256th of the nonzeros."""
+    n = 1 << 22
+    rng = np.random.default_rng(rows + len(shape))
+    nnz = rows * per_row
+    if shape == "one_bucket":
+        col = rng.integers(5 * 16384, 6 * 16384, nnz)
+    elif shape == "third_in_one":
+        col = np.where(rng.random(nnz) < 0.33, rng.integers(0, 16384, nnz), rng.integers(0, n, nnz))
+    elif shape == "two_buckets":
+        col = np.where(rng.random(nnz) < 0.5, rng.integers(16384, 2 * 16384, nnz), rng.integers(200 * 16384, 201 * 16384, nnz))
+    else:
+        col = rng.integers(n - 16384, n, nnz)
+    a = wl.Csr(rows, n, np.arange(rows + 1) * per_row, col, np.zeros(nnz, dtype))  # duplicates in a row are fine
+    x, y = integer_valued(a, 5)
+    want = np.zeros(n, np.float64)
+    np.add.at(want, col, (a.val.astype(np.float64) * np.repeat(x.astype(np.float64), per_row)))
+    want = 2 * want + y
+    for base in (0, 1):
+        got = run(torch_gpu, handle, a.with_base(base), x, y, 2.0, 1.0)
+        assert np.array_equal(got.astype(np.float64), want), (shape, rows, base)
