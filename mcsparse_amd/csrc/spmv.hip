@@ -609,27 +609,69 @@ __device__ __forceinline__ BucketPart bucket_part(uint32_t group, bool merge, co
         s_parts[b] = count / 2 > share ? (count + share - 1) / share : 1u;  // more than twice the share: split
     }
     __syncthreads();
-    if (threadIdx.x == 0) {
+    if (threadIdx.x < kWave) {  // the first wavefront: four buckets per lane, prefix sums over the lanes
+        static_assert(kBucketDigits == 4 * kWave, "four buckets per lane");
+        const uint32_t lane = threadIdx.x;
+        uint32_t parts[4], extra = 0, planes = 0;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            parts[k] = s_parts[4 * lane + k];
+            extra += parts[k] - 1;
+            planes += parts[k] > 1 ? parts[k] : 0;
+        }
+        uint32_t extra_upto = extra, planes_upto = planes;  // inclusive over lanes
+#pragma unroll
+        for (int d = 1; d < kWave; d *= 2) {
+            const uint32_t e = __shfl_up(extra_upto, d, kWave), q = __shfl_up(planes_upto, d, kWave);
+            if (lane >= static_cast<uint32_t>(d)) {
+                extra_upto += e;
+                planes_upto += q;
+            }
+        }
         uint32_t bucket = kBucketDigits, part = 0;
         if (merge || group < kBucketDigits) {
             bucket = group;
         } else {
-            uint32_t further = group - kBucketDigits;
-            for (uint32_t b = 0; b < kBucketDigits; ++b) {
-                const uint32_t extra = s_parts[b] - 1;
-                if (further < extra) {
-                    bucket = b;
-                    part = further + 1;
-                    break;
+            // the further part number `further` lies with the lane whose buckets hold it
+            const uint32_t further = group - kBucketDigits;
+            const bool here = further >= extra_upto - extra && further < extra_upto;
+            const uint64_t owner = __ballot(here);
+            if (owner != 0) {
+                const int src = __ffsll(static_cast<long long>(owner)) - 1;
+                uint32_t left = further - __shfl(extra_upto - extra, src, kWave);
+                uint32_t found = kBucketDigits, found_part = 0;
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    const uint32_t e = __shfl(parts[k], src, kWave) - 1;
+                    if (found == kBucketDigits) {
+                        if (left < e) {
+                            found = 4 * src + k;
+                            found_part = left + 1;
+                        } else {
+                            left -= e;
+                        }
+                    }
                 }
-                further -= extra;
+                bucket = found;
+                part = found_part;
             }
         }
+        // planes of the split buckets before `bucket`
         uint32_t plane = 0;
-        for (uint32_t b = 0; b < bucket && b < kBucketDigits; ++b) plane += s_parts[b] > 1 ? s_parts[b] : 0;
-        s_out[0] = bucket;
-        s_out[1] = part;
-        s_out[2] = plane;
+        if (bucket < kBucketDigits) {
+            const int src = bucket / 4;
+            plane = __shfl(planes_upto - planes, src, kWave);
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const uint32_t q = __shfl(parts[k], src, kWave);
+                if (static_cast<uint32_t>(k) < bucket % 4) plane += q > 1 ? q : 0;
+            }
+        }
+        if (lane == 0) {
+            s_out[0] = bucket;
+            s_out[1] = part;
+            s_out[2] = plane;
+        }
     }
     __syncthreads();
     BucketPart p;
