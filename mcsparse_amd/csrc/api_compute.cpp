@@ -811,6 +811,10 @@ mcsparseStatus_t mcsparseSpMV_preprocess(mcsparseHandle_t handle, mcsparseOperat
     b.format = matA->format;
     b.transposed = v.transpose;
     b.shape = shape;
+    // the longest row is known from the analysis above; for a transposing direction (rows = the view's columns) it
+    // is not, and the plain kernel is used
+    b.shape.crowded_rows = shape.by_column && !v.transpose && matA->plan.valid && shape.chunks != 0 &&
+                           2 * static_cast<uint64_t>(matA->plan.max_row_len) > static_cast<uint64_t>(nnz) / shape.chunks;
     b.region = banded_region_offset(matA, opA, vb);
     b.grid = 0;
     char* region = static_cast<char*>(externalBuffer) + b.region;

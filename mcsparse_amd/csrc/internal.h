@@ -108,6 +108,9 @@ struct BandedShape {
     // true: entries of a tile in column order, products added to the row sums in LDS as they come
     bool by_column = false;
     uint32_t sub = 1;        // by_column: bands per group; `bands` then counts the groups (planes of partial sums)
+    // by_column: some row holds more than half of what a row chunk holds on average, so that the wavefronts of its
+    // tile would queue on its sum in LDS; the kernel variant that sums such a row's products in registers is used
+    bool crowded_rows = false;
 };
 struct SpmvBanded {
     bool valid = false;

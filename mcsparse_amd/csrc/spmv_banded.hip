@@ -339,7 +339,22 @@ __global__ __launch_bounds__(kBlock) void column_order_split_kernel(idx_t nnz, u
     if (tid <= kXcds) xcd_start[tid] = s_start[s_worst[1] <= s_worst[0] ? 1 : 0][tid];
 }
 
-template <typename T>
+// Adds product p to the sum of row r of the tile, for one entry per lane of a wavefront of which most lanes hold row
+// `lead` (a row with an entry in nearly every column of the band: LDS would take the adds to its sum one after the
+// other).  Those lanes are summed in registers and added once.  live: this lane's entry exists.
+__device__ __forceinline__ void add_to_crowded_row(double* s_acc, uint32_t r, double p, bool live, uint32_t lead) {
+    const bool with_lead = live && r == lead;
+    const double sum = group_sum<kWave>(with_lead ? p : 0.0);
+    if (lane_id() == 0) unsafeAtomicAdd(&s_acc[lead], sum);
+    if (live && !with_lead) unsafeAtomicAdd(&s_acc[r], p);
+}
+constexpr int kCrowdedLanes = 40;  // lanes of a wavefront on one row from which they are summed in registers first
+
+// CROWD: the matrix has a row that holds a large share of a tile (BandedShape::crowded_rows): where most lanes of a
+// wavefront meet on one row in the first entries of a slab, the slab's products for that row are summed in registers
+// (a matrix with dense rows: 0.78 -> 0.44 ms with one such row among 4 M, 0.99 -> 0.67 ms with four).  The test and
+// the second copy of the loop cost the kernel 2 to 10 % on matrices without such rows, which is why it is a variant.
+template <typename T, bool CROWD>
 __global__ __launch_bounds__(kColumnBlock) void spmv_column_order_kernel(idx_t m, idx_t n, idx_t nnz, idx_t base,
                                                                         uint32_t band_shift, uint32_t rows_per_tile,
                                                                         uint32_t chunks, uint32_t units, uint32_t sub,
@@ -413,10 +428,23 @@ __global__ __launch_bounds__(kColumnBlock) void spmv_column_order_kernel(idx_t m
                         key = key > base ? key : base;
                         xv[i] = x[min(key - base, n - 1)];
                     }
+                    // a row past the end of the tile (an overwritten layout) still lies inside the sums
+                    if constexpr (CROWD) {
+                        const uint32_t r_first = min(packed[h][0] >> band_shift, rows_per_tile - 1);
+                        const uint32_t lead = __builtin_amdgcn_readfirstlane(r_first);
+                        if (__popcll(__ballot(r_first == lead)) >= kCrowdedLanes) {  // whole wavefront
+#pragma unroll
+                            for (int i = 0; i < kHalf; ++i) {
+                                const uint32_t k = static_cast<uint32_t>(h * kHalf + i) * kColumnBlock + tid;
+                                const uint32_t r = min(packed[h][i] >> band_shift, rows_per_tile - 1);
+                                add_to_crowded_row(s_acc, r, static_cast<double>(v[h][i] * xv[i]), k < cnt, lead);
+                            }
+                            return;
+                        }
+                    }
 #pragma unroll
                     for (int i = 0; i < kHalf; ++i) {
                         const uint32_t k = static_cast<uint32_t>(h * kHalf + i) * kColumnBlock + tid;
-                        // a row past the end of the tile (an overwritten layout) still lies inside the sums
                         const uint32_t r = min(packed[h][i] >> band_shift, rows_per_tile - 1);
                         if (k < cnt) unsafeAtomicAdd(&s_acc[r], static_cast<double>(v[h][i] * xv[i]));
                     }
@@ -451,12 +479,28 @@ __global__ __launch_bounds__(kColumnBlock) void spmv_column_order_kernel(idx_t m
                         key = key > base ? key : base;
                         xv[i] = x[min(key - base, n - 1)];
                     }
+                    // a row past the end of the tile (an overwritten layout) still lies inside the sums
+                    bool crowded = false;
+                    uint32_t lead = 0;
+                    if constexpr (CROWD) {
+                        const uint32_t r_first = min(packed[0] >> band_shift, rows_per_tile - 1);
+                        lead = __builtin_amdgcn_readfirstlane(r_first);
+                        crowded = __popcll(__ballot(r_first == lead)) >= kCrowdedLanes;  // the same for the wavefront
+                    }
+                    if (CROWD && crowded) {
 #pragma unroll
-                    for (int i = 0; i < kColumnIpt; ++i) {
-                        const uint32_t k = static_cast<uint32_t>(i) * kColumnBlock + tid;
-                        // a row past the end of the tile (an overwritten layout) still lies inside the sums
-                        const uint32_t r = min(packed[i] >> band_shift, rows_per_tile - 1);
-                        if (k < cnt) unsafeAtomicAdd(&s_acc[r], static_cast<double>(v[i] * xv[i]));
+                        for (int i = 0; i < kColumnIpt; ++i) {
+                            const uint32_t k = static_cast<uint32_t>(i) * kColumnBlock + tid;
+                            const uint32_t r = min(packed[i] >> band_shift, rows_per_tile - 1);
+                            add_to_crowded_row(s_acc, r, static_cast<double>(v[i] * xv[i]), k < cnt, lead);
+                        }
+                    } else {
+#pragma unroll
+                        for (int i = 0; i < kColumnIpt; ++i) {
+                            const uint32_t k = static_cast<uint32_t>(i) * kColumnBlock + tid;
+                            const uint32_t r = min(packed[i] >> band_shift, rows_per_tile - 1);
+                            if (k < cnt) unsafeAtomicAdd(&s_acc[r], static_cast<double>(v[i] * xv[i]));
+                        }
                     }
                 }
             }
@@ -617,10 +661,10 @@ void launch_spmv_banded(hipStream_t stream, const BandedShape& s, uint32_t grid,
     T* partials = reinterpret_cast<T*>(w + l.partials);
     if (s.by_column) {
         const int lds = static_cast<int>(s.rows_per_tile * sizeof(double));
-        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(spmv_column_order_kernel<T>),
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, lds);
-        hipLaunchKernelGGL((spmv_column_order_kernel<T>), dim3(kColumnGroupsPerXcd * kXcds), dim3(kColumnBlock), lds,
-                           stream, a.m, a.n, a.nnz, a.base, s.band_shift, s.rows_per_tile, s.chunks, s.tiles / s.sub, s.sub,
+        auto* kernel = s.crowded_rows ? spmv_column_order_kernel<T, true> : spmv_column_order_kernel<T, false>;
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+        hipLaunchKernelGGL(kernel, dim3(kColumnGroupsPerXcd * kXcds), dim3(kColumnBlock), lds, stream, a.m, a.n, a.nnz,
+                           a.base, s.band_shift, s.rows_per_tile, s.chunks, s.tiles / s.sub, s.sub,
                            reinterpret_cast<const uint32_t*>(w + l.xcd_start), reinterpret_cast<uint32_t*>(w + l.next_unit),
                            reinterpret_cast<const idx_t*>(w + l.tile_ptr), reinterpret_cast<const idx_t*>(w + l.entries),
                            reinterpret_cast<const T*>(w + l.vals), static_cast<const T*>(a.x), partials);

@@ -108,6 +108,43 @@ def test_long_rows(torch_gpu, handle, oracle, dtype):
     run(torch_gpu, handle, oracle, a, -1.5, 0.5, op=api.OP_T, band_bytes=1 << 17)
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("dense", [1, 3])
+def test_rows_with_an_entry_in_every_column(torch_gpu, handle, oracle, dtype, dense):
+    """A row that holds more than half of what a row chunk holds on average selects the kernel variant that sums
+    the products of such a row in registers before they go to LDS; integer values make every order exact."""
+    torch = torch_gpu
+    m, n, per_row = 40000, 60000, 6
+    rng = np.random.default_rng(50 + dense)
+    base = wl.uniform_rows(m=m, n=n, per_row=per_row, dtype=dtype, config_id=95)
+    lens = base.row_lengths().copy()
+    full = rng.choice(m, dense, replace=False)
+    lens[full] = n
+    ptr = np.concatenate([[0], np.cumsum(lens)])
+    col = np.empty(int(ptr[-1]), np.int64)
+    for r in range(m):
+        col[ptr[r]:ptr[r + 1]] = np.arange(n) if lens[r] == n else base.col[base.ptr[r]:base.ptr[r + 1]]
+    a = wl.Csr(m, n, ptr, col, rng.integers(-3, 4, col.size).astype(dtype))
+    x = rng.integers(-4, 5, n).astype(dtype)
+    y = rng.integers(-8, 9, m).astype(dtype)
+    d_ptr, d_col, d_val, d_x, d_y = (dev(torch, v) for v in (a.ptr, a.col, a.val, x, y))
+    mat = api.SpMat(a.m, a.n, a.nnz, d_ptr, d_col, d_val)
+    mat.set_band_bytes(1 << 14)
+    vx, vy = api.DnVec(d_x), api.DnVec(d_y)
+    ct = api.maca_type(dtype)
+    st, size = api.spmv_preprocess_buffer_size(handle, api.OP_N, 2.0, mat, vx, -1.0, vy, ct)
+    assert st == api.STATUS_SUCCESS
+    buf = torch.empty(size, dtype=torch.uint8, device="cuda")
+    assert api.spmv_preprocess(handle, api.OP_N, 2.0, mat, vx, -1.0, vy, ct, buf) == api.STATUS_SUCCESS
+    assert mat.spmv_preprocess_state()[0] == 3
+    want = 2 * (a.to_scipy().astype(np.float64) @ x.astype(np.float64)) - y
+    for _ in range(2):
+        d_y.copy_(torch.from_numpy(y))
+        assert api.spmv(handle, api.OP_N, 2.0, mat, vx, -1.0, vy, ct, buf) == api.STATUS_SUCCESS
+        torch.cuda.synchronize()
+        assert np.array_equal(d_y.cpu().numpy().astype(np.float64), want)
+
+
 def test_alg2_does_not_use_the_copy(torch_gpu, handle, oracle):
     """MCSPARSE_SPMV_CSR_ALG2 promises the same bits on every run: the call runs the row kernels."""
     a = wl.uniform_rows(m=20000, n=300000, per_row=8, dtype=np.float64, config_id=91)
