@@ -34,6 +34,7 @@ HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 OTHERS = ["c4-64", "c3", "c3t", "c5", "c5-spmv", "c5-coo", "c4-8", "c4-256", "c4-64-col", "c1",
           "c2-alg2", "c3-alg2", "c3t-alg2", "c2-direct", "c3-direct", "c3t-direct", "c4-64-direct"]
 OTHERS_BUDGET_S = 200.0  # wall-clock budget of the default invocation for the workloads above
+SPIN_UP_S = 0.03  # every workload runs its steps for this long before the warmup steps (see run_workload)
 
 
 # HBM/fabric bytes per call (all kernels of one step together), from rocprofv3 FETCH_SIZE and
@@ -309,25 +310,49 @@ def run_workload(name, args, ctx, steps=None, warmup=None, with_cpu=True):
     torch.cuda.synchronize()
     first_pass_ms = (time.perf_counter() - t0) * 1e3 / copies
 
+    # A device that has been idle runs its first 10 to 20 ms of work slower (the clocks come up, the page
+    # tables of the rotated operand copies fill): SpMM with 64 columns 0.55 ms per step straight after 3
+    # warmup steps and 0.50 ms from the 30th step on.  The steps are therefore repeated for SPIN_UP_S before
+    # the warmup steps proper; the count goes into the output line.
+    spin_up_steps = 0
+    t_spin = time.perf_counter()
+    while time.perf_counter() - t_spin < SPIN_UP_S:
+        for i in range(max(copies, 4)):
+            step(spin_up_steps + i)
+        spin_up_steps += max(copies, 4)
+        torch.cuda.synchronize()
+
     for i in range(warmup):
         step(i)
     torch.cuda.synchronize()
 
-    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+    # The timed region: exactly `steps` steps between two synchronisations, with one HIP event at each end
+    # and none inside (an event record is a packet of its own on the stream: a pair around every step costs
+    # about 5 us per step, which is 6 % of a step of the headline workload).
+    region = (torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
     torch.cuda.synchronize()
     t0 = time.perf_counter()
+    region[0].record(stream)
+    for i in range(steps):
+        step(i)
+    region[1].record(stream)
+    torch.cuda.synchronize()
+    wall_s = time.perf_counter() - t0
+    ms_per_step = wall_s * 1e3 / steps
+    region_ms = region[0].elapsed_time(region[1]) / steps
+    # The same steps once more with an event pair around each, for the spread between steps (the pairs
+    # themselves keep a step's first kernel from starting under the last one's tail: about 2 us per step).
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
     for i in range(steps):
         ev[i][0].record(stream)
         step(i)
         ev[i][1].record(stream)
     torch.cuda.synchronize()
-    wall_s = time.perf_counter() - t0
-    ms_per_step = wall_s * 1e3 / steps
     dev_ms = np.array([e0.elapsed_time(e1) for e0, e1 in ev])
     dev_avg_ms = float(dev_ms.mean())
 
     value = algo_bytes / (ms_per_step * 1e-3) / 1e9
-    achieved = algo_bytes / (dev_avg_ms * 1e-3) / 1e9
+    achieved = algo_bytes / (region_ms * 1e-3) / 1e9
     mat0 = sets[0].get("mat")
     plan = mat0.plan() if mat0 is not None and kind in ("spmv", "spmv-csc") else None
     banded = mat0.spmv_preprocess_state() if mat0 is not None and kind in ("spmv", "spmv-csc") else None
@@ -344,6 +369,7 @@ def run_workload(name, args, ctx, steps=None, warmup=None, with_cpu=True):
         "n_gpus": 1,
         "steps": steps,
         "warmup": warmup,
+        "spin_up_steps_before_warmup": spin_up_steps,
         "ms_per_step": round(ms_per_step, 5),
         "higher_is_better": True,
         "scaling": "weak",
@@ -360,7 +386,11 @@ def run_workload(name, args, ctx, steps=None, warmup=None, with_cpu=True):
         "first_call_ms": round(first_pass_ms, 4),
         "preprocess_ms": round(min(preprocess_ms), 4) if preprocess_ms else None,
         "device_ms_per_step": {"mean": round(dev_avg_ms, 5), "median": round(float(np.median(dev_ms)), 5),
-                               "min": round(float(dev_ms.min()), 5)},
+                               "min": round(float(dev_ms.min()), 5),
+                               "timed_region_mean": round(region_ms, 5),
+                               "how": "timed_region_mean (what roofline.achieved uses): two HIP events around the "
+                                      "timed region / steps; mean, median, min: event pairs around every step in a "
+                                      "second pass of the same steps"},
         "spmv_plan": {"family": plan[0], "lanes_per_row": plan[1]} if plan else None,
         "spmv_preprocess": {"state": banded[0], "bands": banded[1], "rows_per_tile": banded[2]} if banded else None,
         "roofline": {"bound": "hbm", "achieved": round(achieved, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
