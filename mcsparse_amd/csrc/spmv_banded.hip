@@ -298,9 +298,12 @@ __global__ __launch_bounds__(kBlock) void column_order_pack_kernel(idx_t nnz, id
 // One workgroup per compute unit: workgroup i belongs to XCD i % 8 and takes every 32nd unit (the tiles
 // of one row chunk in one band group) of that XCD's stretch.  The row sums of a unit live in LDS as
 // doubles (fp32 products are widened: ds_add_f32 runs at a quarter of the rate of ds_add_f64 on this
-// chip); a thread has kColumnIpt gathers in flight (4, 8, 16 measured: 16 is 1-4 % ahead).
+// chip).  A thread keeps two sets of entries in registers, kColumnSet32 or kColumnSet64 each: the largest that fit
+// the 128 registers a thread of a 1024-thread workgroup can have (fp32 12 / 14 / 16 / 18 / 20: 16 and 18 level, the
+// others 1-3 % behind; fp64 8 / 10 / 12 / 13: 75.0 / 73.7 / 72.5 / 70.3 us on 1 M rows x 16, 14 spills registers).
 constexpr int kColumnBlock = 1024;
-constexpr int kColumnIpt = 16;
+constexpr int kColumnSet32 = 16;
+constexpr int kColumnSet64 = 13;
 
 // xcd_start for the kernel below, in units.  A stretch is dealt to the kColumnGroupsPerXcd workgroups of
 // its XCD in turns, so what counts is the largest number of nonzeros any one workgroup ends up with.
@@ -400,109 +403,86 @@ __global__ __launch_bounds__(kColumnBlock) void spmv_column_order_kernel(idx_t m
             e1 = e1 < nnz ? e1 : nnz;
             e1 = e1 > e0 ? e1 : e0;
             const idx_t band_key = (group * sub + b) << band_shift;
-            if constexpr (sizeof(T) == 4) {
-                // fp32: two sets of kColumnIpt entries per thread take turns.  While the gathers and LDS adds of one
-                // run, the entries of the other are on their way, and the next ones are asked for as soon as a set
-                // has been used up (power-law matrix 434 -> 399 us, its transpose 359 -> 341 us; sets of half the
-                // size 416, 351 us).  With fp64 values two sets of that size do not fit the registers, and sets of
-                // half the size lost 3 % on the uniform matrix: the plain loop below stays.
-                constexpr int kHalf = kColumnIpt;
-                constexpr idx_t kSlab = kColumnBlock * kHalf * 2;
-                idx_t packed[2][kHalf];
-                T v[2][kHalf];
-                auto ask = [&](int h, idx_t slab) {
-                    const uint32_t cnt = e1 - slab < kSlab ? e1 - slab : kSlab;  // slab < e1
+            // Two sets of kSet entries per thread take turns.  A set is gathered for and added while the loads of
+            // the other are on their way: the gathers of a set are issued first, then the loads of the next set,
+            // and only then are the gathers waited for (loads return in the order they were issued, so a wait for
+            // gathers that had been issued after the next set's loads would wait for those as well; in that order
+            // 1 M rows x 16 in fp64 took 78.3 us and the power-law matrix in fp32 395 us, in this one 70.3 and 384).
+            constexpr int kSet = sizeof(T) == 4 ? kColumnSet32 : kColumnSet64;
+            constexpr idx_t kPart = kColumnBlock * kSet;  // entries the workgroup takes per set
+            idx_t packed[2][kSet];
+            T v[2][kSet];
+            auto ask = [&](int h, idx_t start) {  // start < e1
+                const uint32_t cnt = e1 - start < kPart ? e1 - start : kPart;
 #pragma unroll
-                    for (int i = 0; i < kHalf; ++i) {
-                        const uint32_t k = min(static_cast<uint32_t>(h * kHalf + i) * kColumnBlock + tid, cnt - 1);
-                        packed[h][i] = load_stream(entries + slab + k);
-                        v[h][i] = load_stream(vals + slab + k);
-                    }
-                };
-                auto use = [&](int h, idx_t slab) {
-                    const uint32_t cnt = e1 - slab < kSlab ? e1 - slab : kSlab;
-                    T xv[kHalf];
-#pragma unroll
-                    for (int i = 0; i < kHalf; ++i) {
-                        idx_t key = band_key | (packed[h][i] & band_mask);  // column + base
-                        key = key > base ? key : base;
-                        xv[i] = x[min(key - base, n - 1)];
-                    }
-                    // a row past the end of the tile (an overwritten layout) still lies inside the sums
-                    if constexpr (CROWD) {
-                        const uint32_t r_first = min(packed[h][0] >> band_shift, rows_per_tile - 1);
-                        const uint32_t lead = __builtin_amdgcn_readfirstlane(r_first);
-                        if (__popcll(__ballot(r_first == lead)) >= kCrowdedLanes) {  // whole wavefront
-#pragma unroll
-                            for (int i = 0; i < kHalf; ++i) {
-                                const uint32_t k = static_cast<uint32_t>(h * kHalf + i) * kColumnBlock + tid;
-                                const uint32_t r = min(packed[h][i] >> band_shift, rows_per_tile - 1);
-                                add_to_crowded_row(s_acc, r, static_cast<double>(v[h][i] * xv[i]), k < cnt, lead);
-                            }
-                            return;
-                        }
-                    }
-#pragma unroll
-                    for (int i = 0; i < kHalf; ++i) {
-                        const uint32_t k = static_cast<uint32_t>(h * kHalf + i) * kColumnBlock + tid;
-                        const uint32_t r = min(packed[h][i] >> band_shift, rows_per_tile - 1);
-                        if (k < cnt) unsafeAtomicAdd(&s_acc[r], static_cast<double>(v[h][i] * xv[i]));
-                    }
-                };
-                if (e0 < e1) {
-                    ask(0, e0);
-                    ask(1, e0);
+                for (int i = 0; i < kSet; ++i) {
+                    const uint32_t k = min(static_cast<uint32_t>(i) * kColumnBlock + tid, cnt - 1);
+                    packed[h][i] = load_stream(entries + start + k);
+                    v[h][i] = load_stream(vals + start + k);
                 }
-                for (idx_t slab = e0; slab < e1; slab += kSlab) {
-                    const bool more = e1 - slab > kSlab;  // whole workgroup
-                    use(0, slab);
-                    if (more) ask(0, slab + kSlab);
-                    use(1, slab);
-                    if (more) ask(1, slab + kSlab);
+            };
+            auto gather = [&](int h, T (&xv)[kSet]) {
+#pragma unroll
+                for (int i = 0; i < kSet; ++i) {
+                    idx_t key = band_key | (packed[h][i] & band_mask);  // column + base
+                    key = key > base ? key : base;
+                    xv[i] = x[min(key - base, n - 1)];
                 }
-            } else {
-                for (idx_t slab = e0; slab < e1; slab += kColumnBlock * kColumnIpt) {
-                    const uint32_t cnt = e1 - slab < static_cast<idx_t>(kColumnBlock * kColumnIpt)
-                                             ? e1 - slab
-                                             : kColumnBlock * kColumnIpt;
-                    idx_t packed[kColumnIpt];
-                    T v[kColumnIpt], xv[kColumnIpt];
+            };
+            auto add = [&](int h, idx_t start, const T (&xv)[kSet]) {
+                const uint32_t cnt = e1 - start < kPart ? e1 - start : kPart;
+                // a row past the end of the tile (an overwritten layout) still lies inside the sums
+                if constexpr (CROWD) {
+                    const uint32_t r_first = min(packed[h][0] >> band_shift, rows_per_tile - 1);
+                    const uint32_t lead = __builtin_amdgcn_readfirstlane(r_first);
+                    if (__popcll(__ballot(r_first == lead)) >= kCrowdedLanes) {  // whole wavefront
 #pragma unroll
-                    for (int i = 0; i < kColumnIpt; ++i) {
-                        const uint32_t k = min(static_cast<uint32_t>(i) * kColumnBlock + tid, cnt - 1);
-                        packed[i] = load_stream(entries + slab + k);
-                        v[i] = load_stream(vals + slab + k);
-                    }
-#pragma unroll
-                    for (int i = 0; i < kColumnIpt; ++i) {
-                        idx_t key = band_key | (packed[i] & band_mask);  // column + base
-                        key = key > base ? key : base;
-                        xv[i] = x[min(key - base, n - 1)];
-                    }
-                    // a row past the end of the tile (an overwritten layout) still lies inside the sums
-                    bool crowded = false;
-                    uint32_t lead = 0;
-                    if constexpr (CROWD) {
-                        const uint32_t r_first = min(packed[0] >> band_shift, rows_per_tile - 1);
-                        lead = __builtin_amdgcn_readfirstlane(r_first);
-                        crowded = __popcll(__ballot(r_first == lead)) >= kCrowdedLanes;  // the same for the wavefront
-                    }
-                    if (CROWD && crowded) {
-#pragma unroll
-                        for (int i = 0; i < kColumnIpt; ++i) {
+                        for (int i = 0; i < kSet; ++i) {
                             const uint32_t k = static_cast<uint32_t>(i) * kColumnBlock + tid;
-                            const uint32_t r = min(packed[i] >> band_shift, rows_per_tile - 1);
-                            add_to_crowded_row(s_acc, r, static_cast<double>(v[i] * xv[i]), k < cnt, lead);
+                            const uint32_t r = min(packed[h][i] >> band_shift, rows_per_tile - 1);
+                            add_to_crowded_row(s_acc, r, static_cast<double>(v[h][i] * xv[i]), k < cnt, lead);
                         }
-                    } else {
-#pragma unroll
-                        for (int i = 0; i < kColumnIpt; ++i) {
-                            const uint32_t k = static_cast<uint32_t>(i) * kColumnBlock + tid;
-                            const uint32_t r = min(packed[i] >> band_shift, rows_per_tile - 1);
-                            if (k < cnt) unsafeAtomicAdd(&s_acc[r], static_cast<double>(v[i] * xv[i]));
-                        }
+                        return;
                     }
                 }
+#pragma unroll
+                for (int i = 0; i < kSet; ++i) {
+                    const uint32_t k = static_cast<uint32_t>(i) * kColumnBlock + tid;
+                    const uint32_t r = min(packed[h][i] >> band_shift, rows_per_tile - 1);
+                    if (k < cnt) unsafeAtomicAdd(&s_acc[r], static_cast<double>(v[h][i] * xv[i]));
+                }
+            };
+            // A set with a successor: gathers, then the successor's loads, then the adds.  The loads are not
+            // made conditional inside it: the compiler then counts the loads in flight for the path without them
+            // and waits for all of them before the first add.  The last set of a tile runs without.
+            auto step = [&](int h, idx_t start) {
+                T xv[kSet];
+                gather(h, xv);
+                __builtin_amdgcn_sched_barrier(0);
+                ask(h ^ 1, start + kPart);
+                __builtin_amdgcn_sched_barrier(0);
+                add(h, start, xv);
+            };
+            auto last = [&](int h, idx_t start) {
+                T xv[kSet];
+                gather(h, xv);
+                add(h, start, xv);
+            };
+            if (e0 < e1) {
+                ask(0, e0);
+                idx_t start = e0;
+                int h = 0;  // the set that holds the entries from `start` (the same for the workgroup)
+                while (e1 - start > kPart) {
+                    step(0, start);
+                    start += kPart;
+                    h = 1;
+                    if (e1 - start <= kPart) break;
+                    step(1, start);
+                    start += kPart;
+                    h = 0;
+                }
+                if (h == 0) last(0, start);
+                else last(1, start);
             }
         }
         __syncthreads();

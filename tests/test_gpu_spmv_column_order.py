@@ -145,6 +145,50 @@ def test_rows_with_an_entry_in_every_column(torch_gpu, handle, oracle, dtype, de
         assert np.array_equal(d_y.cpu().numpy().astype(np.float64), want)
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_tiles_around_whole_sets_of_entries(torch_gpu, handle, oracle, dtype):
+    """The kernel takes a tile in sets of 1024 x 16 (fp32) or 1024 x 13 (fp64) entries, the loads of a set issued
+    under the arithmetic of the one before: tiles of 0, 1, and one less than, exactly and one more than one, two and
+    three sets, each several times, with integer values so that any order of the sums is exact."""
+    torch = torch_gpu
+    rows_per_tile, groups, chunks = 16384, 32, 8
+    keys = (1 << 12) // np.dtype(dtype).itemsize  # columns per group with 4 KiB bands
+    per_set = 1024 * (16 if dtype == np.float32 else 13)
+    sizes = [0, 1, per_set - 1, per_set, per_set + 1, 2 * per_set - 1, 2 * per_set, 2 * per_set + 1, 3 * per_set,
+             3 * per_set + 1, 777, per_set // 2]
+    rng = np.random.default_rng(77)
+    rows, cols = [], []
+    for t in range(groups * chunks):
+        g, c = divmod(t, chunks)
+        count = sizes[(t * 5 + g) % len(sizes)]
+        rows.append(rng.integers(0, rows_per_tile, count) + c * rows_per_tile)
+        cols.append(rng.integers(0, keys, count) + g * keys)
+    rows, cols = np.concatenate(rows), np.concatenate(cols)
+    order = np.lexsort((cols, rows))
+    rows, cols = rows[order], cols[order]
+    m, n = rows_per_tile * chunks, keys * groups
+    ptr = np.concatenate([[0], np.cumsum(np.bincount(rows, minlength=m))])
+    a = wl.Csr(m, n, ptr, cols, rng.integers(-3, 4, cols.size).astype(dtype))
+    x = rng.integers(-4, 5, n).astype(dtype)
+    y = rng.integers(-8, 9, m).astype(dtype)
+    d_ptr, d_col, d_val, d_x, d_y = (dev(torch, v) for v in (a.ptr, a.col, a.val, x, y))
+    mat = api.SpMat(a.m, a.n, a.nnz, d_ptr, d_col, d_val)
+    mat.set_band_bytes(1 << 12)
+    vx, vy = api.DnVec(d_x), api.DnVec(d_y)
+    ct = api.maca_type(dtype)
+    st, size = api.spmv_preprocess_buffer_size(handle, api.OP_N, 1.0, mat, vx, 1.0, vy, ct)
+    assert st == api.STATUS_SUCCESS
+    buf = torch.empty(size, dtype=torch.uint8, device="cuda")
+    assert api.spmv_preprocess(handle, api.OP_N, 1.0, mat, vx, 1.0, vy, ct, buf) == api.STATUS_SUCCESS
+    assert mat.spmv_preprocess_state() == (3, groups, rows_per_tile)
+    want = a.to_scipy().astype(np.float64) @ x.astype(np.float64) + y
+    for _ in range(2):
+        d_y.copy_(torch.from_numpy(y))
+        assert api.spmv(handle, api.OP_N, 1.0, mat, vx, 1.0, vy, ct, buf) == api.STATUS_SUCCESS
+        torch.cuda.synchronize()
+        assert np.array_equal(d_y.cpu().numpy().astype(np.float64), want)
+
+
 def test_alg2_does_not_use_the_copy(torch_gpu, handle, oracle):
     """MCSPARSE_SPMV_CSR_ALG2 promises the same bits on every run: the call runs the row kernels."""
     a = wl.uniform_rows(m=20000, n=300000, per_row=8, dtype=np.float64, config_id=91)
