@@ -267,6 +267,39 @@ __global__ __launch_bounds__(kBlock) void banded_reduce_kernel(idx_t m, uint32_t
     }
 }
 
+// The same with 16 bytes per access: V = 16 / sizeof(T) neighbouring rows per thread.  m is a multiple of V and
+// partials and y are 16-byte aligned (the launch checks).
+template <typename T, bool BETA0>
+__global__ __launch_bounds__(kBlock) void banded_reduce_wide_kernel(idx_t m, uint32_t bands, const T* __restrict__ partials,
+                                                                    T* __restrict__ y, T alpha, T beta,
+                                                                    uint32_t* __restrict__ next_unit) {
+    constexpr int V = 16 / sizeof(T);
+    typedef T vec_t __attribute__((ext_vector_type(V)));
+    if (next_unit != nullptr && blockIdx.x == 0 && threadIdx.x < kXcds) next_unit[threadIdx.x] = kColumnGroupsPerXcd;
+    const uint64_t r = (static_cast<uint64_t>(blockIdx.x) * kBlock + threadIdx.x) * V;
+    if (r >= m) return;
+    constexpr uint32_t kAhead = 8;
+    vec_t sum = vec_t(0);
+    for (uint32_t b0 = 0; b0 < bands; b0 += kAhead) {
+        vec_t p[kAhead];
+#pragma unroll
+        for (uint32_t i = 0; i < kAhead; ++i) {
+            const uint32_t b = min(b0 + i, bands - 1);
+            p[i] = __builtin_nontemporal_load(reinterpret_cast<const vec_t*>(partials + static_cast<uint64_t>(b) * m + r));
+        }
+#pragma unroll
+        for (uint32_t i = 0; i < kAhead; ++i) {
+            if (b0 + i < bands) sum = (b0 + i == 0) ? p[i] : sum + p[i];
+        }
+    }
+    vec_t* out = reinterpret_cast<vec_t*>(y + r);
+    if constexpr (BETA0) {
+        *out = alpha * sum;
+    } else {
+        *out = beta * *out + alpha * sum;
+    }
+}
+
 // ------------------------------------------------------------------------------------------
 // tiles in column order
 // ------------------------------------------------------------------------------------------
@@ -655,8 +688,22 @@ void launch_spmv_banded(hipStream_t stream, const BandedShape& s, uint32_t grid,
                            reinterpret_cast<const idx_t*>(w + l.tile_ptr), reinterpret_cast<const idx_t*>(w + l.entries),
                            reinterpret_cast<const T*>(w + l.vals), static_cast<const T*>(a.x), partials);
     }
-    const dim3 rows_grid((a.m + kBlock - 1) / kBlock);
     uint32_t* next_unit = s.by_column ? reinterpret_cast<uint32_t*>(w + l.next_unit) : nullptr;
+    constexpr idx_t kWide = 16 / sizeof(T);
+    // 16 bytes per access: 1 M rows, four planes of fp64 10.9 -> 8.8 us; eight planes of fp32 (four rows per thread) 1 us slower
+    if (sizeof(T) == 8 && a.m % kWide == 0 &&
+        ((reinterpret_cast<uintptr_t>(partials) | reinterpret_cast<uintptr_t>(a.y)) & 15u) == 0) {
+        const dim3 wide_grid((a.m / kWide + kBlock - 1) / kBlock);
+        if (beta == T(0)) {
+            hipLaunchKernelGGL((banded_reduce_wide_kernel<T, true>), wide_grid, dim3(kBlock), 0, stream, a.m, s.bands,
+                               static_cast<const T*>(partials), static_cast<T*>(a.y), alpha, beta, next_unit);
+        } else {
+            hipLaunchKernelGGL((banded_reduce_wide_kernel<T, false>), wide_grid, dim3(kBlock), 0, stream, a.m, s.bands,
+                               static_cast<const T*>(partials), static_cast<T*>(a.y), alpha, beta, next_unit);
+        }
+        return;
+    }
+    const dim3 rows_grid((a.m + kBlock - 1) / kBlock);
     if (beta == T(0)) {
         hipLaunchKernelGGL((banded_reduce_kernel<T, true>), rows_grid, dim3(kBlock), 0, stream, a.m, s.bands,
                            static_cast<const T*>(partials), static_cast<T*>(a.y), alpha, beta, next_unit);
