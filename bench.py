@@ -54,7 +54,7 @@ MEASURED_TRAFFIC = {
     ("c5-spmv", 2): (_traffic(481330.8 + 65544.6, 131202.3 + 16384.0),
                         "profiles/spmv_banded_f32_c3_powerlaw.txt"),
     # spmv_column_order_kernel + banded_reduce_kernel
-    ("c2", 3): (_traffic(115043.4 + 20557.7, 32776.0 + 8192.0), "profiles/spmv_column_order_f64_c2_1Mx16.txt"),
+    ("c2", 3): (_traffic(115061.1 + 20621.1, 32776.0 + 8192.0), "profiles/spmv_column_order_f64_c2_1Mx16.txt"),
     ("c3", 3): (_traffic(555599.1 + 65550.5, 131136.0 + 16384.0), "profiles/spmv_column_order_f32_c3_powerlaw.txt"),
     ("c3t", 3): (_traffic(583253.5 + 65550.5, 131136.0 + 16384.0), "profiles/spmv_column_order_f32_c3_powerlaw.txt"),
     ("c5-spmv", 3): (_traffic(601424.1 + 65548.9, 131072.0 + 16384.0),
