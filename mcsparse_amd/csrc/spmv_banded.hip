@@ -331,12 +331,69 @@ __global__ __launch_bounds__(kBlock) void column_order_pack_kernel(idx_t nnz, id
 // One workgroup per compute unit: workgroup i belongs to XCD i % 8 and takes every 32nd unit (the tiles
 // of one row chunk in one band group) of that XCD's stretch.  The row sums of a unit live in LDS as
 // doubles (fp32 products are widened: ds_add_f32 runs at a quarter of the rate of ds_add_f64 on this
-// chip).  A thread keeps two sets of entries in registers, kColumnSet32 or kColumnSet64 each: the largest that fit
-// the 128 registers a thread of a 1024-thread workgroup can have (fp32 12 / 14 / 16 / 18 / 20: 16 and 18 level, the
-// others 1-3 % behind; fp64 8 / 10 / 12 / 13: 75.0 / 73.7 / 72.5 / 70.3 us on 1 M rows x 16, 14 spills registers).
+// chip).  A thread keeps two sets of entries in registers, kColumnSet32 or kColumnSet64 each: what fits the 128
+// registers a thread of a 1024-thread workgroup can have (fp64, one entry per load, 8 / 10 / 12 / 13: 75.0 / 73.7 /
+// 72.5 / 70.3 us on 1 M rows x 16, 14 spills registers; fp32, four entries per load, 12: 343 us on the power-law
+// matrix, 16 spills registers: 362 us).
 constexpr int kColumnBlock = 1024;
-constexpr int kColumnSet32 = 16;
+constexpr int kColumnSet32 = 12;
 constexpr int kColumnSet64 = 13;
+// fp32: the entries of a tile lie in blocks of kColumnQuad * 64, counted from the tile's first entry at a multiple
+// of kColumnQuad (the up to three entries ahead of it are taken one by one).  A block of L entries in column order is
+// stored so that lane l < L / 4 finds its entries l, L/4 + l, 2 L/4 + l, 3 L/4 + l of the block side by side at
+// 4 l .. 4 l + 3 (the last L % 4 entries stay where they are): one 128-bit load per lane brings a wavefront four
+// runs of neighbouring entries (the vector memory unit takes a load instruction in the same time whatever its
+// width: power-law matrix 384 -> 343 us, its transpose 324 -> 295 us), an element is an entry of the block exactly
+// when its place is below L, and a tile's last, partial block needs no code of its own.  With fp64 values two sets
+// of 12 do not fit the registers next to the 128-bit loads and sets of 8 lose more than the loads gain (75 against
+// 69 us on 1 M rows x 16): that copy keeps its entries in column order, one per load.
+constexpr int kColumnQuad = 4;
+constexpr uint32_t kColumnQuadBlock = kColumnQuad * kWave;
+static_assert(kColumnSet32 % kColumnQuad == 0, "whole blocks per set");
+template <typename T>
+constexpr bool column_order_quads() { return sizeof(T) == 4; }
+
+// Puts the blocks of every tile into that order, in place.  One workgroup per tile, kInterleaveBlocks blocks per
+// round: a thread reads its element of each of them, then writes.
+constexpr int kInterleaveBlocks = 8;
+template <typename T>
+__global__ __launch_bounds__(kColumnQuadBlock) void column_order_interleave_kernel(idx_t nnz,
+                                                                                  const idx_t* __restrict__ tile_ptr,
+                                                                                  idx_t* entries, T* vals) {
+    idx_t e0 = tile_ptr[blockIdx.x];
+    idx_t e1 = tile_ptr[blockIdx.x + 1];
+    e0 = e0 < nnz ? e0 : nnz;
+    e1 = e1 < nnz ? e1 : nnz;
+    e1 = e1 > e0 ? e1 : e0;
+    const idx_t a0 = (e0 + kColumnQuad - 1) / kColumnQuad * kColumnQuad;
+    if (a0 >= e1) return;  // whole workgroup
+    const uint32_t len = e1 - a0;
+    const uint32_t blocks = (len + kColumnQuadBlock - 1) / kColumnQuadBlock;
+    const uint32_t p = threadIdx.x;
+    for (uint32_t b0 = 0; b0 < blocks; b0 += kInterleaveBlocks) {
+        idx_t w[kInterleaveBlocks];
+        T v[kInterleaveBlocks];
+#pragma unroll
+        for (int i = 0; i < kInterleaveBlocks; ++i) {
+            const uint32_t at = min((b0 + i) * kColumnQuadBlock + p, len - 1);
+            w[i] = entries[a0 + at];
+            v[i] = vals[a0 + at];
+        }
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < kInterleaveBlocks; ++i) {
+            const uint32_t first = (b0 + i) * kColumnQuadBlock;
+            if (first + p < len) {
+                const uint32_t in_block = len - first < kColumnQuadBlock ? len - first : kColumnQuadBlock;
+                const uint32_t q = in_block / kColumnQuad;
+                const uint32_t to = p < q * kColumnQuad ? (p % q) * kColumnQuad + p / q : p;
+                entries[a0 + first + to] = w[i];
+                vals[a0 + first + to] = v[i];
+            }
+        }
+        __syncthreads();
+    }
+}
 
 // xcd_start for the kernel below, in units.  A stretch is dealt to the kColumnGroupsPerXcd workgroups of
 // its XCD in turns, so what counts is the largest number of nonzeros any one workgroup ends up with.
@@ -445,13 +502,44 @@ __global__ __launch_bounds__(kColumnBlock) void spmv_column_order_kernel(idx_t m
             constexpr idx_t kPart = kColumnBlock * kSet;  // entries the workgroup takes per set
             idx_t packed[2][kSet];
             T v[2][kSet];
-            auto ask = [&](int h, idx_t start) {  // start < e1
+            // Element i of a thread's set lies at place(i) of the set.  In blocks: block i / 4 of the wavefront, at
+            // 4 * lane + i % 4; else entry by entry across the workgroup.
+            constexpr bool kQuads = column_order_quads<T>();
+            const uint32_t lane_first = (tid / kWave) * kColumnQuadBlock + (tid % kWave) * kColumnQuad;
+            auto place = [&](int i) {
+                if constexpr (kQuads) {
+                    return static_cast<uint32_t>(i / kColumnQuad) * (kColumnBlock * kColumnQuad) + lane_first +
+                           static_cast<uint32_t>(i % kColumnQuad);
+                } else {
+                    return static_cast<uint32_t>(i) * kColumnBlock + tid;
+                }
+            };
+            auto ask = [&](int h, idx_t start) {  // start < e1 (and a multiple of kColumnQuad where that matters)
                 const uint32_t cnt = e1 - start < kPart ? e1 - start : kPart;
+                if constexpr (kQuads) {
+                    typedef idx_t quad_t __attribute__((ext_vector_type(4)));
+                    const uint32_t last_quad = (cnt - 1) / kColumnQuad * kColumnQuad;
 #pragma unroll
-                for (int i = 0; i < kSet; ++i) {
-                    const uint32_t k = min(static_cast<uint32_t>(i) * kColumnBlock + tid, cnt - 1);
-                    packed[h][i] = load_stream(entries + start + k);
-                    v[h][i] = load_stream(vals + start + k);
+                    for (int j = 0; j < kSet / kColumnQuad; ++j) {
+                        const idx_t at = start + min(place(j * kColumnQuad), last_quad);
+                        const quad_t q = __builtin_nontemporal_load(reinterpret_cast<const quad_t*>(entries + at));
+                        const quad_t f = __builtin_nontemporal_load(reinterpret_cast<const quad_t*>(vals + at));
+                        packed[h][j * 4 + 0] = q.x;
+                        packed[h][j * 4 + 1] = q.y;
+                        packed[h][j * 4 + 2] = q.z;
+                        packed[h][j * 4 + 3] = q.w;
+                        v[h][j * 4 + 0] = __uint_as_float(f.x);
+                        v[h][j * 4 + 1] = __uint_as_float(f.y);
+                        v[h][j * 4 + 2] = __uint_as_float(f.z);
+                        v[h][j * 4 + 3] = __uint_as_float(f.w);
+                    }
+                } else {
+#pragma unroll
+                    for (int i = 0; i < kSet; ++i) {
+                        const uint32_t k = min(place(i), cnt - 1);
+                        packed[h][i] = load_stream(entries + start + k);
+                        v[h][i] = load_stream(vals + start + k);
+                    }
                 }
             };
             auto gather = [&](int h, T (&xv)[kSet]) {
@@ -462,7 +550,7 @@ __global__ __launch_bounds__(kColumnBlock) void spmv_column_order_kernel(idx_t m
                     xv[i] = x[min(key - base, n - 1)];
                 }
             };
-            auto add = [&](int h, idx_t start, const T (&xv)[kSet]) {
+            auto add = [&](int h, idx_t start, const T (&xv)[kSet], bool whole_set) {
                 const uint32_t cnt = e1 - start < kPart ? e1 - start : kPart;
                 // a row past the end of the tile (an overwritten layout) still lies inside the sums
                 if constexpr (CROWD) {
@@ -471,18 +559,18 @@ __global__ __launch_bounds__(kColumnBlock) void spmv_column_order_kernel(idx_t m
                     if (__popcll(__ballot(r_first == lead)) >= kCrowdedLanes) {  // whole wavefront
 #pragma unroll
                         for (int i = 0; i < kSet; ++i) {
-                            const uint32_t k = static_cast<uint32_t>(i) * kColumnBlock + tid;
+                            const uint32_t k = place(i);
                             const uint32_t r = min(packed[h][i] >> band_shift, rows_per_tile - 1);
-                            add_to_crowded_row(s_acc, r, static_cast<double>(v[h][i] * xv[i]), k < cnt, lead);
+                            add_to_crowded_row(s_acc, r, static_cast<double>(v[h][i] * xv[i]), whole_set || k < cnt, lead);
                         }
                         return;
                     }
                 }
 #pragma unroll
                 for (int i = 0; i < kSet; ++i) {
-                    const uint32_t k = static_cast<uint32_t>(i) * kColumnBlock + tid;
+                    const uint32_t k = place(i);
                     const uint32_t r = min(packed[h][i] >> band_shift, rows_per_tile - 1);
-                    if (k < cnt) unsafeAtomicAdd(&s_acc[r], static_cast<double>(v[h][i] * xv[i]));
+                    if (whole_set || k < cnt) unsafeAtomicAdd(&s_acc[r], static_cast<double>(v[h][i] * xv[i]));
                 }
             };
             // A set with a successor: gathers, then the successor's loads, then the adds.  The loads are not
@@ -494,13 +582,25 @@ __global__ __launch_bounds__(kColumnBlock) void spmv_column_order_kernel(idx_t m
                 __builtin_amdgcn_sched_barrier(0);
                 ask(h ^ 1, start + kPart);
                 __builtin_amdgcn_sched_barrier(0);
-                add(h, start, xv);
+                add(h, start, xv, true);
             };
             auto last = [&](int h, idx_t start) {
                 T xv[kSet];
                 gather(h, xv);
-                add(h, start, xv);
+                add(h, start, xv, false);
             };
+            if constexpr (kQuads) {  // the entries ahead of the first multiple of kColumnQuad, a lane each
+                const idx_t a0 = (e0 + kColumnQuad - 1) / kColumnQuad * kColumnQuad;
+                const idx_t head_end = a0 < e1 ? a0 : e1;
+                if (tid < head_end - e0) {
+                    const idx_t w = entries[e0 + tid];
+                    idx_t key = band_key | (w & band_mask);
+                    key = key > base ? key : base;
+                    const uint32_t r = min(w >> band_shift, rows_per_tile - 1);
+                    unsafeAtomicAdd(&s_acc[r], static_cast<double>(vals[e0 + tid] * x[min(key - base, n - 1)]));
+                }
+                e0 = head_end;
+            }
             if (e0 < e1) {
                 ask(0, e0);
                 idx_t start = e0;
@@ -634,6 +734,12 @@ void launch_column_order_build(hipStream_t stream, const BandedShape& s, idx_t m
     launch_sort_triples(stream, nnz, bit_length(s.tiles - 1), ids, packed, vals, sorted_ids,
                         reinterpret_cast<idx_t*>(w + l.entries), w + l.vals, value_bytes, w + l.sort_ws);
     launch_coo2csr(stream, nnz, s.tiles, sorted_ids, 0, reinterpret_cast<idx_t*>(w + l.tile_ptr));
+    if (value_bytes == 4) {
+        static_assert(column_order_quads<float>() && !column_order_quads<double>(), "the kernel's reading of the copy");
+        hipLaunchKernelGGL(column_order_interleave_kernel<float>, dim3(s.tiles), dim3(kColumnQuadBlock), 0, stream, nnz,
+                           reinterpret_cast<const idx_t*>(w + l.tile_ptr), reinterpret_cast<idx_t*>(w + l.entries),
+                           reinterpret_cast<float*>(w + l.vals));
+    }
     hipLaunchKernelGGL(column_order_split_kernel, dim3(1), dim3(kBlock), 0, stream, nnz, s.tiles / s.sub, s.sub,
                        reinterpret_cast<const idx_t*>(w + l.tile_ptr), reinterpret_cast<uint32_t*>(w + l.xcd_start),
                        reinterpret_cast<uint32_t*>(w + l.next_unit));

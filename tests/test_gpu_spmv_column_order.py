@@ -147,15 +147,18 @@ def test_rows_with_an_entry_in_every_column(torch_gpu, handle, oracle, dtype, de
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
 def test_tiles_around_whole_sets_of_entries(torch_gpu, handle, oracle, dtype):
-    """The kernel takes a tile in sets of 1024 x 16 (fp32) or 1024 x 13 (fp64) entries, the loads of a set issued
-    under the arithmetic of the one before: tiles of 0, 1, and one less than, exactly and one more than one, two and
-    three sets, each several times, with integer values so that any order of the sums is exact."""
+    """The kernel takes a tile in sets of 1024 x 12 (fp32) or 1024 x 13 (fp64) entries, the loads of a set issued
+    under the arithmetic of the one before; with fp32 values the entries lie in blocks of 256 that are stored lane by
+    lane, a tile's last block with fewer lanes.  Tiles of 0 to 9 entries, around one block, and one less than,
+    exactly and one more than one, two and three sets, each several times and with their first entry at varying
+    alignments, with integer values so that any order of the sums is exact."""
     torch = torch_gpu
     rows_per_tile, groups, chunks = 16384, 32, 8
     keys = (1 << 12) // np.dtype(dtype).itemsize  # columns per group with 4 KiB bands
-    per_set = 1024 * (16 if dtype == np.float32 else 13)
+    per_set = 1024 * (12 if dtype == np.float32 else 13)
     sizes = [0, 1, per_set - 1, per_set, per_set + 1, 2 * per_set - 1, 2 * per_set, 2 * per_set + 1, 3 * per_set,
-             3 * per_set + 1, 777, per_set // 2]
+             3 * per_set + 1, 777, per_set // 2, 2, 3, 4, 5, 7, 9, 255, 256, 257, 259, 511, 513, per_set + 255,
+             per_set + 258]
     rng = np.random.default_rng(77)
     rows, cols = [], []
     for t in range(groups * chunks):
