@@ -354,7 +354,7 @@ template <typename T>
 constexpr bool column_order_quads() { return sizeof(T) == 4; }
 
 // Puts the blocks of every tile into that order, in place.  One workgroup per tile, kInterleaveBlocks blocks per
-// round: a thread reads its element of each of them, then writes.
+// round, turned round in LDS so that reads and writes both run along the arrays.
 constexpr int kInterleaveBlocks = 8;
 template <typename T>
 __global__ __launch_bounds__(kColumnQuadBlock) void column_order_interleave_kernel(idx_t nnz,
@@ -369,6 +369,8 @@ __global__ __launch_bounds__(kColumnQuadBlock) void column_order_interleave_kern
     if (a0 >= e1) return;  // whole workgroup
     const uint32_t len = e1 - a0;
     const uint32_t blocks = (len + kColumnQuadBlock - 1) / kColumnQuadBlock;
+    __shared__ idx_t s_w[kInterleaveBlocks][kColumnQuadBlock];
+    __shared__ T s_v[kInterleaveBlocks][kColumnQuadBlock];
     const uint32_t p = threadIdx.x;
     for (uint32_t b0 = 0; b0 < blocks; b0 += kInterleaveBlocks) {
         idx_t w[kInterleaveBlocks];
@@ -379,7 +381,6 @@ __global__ __launch_bounds__(kColumnQuadBlock) void column_order_interleave_kern
             w[i] = entries[a0 + at];
             v[i] = vals[a0 + at];
         }
-        __syncthreads();
 #pragma unroll
         for (int i = 0; i < kInterleaveBlocks; ++i) {
             const uint32_t first = (b0 + i) * kColumnQuadBlock;
@@ -387,8 +388,17 @@ __global__ __launch_bounds__(kColumnQuadBlock) void column_order_interleave_kern
                 const uint32_t in_block = len - first < kColumnQuadBlock ? len - first : kColumnQuadBlock;
                 const uint32_t q = in_block / kColumnQuad;
                 const uint32_t to = p < q * kColumnQuad ? (p % q) * kColumnQuad + p / q : p;
-                entries[a0 + first + to] = w[i];
-                vals[a0 + first + to] = v[i];
+                s_w[i][to] = w[i];
+                s_v[i][to] = v[i];
+            }
+        }
+        __syncthreads();  // every element of the round has been read and lies in its new place in LDS
+#pragma unroll
+        for (int i = 0; i < kInterleaveBlocks; ++i) {
+            const uint32_t first = (b0 + i) * kColumnQuadBlock;
+            if (first + p < len) {
+                entries[a0 + first + p] = s_w[i][p];
+                vals[a0 + first + p] = s_v[i][p];
             }
         }
         __syncthreads();
