@@ -333,8 +333,8 @@ __global__ __launch_bounds__(kBlock) void column_order_pack_kernel(idx_t nnz, id
 // doubles (fp32 products are widened: ds_add_f32 runs at a quarter of the rate of ds_add_f64 on this
 // chip).  A thread keeps two sets of entries in registers, kColumnSet32 or kColumnSet64 each: what fits the 128
 // registers a thread of a 1024-thread workgroup can have (fp64, one entry per load, 8 / 10 / 12 / 13: 75.0 / 73.7 /
-// 72.5 / 70.3 us on 1 M rows x 16, 14 spills registers; fp32, four entries per load, 12: 343 us on the power-law
-// matrix, 16 spills registers: 362 us).
+// 72.5 / 70.3 us on 1 M rows x 16, 14 spills registers; fp32, four entries per load, 12 / 16: 340 / 346 us on the
+// power-law matrix, 294 / 292 us on its transpose).
 constexpr int kColumnBlock = 1024;
 constexpr int kColumnSet32 = 12;
 constexpr int kColumnSet64 = 13;
@@ -344,9 +344,9 @@ constexpr int kColumnSet64 = 13;
 // 4 l .. 4 l + 3 (the last L % 4 entries stay where they are): one 128-bit load per lane brings a wavefront four
 // runs of neighbouring entries (the vector memory unit takes a load instruction in the same time whatever its
 // width: power-law matrix 384 -> 343 us, its transpose 324 -> 295 us), an element is an entry of the block exactly
-// when its place is below L, and a tile's last, partial block needs no code of its own.  With fp64 values two sets
-// of 12 do not fit the registers next to the 128-bit loads and sets of 8 lose more than the loads gain (75 against
-// 69 us on 1 M rows x 16): that copy keeps its entries in column order, one per load.
+// when its place is below L, and a tile's last, partial block needs no code of its own.  With fp64 values the same
+// layout with sets of 12 measured slower than one entry per load with sets of 13 (73.8 against 68.5 us on 1 M rows
+// x 16; sets of 8: 75 us): that copy keeps its entries in column order, one per load.
 constexpr int kColumnQuad = 4;
 constexpr uint32_t kColumnQuadBlock = kColumnQuad * kWave;
 static_assert(kColumnSet32 % kColumnQuad == 0, "whole blocks per set");
@@ -531,9 +531,10 @@ __global__ __launch_bounds__(kColumnBlock) void spmv_column_order_kernel(idx_t m
                     const uint32_t last_quad = (cnt - 1) / kColumnQuad * kColumnQuad;
 #pragma unroll
                     for (int j = 0; j < kSet / kColumnQuad; ++j) {
-                        const idx_t at = start + min(place(j * kColumnQuad), last_quad);
-                        const quad_t q = __builtin_nontemporal_load(reinterpret_cast<const quad_t*>(entries + at));
-                        const quad_t f = __builtin_nontemporal_load(reinterpret_cast<const quad_t*>(vals + at));
+                        // (array + start) + place: a uniform base and a small offset per lane, one register
+                        const uint32_t at = min(place(j * kColumnQuad), last_quad);
+                        const quad_t q = __builtin_nontemporal_load(reinterpret_cast<const quad_t*>((entries + start) + at));
+                        const quad_t f = __builtin_nontemporal_load(reinterpret_cast<const quad_t*>((vals + start) + at));
                         packed[h][j * 4 + 0] = q.x;
                         packed[h][j * 4 + 1] = q.y;
                         packed[h][j * 4 + 2] = q.z;
