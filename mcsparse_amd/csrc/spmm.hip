@@ -679,7 +679,9 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(LR <= 16
             for (int r = 0; r < R; ++r) {
                 const bool mine = (ent >> r) & 1u;
                 const uint64_t in = (__ballot(mine) >> group_first) & group_bits;
-                v[r] = mine ? val[min(i[r] + static_cast<idx_t>(__popcll(in & below)), last_value)] : T(0);
+                // loaded whether or not it is wanted (the place is clamped anyway): a select costs less than a branch
+                const T loaded = val[min(i[r] + static_cast<idx_t>(__popcll(in & below)), last_value)];
+                v[r] = mine ? loaded : T(0);
                 i[r] += __popcll(in);
                 take[r] = __brev(static_cast<uint32_t>(in));
             }
