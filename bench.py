@@ -68,8 +68,8 @@ MEASURED_TRAFFIC = {
     ("c3t", 0): (_traffic(229180.3 + 14342.5 + 2 * 7207.2 + 21132.3 + 489308.2 + 421987.3,
                           28832.0 + 56.0 + 2 * 14325.6 + 223.8 + 692310.6 + 16384.0),
                  "profiles/spmv_transposed_buckets_f32_c3_powerlaw.txt"),
-    ("c4-64", 0): (_traffic(613893.3, 524288.0), "profiles/spmm_group_f32_c4_stencil128.txt"),
-    ("c4-256", 0): (_traffic(3673719.8, 2097152.0), "profiles/spmm_group_f32_c4_stencil128.txt"),
+    ("c4-64", 0): (_traffic(492232.8, 524288.0), "profiles/spmm_group_f32_c4_stencil128.txt"),
+    ("c4-256", 0): (_traffic(3630735.8, 2097152.0), "profiles/spmm_group_f32_c4_stencil128.txt"),
     # group kernel (writes the column-major C itself) + the transpose of B
     ("c4-64-col", 0): (_traffic(589819.9 + 262180.0, 537321.5 + 524288.0),
                            "profiles/spmm_colmajor_f32_c4_stencil128_n64.txt"),
