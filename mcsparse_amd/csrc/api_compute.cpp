@@ -856,6 +856,7 @@ mcsparseStatus_t mcsparseSpMV_preprocess(mcsparseHandle_t handle, mcsparseOperat
         hipStreamSynchronize(handle->stream) != hipSuccess)
         return to_public_status(MCSP_STATUS_INTERNAL_ERROR);
     b.grid = mcsp::banded_grid(xcd_start);
+    for (int i = 0; i < 9; ++i) b.shape.xcd_start[i] = xcd_start[i];
     b.useful = true;
     b.valid = true;
     return MCSPARSE_STATUS_SUCCESS;

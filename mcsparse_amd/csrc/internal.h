@@ -111,6 +111,9 @@ struct BandedShape {
     // by_column: some row holds more than half of what a row chunk holds on average, so that the wavefronts of its
     // tile would queue on its sum in LDS; the kernel variant that sums such a row's products in registers is used
     bool crowded_rows = false;
+    // by_column: where each XCD's stretch of units begins (what the build left at BandedLayout::xcd_start, read back
+    // once): handed to the kernel with its arguments, which saves its workgroups a dependent load from memory
+    uint32_t xcd_start[9] = {0, 0, 0, 0, 0, 0, 0, 0, 0};
 };
 struct SpmvBanded {
     bool valid = false;

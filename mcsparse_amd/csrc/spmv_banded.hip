@@ -453,6 +453,11 @@ __device__ __forceinline__ void add_to_crowded_row(double* s_acc, uint32_t r, do
 }
 constexpr int kCrowdedLanes = 40;  // lanes of a wavefront on one row from which they are summed in registers first
 
+// Where the stretch of units of each XCD begins (and the last one ends), by value among the kernel's arguments.
+struct XcdStarts {
+    uint32_t first[kXcds + 1];
+};
+
 // CROWD: the matrix has a row that holds a large share of a tile (BandedShape::crowded_rows): where most lanes of a
 // wavefront meet on one row in the first entries of a slab, the slab's products for that row are summed in registers
 // (a matrix with dense rows: 0.78 -> 0.44 ms with one such row among 4 M, 0.99 -> 0.67 ms with four).  The test and
@@ -461,13 +466,14 @@ template <typename T, bool CROWD>
 __global__ __launch_bounds__(kColumnBlock) void spmv_column_order_kernel(idx_t m, idx_t n, idx_t nnz, idx_t base,
                                                                         uint32_t band_shift, uint32_t rows_per_tile,
                                                                         uint32_t chunks, uint32_t units, uint32_t sub,
-                                                                        const uint32_t* __restrict__ xcd_start,
+                                                                        const XcdStarts stretches,
                                                                         uint32_t* __restrict__ next_unit,
                                                                         const idx_t* __restrict__ tile_ptr,
                                                                         const idx_t* __restrict__ entries,
                                                                         const T* __restrict__ vals,
                                                                         const T* __restrict__ x,
                                                                         T* __restrict__ partials) {
+    const uint32_t* xcd_start = stretches.first;
     extern __shared__ __align__(16) unsigned char s_raw[];
     __shared__ uint32_t s_unit;
     double* s_acc = reinterpret_cast<double*>(s_raw);
@@ -791,11 +797,13 @@ void launch_spmv_banded(hipStream_t stream, const BandedShape& s, uint32_t grid,
     T* partials = reinterpret_cast<T*>(w + l.partials);
     if (s.by_column) {
         const int lds = static_cast<int>(s.rows_per_tile * sizeof(double));
+        XcdStarts stretches;
+        for (uint32_t i = 0; i <= kXcds; ++i) stretches.first[i] = s.xcd_start[i];
         auto* kernel = s.crowded_rows ? spmv_column_order_kernel<T, true> : spmv_column_order_kernel<T, false>;
         (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, lds);
         hipLaunchKernelGGL(kernel, dim3(kColumnGroupsPerXcd * kXcds), dim3(kColumnBlock), lds, stream, a.m, a.n, a.nnz,
                            a.base, s.band_shift, s.rows_per_tile, s.chunks, s.tiles / s.sub, s.sub,
-                           reinterpret_cast<const uint32_t*>(w + l.xcd_start), reinterpret_cast<uint32_t*>(w + l.next_unit),
+                           stretches, reinterpret_cast<uint32_t*>(w + l.next_unit),
                            reinterpret_cast<const idx_t*>(w + l.tile_ptr), reinterpret_cast<const idx_t*>(w + l.entries),
                            reinterpret_cast<const T*>(w + l.vals), static_cast<const T*>(a.x), partials);
     } else if (grid != 0) {
