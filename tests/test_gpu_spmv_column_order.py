@@ -192,6 +192,37 @@ def test_tiles_around_whole_sets_of_entries(torch_gpu, handle, oracle, dtype):
         assert np.array_equal(d_y.cpu().numpy().astype(np.float64), want)
 
 
+@pytest.mark.parametrize("alg", [api.SPMV_CSR_ALG1, api.SPMV_CSR_ALG2])
+@pytest.mark.parametrize("m,offset", [(70000, 0), (70000, 1), (70001, 0), (70001, 1)])
+def test_fp64_reduce_with_any_alignment_of_y(torch_gpu, handle, oracle, alg, m, offset):
+    """The reduce over the planes takes two rows per thread with 16-byte accesses when the number of rows is even and
+    y is 16-byte aligned, and one row per thread otherwise: both kernels, both copies, same result."""
+    torch = torch_gpu
+    a = wl.random_ragged(m, 50000, 6, dtype=np.float64, seed=12)
+    rng = np.random.default_rng(12)
+    x = rng.uniform(-1, 1, a.n)
+    y = rng.uniform(-1, 1, a.m)
+    d_ptr, d_col, d_val, d_x = (dev(torch, v) for v in (a.ptr, a.col, a.val, x))
+    backing = torch.zeros(m + 2, dtype=torch.float64, device="cuda")
+    d_y = backing[offset:offset + m]  # offset 1: 8 bytes past a 16-byte boundary
+    assert (d_y.data_ptr() % 16 == 0) == (offset == 0)
+    mat = api.SpMat(a.m, a.n, a.nnz, d_ptr, d_col, d_val)
+    mat.set_band_bytes(1 << 14)
+    vx, vy = api.DnVec(d_x), api.DnVec(d_y)
+    ct = api.maca_type(np.float64)
+    st, size = api.spmv_preprocess_buffer_size(handle, api.OP_N, -0.5, mat, vx, 2.0, vy, ct, alg=alg)
+    assert st == api.STATUS_SUCCESS
+    buf = torch.empty(size, dtype=torch.uint8, device="cuda")
+    assert api.spmv_preprocess(handle, api.OP_N, -0.5, mat, vx, 2.0, vy, ct, buf, alg=alg) == api.STATUS_SUCCESS
+    assert mat.spmv_preprocess_state()[0] == (2 if alg == api.SPMV_CSR_ALG2 else 3)
+    y_ref, bound = oracle.spmv(False, a.m, a.n, a.base, a.ptr, a.col, a.val, -0.5, 2.0, x, y)
+    d_y.copy_(torch.from_numpy(y))
+    assert api.spmv(handle, api.OP_N, -0.5, mat, vx, 2.0, vy, ct, buf, alg=alg) == api.STATUS_SUCCESS
+    torch.cuda.synchronize()
+    assert_within(d_y.cpu().numpy(), y_ref, bound, np.float64, what="reduce, m %d, y offset %d" % (m, offset))
+    assert backing[offset + m:].abs().sum().item() == 0 and (offset == 0 or backing[0].item() == 0)
+
+
 def test_alg2_does_not_use_the_copy(torch_gpu, handle, oracle):
     """MCSPARSE_SPMV_CSR_ALG2 promises the same bits on every run: the call runs the row kernels."""
     a = wl.uniform_rows(m=20000, n=300000, per_row=8, dtype=np.float64, config_id=91)
