@@ -460,7 +460,7 @@ struct XcdStarts {
 
 // CROWD: the matrix has a row that holds a large share of a tile (BandedShape::crowded_rows): where most lanes of a
 // wavefront meet on one row in the first entries of a slab, the slab's products for that row are summed in registers
-// (a matrix with dense rows: 0.78 -> 0.44 ms with one such row among 4 M, 0.99 -> 0.67 ms with four).  The test and
+// (a matrix with dense rows: 0.78 -> 0.36 ms with one such row among 4 M, 0.99 -> 0.55 ms with four).  The test and
 // the second copy of the loop cost the kernel 2 to 10 % on matrices without such rows, which is why it is a variant.
 template <typename T, bool CROWD>
 __global__ __launch_bounds__(kColumnBlock) void spmv_column_order_kernel(idx_t m, idx_t n, idx_t nnz, idx_t base,
