@@ -353,8 +353,9 @@ static_assert(kColumnSet32 % kColumnQuad == 0, "whole blocks per set");
 template <typename T>
 constexpr bool column_order_quads() { return sizeof(T) == 4; }
 
-// Puts the blocks of every tile into that order, in place.  One workgroup per tile, kInterleaveBlocks blocks per
-// round, turned round in LDS so that reads and writes both run along the arrays.
+// Puts the blocks of every tile into that order, in place.  kInterleaveParts workgroups per tile take turns at
+// rounds of kInterleaveBlocks blocks, turned round in LDS so that reads and writes both run along the arrays.
+constexpr uint32_t kInterleaveParts = 8;
 constexpr int kInterleaveBlocks = 8;
 template <typename T>
 __global__ __launch_bounds__(kColumnQuadBlock) void column_order_interleave_kernel(idx_t nnz,
@@ -372,7 +373,7 @@ __global__ __launch_bounds__(kColumnQuadBlock) void column_order_interleave_kern
     __shared__ idx_t s_w[kInterleaveBlocks][kColumnQuadBlock];
     __shared__ T s_v[kInterleaveBlocks][kColumnQuadBlock];
     const uint32_t p = threadIdx.x;
-    for (uint32_t b0 = 0; b0 < blocks; b0 += kInterleaveBlocks) {
+    for (uint32_t b0 = blockIdx.y * kInterleaveBlocks; b0 < blocks; b0 += gridDim.y * kInterleaveBlocks) {  // whole workgroup
         idx_t w[kInterleaveBlocks];
         T v[kInterleaveBlocks];
 #pragma unroll
@@ -753,7 +754,7 @@ void launch_column_order_build(hipStream_t stream, const BandedShape& s, idx_t m
     launch_coo2csr(stream, nnz, s.tiles, sorted_ids, 0, reinterpret_cast<idx_t*>(w + l.tile_ptr));
     if (value_bytes == 4) {
         static_assert(column_order_quads<float>() && !column_order_quads<double>(), "the kernel's reading of the copy");
-        hipLaunchKernelGGL(column_order_interleave_kernel<float>, dim3(s.tiles), dim3(kColumnQuadBlock), 0, stream, nnz,
+        hipLaunchKernelGGL(column_order_interleave_kernel<float>, dim3(s.tiles, kInterleaveParts), dim3(kColumnQuadBlock), 0, stream, nnz,
                            reinterpret_cast<const idx_t*>(w + l.tile_ptr), reinterpret_cast<idx_t*>(w + l.entries),
                            reinterpret_cast<float*>(w + l.vals));
     }
