@@ -798,6 +798,31 @@ mcsparseStatus_t mcsparseSpMV_preprocess(mcsparseHandle_t handle, mcsparseOperat
                                             v.n * static_cast<int64_t>(vb), externalBuffer, true);
         if (ps != MCSP_STATUS_SUCCESS) return to_public_status(ps);
     }
+    // Where a few lines of x take most of the gathers (long rows under a transposing direction, popular columns),
+    // one band group over all of x does better than groups that fit an XCD's L2: the hot lines stay in L2 anyway
+    // and the planes of partial sums go.  Measured on the matrix, unless the caller has set the width.
+    if (shape.by_column && matA->banded.band_bytes == 0 && shape.bands > 1) {
+        const idx_t gathered = static_cast<idx_t>(v.transpose ? v.m : v.n);
+        const size_t region_at = banded_region_offset(matA, opA, vb);
+        const size_t room = align_up(mcsp::banded_layout(shape, m, nnz, vb).total);
+        if (mcsp::line_gathers_workspace_bytes(gathered, vb) <= room) {
+            char* ws = static_cast<char*>(externalBuffer) + region_at;
+            mcsp::launch_line_gathers(handle->stream, v.transpose, gathered, nnz, base, v.ptr, v.ind, vb, ws);
+            unsigned long long bins[2 * mcsp::kLineGatherBins];
+            if (hipMemcpyAsync(bins, ws, sizeof(bins), hipMemcpyDeviceToHost, handle->stream) != hipSuccess ||
+                hipStreamSynchronize(handle->stream) != hipSuccess)
+                return to_public_status(MCSP_STATUS_INTERNAL_ERROR);
+            if (mcsp::gathers_favour_wide_groups(bins)) {
+                size_t all_of_x = mcsp::kBandedBandBytes;
+                while (all_of_x < (static_cast<size_t>(gathered) + base) * vb) all_of_x *= 2;
+                BandedShape wide;
+                if (mcsp::column_order_shape(m, gathered, nnz, base, vb, all_of_x, &wide) &&
+                    wide.rows_per_tile == shape.rows_per_tile &&
+                    align_up(mcsp::banded_layout(wide, m, nnz, vb).total) <= room)
+                    shape = wide;
+            }
+        }
+    }
     SpmvBanded& b = matA->banded;
     b.buffer = externalBuffer;
     b.rows = matA->rows;

@@ -280,6 +280,16 @@ constexpr uint32_t kColumnOrderRows = 16384;
 constexpr uint32_t kColumnOrderMinRows = 2048;
 bool column_order_shape(idx_t m, idx_t n, idx_t nnz, idx_t base, size_t value_bytes, size_t band_bytes,
                         BandedShape* out);
+// How the gathers of an SpMV are spread over the 128-byte lines of x: launch_line_gathers fills, at the head of
+// `workspace` (line_gathers_workspace_bytes), kLineGatherBins pairs (lines, gathers) binned by the highest bit of a
+// line's count: of_rows from the row lengths (the gathered element is the row: a transposing direction), else from
+// a sample of the indices.  gathers_favour_wide_groups reads the pairs once they are on the host.
+constexpr uint32_t kLineGatherBins = 32;
+constexpr double kHotLines = 16384;
+size_t line_gathers_workspace_bytes(idx_t gathered, size_t value_bytes);
+void launch_line_gathers(hipStream_t stream, bool of_rows, idx_t gathered, idx_t nnz, idx_t base, const idx_t* ptr,
+                         const idx_t* ind, size_t value_bytes, void* workspace);
+bool gathers_favour_wide_groups(const unsigned long long* bins);
 // r_keys / c_keys: row + base and column + base of every nonzero of the matrix to copy, in an order
 // sorted by the 128-byte line of x the column lies in (any order inside a line); vals in the same
 // order.  Neither is written.

@@ -674,6 +674,102 @@ bool banded_shape(idx_t m, idx_t n, idx_t nnz, idx_t base, size_t value_bytes, s
     return true;
 }
 
+// ------------------------------------------------------------------------------------------
+// how the gathers are spread over the lines of x
+// ------------------------------------------------------------------------------------------
+namespace {
+
+__global__ __launch_bounds__(kBlock) void fill_u32_kernel(uint64_t n, uint32_t value, uint32_t* p) {
+    const uint64_t i = static_cast<uint64_t>(blockIdx.x) * kBlock + threadIdx.x;
+    if (i < n) p[i] = value;
+}
+
+// counts[line] += gathers of that line.  Rows: the gathered element is the row itself (a transposing direction:
+// element r is read once per nonzero of row r).  Indices: every stride-th index names the gathered element.
+__global__ __launch_bounds__(kBlock) void line_gathers_of_rows_kernel(idx_t rows, const idx_t* __restrict__ ptr,
+                                                                      uint32_t line_shift, uint32_t lines,
+                                                                      uint32_t* counts) {
+    const uint64_t r = static_cast<uint64_t>(blockIdx.x) * kBlock + threadIdx.x;
+    if (r >= rows) return;
+    const idx_t len = ptr[r + 1] - ptr[r];
+    if (len != 0) atomicAdd(&counts[min(static_cast<uint32_t>(r >> line_shift), lines - 1)], len);
+}
+__global__ __launch_bounds__(kBlock) void line_gathers_of_indices_kernel(idx_t nnz, uint32_t stride, idx_t base,
+                                                                         const idx_t* __restrict__ ind,
+                                                                         uint32_t line_shift, uint32_t lines,
+                                                                         uint32_t* counts) {
+    const uint64_t k = (static_cast<uint64_t>(blockIdx.x) * kBlock + threadIdx.x) * stride;
+    if (k >= nnz) return;
+    const idx_t key = ind[k];
+    const idx_t c = key > base ? key - base : 0;
+    atomicAdd(&counts[min(static_cast<uint32_t>(c >> line_shift), lines - 1)], 1u);
+}
+// bins[2 b] = lines whose count has b as its highest bit, bins[2 b + 1] = their gathers
+__global__ __launch_bounds__(kBlock) void line_gather_bins_kernel(uint32_t lines, const uint32_t* __restrict__ counts,
+                                                                  unsigned long long* bins) {
+    __shared__ unsigned long long s_bins[64];
+    if (threadIdx.x < 64) s_bins[threadIdx.x] = 0;
+    __syncthreads();
+    const uint64_t i = static_cast<uint64_t>(blockIdx.x) * kBlock + threadIdx.x;
+    const uint32_t c = i < lines ? counts[i] : 0;
+    if (c != 0) {
+        const uint32_t b = 31 - __clz(static_cast<int>(c));
+        atomicAdd(&s_bins[2 * b], 1ull);
+        atomicAdd(&s_bins[2 * b + 1], static_cast<unsigned long long>(c));
+    }
+    __syncthreads();
+    if (threadIdx.x < 64 && s_bins[threadIdx.x] != 0) atomicAdd(&bins[threadIdx.x], s_bins[threadIdx.x]);
+}
+
+}  // namespace
+
+size_t line_gathers_workspace_bytes(idx_t gathered, size_t value_bytes) {
+    const uint32_t line_shift = value_bytes == 8 ? 4 : 5;
+    const uint64_t lines = (static_cast<uint64_t>(gathered) >> line_shift) + 1;
+    return 2 * kLineGatherBins * sizeof(unsigned long long) + lines * sizeof(uint32_t);
+}
+
+void launch_line_gathers(hipStream_t stream, bool of_rows, idx_t gathered, idx_t nnz, idx_t base, const idx_t* ptr,
+                         const idx_t* ind, size_t value_bytes, void* workspace) {
+    const uint32_t line_shift = value_bytes == 8 ? 4 : 5;
+    const uint32_t lines = static_cast<uint32_t>((static_cast<uint64_t>(gathered) >> line_shift) + 1);
+    unsigned long long* bins = static_cast<unsigned long long*>(workspace);
+    uint32_t* counts = reinterpret_cast<uint32_t*>(bins + 2 * kLineGatherBins);
+    const uint64_t words = 4ull * kLineGatherBins + lines;  // the pairs as 32-bit words, then the counts
+    hipLaunchKernelGGL(fill_u32_kernel, dim3(static_cast<uint32_t>((words + kBlock - 1) / kBlock)), dim3(kBlock), 0, stream,
+                       words, 0u, static_cast<uint32_t*>(workspace));
+    if (of_rows) {
+        hipLaunchKernelGGL(line_gathers_of_rows_kernel, dim3((gathered + kBlock - 1) / kBlock), dim3(kBlock), 0, stream,
+                           gathered, ptr, line_shift, lines, counts);
+    } else {
+        const uint32_t stride = static_cast<uint32_t>((static_cast<uint64_t>(nnz) >> 22) + 1);  // about 4 M samples at most
+        const uint64_t samples = (static_cast<uint64_t>(nnz) + stride - 1) / stride;
+        hipLaunchKernelGGL(line_gathers_of_indices_kernel, dim3(static_cast<uint32_t>((samples + kBlock - 1) / kBlock)),
+                           dim3(kBlock), 0, stream, nnz, stride, base, ind, line_shift, lines, counts);
+    }
+    hipLaunchKernelGGL(line_gather_bins_kernel, dim3((lines + kBlock - 1) / kBlock), dim3(kBlock), 0, stream, lines, counts,
+                       bins);
+}
+
+// bins: what line_gather_bins_kernel left (read back).  True when the kHotLines most gathered lines of x (half of what
+// an XCD's L2 holds) take more than half of the gathers: the hot lines then stay in L2 whatever the width of a band
+// group, and one group over all of x saves the planes of partial sums (power-law matrix, op T: 78 % of the gathers
+// in the 16384 hottest lines, 294 -> 253 us; uniform columns: 12 %, 340 -> 425 us with groups of 8 MiB).
+bool gathers_favour_wide_groups(const unsigned long long* bins) {
+    unsigned long long all = 0;
+    for (uint32_t b = 0; b < 32; ++b) all += bins[2 * b + 1];
+    if (all == 0) return false;
+    double lines = 0, gathers = 0;
+    for (int b = 31; b >= 0 && lines < kHotLines; --b) {
+        const double n = static_cast<double>(bins[2 * b]);
+        if (n == 0) continue;
+        const double take = n <= kHotLines - lines ? 1.0 : (kHotLines - lines) / n;
+        lines += n * take;
+        gathers += static_cast<double>(bins[2 * b + 1]) * take;
+    }
+    return 2.0 * gathers > static_cast<double>(all);
+}
+
 bool column_order_shape(idx_t m, idx_t n, idx_t nnz, idx_t base, size_t value_bytes, size_t band_bytes,
                         BandedShape* out) {
     if (m == 0 || n == 0 || nnz == 0 || (value_bytes != 4 && value_bytes != 8)) return false;

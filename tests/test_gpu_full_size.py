@@ -13,6 +13,7 @@ from gpu_util import assert_within, dev, run_spmv
 from test_gpu_convert import gpu_csr2coo, gpu_csr2csc
 from test_gpu_spmm import run_spmm
 from test_gpu_spmv_banded import run_banded
+from test_gpu_spmv_column_order import run as run_column_order
 
 pytestmark = pytest.mark.gpu
 
@@ -50,6 +51,11 @@ def test_config3_power_law_full_size(torch_gpu, handle, oracle, power_law_full):
     assert st == 0
     yt_ref, bound_t = oracle.spmv(True, a.m, a.n, 0, a.ptr, a.col, a.val, 1.0, 0.0, xt, None)
     assert_within(yt, yt_ref, bound_t, np.float32, what="C3 op T")
+    # op T from the copy in column order: x is gathered by row, and the long rows take most of the gathers (the row
+    # lengths tell the preprocess call), so one band group spans all of x
+    state, bands, rows, _, _ = run_column_order(torch_gpu, handle, oracle, a, 1.0, 0.0, op=api.OP_T,
+                                                what="C3 op T, column order")
+    assert (state, bands, rows) == (3, 1, 16384)
 
 
 def test_config5_conversions_full_size(torch_gpu, handle, oracle, power_law_full):
@@ -77,6 +83,12 @@ def test_config5_conversions_full_size(torch_gpu, handle, oracle, power_law_full
     state, bands, rows = run_banded(torch_gpu, handle, oracle, csc_as_csr, 1.0, 0.0, as_csc=True,
                                     what="C5 A^T x from CSC, banded", reference=(xt, yt_ref, bound_t))
     assert (state, bands) == (2, 8)
+    # and from the copy in column order: the long rows of A make a few lines of x take most of the gathers (78 % in
+    # the 16384 hottest lines), which a sample of the indices shows the preprocess call: one band group over all of x
+    state, bands, rows = run_banded(torch_gpu, handle, oracle, csc_as_csr, 1.0, 0.0, as_csc=True, calls=2,
+                                    what="C5 A^T x from CSC, column order", reference=(xt, yt_ref, bound_t),
+                                    alg=api.SPMV_CSR_ALG1, expect_state=3)
+    assert (bands, rows) == (1, 16384)
 
 
 def test_config2_full_size_banded(torch_gpu, handle, oracle):
