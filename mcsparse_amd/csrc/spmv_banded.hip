@@ -690,9 +690,11 @@ __global__ __launch_bounds__(kBlock) void line_gathers_of_rows_kernel(idx_t rows
                                                                       uint32_t line_shift, uint32_t lines,
                                                                       uint32_t* counts) {
     const uint64_t r = static_cast<uint64_t>(blockIdx.x) * kBlock + threadIdx.x;
-    if (r >= rows) return;
-    const idx_t len = ptr[r + 1] - ptr[r];
-    if (len != 0) atomicAdd(&counts[min(static_cast<uint32_t>(r >> line_shift), lines - 1)], len);
+    uint32_t len = r < rows ? ptr[r + 1] - ptr[r] : 0;
+    // the rows of a line are neighbouring lanes (16 or 32 of them, aligned): summed first, one add per line
+    for (uint32_t d = 1; d < (1u << line_shift); d <<= 1) len += __shfl_xor(len, static_cast<int>(d));
+    if ((r & ((1u << line_shift) - 1u)) == 0 && r < rows && len != 0)
+        atomicAdd(&counts[min(static_cast<uint32_t>(r >> line_shift), lines - 1)], len);
 }
 __global__ __launch_bounds__(kBlock) void line_gathers_of_indices_kernel(idx_t nnz, uint32_t stride, idx_t base,
                                                                          const idx_t* __restrict__ ind,
@@ -742,7 +744,7 @@ void launch_line_gathers(hipStream_t stream, bool of_rows, idx_t gathered, idx_t
         hipLaunchKernelGGL(line_gathers_of_rows_kernel, dim3((gathered + kBlock - 1) / kBlock), dim3(kBlock), 0, stream,
                            gathered, ptr, line_shift, lines, counts);
     } else {
-        const uint32_t stride = static_cast<uint32_t>((static_cast<uint64_t>(nnz) >> 22) + 1);  // about 4 M samples at most
+        const uint32_t stride = static_cast<uint32_t>((static_cast<uint64_t>(nnz) >> 20) + 1);  // about 1 M samples at most
         const uint64_t samples = (static_cast<uint64_t>(nnz) + stride - 1) / stride;
         hipLaunchKernelGGL(line_gathers_of_indices_kernel, dim3(static_cast<uint32_t>((samples + kBlock - 1) / kBlock)),
                            dim3(kBlock), 0, stream, nnz, stride, base, ind, line_shift, lines, counts);
