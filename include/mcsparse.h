@@ -505,7 +505,8 @@ mcsparseStatus_t mcsparseSpMV_preprocess(mcsparseHandle_t handle, mcsparseOperat
 mcsparseStatus_t mcsparseSpMatGetSpMVPreprocess(mcsparseSpMatDescr_t spMatDescr, int* state, int* bands,
                                                 int* rows_per_tile);
 
-/* Width, in bytes of x, of the column bands mcsparseSpMV_preprocess cuts (0 = the default, 2 MiB;
+/* Width, in bytes of x, of the column bands mcsparseSpMV_preprocess cuts (0 = the default: 2 MiB, or, for
+ * the copy in column order, all of x where the call finds that a few lines of x take most of the gathers;
  * rounded down to a power of two).  Drops a banded copy already built.  For tests and benchmarks. */
 mcsparseStatus_t mcsparseSpMatSetSpMVBandBytes(mcsparseSpMatDescr_t spMatDescr, size_t band_bytes);
 
