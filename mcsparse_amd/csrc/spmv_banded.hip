@@ -420,6 +420,7 @@ __global__ __launch_bounds__(kBlock) void column_order_split_kernel(idx_t nnz, u
     __shared__ unsigned long long s_worst[2];
     const uint32_t tid = threadIdx.x;
     if (tid < kXcds) next_unit[tid] = kColumnGroupsPerXcd;  // the work counters of the SpMV kernel: see there
+    if (tid == kXcds) next_unit[kXcds] = 0;                 // and its count of workgroups that are through
     if (tid <= kXcds) {
         const uint64_t target = static_cast<uint64_t>(nnz) * tid / kXcds;
         uint32_t lo = 0, hi = units;  // first unit whose offset is >= target
@@ -463,7 +464,10 @@ struct XcdStarts {
 // wavefront meet on one row in the first entries of a slab, the slab's products for that row are summed in registers
 // (a matrix with dense rows: 0.78 -> 0.36 ms with one such row among 4 M, 0.99 -> 0.55 ms with four).  The test and
 // the second copy of the loop cost the kernel 2 to 10 % on matrices without such rows, which is why it is a variant.
-template <typename T, bool CROWD>
+// DIRECT: one band group spans all of x, so a unit's sums are the rows of y themselves: the kernel writes
+// y = alpha * sums + beta * y and no reduce kernel follows (11.7 us of 254 on the power-law matrix under op T).
+// The work counters are then put back by the workgroup that is through last: next_unit[kXcds] counts them.
+template <typename T, bool CROWD, bool DIRECT>
 __global__ __launch_bounds__(kColumnBlock) void spmv_column_order_kernel(idx_t m, idx_t n, idx_t nnz, idx_t base,
                                                                         uint32_t band_shift, uint32_t rows_per_tile,
                                                                         uint32_t chunks, uint32_t units, uint32_t sub,
@@ -473,7 +477,8 @@ __global__ __launch_bounds__(kColumnBlock) void spmv_column_order_kernel(idx_t m
                                                                         const idx_t* __restrict__ entries,
                                                                         const T* __restrict__ vals,
                                                                         const T* __restrict__ x,
-                                                                        T* __restrict__ partials) {
+                                                                        T* __restrict__ partials, T* __restrict__ y,
+                                                                        T alpha, T beta) {
     const uint32_t* xcd_start = stretches.first;
     extern __shared__ __align__(16) unsigned char s_raw[];
     __shared__ uint32_t s_unit;
@@ -637,12 +642,30 @@ __global__ __launch_bounds__(kColumnBlock) void spmv_column_order_kernel(idx_t m
             }
         }
         __syncthreads();
-        T* out = partials + static_cast<uint64_t>(group) * m + row0;
-        for (uint32_t r = tid; r < rows_per_tile; r += kColumnBlock) {
-            if (r < tile_rows) out[r] = static_cast<T>(s_acc[r]);
-            s_acc[r] = 0.0;
+        if constexpr (DIRECT) {
+            T* out = y + row0;
+            for (uint32_t r = tid; r < rows_per_tile; r += kColumnBlock) {
+                if (r < tile_rows) {
+                    const T sum = alpha * static_cast<T>(s_acc[r]);
+                    out[r] = beta == T(0) ? sum : sum + beta * out[r];
+                }
+                s_acc[r] = 0.0;
+            }
+        } else {
+            T* out = partials + static_cast<uint64_t>(group) * m + row0;
+            for (uint32_t r = tid; r < rows_per_tile; r += kColumnBlock) {
+                if (r < tile_rows) out[r] = static_cast<T>(s_acc[r]);
+                s_acc[r] = 0.0;
+            }
         }
         __syncthreads();
+    }
+    if constexpr (DIRECT) {
+        // every workgroup comes here once, after its last look at a work counter
+        if (tid == 0 && atomicAdd(&next_unit[kXcds], 1u) == gridDim.x - 1) {
+            for (uint32_t i = 0; i < kXcds; ++i) atomicExch(&next_unit[i], static_cast<uint32_t>(kColumnGroupsPerXcd));
+            atomicExch(&next_unit[kXcds], 0u);
+        }
     }
 }
 
@@ -812,7 +835,7 @@ BandedLayout banded_layout(const BandedShape& s, idx_t m, idx_t nnz, size_t valu
     size_t off = 0;
     l.tile_ptr = off; off += align_up((static_cast<size_t>(s.tiles) + 1) * sizeof(idx_t));
     l.xcd_start = off; off += align_up((kXcds + 1) * sizeof(uint32_t));
-    l.next_unit = off; off += align_up(kXcds * sizeof(uint32_t));
+    l.next_unit = off; off += align_up((kXcds + 1) * sizeof(uint32_t));  // the counters and the count of finished workgroups
     l.entries = off; off += idx_bytes;
     l.vals = off; off += align_up(static_cast<size_t>(nnz) * value_bytes);
     l.partials = off; off += align_up(static_cast<size_t>(s.bands) * m * value_bytes);
@@ -898,13 +921,20 @@ void launch_spmv_banded(hipStream_t stream, const BandedShape& s, uint32_t grid,
         const int lds = static_cast<int>(s.rows_per_tile * sizeof(double));
         XcdStarts stretches;
         for (uint32_t i = 0; i <= kXcds; ++i) stretches.first[i] = s.xcd_start[i];
-        auto* kernel = s.crowded_rows ? spmv_column_order_kernel<T, true> : spmv_column_order_kernel<T, false>;
+        // one band group: the kernel writes y itself, and no reduce follows
+        const bool direct = s.bands == 1;
+        auto* kernel = direct ? (s.crowded_rows ? spmv_column_order_kernel<T, true, true>
+                                                : spmv_column_order_kernel<T, false, true>)
+                              : (s.crowded_rows ? spmv_column_order_kernel<T, true, false>
+                                                : spmv_column_order_kernel<T, false, false>);
         (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, lds);
         hipLaunchKernelGGL(kernel, dim3(kColumnGroupsPerXcd * kXcds), dim3(kColumnBlock), lds, stream, a.m, a.n, a.nnz,
                            a.base, s.band_shift, s.rows_per_tile, s.chunks, s.tiles / s.sub, s.sub,
                            stretches, reinterpret_cast<uint32_t*>(w + l.next_unit),
                            reinterpret_cast<const idx_t*>(w + l.tile_ptr), reinterpret_cast<const idx_t*>(w + l.entries),
-                           reinterpret_cast<const T*>(w + l.vals), static_cast<const T*>(a.x), partials);
+                           reinterpret_cast<const T*>(w + l.vals), static_cast<const T*>(a.x), partials,
+                           static_cast<T*>(a.y), alpha, beta);
+        if (direct) return;
     } else if (grid != 0) {
         hipLaunchKernelGGL((spmv_banded_kernel<T>), dim3(grid), dim3(kBlock), 0, stream, a.m, a.n, a.nnz, a.base,
                            s.band_shift, s.rows_per_tile, s.chunks, s.tiles,

@@ -118,17 +118,21 @@ def test_calls_replay_in_a_hip_graph(torch_gpu, oracle):
     handle.destroy()
 
 
-@pytest.mark.parametrize("alg,state", [(api.SPMV_ALG_DEFAULT, 3), (api.SPMV_CSR_ALG2, 2)])
-def test_preprocessed_spmv_replays_in_a_hip_graph(torch_gpu, oracle, alg, state):
-    """mcsparseSpMV on a copy built by mcsparseSpMV_preprocess (before the capture: it blocks) is two kernels."""
+@pytest.mark.parametrize("alg,state,tall", [(api.SPMV_ALG_DEFAULT, 3, False), (api.SPMV_CSR_ALG2, 2, False),
+                                            (api.SPMV_ALG_DEFAULT, 3, True)])
+def test_preprocessed_spmv_replays_in_a_hip_graph(torch_gpu, oracle, alg, state, tall):
+    """mcsparseSpMV on a copy built by mcsparseSpMV_preprocess (before the capture: it blocks) is two kernels; one
+    (which also puts its work counters back for the next replay) where x lies inside one band group (tall)."""
     torch = torch_gpu
     rng = np.random.default_rng(22)
     side = torch.cuda.Stream()
     handle = api.Handle(stream=side.cuda_stream)
-    a = wl.random_ragged(20000, 40000, 10, dtype=np.float64, seed=9)
+    a = wl.random_ragged(600000, 100000, 4, dtype=np.float64, seed=9) if tall else \
+        wl.random_ragged(20000, 40000, 10, dtype=np.float64, seed=9)
     d_ptr, d_col, d_val = dev(torch, a.ptr), dev(torch, a.col), dev(torch, a.val)
     A = api.SpMat(a.m, a.n, a.nnz, d_ptr, d_col, d_val, base=a.base)
-    A.set_band_bytes(1 << 13)
+    if not tall:
+        A.set_band_bytes(1 << 13)
     x = torch.zeros(a.n, dtype=torch.float64, device="cuda")
     y = torch.zeros(a.m, dtype=torch.float64, device="cuda")
     vx, vy = api.DnVec(x), api.DnVec(y)
@@ -140,6 +144,7 @@ def test_preprocessed_spmv_replays_in_a_hip_graph(torch_gpu, oracle, alg, state)
         assert api.spmv(handle, api.OP_N, 1.5, A, vx, 0.5, vy, api.R_64F, buf, alg=alg) == 0
     torch.cuda.synchronize()
     assert A.spmv_preprocess_state()[0] == state
+    assert not tall or A.spmv_preprocess_state()[1] == 1
     graph = torch.cuda.CUDAGraph()
     with torch.cuda.graph(graph, stream=side):
         # a preprocess call would have to block: refused on a capturing stream, the copy stays as it is

@@ -223,6 +223,37 @@ def test_fp64_reduce_with_any_alignment_of_y(torch_gpu, handle, oracle, alg, m, 
     assert backing[offset + m:].abs().sum().item() == 0 and (offset == 0 or backing[0].item() == 0)
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("alpha,beta", [(1.0, 0.0), (-1.5, 0.75), (0.0, 2.0)])
+def test_one_band_group_writes_y_itself(torch_gpu, handle, oracle, dtype, alpha, beta):
+    """x inside one band group: no planes of partial sums and no reduce kernel; the SpMV kernel applies alpha and
+    beta, must not read y under beta = 0 (NaN in it), and puts its work counters back itself: three calls."""
+    torch = torch_gpu
+    a = wl.random_ragged(600000, 100000, 5, dtype=dtype, seed=21)
+    rng = np.random.default_rng(21)
+    x = rng.uniform(-1, 1, a.n).astype(dtype)
+    y = rng.uniform(-1, 1, a.m).astype(dtype)
+    if beta == 0.0:
+        y[::7] = np.nan
+    d_ptr, d_col, d_val, d_x, d_y = (dev(torch, v) for v in (a.ptr, a.col, a.val, x, y))
+    mat = api.SpMat(a.m, a.n, a.nnz, d_ptr, d_col, d_val)
+    vx, vy = api.DnVec(d_x), api.DnVec(d_y)
+    ct = api.maca_type(dtype)
+    st, size = api.spmv_preprocess_buffer_size(handle, api.OP_N, alpha, mat, vx, beta, vy, ct)
+    assert st == api.STATUS_SUCCESS
+    buf = torch.empty(size, dtype=torch.uint8, device="cuda")
+    assert api.spmv_preprocess(handle, api.OP_N, alpha, mat, vx, beta, vy, ct, buf) == api.STATUS_SUCCESS
+    state, bands, rows = mat.spmv_preprocess_state()
+    assert (state, bands) == (3, 1), (state, bands, rows)
+    y_ref, bound = oracle.spmv(False, a.m, a.n, a.base, a.ptr, a.col, a.val, alpha, beta, x,
+                               np.where(np.isnan(y), 0, y).astype(dtype))
+    for _ in range(3):
+        d_y.copy_(torch.from_numpy(y))
+        assert api.spmv(handle, api.OP_N, alpha, mat, vx, beta, vy, ct, buf) == api.STATUS_SUCCESS
+        torch.cuda.synchronize()
+        assert_within(d_y.cpu().numpy(), y_ref, bound, dtype, what="one band group")
+
+
 def test_alg2_does_not_use_the_copy(torch_gpu, handle, oracle):
     """MCSPARSE_SPMV_CSR_ALG2 promises the same bits on every run: the call runs the row kernels."""
     a = wl.uniform_rows(m=20000, n=300000, per_row=8, dtype=np.float64, config_id=91)
