@@ -56,8 +56,8 @@ MEASURED_TRAFFIC = {
     # spmv_column_order_kernel + banded_reduce_kernel
     ("c2", 3): (_traffic(115061.1 + 20621.1, 32776.0 + 8192.0), "profiles/spmv_column_order_f64_c2_1Mx16.txt"),
     ("c3", 3): (_traffic(491030.7 + 65551.5, 131136.0 + 16384.0), "profiles/spmv_column_order_f32_c3_powerlaw.txt"),
-    ("c3t", 3): (_traffic(582000.8 + 8208.5, 16392.0 + 16384.0), "profiles/spmv_column_order_f32_c3_powerlaw.txt"),
-    ("c5-spmv", 3): (_traffic(582000.8 + 8208.5, 16392.0 + 16384.0),
+    ("c3t", 3): (_traffic(581912.9, 16400.3), "profiles/spmv_column_order_f32_c3_powerlaw.txt"),
+    ("c5-spmv", 3): (_traffic(581912.9, 16400.3),
                      "profiles/spmv_column_order_f32_c3_powerlaw.txt"),
     # without the preprocess call: vector kernel; merge kernel (tiles in column order) + partition
     # + tile order + fix-up
