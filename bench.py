@@ -7,9 +7,11 @@ A step is one pass of the hot path (one mcsparseSpMV / mcsparseSpMM / mcsparseCs
 through the C ABI) over one synthetic operand set that is already resident in HBM.  Several
 independent copies of all operands are rotated so the 256 MB Infinity Cache cannot hold a
 matrix between steps.  The default workload is the configuration the metric is quoted on:
-fp64 CSR SpMV, 1,048,576 rows x 16 nonzeros per row.  Prints one JSON line; the default
-invocation also measures the other configurations (fewer steps each, inside a wall-clock budget)
-and reports them under "others" of the same line.
+fp64 CSR SpMV, 1,048,576 rows x 16 nonzeros per row.  The last line of stdout is one compact JSON
+object (about 2 KB) with the headline figures; the default invocation also measures the other
+configurations (50 timed steps each, inside a wall-clock budget) and lists them under "others" of
+that line as workload: [ms_per_step, roofline.frac].  The full object of every workload measured
+goes to stderr, one JSON line each, and to gpurun_out/bench_details.json when that directory exists.
 
 Workloads: c1 (5-pt Laplacian 256^2 fp32), c2 (default), c3 / c3t (power-law fp32, op N / T),
 c4-8 / c4-64 / c4-256 (27-pt stencil 128^3 SpMM, row-major B and C), c4-64-col (the same with
@@ -34,6 +36,8 @@ HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 OTHERS = ["c4-64", "c3", "c3t", "c5", "c5-spmv", "c5-coo", "c4-8", "c4-256", "c4-64-col", "c1",
           "c2-alg2", "c3-alg2", "c3t-alg2", "c2-direct", "c3-direct", "c3t-direct", "c4-64-direct"]
 OTHERS_BUDGET_S = 200.0  # wall-clock budget of the default invocation for the workloads above
+OTHER_STEPS = {"c5": 20}  # timed steps of the workloads above: 50 unless named here (a step of c5 takes milliseconds)
+OTHERS_WITH_CPU = ("c4-64", "c3", "c3t", "c5")  # the OpenMP port is timed beside these (and beside the headline)
 SPIN_UP_S = 0.03  # every workload runs its steps for this long before the warmup steps (see run_workload)
 
 
@@ -446,24 +450,48 @@ def main():
     default_run = (name == "c2" and not args.no_others and not args.no_preprocess and not args.alg2 and
                    not args.no_cpu_baseline and args.scale == 1.0 and
                    not (args.family or args.lanes or args.band_bytes or args.copies))
+    details = [out]
     if default_run:
         others, skipped = {}, []
         for w in OTHERS:
             if time.perf_counter() - t_start > OTHERS_BUDGET_S:
                 skipped.append(w)
                 continue
-            r = run_workload(w, args, ctx, steps=12, warmup=3)
-            others[w] = {k: r[k] for k in ("value", "unit", "ms_per_step", "pct_of_hbm_peak", "gflops", "steps",
-                                           "algorithmic_bytes_per_step", "device_ms_per_step", "preprocess_ms",
-                                           "first_call_ms", "spmv_plan", "spmv_preprocess", "roofline") if k in r}
-            others[w]["workload"] = r["config"]["workload"]
-            others[w]["nnz"] = r["config"]["nnz"]
-            if "cpu_baseline" in r:
-                others[w]["cpu_baseline"] = r["cpu_baseline"]
+            r = run_workload(w, args, ctx, steps=OTHER_STEPS.get(w, 50), warmup=5, with_cpu=w in OTHERS_WITH_CPU)
+            details.append(r)
+            others[w] = [r["ms_per_step"], r["roofline"]["frac"]]
         out["others"] = others
+        out["others_are"] = "workload: [ms_per_step, roofline.frac]"
         out["others_skipped"] = skipped
-    print(json.dumps(out))
+    write_details(details)
+    print(compact_line(out))
     return 0
+
+
+HEADLINE_KEYS = ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step", "higher_is_better", "scaling",
+                 "vs_baseline", "dtype", "data", "config", "pct_of_hbm_peak", "gflops", "algorithmic_bytes_per_step",
+                 "preprocess_ms", "roofline", "cpu_baseline", "others", "others_are", "others_skipped")
+
+
+def compact_line(out):
+    """The one JSON line a run ends with: the headline keys only, short enough (about 2 KB) that a reader who keeps
+    the last few KB of the output still has all of it.  Everything else a workload measured goes to write_details."""
+    line = {k: out[k] for k in HEADLINE_KEYS if k in out}
+    return json.dumps(line, separators=(",", ":"))
+
+
+def write_details(objects):
+    """Every workload's full object: one JSON line each on stderr, and the list as bench_details.json in the
+    directory named by BENCH_DETAILS_DIR (default: gpurun_out beside this script, when it exists)."""
+    for o in objects:
+        print(json.dumps(o), file=sys.stderr)
+    directory = os.environ.get("BENCH_DETAILS_DIR") or os.path.join(ROOT, "gpurun_out")
+    if os.path.isdir(directory):
+        try:
+            with open(os.path.join(directory, "bench_details.json"), "w") as f:
+                json.dump(objects, f, indent=1)
+        except OSError:
+            pass
 
 
 def copy_probe(torch, args):
@@ -600,16 +628,12 @@ def cpu_baseline(kind, a, alpha, beta, n_cols, algo_bytes, op_t):
             oracle.csr2coo_omp(a.m, a.base, ptr, a.nnz)
         sample = "whole workload per repetition"
     elif kind == "spmm":
-        rows = min(a.m, max(1024, int(2e9 / max(1, 27 * n_cols * 4 * 10))))
-        sub_ptr = ptr[:rows + 1]
         B = ft(rng.uniform(-1, 1, (a.n, n_cols)).astype(dt))
-        C = ft(np.zeros((rows, n_cols), dtype=dt))
+        C = ft(np.zeros((a.m, n_cols), dtype=dt))
 
         def run():
-            oracle.spmm_omp_f32(rows, n_cols, a.base, sub_ptr, col, val, alpha, beta, B, C)
-        frac = rows / a.m
-        algo_bytes = algo_bytes * frac
-        sample = "first %d of %d rows per repetition, rate scaled by bytes" % (rows, a.m)
+            oracle.spmm_omp_f32(a.m, n_cols, a.base, ptr, col, val, alpha, beta, B, C)
+        sample = "whole workload per repetition"
     else:
         return {"value": None, "unit": "GB/s", "cores": threads, "kind": "port",
                 "sample": "no OpenMP port of this workload"}

@@ -327,6 +327,11 @@ mcspStatus_t spmv_typed(mcsparseHandle_t h, mcsparseSpMatDescr* A, mcsparseOpera
                                     buf + A->banded.region);
         return MCSP_STATUS_SUCCESS;
     }
+    // A call that does not run from the copy but is handed the copy's buffer may write over it: the copy
+    // sits behind the scratch of its own direction only, and the scratch of this call (the other
+    // direction, another value size) can reach further.  Such a call ends the copy; the next matching
+    // call runs the direct kernels until preprocess is called again.
+    if (A->banded.valid && A->banded.buffer == buffer && l.total > A->banded.region) A->banded.valid = false;
     if (wide_indices(A)) {
         const IndexArrays ia = index_arrays(h, A, buf + l.narrow);
         v = make_view(A, op, ia.rows, ia.cols);

@@ -393,3 +393,41 @@ def test_copies_of_coo_and_64_bit_inputs(torch_gpu, handle, oracle, alg, state, 
             assert api.spmv(handle, op, 1.5, mat, vx, -0.5, vy, api.R_64F, buf, alg=alg) == api.STATUS_SUCCESS
             torch.cuda.synchronize()
             assert_within(d_y.cpu().numpy(), y_ref, bound, np.float64, what="fmt %d index %d op %d" % (fmt, index_type, op))
+
+
+@pytest.mark.parametrize("alg", [api.SPMV_ALG_DEFAULT, api.SPMV_CSR_ALG2])
+def test_a_call_in_the_other_direction_on_the_same_buffer_ends_the_copy(torch_gpu, handle, oracle, alg):
+    """The copy of op N sits behind the scratch of op N only.  A^T x on the same buffer (sized for both) writes its
+    far larger scratch over the copy: the descriptor must drop the copy, so that the next A x reads the caller's
+    arrays again instead of the overwritten region."""
+    torch = torch_gpu
+    a = wl.random_ragged(90001, 70003, 8, dtype=np.float64, seed=31)
+    rng = np.random.default_rng(31)
+    x_n, y_n = rng.uniform(-1, 1, a.n), rng.uniform(-1, 1, a.m)
+    x_t, y_t = rng.uniform(-1, 1, a.m), rng.uniform(-1, 1, a.n)
+    d_ptr, d_col, d_val = (dev(torch, v) for v in (a.ptr, a.col, a.val))
+    d_xn, d_yn, d_xt, d_yt = (dev(torch, v) for v in (x_n, y_n, x_t, y_t))
+    mat = api.SpMat(a.m, a.n, a.nnz, d_ptr, d_col, d_val)
+    mat.set_band_bytes(1 << 14)
+    vxn, vyn, vxt, vyt = api.DnVec(d_xn), api.DnVec(d_yn), api.DnVec(d_xt), api.DnVec(d_yt)
+    ct = api.R_64F
+    st, size_pre = api.spmv_preprocess_buffer_size(handle, api.OP_N, 1.5, mat, vxn, 0.5, vyn, ct, alg=alg)
+    assert st == api.STATUS_SUCCESS
+    st, size_t = api.spmv_buffer_size(handle, api.OP_T, 1.5, mat, vxt, 0.5, vyt, ct)
+    assert st == api.STATUS_SUCCESS
+    buf = torch.empty(max(size_pre, size_t), dtype=torch.uint8, device="cuda")
+    assert api.spmv_preprocess(handle, api.OP_N, 1.5, mat, vxn, 0.5, vyn, ct, buf, alg=alg) == api.STATUS_SUCCESS
+    assert mat.spmv_preprocess_state()[0] in (2, 3)
+    ref_n, bound_n = oracle.spmv(False, a.m, a.n, 0, a.ptr, a.col, a.val, 1.5, 0.5, x_n, y_n)
+    ref_t, bound_t = oracle.spmv(True, a.m, a.n, 0, a.ptr, a.col, a.val, 1.5, 0.5, x_t, y_t)
+    assert api.spmv(handle, api.OP_N, 1.5, mat, vxn, 0.5, vyn, ct, buf, alg=alg) == api.STATUS_SUCCESS
+    torch.cuda.synchronize()
+    assert_within(d_yn.cpu().numpy(), ref_n, bound_n, np.float64, what="A x from the copy")
+    assert api.spmv(handle, api.OP_T, 1.5, mat, vxt, 0.5, vyt, ct, buf, alg=alg) == api.STATUS_SUCCESS
+    torch.cuda.synchronize()
+    assert_within(d_yt.cpu().numpy(), ref_t, bound_t, np.float64, what="A^T x on the copy's buffer")
+    assert mat.spmv_preprocess_state()[0] == 0  # the copy is gone
+    d_yn.copy_(torch.from_numpy(y_n))
+    assert api.spmv(handle, api.OP_N, 1.5, mat, vxn, 0.5, vyn, ct, buf, alg=alg) == api.STATUS_SUCCESS
+    torch.cuda.synchronize()
+    assert_within(d_yn.cpu().numpy(), ref_n, bound_n, np.float64, what="A x after the copy was written over")
