@@ -555,7 +555,11 @@ mcspStatus_t spmm_typed(mcsparseHandle_t h, const mcsparseSpMatDescr* A, mcspars
         // The kernel that works from the schedule owns four consecutive rows per lane group and writes them
         // into a column-major C as they lie there, 16 bytes per column: no row-major copy of C then.
         const bool scheduled_here = (b == 0 || shared_structure) && schedule_matches(A, buffer);
-        const bool direct_c = l.copy_c && scheduled_here && mcsp::spmm_schedule_usable(a, sizeof(T)) &&
+        const bool by_blocks = A->schedule.blocks;
+        auto schedule_usable = [&]() {
+            return by_blocks ? mcsp::spmm_blocks_usable(a, sizeof(T)) : mcsp::spmm_schedule_usable(a, sizeof(T));
+        };
+        const bool direct_c = l.copy_c && scheduled_here && schedule_usable() &&
                               reinterpret_cast<uintptr_t>(c_user) % 16 == 0 &&
                               (static_cast<uint64_t>(C->ld) * sizeof(T)) % 16 == 0;
         const bool copy_c = l.copy_c && !direct_c;
@@ -568,9 +572,14 @@ mcspStatus_t spmm_typed(mcsparseHandle_t h, const mcsparseSpMatDescr* A, mcspars
             if (l.copy_b && A->nnz != 0) a.n = static_cast<idx_t>(l.n_padded);
         }
         // the schedule was built from batch 0's structure
-        if (scheduled_here && mcsp::spmm_schedule_usable(a, sizeof(T))) {
-            mcsp::launch_spmm_scheduled<T>(h->stream, a, buffer, A->schedule.entries, A->schedule.mean_span, h_alpha,
-                                           beta_inner);
+        if (scheduled_here && schedule_usable()) {
+            if (by_blocks)
+                mcsp::launch_spmm_blocks<T>(h->stream, a, buffer, A->schedule.entries, A->schedule.longest_group,
+                                            A->schedule.mean_span, h_alpha,
+                                            beta_inner);
+            else
+                mcsp::launch_spmm_scheduled<T>(h->stream, a, buffer, A->schedule.entries, A->schedule.mean_span, h_alpha,
+                                               beta_inner);
         } else {
             mcsp::launch_spmm<T>(h->stream, a, h_alpha, beta_inner);
         }
@@ -938,18 +947,7 @@ mcsparseStatus_t mcsparseSpMM_preprocess(mcsparseHandle_t handle, mcsparseOperat
     const idx_t nnz = static_cast<idx_t>(matA->nnz);
     const IndexArrays ia = index_arrays(handle, matA, static_cast<char*>(externalBuffer) +
                                                           spmm_layout(matA, matB, matC, opB, value_size(matA->valueType)).narrow);
-    mcsp::launch_spmm_schedule(handle->stream, m, nnz, static_cast<idx_t>(matA->idxBase), ia.rows, ia.cols,
-                               externalBuffer);
     const mcsp::SpmmScheduleLayout l = mcsp::spmm_schedule_layout(m, nnz);
-    const uint64_t groups = mcsp::spmm_groups(m);
-    uint32_t entries = 0;
-    const char* total_slot = static_cast<const char*>(externalBuffer) + l.group_ptr + groups * sizeof(uint32_t);
-    unsigned long long span_sum = 0;
-    const char* span_slot = static_cast<const char*>(externalBuffer) + l.span_sum;
-    if (hipMemcpyAsync(&entries, total_slot, sizeof(entries), hipMemcpyDeviceToHost, handle->stream) != hipSuccess ||
-        hipMemcpyAsync(&span_sum, span_slot, sizeof(span_sum), hipMemcpyDeviceToHost, handle->stream) != hipSuccess ||
-        hipStreamSynchronize(handle->stream) != hipSuccess)
-        return to_public_status(MCSP_STATUS_INTERNAL_ERROR);
     SpmmSchedule& s = matA->schedule;
     s.buffer = externalBuffer;
     s.rows = matA->rows;
@@ -957,6 +955,53 @@ mcsparseStatus_t mcsparseSpMM_preprocess(mcsparseHandle_t handle, mcsparseOperat
     s.m = matA->row_num;
     s.nnz = matA->nnz;
     s.base = static_cast<int>(matA->idxBase);
+    s.blocks = false;
+    const char* span_slot = static_cast<const char*>(externalBuffer) + l.span_sum;
+
+    // First choice, for operands of 65 to 512 bytes per row (the widths its kernel was measured faster at: 19 %,
+    // 4 % and 20 % at 32, 64 and 128 fp32 columns of a 27-point stencil; at 256 columns the merged lists below
+    // win by 7 %): diagonal blocks over groups of eight rows.  Kept when the blocks are large (a stencil's are 24
+    // nonzeros each) and each loaded row of op(B) serves about two nonzeros or more; matrices without such
+    // structure get the merged column lists.
+    const size_t vb = value_size(matA->valueType);
+    const int64_t row_bytes = matC->col_num * static_cast<int64_t>(vb);
+    const bool wide_enough = row_bytes > 64 && row_bytes <= 512 && matA->row_num < (int64_t(1) << 31);
+    if (wide_enough) {
+        mcsp::launch_spmm_block_count(handle->stream, m, nnz, static_cast<idx_t>(matA->idxBase), ia.rows, ia.cols,
+                                      externalBuffer);
+        const uint64_t block_groups = mcsp::spmm_block_groups(m);
+        uint32_t blocks = 0;
+        unsigned long long counters[3] = {0, 0, 0};  // span sum, rows of op(B) loaded, longest group (low 32 bits)
+        const char* total_slot = static_cast<const char*>(externalBuffer) + l.group_ptr + block_groups * sizeof(uint32_t);
+        if (hipMemcpyAsync(&blocks, total_slot, sizeof(blocks), hipMemcpyDeviceToHost, handle->stream) != hipSuccess ||
+            hipMemcpyAsync(counters, span_slot, sizeof(counters), hipMemcpyDeviceToHost, handle->stream) != hipSuccess ||
+            hipStreamSynchronize(handle->stream) != hipSuccess)
+            return to_public_status(MCSP_STATUS_INTERNAL_ERROR);
+        const uint64_t nz = static_cast<uint64_t>(matA->nnz);
+        if (blocks != 0 && static_cast<uint64_t>(blocks) * 8 <= nz && counters[1] * 9 <= nz * 5 &&
+            mcsp::spmm_block_schedule_fits(m, nnz, blocks)) {
+            mcsp::launch_spmm_block_fill(handle->stream, m, nnz, static_cast<idx_t>(matA->idxBase), ia.rows, ia.cols,
+                                         externalBuffer);
+            s.entries = blocks;
+            s.mean_span = block_groups != 0 ? counters[0] / block_groups : 0;
+            s.blocks = true;
+            s.longest_group = static_cast<uint32_t>(counters[2] & 0xffffffffull);
+            s.useful = true;
+            s.valid = true;
+            return MCSPARSE_STATUS_SUCCESS;
+        }
+    }
+
+    mcsp::launch_spmm_schedule(handle->stream, m, nnz, static_cast<idx_t>(matA->idxBase), ia.rows, ia.cols,
+                               externalBuffer);
+    const uint64_t groups = mcsp::spmm_groups(m);
+    uint32_t entries = 0;
+    const char* total_slot = static_cast<const char*>(externalBuffer) + l.group_ptr + groups * sizeof(uint32_t);
+    unsigned long long span_sum = 0;
+    if (hipMemcpyAsync(&entries, total_slot, sizeof(entries), hipMemcpyDeviceToHost, handle->stream) != hipSuccess ||
+        hipMemcpyAsync(&span_sum, span_slot, sizeof(span_sum), hipMemcpyDeviceToHost, handle->stream) != hipSuccess ||
+        hipStreamSynchronize(handle->stream) != hipSuccess)
+        return to_public_status(MCSP_STATUS_INTERNAL_ERROR);
     s.entries = entries;
     s.mean_span = groups != 0 ? span_sum / groups : 0;
     // Worth it when the merged lists are clearly shorter than the rows they replace; groups too

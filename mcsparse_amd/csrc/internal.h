@@ -89,8 +89,10 @@ struct SpmmSchedule {
     const void* cols = nullptr;
     int64_t m = 0, nnz = 0;
     int base = 0;
-    uint32_t entries = 0;  // length of all merged lists together
+    uint32_t entries = 0;  // length of all merged lists together, or the number of diagonal blocks
     uint64_t mean_span = 0;  // mean distance between the first and the last column of a group
+    bool blocks = false;   // the schedule holds diagonal blocks (spmm_blocks.hip) instead of merged lists
+    uint32_t longest_group = 0;  // blocks: the most nonzeros in one group of rows
 };
 
 // Column-banded copy of a CSR matrix built by mcsparseSpMV_preprocess inside the caller's buffer
@@ -347,6 +349,31 @@ bool spmm_schedule_usable(const SpmmArgs& a, size_t value_bytes);
 template <typename T>
 void launch_spmm_scheduled(hipStream_t stream, const SpmmArgs& a, const void* schedule, uint32_t total_entries,
                            uint64_t mean_span, T alpha, T beta);
+
+// Diagonal-block schedule of a CSR structure (spmm_blocks.hip), the second kind mcsparseSpMM_preprocess can leave in
+// the region spmm_schedule_layout describes: for every group of kSpmmBlockRows consecutive rows a list of blocks
+// {int32 c, uint32 n | lo << 8 | hi << 16}: each row r in [lo, hi) of the group holds the n <= kSpmmBlockMaxDiagonals
+// consecutive columns c + r .. c + r + n - 1 (zero-based), and the blocks of a group consume every row's nonzeros
+// in storage order.  group_ptr's place holds the groups+1 offsets into the blocks, entries' place the blocks
+// (8 bytes each: the schedule is only kept when they fit), span_sum's place three counters: the sum of the
+// groups' column spans and the number of rows of op(B) all blocks load (u64), the most nonzeros in one group (u32).
+constexpr int kSpmmBlockRows = 8;
+constexpr int kSpmmBlockMaxDiagonals = 3;
+constexpr uint64_t spmm_block_groups(idx_t m) { return (static_cast<uint64_t>(m) + kSpmmBlockRows - 1) / kSpmmBlockRows; }
+// Counts the blocks of every group and scans the counts (the total lands in slot `groups` of the offsets).
+void launch_spmm_block_count(hipStream_t stream, idx_t m, idx_t nnz, idx_t base, const idx_t* row_ptr, const idx_t* col,
+                             void* schedule);
+// Whether `blocks` blocks of 8 bytes and the order of the groups (4 bytes each) fit the entries' place.
+bool spmm_block_schedule_fits(idx_t m, idx_t nnz, uint32_t blocks);
+// Writes the blocks and the order in which the kernel takes the groups; only after the count, and only when
+// spmm_block_schedule_fits says so.
+void launch_spmm_block_fill(hipStream_t stream, idx_t m, idx_t nnz, idx_t base, const idx_t* row_ptr, const idx_t* col,
+                            void* schedule);
+bool spmm_blocks_usable(const SpmmArgs& a, size_t value_bytes);
+// longest_group: the most nonzeros any group with blocks holds (the third counter the count leaves).
+template <typename T>
+void launch_spmm_blocks(hipStream_t stream, const SpmmArgs& a, const void* schedule, uint32_t total_blocks,
+                        uint32_t longest_group, uint64_t mean_span, T alpha, T beta);
 
 // Dense transposes for column-major SpMM operands (spmm.hip).  src is rows x cols, row-major with
 // leading dimension lds.  launch_transpose: dst (cols x rows_padded, ldd) = transpose(src), the columns

@@ -47,7 +47,8 @@ def run_spmm(torch, handle, a, B, C0, alpha, beta, op_b=api.OP_N, b_order=api.OR
     if preprocess:
         assert api.spmm_preprocess(handle, api.OP_N, op_b, alpha, mat, mB, beta, mC, ct, buf) == 0
         if expect_schedule is not None:
-            assert mat.spmm_schedule()[0] == expect_schedule, mat.spmm_schedule()
+            wanted = expect_schedule if isinstance(expect_schedule, tuple) else (expect_schedule,)
+            assert mat.spmm_schedule()[0] in wanted, mat.spmm_schedule()
     st = api.spmm(handle, api.OP_N, op_b, alpha, mat, mB, beta, mC, ct, buf)
     torch.cuda.synchronize()
     out = d_C.cpu().numpy()
@@ -120,10 +121,11 @@ def test_exact_cases(torch_gpu, handle):
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
 def test_preprocessed_stencil(torch_gpu, handle, oracle, n, dtype):
     a = wl.stencil_27pt(13, dtype=dtype).with_base(1)  # row count not a multiple of the group size: the last group is short
+    # state 2: merged column lists; state 3: diagonal blocks, for operands of more than 64 bytes per row
     for c_order in (api.ORDER_ROW, api.ORDER_COL):
-        check(torch_gpu, handle, oracle, a, n, 1.0, 0.0, preprocess=True, expect_schedule=2, c_order=c_order)
-        check(torch_gpu, handle, oracle, a, n, -1.5, 0.75, preprocess=True, expect_schedule=2, c_order=c_order, pad_b=4,
-              pad_c=8)
+        check(torch_gpu, handle, oracle, a, n, 1.0, 0.0, preprocess=True, expect_schedule=(2, 3), c_order=c_order)
+        check(torch_gpu, handle, oracle, a, n, -1.5, 0.75, preprocess=True, expect_schedule=(2, 3), c_order=c_order,
+              pad_b=4, pad_c=8)
 
 
 def test_preprocessed_stencil_in_xcd_stretches(torch_gpu, handle, oracle):
@@ -132,8 +134,9 @@ def test_preprocessed_stencil_in_xcd_stretches(torch_gpu, handle, oracle):
     partly filled."""
     a = wl.stencil_27pt(48, dtype=np.float32)
     for n in (64, 40):
-        check(torch_gpu, handle, oracle, a, n, 1.0, 0.0, preprocess=True, expect_schedule=2)
-    check(torch_gpu, handle, oracle, a, 64, 0.5, -1.0, preprocess=True, expect_schedule=2, c_order=api.ORDER_COL)
+        check(torch_gpu, handle, oracle, a, n, 1.0, 0.0, preprocess=True, expect_schedule=3)
+    check(torch_gpu, handle, oracle, a, 64, 0.5, -1.0, preprocess=True, expect_schedule=3, c_order=api.ORDER_COL)
+    check(torch_gpu, handle, oracle, a, 16, 1.0, 0.0, preprocess=True, expect_schedule=2)  # too narrow for blocks
 
 
 def test_preprocessed_ragged_rows_with_overlap(torch_gpu, handle, oracle):
@@ -207,13 +210,13 @@ def test_schedule_is_dropped_with_other_buffer_or_pointers(torch_gpu, handle, or
     assert mat.spmm_schedule()[0] == 0
 
 
-def test_overwritten_schedule_stays_in_bounds(torch_gpu, handle):
+@pytest.mark.parametrize("grid,n", [(10, 64), (40, 64), (40, 128), (10, 16)])
+def test_overwritten_schedule_stays_in_bounds(torch_gpu, handle, grid, n):
     """The reference's preprocess is a no-op, so a caller written against it may reuse the scratch
     buffer between preprocess and SpMM.  The schedule is then garbage: the product may be wrong, but
     every access stays inside the arrays (the call returns and the device stays healthy)."""
     torch = torch_gpu
-    a = wl.stencil_27pt(10, dtype=np.float32)
-    n = 64
+    a = wl.stencil_27pt(grid, dtype=np.float32)
     d_ptr, d_col, d_val = dev(torch, a.ptr), dev(torch, a.col), dev(torch, a.val)
     d_B = torch.ones((a.n, n), dtype=torch.float32, device="cuda")
     d_C = torch.zeros((a.m, n), dtype=torch.float32, device="cuda")
@@ -222,7 +225,7 @@ def test_overwritten_schedule_stays_in_bounds(torch_gpu, handle):
     st, size = api.spmm_buffer_size(handle, api.OP_N, api.OP_N, 1.0, mat, mB, 0.0, mC, api.R_32F)
     buf = torch.empty(size, dtype=torch.uint8, device="cuda")
     assert api.spmm_preprocess(handle, api.OP_N, api.OP_N, 1.0, mat, mB, 0.0, mC, api.R_32F, buf) == 0
-    assert mat.spmm_schedule()[0] == 2
+    assert mat.spmm_schedule()[0] in (2, 3)
     gen = torch.Generator(device="cuda")
     gen.manual_seed(3)
     for fill in (0xFF, None, 0x00):
@@ -239,3 +242,151 @@ def test_overwritten_schedule_stays_in_bounds(torch_gpu, handle):
     want = np.asarray(a.to_scipy().sum(axis=1)).ravel()  # B = ones: row sums of A
     got = d_C.cpu().numpy()
     assert np.allclose(got, want[:, None].repeat(n, 1), rtol=1e-5, atol=1e-5)
+
+
+# ---- diagonal blocks (mcsparseSpMM_preprocess on matrices whose neighbouring rows hold the same diagonals) ----
+
+def read_blocks(torch, buf, m):
+    """The block schedule as it lies in the buffer: offsets per group of 8 rows, then (c, n | lo << 8 | hi << 16)."""
+    def align(x):
+        return (x + 127) // 128 * 128
+    raw = buf.cpu().numpy()
+    groups = (m + 7) // 8
+    ptr = raw[:4 * (groups + 1)].view(np.uint32)
+    at = align(4 * ((m + 3) // 4 + 1)) + 128  # behind the offsets of the 4-row groups and the counters
+    words = raw[at:at + 8 * int(ptr[groups])].view(np.uint32).reshape(-1, 2)
+    return ptr, words
+
+
+def columns_from_blocks(ptr, words, m):
+    """Expands the blocks into every row's column sequence (zero-based)."""
+    rows = [[] for _ in range(m)]
+    for g in range(len(ptr) - 1):
+        for c, shape in words[ptr[g]:ptr[g + 1]]:
+            c = int(np.int32(c))
+            n, lo, hi = int(shape & 7), int((shape >> 8) & 15), int((shape >> 16) & 31)
+            assert 1 <= n <= 4 and 0 <= lo < hi <= 8
+            for r in range(lo, hi):
+                rows[8 * g + r].extend(range(c + r, c + r + n))
+    return rows
+
+
+@pytest.mark.parametrize("shape", ["stencil", "banded", "unsorted"])
+def test_blocks_cover_every_nonzero_once_and_in_storage_order(torch_gpu, handle, shape):
+    """Structural outputs are bit-exact: the blocks of a group, expanded, are the rows' column indices as stored."""
+    torch = torch_gpu
+    rng = np.random.default_rng(3)
+    if shape == "stencil":
+        a = wl.stencil_27pt(40, dtype=np.float32).with_base(1)
+    else:
+        m = 4099
+        offsets = np.array([-70, -69, -68, -2, -1, 0, 1, 2, 3, 64, 65, 66, 67, 68, 69])  # runs of 3, 6 (cut at 4) and 6
+        rows = []
+        for r in range(m):
+            c = r + offsets
+            c = c[(c >= 0) & (c < m)]
+            if r % 97 == 5:
+                c = c[::2]                      # a row with holes breaks the blocks around it
+            if r % 211 == 7:
+                c = np.zeros(0, np.int64)       # an empty row
+            if shape == "unsorted" and r % 120 == 0:
+                c = rng.permutation(c)          # consumed in storage order: single nonzeros around intact blocks
+            rows.append(c)
+        ptr = np.concatenate([[0], np.cumsum([len(c) for c in rows])]).astype(np.int32)
+        a = wl.Csr(m, m, ptr, np.concatenate(rows).astype(np.int32), rng.uniform(-1, 1, int(ptr[-1])).astype(np.float32))
+    n = 64
+    d_ptr, d_col, d_val = dev(torch, a.ptr), dev(torch, a.col), dev(torch, a.val)
+    d_B = torch.ones((a.n, n), dtype=torch.float32, device="cuda")
+    d_C = torch.zeros((a.m, n), dtype=torch.float32, device="cuda")
+    mat = api.SpMat(a.m, a.n, a.nnz, d_ptr, d_col, d_val, base=a.base)
+    mB, mC = api.DnMat(a.n, n, n, d_B), api.DnMat(a.m, n, n, d_C)
+    st, size = api.spmm_buffer_size(handle, api.OP_N, api.OP_N, 1.0, mat, mB, 0.0, mC, api.R_32F)
+    buf = torch.zeros(size, dtype=torch.uint8, device="cuda")
+    assert api.spmm_preprocess(handle, api.OP_N, api.OP_N, 1.0, mat, mB, 0.0, mC, api.R_32F, buf) == 0
+    state, blocks = mat.spmm_schedule()
+    assert state == 3, (state, blocks)
+    torch.cuda.synchronize()
+    ptr, words = read_blocks(torch, buf, a.m)
+    assert int(ptr[-1]) == blocks and (np.diff(ptr.astype(np.int64)) >= 0).all()
+    got = columns_from_blocks(ptr, words, a.m)
+    for r in range(a.m):
+        want = (a.col[a.ptr[r] - a.base:a.ptr[r + 1] - a.base].astype(np.int64) - a.base).tolist()
+        assert got[r] == want, (r, got[r], want)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("n", [20, 36, 64, 72, 128])
+def test_blocks_banded_matrix_with_broken_rows(torch_gpu, handle, oracle, dtype, n):
+    """Diagonal runs of one to six, rows with holes, empty rows, unsorted rows, a group too long to cover, a row
+    count that leaves the last group short; every width of lane group; both layouts of C."""
+    rng = np.random.default_rng(5)
+    m, k = 3003, 3100
+    offsets = np.array([-70, -69, -68, -2, -1, 0, 1, 2, 3, 64, 65, 66, 67, 68, 69, 200])
+    rows = []
+    for r in range(m):
+        c = r + offsets
+        c = c[(c >= 0) & (c < k)]
+        if r % 97 == 5:
+            c = c[::2]
+        if r % 211 == 7:
+            c = np.zeros(0, np.int64)
+        if r in (1000, 1001):
+            c = rng.choice(k, 1500, replace=False)   # 3000 nonzeros in their group: not covered, row by row
+        if r % 120 == 0:
+            c = rng.permutation(c)
+        rows.append(c)
+    ptr = np.concatenate([[0], np.cumsum([len(c) for c in rows])]).astype(np.int32)
+    a = wl.Csr(m, k, ptr, np.concatenate(rows).astype(np.int32), rng.uniform(-1, 1, int(ptr[-1])).astype(dtype))
+    # blocks for operands of 65 to 512 bytes per row, merged column lists beyond
+    want = 3 if 64 < n * np.dtype(dtype).itemsize <= 512 else (1, 2)
+    for c_order in (api.ORDER_ROW, api.ORDER_COL):
+        check(torch_gpu, handle, oracle, a, n, 1.0, 0.0, preprocess=True, expect_schedule=want, c_order=c_order)
+    check(torch_gpu, handle, oracle, a.with_base(1), n, -0.5, 1.5, preprocess=True, expect_schedule=want, pad_b=4, pad_c=8)
+
+
+def test_blocks_row_ignores_rows_of_b_only_its_neighbours_use(torch_gpu, handle):
+    """A block loads rows of op(B) for all its rows of A; a row must only see the ones it names (0 * inf = NaN)."""
+    m = 64
+    rows = [np.array([r, r + 1, r + 2]) for r in range(m)]
+    ptr = np.concatenate([[0], np.cumsum([len(c) for c in rows])]).astype(np.int32)
+    a = wl.Csr(m, m + 2, ptr, np.concatenate(rows).astype(np.int32), np.ones(3 * m, np.float32))
+    n = 64
+    B = np.ones((m + 2, n), np.float32)
+    B[10, :] = np.inf   # named by rows 8, 9, 10 only
+    st, got, _ = run_spmm(torch_gpu, handle, a, B, np.zeros((m, n), np.float32), 1.0, 0.0, preprocess=True,
+                          expect_schedule=3)
+    assert st == 0
+    for r in range(m):
+        if r in (8, 9, 10):
+            assert np.all(np.isinf(got[r]))
+        else:
+            assert np.all(got[r] == 3.0), r
+
+
+def test_blocks_schedule_used_with_a_wider_operand_than_it_was_built_for(torch_gpu, handle, oracle):
+    """The schedule belongs to the structure of A: built with a 64-column operand it also serves 256 columns (cut into
+    panels) and 8 columns (too narrow for its kernel: the schedule-free kernel runs)."""
+    torch = torch_gpu
+    a = wl.stencil_27pt(40, dtype=np.float32)
+    rng = np.random.default_rng(9)
+    d_ptr, d_col, d_val = dev(torch, a.ptr), dev(torch, a.col), dev(torch, a.val)
+    mat = api.SpMat(a.m, a.n, a.nnz, d_ptr, d_col, d_val)
+    sizes = {}
+    ops = {}
+    for n in (64, 256, 8):
+        B = rng.uniform(-1, 1, (a.n, n)).astype(np.float32)
+        d_B = dev(torch, B)
+        d_C = torch.zeros((a.m, n), dtype=torch.float32, device="cuda")
+        ops[n] = (B, d_B, d_C, api.DnMat(a.n, n, n, d_B), api.DnMat(a.m, n, n, d_C))
+        st, sizes[n] = api.spmm_buffer_size(handle, api.OP_N, api.OP_N, 1.0, mat, ops[n][3], 0.0, ops[n][4], api.R_32F)
+        assert st == 0
+    buf = torch.empty(max(sizes.values()), dtype=torch.uint8, device="cuda")
+    assert api.spmm_preprocess(handle, api.OP_N, api.OP_N, 1.0, mat, ops[64][3], 0.0, ops[64][4], api.R_32F, buf) == 0
+    assert mat.spmm_schedule()[0] == 3
+    for n in (64, 256, 8):
+        B, d_B, d_C, mB, mC = ops[n]
+        assert api.spmm(handle, api.OP_N, api.OP_N, 1.0, mat, mB, 0.0, mC, api.R_32F, buf) == 0
+        torch.cuda.synchronize()
+        c_ref, bound = oracle.spmm(a.m, n, 0, a.ptr, a.col, a.val, 1.0, 0.0, B.ravel(), n, True,
+                                   np.zeros(a.m * n, np.float32), n, True)
+        assert_within(d_C.cpu().numpy(), c_ref, bound, np.float32, what="n=%d" % n)
