@@ -13,12 +13,14 @@ configurations (50 timed steps each, inside a wall-clock budget) and lists them 
 that line as workload: [ms_per_step, roofline.frac].  The full object of every workload measured
 goes to stderr, one JSON line each, and to gpurun_out/bench_details.json when that directory exists.
 
-Workloads: c1 (5-pt Laplacian 256^2 fp32), c2 (default), c3 / c3t (power-law fp32, op N / T),
+Workloads: mixed (1 M rows of 16 and 64 rows of 100000, fp32), c1 (5-pt Laplacian 256^2 fp32), c2 (default), c3 / c3t (power-law fp32, op N / T),
 c4-8 / c4-64 / c4-256 (27-pt stencil 128^3 SpMM, row-major B and C), c4-64-col (the same with
 column-major B and C, the layout of csrmm2), c5 (csr2csc on the c3 matrix), c5-coo (csr2coo on it),
 c5-spmv (A^T x from the converted CSC).  Probes: copy (a plain device copy, the yardstick of the
 traffic counters), gather-probe (16.8 M random 8-byte reads through mcsparseDgthr: what the x[col]
-reads of c2 cost on their own, from an 8 MB table and from one that fits every L2).
+reads of c2 cost on their own, from an 8 MB table and from one that fits every L2), stream-probe (the library's own
+streaming kernels reading, writing and copying 1 GiB buffers: what the memory takes by itself; the default run holds
+the headline against these rates as roofline.stream_ceiling_frac).
 """
 import argparse
 import json
@@ -34,55 +36,37 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 
 OTHERS = ["c4-64", "c3", "c3t", "c5", "c5-spmv", "c5-coo", "c4-8", "c4-256", "c4-64-col", "c1",
-          "c2-alg2", "c3-alg2", "c3t-alg2", "c2-direct", "c3-direct", "c3t-direct", "c4-64-direct"]
+          "c2-alg2", "c3-alg2", "c3t-alg2", "c2-direct", "c3-direct", "c3t-direct", "c4-64-direct", "mixed-direct"]
 OTHERS_BUDGET_S = 200.0  # wall-clock budget of the default invocation for the workloads above
 OTHER_STEPS = {"c5": 20}  # timed steps of the workloads above: 50 unless named here (a step of c5 takes milliseconds)
 OTHERS_WITH_CPU = ("c4-64", "c3", "c3t", "c5")  # the OpenMP port is timed beside these (and beside the headline)
 SPIN_UP_S = 0.03  # every workload runs its steps for this long before the warmup steps (see run_workload)
 
 
-# HBM/fabric bytes per call (all kernels of one step together), from rocprofv3 FETCH_SIZE and
-# WRITE_SIZE, each scaled by what the same counter reads on a 1 GiB copy: 2 KiB and 1 KiB per
-# count.  These are constants taken from the counter summaries under profiles/ (named beside each),
-# not counters read during the run.
-def _traffic(fetch_counts, write_counts):
-    return int((fetch_counts * 2 + write_counts) * 1024)
+def measured_traffic():
+    """{(workload, preprocess state): (bytes per step, file)} from the "traffic" lines of the counter summaries under
+    profiles/: FETCH_SIZE and WRITE_SIZE counts of all kernels of one step, each scaled by what the same counter
+    reads on a 1 GiB copy (2 KiB and 1 KiB per count, profiles/copy_kernel_counter_calibration.txt).  Constants
+    taken from those summaries, not counters read during the run."""
+    out = {}
+    directory = os.path.join(ROOT, "profiles")
+    if not os.path.isdir(directory):
+        return out
+    for name in sorted(os.listdir(directory)):
+        if not name.endswith(".txt"):
+            continue
+        with open(os.path.join(directory, name)) as f:
+            for line in f:
+                parts = line.split()
+                if len(parts) == 5 and parts[0] == "traffic" and parts[2].startswith("state="):
+                    fetch = float(parts[3].split("=", 1)[1])
+                    write = float(parts[4].split("=", 1)[1])
+                    out[(parts[1], int(parts[2].split("=", 1)[1]))] = (int((fetch * 2 + write) * 1024),
+                                                                        "profiles/" + name)
+    return out
 
 
-MEASURED_TRAFFIC = {
-    # keys: (workload, state of mcsparseSpMV_preprocess: 2 banded copy, 3 copy in column order, 0 neither).
-    # spmv_banded_kernel + banded_reduce_kernel
-    ("c2", 2): (_traffic(108483.2 + 20567.1, 32768.0 + 8192.0), "profiles/spmv_banded_f64_c2_1Mx16.txt"),
-    ("c3", 2): (_traffic(479341.2 + 65545.2, 133136.1 + 16384.0), "profiles/spmv_banded_f32_c3_powerlaw.txt"),
-    ("c3t", 2): (_traffic(481300.5 + 65544.8, 131206.2 + 16384.0), "profiles/spmv_banded_f32_c3_powerlaw.txt"),
-    ("c5-spmv", 2): (_traffic(481330.8 + 65544.6, 131202.3 + 16384.0),
-                        "profiles/spmv_banded_f32_c3_powerlaw.txt"),
-    # spmv_column_order_kernel + banded_reduce_kernel
-    ("c2", 3): (_traffic(115061.1 + 20621.1, 32776.0 + 8192.0), "profiles/spmv_column_order_f64_c2_1Mx16.txt"),
-    ("c3", 3): (_traffic(491030.7 + 65551.5, 131136.0 + 16384.0), "profiles/spmv_column_order_f32_c3_powerlaw.txt"),
-    ("c3t", 3): (_traffic(581912.9, 16400.3), "profiles/spmv_column_order_f32_c3_powerlaw.txt"),
-    ("c5-spmv", 3): (_traffic(581912.9, 16400.3),
-                     "profiles/spmv_column_order_f32_c3_powerlaw.txt"),
-    # without the preprocess call: vector kernel; merge kernel (tiles in column order) + partition
-    # + tile order + fix-up
-    ("c2", 0): (_traffic(653904.5, 10047.2), "profiles/spmv_vector_f64_c2_1Mx16.txt"),
-    ("c3", 0): (_traffic(3305285.9 + 17229.2 + 251.2 + 3154.3, 25157.0 + 1391.2 + 1994.3 + 1375.1),
-                    "profiles/spmv_merge_f32_c3_powerlaw.txt"),
-    # op T without the preprocess call: key histogram + scans + row starts per tile + one scatter pass + bucket sums
-    ("c3t", 0): (_traffic(229180.3 + 14342.5 + 2 * 7207.2 + 21132.3 + 489308.2 + 421987.3,
-                          28832.0 + 56.0 + 2 * 14325.6 + 223.8 + 692310.6 + 16384.0),
-                 "profiles/spmv_transposed_buckets_f32_c3_powerlaw.txt"),
-    ("c4-64", 0): (_traffic(492232.8, 524288.0), "profiles/spmm_group_f32_c4_stencil128.txt"),
-    ("c4-256", 0): (_traffic(3630735.8, 2097152.0), "profiles/spmm_group_f32_c4_stencil128.txt"),
-    # group kernel (writes the column-major C itself) + the transpose of B
-    ("c4-64-col", 0): (_traffic(589819.9 + 262180.0, 537321.5 + 524288.0),
-                           "profiles/spmm_colmajor_f32_c4_stencil128_n64.txt"),
-    # csr2csc: 2 x scatter + the scatter that reads the CSR arrays in place + 3 x (histogram + scans)
-    # + row starts per tile + coo2csr
-    ("c5", 0): (_traffic(2 * 701979.0 + 481119.4 + 3 * (229171.1 + 2 * 7206.6 + 14342.5) + 21136.0 + 237161.6,
-                             2 * 1387754.6 + 1421432.8 + 3 * (28789.0 + 2 * 14326.3 + 56.0) + 223.8 + 19514.6),
-                    "profiles/csr2csc_radix_f32_c5_powerlaw.txt"),
-}
+MEASURED_TRAFFIC = measured_traffic()
 
 
 def parse():
@@ -125,6 +109,9 @@ class Matrices:
         elif key == "power_law":
             a = cached(self.cache, "power_law_%g" % s, lambda: wl.power_law(
                 m=max(64, int((1 << 22) * s)), max_len=max(8, int(200000 * min(1.0, s * 4))), dtype=np.float32))
+        elif key == "mixed":
+            a = wl.mixed_rows(m=max(4096, int((1 << 20) * s)), long_len=max(64, int(100000 * min(1.0, s * 4))),
+                              dtype=np.float32)
         elif key == "stencil":
             a = wl.stencil_27pt(max(4, int(round(128 * s ** (1 / 3)))), dtype=np.float32)
         else:
@@ -157,6 +144,9 @@ def describe(name):
     if name == "c5-spmv":
         return ("power_law", "spmv-csc", False, 0, 1.0, 0.0,
                 "fp32 SpMV op T from the CSC produced by csr2csc (power-law matrix)")
+    if name == "mixed":
+        return ("mixed", "spmv", False, 0, 1.0, 0.0,
+                "fp32 CSR SpMV, 1048576 rows x 16 nnz/row uniform + 64 rows of 100000")
     if name.startswith("c4-"):
         parts = name.split("-")
         n_cols = int(parts[1])
@@ -433,6 +423,9 @@ def main():
         return copy_probe(torch, args)
     if name == "gather-probe":
         return gather_probe(torch, api, handle, args)
+    if name == "stream-probe":
+        print(json.dumps(stream_probe(torch, api, handle, stream, steps=args.steps or 40)))
+        return 0
     try:
         describe(name)
     except (KeyError, ValueError, IndexError):
@@ -451,6 +444,19 @@ def main():
                    not args.no_cpu_baseline and args.scale == 1.0 and
                    not (args.family or args.lanes or args.band_bytes or args.copies))
     details = [out]
+    if default_run or name == "c2":
+        # The same bytes at the rates the memory gives streaming kernels of this library (measured in this run): what
+        # a kernel that only streamed its algorithmic bytes, reads at the read rate and writes at the write rate,
+        # would reach, and the headline as a fraction of that.
+        probe = stream_probe(torch, api, handle, stream, steps=20)
+        details.append(probe)
+        a_bytes = out["algorithmic_bytes_per_step"]
+        writes = out["config"]["rows"] * (8 if out["dtype"] == "f64" else 4)
+        floor_ms = ((a_bytes - writes) / probe["read_GBps"] + writes / probe["write_GBps"]) / 1e6
+        out["roofline"]["stream_ceiling"] = {"read_GBps": probe["read_GBps"], "write_GBps": probe["write_GBps"],
+                                             "copy_GBps": probe["copy_GBps"],
+                                             "algorithmic_bytes_at_these_rates_ms": round(floor_ms, 5)}
+        out["roofline"]["stream_ceiling_frac"] = round(floor_ms / (a_bytes / out["roofline"]["achieved"] / 1e6), 4)
     if default_run:
         others, skipped = {}, []
         for w in OTHERS:
@@ -492,6 +498,39 @@ def write_details(objects):
                 json.dump(objects, f, indent=1)
         except OSError:
             pass
+
+
+def stream_probe(torch, api, handle, stream, steps=40, gib=1):
+    """What the memory takes by itself: the library's own streaming kernels (mcsparseXstreamProbe: 16-byte
+    non-temporal accesses, eight in flight per thread) reading, writing and copying buffers of 1 GiB, rotated over
+    four so that the 256 MB Infinity Cache holds none of them.  GB/s per mode, between two events on the stream."""
+    nbytes = gib << 30
+    bufs = [torch.empty(nbytes, dtype=torch.uint8, device="cuda") for _ in range(4)]
+    for b in bufs:
+        b.fill_(1)
+    sink = torch.zeros(1 << 20, dtype=torch.int32, device="cuda")
+    out = {"workload": "stream-probe", "buffer_bytes": nbytes, "buffers_rotated": len(bufs), "steps": steps}
+
+    def run(mode, i):
+        src, dst = bufs[i % 4], bufs[(i + 1) % 4]
+        api.check(api.stream_probe(handle, mode, src if mode != 1 else None, dst if mode != 0 else None, nbytes,
+                                   sink if mode == 0 else None), "mcsparseXstreamProbe")
+
+    for mode, name, moved in ((0, "read", nbytes), (1, "write", nbytes), (2, "copy", 2 * nbytes)):
+        for i in range(8):
+            run(mode, i)
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(stream)
+        for i in range(steps):
+            run(mode, i)
+        e1.record(stream)
+        torch.cuda.synchronize()
+        ms = e0.elapsed_time(e1) / steps
+        out[name + "_GBps"] = round(moved / ms / 1e6, 1)
+        out[name + "_ms"] = round(ms, 4)
+    del bufs
+    torch.cuda.empty_cache()
+    return out
 
 
 def copy_probe(torch, args):

@@ -510,6 +510,32 @@ mcsparseStatus_t mcsparseSpMatGetSpMVPreprocess(mcsparseSpMatDescr_t spMatDescr,
  * rounded down to a power of two).  Drops a banded copy already built.  For tests and benchmarks. */
 mcsparseStatus_t mcsparseSpMatSetSpMVBandBytes(mcsparseSpMatDescr_t spMatDescr, size_t band_bytes);
 
+/* What the device's memory takes by itself, measured with kernels as plain as this library's can be (16-byte
+ * non-temporal accesses, eight in flight per thread): mode 0 reads `bytes` of src, mode 1 writes `bytes` of dst,
+ * mode 2 copies src to dst.  bytes must be a multiple of 16 and both arrays 16-byte aligned; mode 0 needs `sink`,
+ * device memory of at least 2048 * (compute units of the device) uint32 (sink_words says how many it holds), where
+ * every thread leaves a word so that its loads are not optimised away.  A yardstick for benchmarks: the rates the
+ * kernels of the path are held against besides the published 8 TB/s. */
+mcsparseStatus_t mcsparseXstreamProbe(mcsparseHandle_t handle, int mode, const void* src, void* dst, size_t bytes,
+                                      uint32_t* sink, size_t sink_words);
+
+/* The reference's SpMV adds the products of a row in a fixed order, so two runs of a call give the same bits
+ * whatever `alg` is.  In this library only MCSPARSE_SPMV_CSR_ALG2 promises that: the other values take the faster
+ * paths that add products in LDS in the order the wavefronts reach them (a transposing call without preprocess,
+ * every call after mcsparseSpMV_preprocess), within the same error bound but not bit for bit the same between runs.
+ * deterministic != 0 makes every mcsparseSpMV, mcsparseSpMV_preprocess(_bufferSize) and mcsparseSpMV_staticBuffer
+ * call of the handle run as MCSPARSE_SPMV_CSR_ALG2, for callers that compare runs and cannot change the `alg` they
+ * pass.  Off by default. */
+mcsparseStatus_t mcsparseSetSpMVDeterministic(mcsparseHandle_t handle, int deterministic);
+mcsparseStatus_t mcsparseGetSpMVDeterministic(const mcsparseHandle_t handle, int* deterministic);
+
+/* How many XCDs (dies with an L2 of their own, which take the workgroups of a launch in turn) the library
+ * assumes behind a device that shows `computeUnits` compute units: computeUnits / 32 where that is a whole
+ * number up to 8 (256 -> 8, 128 -> 4, 64 -> 2, 32 -> 1), else 1, in which case the orders that keep
+ * neighbouring work in one L2 turn into the plain order.  A pure host function; the library asks the device for
+ * its compute units at the first launch that needs them.  For tests. */
+mcsparseStatus_t mcsparseXtopologyOfCuCount(int computeUnits, int* xcds);
+
 /* mcsparseSpMV without an externalBuffer, for callers that cannot allocate device memory: code
  * under HIP graph capture, serving loops and harnesses that forbid hipMalloc.  No counterpart in
  * the reference.  The scratch lives in a device array of MCSPARSE_SPMV_STATIC_BUFFER_BYTES inside
@@ -519,7 +545,9 @@ mcsparseStatus_t mcsparseSpMatSetSpMVBandBytes(mcsparseSpMatDescr_t spMatDescr, 
  * copies nothing to the host: it needs MCSPARSE_POINTER_MODE_HOST (NOT_SUPPORTED otherwise), and a
  * structure that has no SpMV plan yet runs the merge-path family instead of being analysed.
  * Results are those of mcsparseSpMV with the same kernel family.  All calls on one GPU share the
- * array: calls that overlap in time on one GPU (different streams or threads) race. */
+ * array: calls that overlap in time on one GPU (different streams or threads) race.  The first call
+ * on a GPU looks the array's address up, which a stream under graph capture cannot hold: that call
+ * must come before the capture (under capture it returns NOT_SUPPORTED and enqueues nothing). */
 #define MCSPARSE_SPMV_STATIC_BUFFER_BYTES (4u << 20)
 mcsparseStatus_t mcsparseSpMV_staticBuffer(mcsparseHandle_t handle, mcsparseOperation_t opA, const void* alpha,
                                            mcsparseSpMatDescr_t matA, mcsparseDnVecDescr_t vecX, const void* beta,

@@ -56,6 +56,10 @@ PROTOTYPES = {
     "mcsparseDnMatSetStridedBatch": (c_int, [vp, c_int, c_i64]),
     "mcsparseDnMatGetStridedBatch": (c_int, [vp, P(c_int), P(c_i64)]),
     "mcsparseSpMV": (c_int, [vp, c_int, vp, vp, vp, vp, vp, c_int, c_int, vp]),
+    "mcsparseSetSpMVDeterministic": (c_int, [vp, c_int]),
+    "mcsparseGetSpMVDeterministic": (c_int, [vp, P(c_int)]),
+    "mcsparseXstreamProbe": (c_int, [vp, c_int, vp, vp, ctypes.c_size_t, vp, ctypes.c_size_t]),
+    "mcsparseXtopologyOfCuCount": (c_int, [c_int, P(c_int)]),
     "mcsparseSpMV_staticBuffer": (c_int, [vp, c_int, vp, vp, vp, vp, vp, c_int, c_int]),
     "mcsparseSpMV_preprocess_bufferSize": (c_int, [vp, c_int, vp, vp, vp, vp, vp, c_int, c_int, P(c_size)]),
     "mcsparseSpMV_preprocess": (c_int, [vp, c_int, vp, vp, vp, vp, vp, c_int, c_int, vp]),

@@ -95,6 +95,14 @@ class Handle:
     def set_pointer_mode(self, mode):
         check(self.lib.mcsparseSetPointerMode(self._h, mode), "mcsparseSetPointerMode")
 
+    def set_spmv_deterministic(self, on):
+        check(self.lib.mcsparseSetSpMVDeterministic(self._h, 1 if on else 0), "mcsparseSetSpMVDeterministic")
+
+    def spmv_deterministic(self):
+        out = ctypes.c_int(-1)
+        check(self.lib.mcsparseGetSpMVDeterministic(self._h, ctypes.byref(out)), "mcsparseGetSpMVDeterministic")
+        return bool(out.value)
+
     def destroy(self):
         if self._h:
             self.lib.mcsparseDestroy(self._h)
@@ -258,6 +266,14 @@ def spmv_static_buffer(handle, op, alpha, mat, x, beta, y, compute_type):
     a, b = _scalar(alpha, compute_type), _scalar(beta, compute_type)
     return handle.lib.mcsparseSpMV_staticBuffer(handle.ptr, op, ctypes.addressof(a), mat.ptr, x.ptr,
                                                 ctypes.addressof(b), y.ptr, compute_type, SPMV_ALG_DEFAULT)
+
+
+def stream_probe(handle, mode, src, dst, nbytes, sink):
+    """mcsparseXstreamProbe: mode 0 reads src, 1 writes dst, 2 copies (torch tensors; sink: int32/uint32 tensor)."""
+    return handle.lib.mcsparseXstreamProbe(handle.ptr, mode, ctypes.c_void_p(src.data_ptr() if src is not None else 0),
+                                           ctypes.c_void_p(dst.data_ptr() if dst is not None else 0), nbytes,
+                                           ctypes.c_void_p(sink.data_ptr() if sink is not None else 0),
+                                           sink.numel() if sink is not None else 0)
 
 
 def spmm_buffer_size(handle, op_a, op_b, alpha, mat, B, beta, C, compute_type):

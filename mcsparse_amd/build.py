@@ -16,7 +16,7 @@ OBJ_DIR = os.path.join(LIB_DIR, "obj")
 LIB_PATH = os.path.join(LIB_DIR, "libmcsparse.so")
 EXPORTS = os.path.join(CSRC, "exports.map")
 
-SOURCES = ["api_helper.cpp", "api_compute.cpp", "api_legacy.cpp", "api_sort.cpp", "analysis.hip", "spmv.hip",
+SOURCES = ["api_helper.cpp", "api_compute.cpp", "api_legacy.cpp", "api_sort.cpp", "topology.cpp", "analysis.hip", "spmv.hip",
            "spmv_banded.hip", "spmm.hip", "spmm_blocks.hip", "convert.hip", "static_scratch.hip"]
 HEADERS = ["internal.h", "device_util.h", "spmm_device.h"]
 

@@ -323,9 +323,11 @@ mcspStatus_t spmv_typed(mcsparseHandle_t h, mcsparseSpMatDescr* A, mcsparseOpera
         a.row_ptr = nullptr;
         a.col = nullptr;
         a.val = nullptr;
-        mcsp::launch_spmv_banded<T>(h->stream, A->banded.shape, A->banded.grid, a, h_alpha, h_beta,
-                                    buf + A->banded.region);
-        return MCSP_STATUS_SUCCESS;
+        // (a device that refuses the kernel's LDS size launches nothing: an error, not a y left unwritten)
+        return mcsp::launch_spmv_banded<T>(h->stream, A->banded.shape, A->banded.grid, a, h_alpha, h_beta,
+                                           buf + A->banded.region)
+                   ? MCSP_STATUS_SUCCESS
+                   : MCSP_STATUS_INTERNAL_ERROR;
     }
     // A call that does not run from the copy but is handed the copy's buffer may write over it: the copy
     // sits behind the scratch of its own direction only, and the scratch of this call (the other
@@ -386,11 +388,12 @@ mcspStatus_t spmv_typed(mcsparseHandle_t h, mcsparseSpMatDescr* A, mcsparseOpera
             mcsp::launch_csr2coo(h->stream, static_cast<idx_t>(v.m), nnz, v.ptr, base, expanded);
             rows = expanded;
         }
-        mcsp::launch_skinny_transpose<T>(h->stream, static_cast<idx_t>(v.m), static_cast<idx_t>(v.n), nnz, base, rows,
-                                         v.ind, static_cast<const T*>(v.val), static_cast<const T*>(x->values),
-                                         static_cast<T*>(y->values), h_alpha, h_beta,
-                                         ws + align_up(static_cast<size_t>(nnz) * sizeof(idx_t)));
-        return MCSP_STATUS_SUCCESS;
+        return mcsp::launch_skinny_transpose<T>(h->stream, static_cast<idx_t>(v.m), static_cast<idx_t>(v.n), nnz, base, rows,
+                                                v.ind, static_cast<const T*>(v.val), static_cast<const T*>(x->values),
+                                                static_cast<T*>(y->values), h_alpha, h_beta,
+                                                ws + align_up(static_cast<size_t>(nnz) * sizeof(idx_t)))
+                   ? MCSP_STATUS_SUCCESS
+                   : MCSP_STATUS_INTERNAL_ERROR;
     }
     uint32_t bucket_shift = 0;
     if (alg != MCSPARSE_SPMV_CSR_ALG2 &&
@@ -398,9 +401,10 @@ mcspStatus_t spmv_typed(mcsparseHandle_t h, mcsparseSpMatDescr* A, mcsparseOpera
         mcsp::BucketedProducts b;
         mcsp::launch_bucketed_products(h->stream, static_cast<idx_t>(v.m), static_cast<idx_t>(v.n), nnz, v.val, v.ptr,
                                        v.ind, x->values, t_val, sizeof(T), base, buf + l.csr2csc_ws, &b);
-        mcsp::launch_bucket_sums<T>(h->stream, static_cast<idx_t>(v.n), nnz, b, static_cast<const T*>(t_val),
-                                    static_cast<T*>(y->values), h_alpha, h_beta);
-        return MCSP_STATUS_SUCCESS;
+        return mcsp::launch_bucket_sums<T>(h->stream, static_cast<idx_t>(v.n), nnz, b, static_cast<const T*>(t_val),
+                                           static_cast<T*>(y->values), h_alpha, h_beta)
+                   ? MCSP_STATUS_SUCCESS
+                   : MCSP_STATUS_INTERNAL_ERROR;
     }
     mcsp::launch_transposed_products(h->stream, static_cast<idx_t>(v.m), static_cast<idx_t>(v.n), nnz, v.val, v.ptr, v.ind,
                                      x->values, t_val, t_ptr, sizeof(T), base, buf + l.csr2csc_ws);
@@ -659,7 +663,16 @@ void spmv_plan_from_bins(const uint32_t* bins, int64_t m, int64_t nnz, int64_t x
         // Rows longer than a tile of the merge path put whole tiles inside one row; when x is too
         // large to stay in an XCD's L2 next to the streamed matrix, those tiles run in the order of
         // their first column (lanes = 1), which costs two small kernels per call.
-        *lanes = max_row_len >= kMergeTileItems && x_bytes > kMergeOrderMinVectorBytes ? 1 : 0;
+        // That order pays where such rows hold most of the nonzeros (the power-law matrix: two thirds); where a few
+        // long rows sit among many short ones it costs more than it brings (1 M rows of 16 plus 64 rows of 100000:
+        // 155 us against 140 us in storage order).
+        double in_long_rows = 0;
+        for (int b = 1; b < MCSPARSE_ROW_BIN_COUNT; ++b) {
+            const double lower_edge = std::ldexp(1.0, b - 1);
+            if (lower_edge >= kMergeTileItems) in_long_rows += static_cast<double>(bins[b]) * lower_edge;
+        }
+        const bool mostly_long = nnz > 0 && in_long_rows * 2 >= static_cast<double>(nnz);  // lower edges: an underestimate
+        *lanes = max_row_len >= kMergeTileItems && x_bytes > kMergeOrderMinVectorBytes && mostly_long ? 1 : 0;
     } else {
         *family = kFamilyVector;
         *lanes = mean_lanes;
@@ -706,6 +719,7 @@ mcspStatus_t spmv_call(mcsparseHandle_t handle, mcsparseOperation_t opA, const v
     const mcspStatus_t st =
         spmv_check(handle, opA, alpha, matA, vecX, beta, vecY, computeType, buffer, buffer_bytes, may_read_back);
     if (st != MCSP_STATUS_SUCCESS) return st;
+    if (handle->spmv_deterministic) alg = MCSPARSE_SPMV_CSR_ALG2;
     if (computeType == MACA_R_32F)
         return spmv_typed<float>(handle, matA, opA, alpha, beta, vecX, vecY, buffer, may_read_back, alg);
     return spmv_typed<double>(handle, matA, opA, alpha, beta, vecX, vecY, buffer, may_read_back, alg);
@@ -759,6 +773,7 @@ mcsparseStatus_t mcsparseSpMV_preprocess_bufferSize(mcsparseHandle_t handle, mcs
     const mcsparseStatus_t st =
         mcsparseSpMV_bufferSize(handle, opA, alpha, matA, vecX, beta, vecY, computeType, alg, bufferSize);
     if (st != MCSPARSE_STATUS_SUCCESS) return st;
+    if (handle->spmv_deterministic) alg = MCSPARSE_SPMV_CSR_ALG2;
     BandedShape shape;
     if (banded_candidate(matA, opA, alg, &shape)) {
         const size_t vb = value_size(matA->valueType);
@@ -782,6 +797,7 @@ mcsparseStatus_t mcsparseSpMV_preprocess(mcsparseHandle_t handle, mcsparseOperat
     if (st != MCSP_STATUS_SUCCESS) return to_public_status(st);
     matA->banded.valid = false;
     if (stream_is_capturing(handle->stream)) return to_public_status(MCSP_STATUS_NOT_IMPLEMENTED);  // it blocks
+    if (handle->spmv_deterministic) alg = MCSPARSE_SPMV_CSR_ALG2;
     BandedShape shape;
     if (matA->nnz == 0 || !banded_candidate(matA, opA, alg, &shape)) return MCSPARSE_STATUS_SUCCESS;  // nothing to prepare
 
@@ -1152,6 +1168,20 @@ mcsparseStatus_t mcsparseXcsrRowBins(mcsparseHandle_t handle, int m, const int* 
     if (csr_rows == nullptr || bin_hist == nullptr) return to_public_status(MCSP_STATUS_INVALID_POINTER);
     mcsp::launch_row_bins(handle->stream, static_cast<idx_t>(m), reinterpret_cast<const idx_t*>(csr_rows),
                           static_cast<idx_t>(idx_base), row_bins, bin_hist);
+    return MCSPARSE_STATUS_SUCCESS;
+}
+
+// EXTENSION: a measuring stick, not part of the path (see include/mcsparse.h)
+mcsparseStatus_t mcsparseXstreamProbe(mcsparseHandle_t handle, int mode, const void* src, void* dst, size_t bytes,
+                                      uint32_t* sink, size_t sink_words) {
+    if (handle == nullptr) return to_public_status(MCSP_STATUS_INVALID_HANDLE);
+    if (mode < 0 || mode > 2 || bytes % 16 != 0) return to_public_status(MCSP_STATUS_INVALID_VALUE);
+    if ((mode != 1 && src == nullptr) || (mode != 0 && dst == nullptr) || (mode == 0 && sink == nullptr))
+        return to_public_status(MCSP_STATUS_INVALID_POINTER);
+    if (((reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst)) & 15u) != 0)
+        return to_public_status(MCSP_STATUS_INVALID_VALUE);
+    if (mode == 0 && sink_words < mcsp::stream_probe_threads()) return to_public_status(MCSP_STATUS_INVALID_SIZE);
+    mcsp::launch_stream_probe(handle->stream, mode, src, dst, bytes, sink);
     return MCSPARSE_STATUS_SUCCESS;
 }
 

@@ -170,6 +170,22 @@ mcsparseStatus_t mcsparseGetPointerMode(const mcsparseHandle_t handle, mcsparseP
     return MCSPARSE_STATUS_SUCCESS;
 }
 
+// EXTENSION.  The reference's SpMV adds every row in a fixed order (csr_vector_device.hpp:40-75), so two runs give
+// the same bits whatever `alg` says.  Here only MCSPARSE_SPMV_CSR_ALG2 promises that; with this switch on, every
+// mcsparseSpMV / mcsparseSpMV_preprocess / mcsparseSpMV_staticBuffer call of the handle runs as that algorithm.
+mcsparseStatus_t mcsparseSetSpMVDeterministic(mcsparseHandle_t handle, int deterministic) {
+    if (handle == nullptr) return to_public_status(MCSP_STATUS_INVALID_HANDLE);
+    handle->spmv_deterministic = deterministic != 0;
+    return MCSPARSE_STATUS_SUCCESS;
+}
+
+mcsparseStatus_t mcsparseGetSpMVDeterministic(const mcsparseHandle_t handle, int* deterministic) {
+    if (handle == nullptr) return to_public_status(MCSP_STATUS_INVALID_HANDLE);
+    if (deterministic == nullptr) return to_public_status(MCSP_STATUS_INVALID_POINTER);
+    *deterministic = handle->spmv_deterministic ? 1 : 0;
+    return MCSPARSE_STATUS_SUCCESS;
+}
+
 // ---- dense vector: src/common/mcsp_helper.cpp:325-387 ------------------------------------
 
 mcsparseStatus_t mcsparseCreateDnVec(mcsparseDnVecDescr_t* dnVecDescr, int64_t size, void* values,

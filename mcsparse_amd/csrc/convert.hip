@@ -465,7 +465,6 @@ constexpr int kSortTile = kSortBlock * kSortIpt;       // 4096 triples per workg
 constexpr int kSortWaves = kSortBlock / kWave;         // 16
 constexpr int kSortWaveItems = kWave * kSortIpt;       // each wave owns 256 consecutive triples
 constexpr int kMaxRadix = 256;
-constexpr uint32_t kXcds = 8;                          // accelerator complex dies of an MI355X
 static_assert(kSortBlock >= kMaxRadix, "one thread per digit");
 
 // counters[digit * tiles + tile] = how many keys of `tile` carry `digit` (the digit of key - bias).  256 threads, 16 keys
@@ -473,15 +472,16 @@ static_assert(kSortBlock >= kMaxRadix, "one thread per digit");
 constexpr int kHistBlock = 256;
 __global__ __launch_bounds__(kHistBlock) void radix_hist_kernel(const idx_t* __restrict__ keys, idx_t count,
                                                                 uint32_t shift, uint32_t bits, uint32_t tiles,
-                                                                uint32_t* __restrict__ counters, idx_t bias) {
+                                                                uint32_t* __restrict__ counters, idx_t bias,
+                                                                uint32_t xcds) {
     typedef idx_t idx4 __attribute__((ext_vector_type(4)));
     __shared__ uint32_t s_cnt[kMaxRadix];
     const uint32_t radix = 1u << bits;
     const uint32_t mask = radix - 1;
     // The same tile order as the scatter kernel below: an XCD counts a contiguous range of tiles,
     // so the sixteen neighbouring tiles whose counters share a cache line write it in one L2.
-    const uint32_t tiles_per_xcd = (tiles + kXcds - 1) / kXcds;
-    const uint32_t tile = (blockIdx.x % kXcds) * tiles_per_xcd + blockIdx.x / kXcds;
+    const uint32_t tiles_per_xcd = (tiles + xcds - 1) / xcds;
+    const uint32_t tile = (blockIdx.x % xcds) * tiles_per_xcd + blockIdx.x / xcds;
     if (tile >= tiles) return;  // whole workgroup
     s_cnt[threadIdx.x] = 0;
     __syncthreads();
@@ -569,7 +569,8 @@ __global__ __launch_bounds__(kSortBlock) void radix_scatter_kernel(
     const idx_t* __restrict__ keys_in, const idx_t* __restrict__ rows_in, const void* __restrict__ vals_in_v,
     idx_t* __restrict__ keys_out, idx_t* __restrict__ rows_out, void* __restrict__ vals_out_v, idx_t count,
     uint32_t shift, uint32_t bits, uint32_t tiles, const uint32_t* __restrict__ counters,
-    const idx_t* __restrict__ tile_rows, idx_t base, const void* __restrict__ x_v, bool short_keys, idx_t bias) {
+    const idx_t* __restrict__ tile_rows, idx_t base, const void* __restrict__ x_v, bool short_keys, idx_t bias,
+    uint32_t xcds) {
     static_assert(AUX || VB != 0, "pairs carry a value");
     static_assert(!TIMES_X || (FROM_CSR && !AUX), "products are formed where the rows are worked out");
     typedef typename ValueOf<VB>::type val_t;
@@ -594,11 +595,11 @@ __global__ __launch_bounds__(kSortBlock) void radix_scatter_kernel(
     const unsigned wave = tid / kWave;
     const uint32_t radix = 1u << bits;
     const uint32_t mask = radix - 1;
-    // Workgroups are handed to the 8 XCDs round-robin.  Tile t+1 appends to the digit runs tile t
+    // Workgroups are handed to the device's XCDs in turn.  Tile t+1 appends to the digit runs tile t
     // started, so each XCD walks a contiguous range of tiles: the partial cache lines at the run
     // ends then meet in one L2 and leave as full lines.
-    const uint32_t tiles_per_xcd = (tiles + kXcds - 1) / kXcds;
-    const uint32_t tile = (blockIdx.x % kXcds) * tiles_per_xcd + blockIdx.x / kXcds;
+    const uint32_t tiles_per_xcd = (tiles + xcds - 1) / xcds;
+    const uint32_t tile = (blockIdx.x % xcds) * tiles_per_xcd + blockIdx.x / xcds;
     if (tile >= tiles) return;  // whole workgroup
     const uint64_t tile_start = static_cast<uint64_t>(tile) * kSortTile;
     const uint32_t tile_count =
@@ -830,30 +831,30 @@ template <int VB>
 void launch_scatter(hipStream_t stream, bool from_csr, uint32_t grid, const idx_t* keys_in, const idx_t* aux_in,
                     const void* vals_in, idx_t* keys_out, idx_t* aux_out, void* vals_out, idx_t count, uint32_t shift,
                     uint32_t bits, uint32_t tiles, const uint32_t* counters, const idx_t* tile_rows, idx_t base,
-                    bool pairs, const void* x, bool short_keys, idx_t bias) {
+                    bool pairs, const void* x, bool short_keys, idx_t bias, uint32_t xcds) {
     const void* none = nullptr;
     if constexpr (VB != 0) {
         if (pairs && from_csr) {
             hipLaunchKernelGGL((radix_scatter_kernel<VB, true, false, true>), dim3(grid), dim3(kSortBlock), 0, stream, keys_in,
                                aux_in, vals_in, keys_out, aux_out, vals_out, count, shift, bits, tiles, counters, tile_rows,
-                               base, x, short_keys, bias);
+                               base, x, short_keys, bias, xcds);
             return;
         }
         if (pairs) {
             hipLaunchKernelGGL((radix_scatter_kernel<VB, false, false, false>), dim3(grid), dim3(kSortBlock), 0, stream, keys_in,
                                aux_in, vals_in, keys_out, aux_out, vals_out, count, shift, bits, tiles, counters, tile_rows,
-                               base, none, false, bias);
+                               base, none, false, bias, xcds);
             return;
         }
     }
     if (from_csr) {
         hipLaunchKernelGGL((radix_scatter_kernel<VB, true, true, false>), dim3(grid), dim3(kSortBlock), 0, stream, keys_in,
                            aux_in, vals_in, keys_out, aux_out, vals_out, count, shift, bits, tiles, counters, tile_rows, base,
-                           none, false, bias);
+                           none, false, bias, xcds);
     } else {
         hipLaunchKernelGGL((radix_scatter_kernel<VB, false, true, false>), dim3(grid), dim3(kSortBlock), 0, stream, keys_in,
                            aux_in, vals_in, keys_out, aux_out, vals_out, count, shift, bits, tiles, counters, tile_rows, base,
-                           none, false, bias);
+                           none, false, bias, xcds);
     }
 }
 
@@ -884,7 +885,8 @@ void radix_sort_triples(hipStream_t stream, idx_t count, uint32_t key_bits, cons
     const uint32_t bits = key_bits == 0 ? 1 : (key_bits + passes - 1) / passes;
     const uint32_t radix = 1u << bits;
     const uint32_t tiles = sort_tiles(count);
-    const uint32_t scatter_grid = (tiles + kXcds - 1) / kXcds * kXcds;
+    const uint32_t xcds = device_topology().xcds;
+    const uint32_t scatter_grid = (tiles + xcds - 1) / xcds * xcds;
     uint32_t shift = csr.first_bit;
     if (csr.rows > 0) {
         const uint32_t waves_per_block = kBlock / kWave;
@@ -898,12 +900,12 @@ void radix_sort_triples(hipStream_t stream, idx_t count, uint32_t key_bits, cons
         idx_t* a_out = last ? aux_out : t.aux[p & 1];
         void* v_out = last ? vals_out : t.vals[p & 1];
         hipLaunchKernelGGL(radix_hist_kernel, dim3(scatter_grid), dim3(kHistBlock), 0, stream, keys_in, count, shift, bits,
-                           tiles, t.counters, csr.bias);
+                           tiles, t.counters, csr.bias, xcds);
         launch_exclusive_scan(stream, t.counters, static_cast<uint64_t>(radix) * tiles, t.scan_ws);
         auto* launch = value_bytes == 0 ? launch_scatter<0> : value_bytes == 4 ? launch_scatter<4> : launch_scatter<8>;
         launch(stream, from_csr, scatter_grid, keys_in, aux_in, vals_in, k_out, a_out, v_out, count, shift, bits, tiles,
                t.counters, t.tile_rows, csr.base, csr.times_x != nullptr, csr.times_x,
-               csr.short_keys && last && from_csr, csr.bias);
+               csr.short_keys && last && from_csr, csr.bias, xcds);
         keys_in = k_out;
         aux_in = a_out;
         vals_in = v_out;

@@ -21,6 +21,8 @@ static constexpr inline size_t align_up(size_t n, size_t a = kAlign) { return (n
 struct mcsparseContext {
     hipStream_t stream = nullptr;
     mcsparsePointerMode_t ptr_mode = MCSPARSE_POINTER_MODE_HOST;
+    // mcsparseSetSpMVDeterministic: every SpMV call of this handle is treated as MCSPARSE_SPMV_CSR_ALG2
+    bool spmv_deterministic = false;
 };
 
 // reference: src/include/mcsp_internal_types.h:86-94
@@ -166,6 +168,27 @@ struct mcsparseSpMatDescr {
     SpmvBanded banded;
 };
 
+// How many compute units the current device shows and how many XCDs (L2 domains that take the workgroups of a
+// launch in turn) they make up: topology.cpp.
+namespace mcsp {
+constexpr uint32_t kMaxXcds = 8;
+struct Topology {
+    uint32_t cus = 256;
+    uint32_t xcds = 8;
+};
+Topology topology_of_cu_count(int cus);
+Topology device_topology();
+}  // namespace mcsp
+
+// The kernels that ask for more dynamic LDS than the default limit: raises the limit for `kernel`; false when the
+// device refuses (another LDS size), in which case the launcher launches nothing and its caller reports
+// MCSP_STATUS_INTERNAL_ERROR instead of returning success with the output unwritten.
+inline bool allow_dynamic_lds(const void* kernel, size_t bytes) {
+    return hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(bytes)) == hipSuccess;
+}
+// After the launches of a path that raised an LDS limit: whether the runtime took them.
+inline bool launches_taken() { return hipGetLastError() == hipSuccess; }
+
 // Internal status, mapped to the public one exactly as the reference's wrapper does
 // (src/include/mcsp_internal_types.h:13-30, src/wrapper/mcsp_interface_wrapper.cpp:5-42).
 enum mcspStatus_t {
@@ -307,8 +330,13 @@ void launch_banded_build(hipStream_t stream, const BandedShape& s, idx_t m, idx_
                          const idx_t* col, const void* val, size_t value_bytes, void* region);
 uint32_t banded_grid(const uint32_t* xcd_start_host);
 template <typename T>
-void launch_spmv_banded(hipStream_t stream, const BandedShape& s, uint32_t grid, const SpmvArgs& a, T alpha, T beta,
+bool launch_spmv_banded(hipStream_t stream, const BandedShape& s, uint32_t grid, const SpmvArgs& a, T alpha, T beta,
                         void* region);
+
+// Streaming kernels that measure what the memory takes by itself (analysis.hip): mode 0 reads src, 1 writes dst,
+// 2 copies; bytes a multiple of 16, arrays 16-byte aligned, sink = stream_probe_threads() uint32 for mode 0.
+uint32_t stream_probe_threads();
+void launch_stream_probe(hipStream_t stream, int mode, const void* src, void* dst, uint64_t bytes, uint32_t* sink);
 
 // ---- SpMM (spmm.hip) ----
 struct SpmmArgs {
@@ -425,7 +453,7 @@ void launch_bucketed_products(hipStream_t stream, idx_t m, idx_t n, idx_t nnz, c
 // y[c] = alpha * (sum of the products of column c) + beta * y[c] for all n columns, from such buckets;
 // the sums are formed in LDS in the order the wavefronts reach the products.
 template <typename T>
-void launch_bucket_sums(hipStream_t stream, idx_t n, idx_t nnz, const BucketedProducts& b, const T* products, T* y,
+bool launch_bucket_sums(hipStream_t stream, idx_t n, idx_t nnz, const BucketedProducts& b, const T* products, T* y,
                         T alpha, T beta);
 
 // y = alpha * A^T x + beta * y for an m x n matrix with at most 2^14 columns and many nonzeros per
@@ -436,7 +464,7 @@ constexpr uint32_t kSkinnyMinNonzerosPerColumn = 128;
 bool skinny_transpose_shape(idx_t n, idx_t nnz);
 size_t skinny_transpose_workspace_bytes(idx_t n);
 template <typename T>
-void launch_skinny_transpose(hipStream_t stream, idx_t m, idx_t n, idx_t nnz, idx_t base, const idx_t* rows,
+bool launch_skinny_transpose(hipStream_t stream, idx_t m, idx_t n, idx_t nnz, idx_t base, const idx_t* rows,
                              const idx_t* col, const T* val, const T* x, T* y, T alpha, T beta, void* workspace);
 
 // One stable radix pass over the nonzeros of a CSR matrix where they lie, on band_bits (<= 8) bits

@@ -460,7 +460,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(LR <= 16
                                                             const uint32_t* __restrict__ entries,
                                                             const T* __restrict__ B, int64_t ldb, T* __restrict__ C,
                                                             int64_t ldc, bool c_row_major, T alpha, T beta,
-                                                            uint32_t xcd_chunk, idx_t k, idx_t nnz,
+                                                            uint32_t xcd_chunk, uint32_t xcds, idx_t k, idx_t nnz,
                                                             uint32_t total_entries) {
     typedef typename ByteOffset<WIDE>::type off_t;
     constexpr int V = 16 / sizeof(T);
@@ -470,7 +470,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(LR <= 16
     constexpr bool kAlternate = LR < kWave;
     constexpr int kBatch = kAlternate ? 2 : 8;
     const idx_t lane = threadIdx.x % LR;
-    const uint64_t group = xcd_position(blockIdx.x, xcd_chunk) * kGroupsPerBlock + threadIdx.x / LR;
+    const uint64_t group = xcd_position(blockIdx.x, xcd_chunk, xcds) * kGroupsPerBlock + threadIdx.x / LR;
     const uint64_t r0 = group * R;
     if (r0 >= static_cast<uint64_t>(m)) return;  // whole lane groups
     const uint64_t c_own = (static_cast<uint64_t>(blockIdx.y) * LR + lane) * V;
@@ -626,22 +626,23 @@ void launch_group(hipStream_t stream, const SpmmArgs& a, const uint32_t* group_p
     // a stencil) in its own L2 -- as long as such a stretch of op(B) is small against the 4 MB of
     // an L2; beyond that the plain round-robin does as well.
     constexpr uint64_t kRowsPerBlock = static_cast<uint64_t>(kBlock / LR) * R;
+    const uint32_t xcds = device_topology().xcds;
     uint32_t xcd_chunk = 1;
     const uint64_t stretch_rows = mean_span / 16;
     if (stretch_rows * a.n * sizeof(T) <= (1u << 20)) {
         while (static_cast<uint64_t>(xcd_chunk) * 2 * kRowsPerBlock <= stretch_rows) xcd_chunk *= 2;
     }
-    const dim3 grid(xcd_padded_grid(group_blocks, xcd_chunk), static_cast<uint32_t>(panels));
+    const dim3 grid(xcd_padded_grid(group_blocks, xcd_chunk, xcds), static_cast<uint32_t>(panels));
     const T* val = static_cast<const T*>(a.val);
     const T* B = static_cast<const T*>(a.B);
     T* C = static_cast<T*>(a.C);
     if (narrow_offsets(a, sizeof(T))) {
         hipLaunchKernelGGL((spmm_group_kernel<T, LR, false>), grid, dim3(kBlock), 0, stream, a.m, a.n, a.base, a.row_ptr,
-                           a.col, val, group_ptr, entries, B, a.ldb, C, a.ldc, a.c_row_major, alpha, beta, xcd_chunk, a.k,
+                           a.col, val, group_ptr, entries, B, a.ldb, C, a.ldc, a.c_row_major, alpha, beta, xcd_chunk, xcds, a.k,
                            a.nnz, total_entries);
     } else {
         hipLaunchKernelGGL((spmm_group_kernel<T, LR, true>), grid, dim3(kBlock), 0, stream, a.m, a.n, a.base, a.row_ptr,
-                           a.col, val, group_ptr, entries, B, a.ldb, C, a.ldc, a.c_row_major, alpha, beta, xcd_chunk, a.k,
+                           a.col, val, group_ptr, entries, B, a.ldb, C, a.ldc, a.c_row_major, alpha, beta, xcd_chunk, xcds, a.k,
                            a.nnz, total_entries);
     }
 }

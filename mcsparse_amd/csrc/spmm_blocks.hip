@@ -228,7 +228,7 @@ __global__ __launch_bounds__(kBlock) void spmm_blocks_kernel(idx_t m, idx_t n, i
                                                              const uint2* __restrict__ blocks,
                                                              const uint32_t* __restrict__ order, const T* __restrict__ B,
                                                              int64_t ldb, T* __restrict__ C, int64_t ldc,
-                                                             bool c_row_major, T alpha, T beta, uint32_t xcd_chunk,
+                                                             bool c_row_major, T alpha, T beta, uint32_t xcd_chunk, uint32_t xcds,
                                                              idx_t k, idx_t nnz, uint32_t total_blocks) {
     typedef typename ByteOffset<WIDE>::type off_t;
     constexpr int V = 16 / sizeof(T);
@@ -237,7 +237,7 @@ __global__ __launch_bounds__(kBlock) void spmm_blocks_kernel(idx_t m, idx_t n, i
     constexpr int kValuesPerLane = (D + kLanesPerRow - 1) / kLanesPerRow;
     static_assert(LR >= K && LR % K == 0, "a lane group fetches the values of its K rows in one go");
     const idx_t lane = threadIdx.x % LR;
-    const uint64_t turn = xcd_position(blockIdx.x, xcd_chunk) * kGroupsPerBlock + threadIdx.x / LR;
+    const uint64_t turn = xcd_position(blockIdx.x, xcd_chunk, xcds) * kGroupsPerBlock + threadIdx.x / LR;
     const uint64_t groups = spmm_block_groups(m);
     if (turn >= groups) return;  // whole lane groups
     // which group takes this turn (held to the groups that exist, whatever the buffer holds)
@@ -503,12 +503,13 @@ void launch_blocks(hipStream_t stream, const SpmmArgs& a, const uint32_t* block_
     // neighbouring stretches share (the neighbouring grid lines of a stencil) stay in its own L2, as long as
     // such a stretch of op(B) is small against the 4 MB of an L2.
     constexpr uint64_t kRowsPerBlock = static_cast<uint64_t>(kBlock / LR) * K;
+    const uint32_t xcds = device_topology().xcds;
     uint32_t xcd_chunk = 1;
     const uint64_t stretch_rows = mean_span / 16;
     if (stretch_rows * a.n * sizeof(T) <= (1u << 20)) {
         while (static_cast<uint64_t>(xcd_chunk) * 2 * kRowsPerBlock <= stretch_rows) xcd_chunk *= 2;
     }
-    const dim3 grid(xcd_padded_grid(group_blocks, xcd_chunk), static_cast<uint32_t>(panels));
+    const dim3 grid(xcd_padded_grid(group_blocks, xcd_chunk, xcds), static_cast<uint32_t>(panels));
     const T* val = static_cast<const T*>(a.val);
     const T* B = static_cast<const T*>(a.B);
     T* C = static_cast<T*>(a.C);
@@ -518,7 +519,7 @@ void launch_blocks(hipStream_t stream, const SpmmArgs& a, const uint32_t* block_
     auto launch = [&](auto wide_c, auto staged_c) {
         hipLaunchKernelGGL((spmm_blocks_kernel<T, LR, decltype(wide_c)::value, decltype(staged_c)::value>), grid, dim3(kBlock),
                            0, stream, a.m, a.n, a.base, a.row_ptr, a.col, val, block_ptr, blocks, order, B, a.ldb, C, a.ldc,
-                           a.c_row_major, alpha, beta, xcd_chunk, a.k, a.nnz, total_blocks);
+                           a.c_row_major, alpha, beta, xcd_chunk, xcds, a.k, a.nnz, total_blocks);
     };
     if (narrow_offsets(a, sizeof(T))) {
         if (staged) launch(std::false_type{}, std::true_type{});

@@ -60,20 +60,19 @@ struct ByteOffset { typedef uint32_t type; };
 template <>
 struct ByteOffset<true> { typedef uint64_t type; };
 
-// Workgroups are handed to the 8 XCDs round-robin (workgroup h runs on XCD h % 8), each XCD with
+// Workgroups are handed to the XCDs of a device in turn (workgroup h runs on XCD h % xcds), each XCD with
 // an L2 of its own.  Rows that are close in the matrix tend to read the same rows of op(B), so
 // an XCD should work on a contiguous stretch of rows: this maps the hardware's workgroup number
-// to a position such that every XCD takes `chunk` consecutive positions at a time.  chunk = 1
+// to a position such that every XCD takes `chunk` consecutive positions at a time.  chunk = 1 (or one XCD)
 // is the identity; positions past `count` (the grid is padded to whole rounds) do no work.
-constexpr uint32_t kXcds = 8;
-__device__ __forceinline__ uint64_t xcd_position(uint32_t hw_block, uint32_t chunk) {
-    const uint32_t per_round = kXcds * chunk;
+__device__ __forceinline__ uint64_t xcd_position(uint32_t hw_block, uint32_t chunk, uint32_t xcds) {
+    const uint32_t per_round = xcds * chunk;
     const uint32_t round = hw_block / per_round;
     const uint32_t rem = hw_block % per_round;
-    return static_cast<uint64_t>(round) * per_round + (rem % kXcds) * chunk + rem / kXcds;
+    return static_cast<uint64_t>(round) * per_round + (rem % xcds) * chunk + rem / xcds;
 }
-inline uint32_t xcd_padded_grid(uint64_t count, uint32_t chunk) {
-    const uint64_t per_round = static_cast<uint64_t>(kXcds) * chunk;
+inline uint32_t xcd_padded_grid(uint64_t count, uint32_t chunk, uint32_t xcds) {
+    const uint64_t per_round = static_cast<uint64_t>(xcds) * chunk;
     return static_cast<uint32_t>((count + per_round - 1) / per_round * per_round);
 }
 

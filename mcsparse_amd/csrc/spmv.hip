@@ -790,9 +790,9 @@ __global__ __launch_bounds__(kBlock) void bucket_merge_kernel(idx_t n, idx_t nnz
 }
 
 template <typename T>
-void launch_bucket_sums(hipStream_t stream, idx_t n, idx_t nnz, const BucketedProducts& b, const T* products, T* y,
+bool launch_bucket_sums(hipStream_t stream, idx_t n, idx_t nnz, const BucketedProducts& b, const T* products, T* y,
                         T alpha, T beta) {
-    if (b.buckets == 0 || b.buckets > kBucketDigits || b.shift > kBucketMaxShift) return;
+    if (b.buckets == 0 || b.buckets > kBucketDigits || b.shift > kBucketMaxShift) return false;
     const size_t lds = sizeof(double) << b.shift;
     // A bucket with more than twice `share` pairs is dealt to several workgroups, ceil(count / share) of them.  share
     // is the mean of a bucket, so that at most 256 further workgroups are needed, or more where the spare scratch is
@@ -808,8 +808,7 @@ void launch_bucket_sums(hipStream_t stream, idx_t n, idx_t nnz, const BucketedPr
         share = nnz;  // no bucket holds more
     }
     double* planes = static_cast<double*>(b.spare);
-    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(bucket_sums_kernel<T>),
-                              hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
+    if (!allow_dynamic_lds(reinterpret_cast<const void*>(bucket_sums_kernel<T>), lds)) return false;
     hipLaunchKernelGGL((bucket_sums_kernel<T>), dim3(split ? 2 * kBucketDigits : b.buckets), dim3(kBucketBlock), lds, stream,
                        n, nnz, b.shift, b.stride, b.buckets, static_cast<uint32_t>(share), b.starts, b.keys, products, y,
                        planes, alpha, beta);
@@ -818,11 +817,12 @@ void launch_bucket_sums(hipStream_t stream, idx_t n, idx_t nnz, const BucketedPr
                            nnz, b.shift, b.stride, b.buckets, static_cast<uint32_t>(share), b.starts,
                            static_cast<const double*>(planes), y, alpha, beta);
     }
+    return launches_taken();
 }
 
-template void launch_bucket_sums<float>(hipStream_t, idx_t, idx_t, const BucketedProducts&, const float*, float*, float,
+template bool launch_bucket_sums<float>(hipStream_t, idx_t, idx_t, const BucketedProducts&, const float*, float*, float,
                                         float);
-template void launch_bucket_sums<double>(hipStream_t, idx_t, idx_t, const BucketedProducts&, const double*, double*,
+template bool launch_bucket_sums<double>(hipStream_t, idx_t, idx_t, const BucketedProducts&, const double*, double*,
                                          double, double);
 // ---- A^T x for a matrix with few columns ----
 // With at most 2^14 columns all of y fits in the LDS of one workgroup, so nothing is sorted: each
@@ -901,22 +901,22 @@ size_t skinny_transpose_workspace_bytes(idx_t n) {
 }
 
 template <typename T>
-void launch_skinny_transpose(hipStream_t stream, idx_t m, idx_t n, idx_t nnz, idx_t base, const idx_t* rows,
+bool launch_skinny_transpose(hipStream_t stream, idx_t m, idx_t n, idx_t nnz, idx_t base, const idx_t* rows,
                              const idx_t* col, const T* val, const T* x, T* y, T alpha, T beta, void* workspace) {
-    if (m == 0 || n == 0 || nnz == 0) return;
+    if (m == 0 || n == 0 || nnz == 0) return true;
     double* planes = static_cast<double*>(workspace);
     const size_t lds = static_cast<size_t>(n) * sizeof(double);
-    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(skinny_products_kernel<T>),
-                              hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
+    if (!allow_dynamic_lds(reinterpret_cast<const void*>(skinny_products_kernel<T>), lds)) return false;
     hipLaunchKernelGGL((skinny_products_kernel<T>), dim3(kSkinnyGroups), dim3(kSkinnyBlock), lds, stream, m, n, nnz, base,
                        rows, col, val, x, planes);
     hipLaunchKernelGGL((skinny_reduce_kernel<T>), dim3((n + kBlock - 1) / kBlock), dim3(kBlock), 0, stream, n,
                        static_cast<const double*>(planes), y, alpha, beta);
+    return launches_taken();
 }
 
-template void launch_skinny_transpose<float>(hipStream_t, idx_t, idx_t, idx_t, idx_t, const idx_t*, const idx_t*,
+template bool launch_skinny_transpose<float>(hipStream_t, idx_t, idx_t, idx_t, idx_t, const idx_t*, const idx_t*,
                                              const float*, const float*, float*, float, float, void*);
-template void launch_skinny_transpose<double>(hipStream_t, idx_t, idx_t, idx_t, idx_t, const idx_t*, const idx_t*,
+template bool launch_skinny_transpose<double>(hipStream_t, idx_t, idx_t, idx_t, idx_t, const idx_t*, const idx_t*,
                                               const double*, const double*, double*, double, double, void*);
 
 template void launch_row_sums_merge<float>(hipStream_t, const SpmvArgs&, float, float, void*);

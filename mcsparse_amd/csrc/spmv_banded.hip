@@ -34,8 +34,12 @@ constexpr int kBlock = 256;
 constexpr int kIpt = 16;
 constexpr int kSlab = kBlock * kIpt;  // entries a workgroup stages at a time
 constexpr int kRowsPerThread = kBandedMaxRowsPerTile / kBlock;
-constexpr uint32_t kXcds = 8;  // accelerator complex dies of an MI355X; workgroup i runs on XCD i % 8
-constexpr uint32_t kColumnGroupsPerXcd = 32;  // workgroups per XCD of the kernel on tiles in column order: one per CU
+// The list of tiles (units) of a copy is cut into this many stretches, and workgroup i works on stretch i % 8: the
+// eight XCDs of a whole MI355X, which take the workgroups of a launch in turn, so that one L2 holds one stretch's
+// band of x.  It is part of the copy's layout, not read from the device: on a device with fewer XCDs (a partition)
+// several stretches share an L2, which costs hit rate and nothing else.
+constexpr uint32_t kXcds = 8;
+constexpr uint32_t kColumnGroupsPerXcd = 32;  // workgroups per stretch of the kernel on tiles in column order (one per CU of an XCD)
 static_assert(kBandedMaxRowsPerTile % kBlock == 0, "rows of a tile are dealt to the threads in rounds");
 static_assert(kSlab <= 65536 && kBandedMaxRowsPerTile <= 65536, "16-bit positions in LDS");
 
@@ -911,9 +915,9 @@ uint32_t banded_grid(const uint32_t* xcd_start_host) {
 }
 
 template <typename T>
-void launch_spmv_banded(hipStream_t stream, const BandedShape& s, uint32_t grid, const SpmvArgs& a, T alpha, T beta,
+bool launch_spmv_banded(hipStream_t stream, const BandedShape& s, uint32_t grid, const SpmvArgs& a, T alpha, T beta,
                         void* region) {
-    if (a.m == 0) return;
+    if (a.m == 0) return true;
     const BandedLayout l = banded_layout(s, a.m, a.nnz, sizeof(T));
     char* w = static_cast<char*>(region);
     T* partials = reinterpret_cast<T*>(w + l.partials);
@@ -927,14 +931,14 @@ void launch_spmv_banded(hipStream_t stream, const BandedShape& s, uint32_t grid,
                                                 : spmv_column_order_kernel<T, false, true>)
                               : (s.crowded_rows ? spmv_column_order_kernel<T, true, false>
                                                 : spmv_column_order_kernel<T, false, false>);
-        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+        if (!allow_dynamic_lds(reinterpret_cast<const void*>(kernel), lds)) return false;
         hipLaunchKernelGGL(kernel, dim3(kColumnGroupsPerXcd * kXcds), dim3(kColumnBlock), lds, stream, a.m, a.n, a.nnz,
                            a.base, s.band_shift, s.rows_per_tile, s.chunks, s.tiles / s.sub, s.sub,
                            stretches, reinterpret_cast<uint32_t*>(w + l.next_unit),
                            reinterpret_cast<const idx_t*>(w + l.tile_ptr), reinterpret_cast<const idx_t*>(w + l.entries),
                            reinterpret_cast<const T*>(w + l.vals), static_cast<const T*>(a.x), partials,
                            static_cast<T*>(a.y), alpha, beta);
-        if (direct) return;
+        if (direct) return launches_taken();
     } else if (grid != 0) {
         hipLaunchKernelGGL((spmv_banded_kernel<T>), dim3(grid), dim3(kBlock), 0, stream, a.m, a.n, a.nnz, a.base,
                            s.band_shift, s.rows_per_tile, s.chunks, s.tiles,
@@ -955,7 +959,7 @@ void launch_spmv_banded(hipStream_t stream, const BandedShape& s, uint32_t grid,
             hipLaunchKernelGGL((banded_reduce_wide_kernel<T, false>), wide_grid, dim3(kBlock), 0, stream, a.m, s.bands,
                                static_cast<const T*>(partials), static_cast<T*>(a.y), alpha, beta, next_unit);
         }
-        return;
+        return launches_taken();
     }
     const dim3 rows_grid((a.m + kBlock - 1) / kBlock);
     if (beta == T(0)) {
@@ -965,9 +969,10 @@ void launch_spmv_banded(hipStream_t stream, const BandedShape& s, uint32_t grid,
         hipLaunchKernelGGL((banded_reduce_kernel<T, false>), rows_grid, dim3(kBlock), 0, stream, a.m, s.bands,
                            static_cast<const T*>(partials), static_cast<T*>(a.y), alpha, beta, next_unit);
     }
+    return launches_taken();
 }
 
-template void launch_spmv_banded<float>(hipStream_t, const BandedShape&, uint32_t, const SpmvArgs&, float, float, void*);
-template void launch_spmv_banded<double>(hipStream_t, const BandedShape&, uint32_t, const SpmvArgs&, double, double, void*);
+template bool launch_spmv_banded<float>(hipStream_t, const BandedShape&, uint32_t, const SpmvArgs&, float, float, void*);
+template bool launch_spmv_banded<double>(hipStream_t, const BandedShape&, uint32_t, const SpmvArgs&, double, double, void*);
 
 }  // namespace mcsp

@@ -20,14 +20,19 @@ static __device__ __align__(256) unsigned char scratch[kScratchBytes];
 std::mutex g_lock;
 void* g_scratch_of_device[kMaxDevices] = {nullptr};
 
-// Address of the current device's copy of `scratch`, looked up once per device.
-hipError_t scratch_of_current_device(void** out) {
+// Address of the current device's copy of `scratch`, looked up once per device.  The lookup may load the
+// library's code object, which is not stream work: while `stream` is being captured into a graph it is not
+// attempted (hipErrorStreamCaptureUnsupported), so the first call on a device must come before the capture.
+hipError_t scratch_of_current_device(hipStream_t stream, void** out) {
     int device = -1;
     hipError_t err = hipGetDevice(&device);
     if (err != hipSuccess) return err;
     if (device < 0 || device >= kMaxDevices) return hipErrorInvalidDevice;
     std::lock_guard<std::mutex> guard(g_lock);
     if (g_scratch_of_device[device] == nullptr) {
+        hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(stream, &capturing) != hipSuccess || capturing != hipStreamCaptureStatusNone)
+            return hipErrorStreamCaptureUnsupported;
         void* ptr = nullptr;
         err = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
         if (err != hipSuccess) return err;
@@ -54,7 +59,10 @@ mcsparseStatus_t mcsparseSpMV_staticBuffer(mcsparseHandle_t handle, mcsparseOper
         mcsp::spmv_check(handle, opA, alpha, matA, vecX, beta, vecY, computeType, &placeholder, kScratchBytes, false);
     if (st != MCSP_STATUS_SUCCESS) return to_public_status(st);
     void* buffer = nullptr;
-    if (scratch_of_current_device(&buffer) != hipSuccess) return to_public_status(MCSP_STATUS_INTERNAL_ERROR);
+    const hipError_t found = scratch_of_current_device(handle->stream, &buffer);
+    // the first call on a device under graph capture: NOT_SUPPORTED, as for everything a capture cannot hold
+    if (found == hipErrorStreamCaptureUnsupported) return to_public_status(MCSP_STATUS_NOT_IMPLEMENTED);
+    if (found != hipSuccess) return to_public_status(MCSP_STATUS_INTERNAL_ERROR);
     return to_public_status(
         mcsp::spmv_call(handle, opA, alpha, matA, vecX, beta, vecY, computeType, buffer, kScratchBytes, false, alg));
 }

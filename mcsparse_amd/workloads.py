@@ -63,6 +63,28 @@ def uniform_rows(m=1 << 20, n=None, per_row=16, dtype=np.float64, base=0, config
     return Csr(m, n, ptr + base, col.reshape(-1) + base, val, base)
 
 
+def mixed_rows(m=1 << 20, n=None, per_row=16, long_rows=64, long_len=100_000, dtype=np.float32, base=0, config_id=6):
+    """Mostly short rows plus a handful of very long ones, spread evenly over the matrix: what a row-length-binned
+    dispatch is for.  Short rows as in uniform_rows; a long row holds long_len distinct sorted columns."""
+    n = m if n is None else n
+    rng = _rng(config_id)
+    lengths = np.full(m, per_row, dtype=np.int64)
+    where = (np.arange(long_rows, dtype=np.int64) * m) // max(long_rows, 1) + m // (2 * max(long_rows, 1))
+    lengths[where] = min(long_len, n)
+    ptr = np.concatenate([[0], np.cumsum(lengths)])
+    col = np.empty(int(ptr[-1]), dtype=np.int64)
+    short = np.ones(m, dtype=bool)
+    short[where] = False
+    d = np.sort(rng.integers(0, n - per_row + 1, size=(int(short.sum()), per_row), dtype=np.int64), axis=1)
+    d += np.arange(per_row, dtype=np.int64)[None, :]
+    starts = ptr[:-1][short]
+    col[(starts[:, None] + np.arange(per_row, dtype=np.int64)[None, :]).reshape(-1)] = d.reshape(-1)
+    for r in where:
+        col[ptr[r]:ptr[r + 1]] = np.sort(rng.choice(n, size=int(lengths[r]), replace=False))
+    val = _uniform_pm1(rng, int(ptr[-1]), dtype)
+    return Csr(m, n, ptr + base, col + base, val, base)
+
+
 def zipf_row_lengths(m, exponent=1.8, max_len=200_000, rng=None):
     """Row lengths with pmf proportional to k^-exponent on [1, max_len] (inverse CDF)."""
     k = np.arange(1, max_len + 1, dtype=np.float64)

@@ -446,14 +446,20 @@ def test_spmv_family_choice_from_row_bins(lib):
     assert _plan(lib, rng.integers(12, 17, m)) == (api.FAMILY_VECTOR, 16)
     # 5-point Laplacian: 3..5 per row
     assert _plan(lib, rng.choice([3, 4, 5], m, p=[0.01, 0.04, 0.95])) == (api.FAMILY_VECTOR, 8)
-    # one row far longer than the rest serialises a wavefront: merge path; in column order when
-    # the rows exceed a tile and x does not fit an L2, in storage order otherwise
+    # rows far longer than the rest serialise a wavefront: merge path; in column order when such rows exceed a
+    # tile, hold most of the nonzeros, and x does not fit an L2; in storage order otherwise
     skew = np.full(m, 4)
-    skew[7] = 100000
+    skew[7:17] = 100000
     assert _plan(lib, skew) == (api.FAMILY_MERGE, 1)
     assert _plan(lib, skew, x_bytes=1 << 20) == (api.FAMILY_MERGE, 0)
-    skew[7] = 700
+    skew[7:17] = 700
     assert _plan(lib, skew) == (api.FAMILY_MERGE, 0)
+    # a handful of long rows among many short ones (1 M rows of 16, 64 rows of 100000: a quarter of the nonzeros):
+    # one merge-path launch over all rows in storage order (measured 140 us; the vector kernel on the short rows
+    # plus the merge kernel on the long ones, as two launches, 107 + 37 us; tiles in column order 155 us)
+    mixed = np.full(1 << 20, 16)
+    mixed[::16384] = 100000
+    assert _plan(lib, mixed) == (api.FAMILY_MERGE, 0)
     # power law: most rows hold one nonzero, the mean is carried by a few long ones
     zipf = np.minimum(rng.zipf(1.8, m), 200000)
     assert _plan(lib, zipf)[0] == api.FAMILY_MERGE
@@ -463,3 +469,29 @@ def test_spmv_family_choice_from_row_bins(lib):
     # argument checks
     fam, lanes = ctypes.c_int(), ctypes.c_int()
     assert lib.mcsparseXcsrRowBinsPlan(None, 1, 1, 1, ctypes.byref(fam), ctypes.byref(lanes)) == api.STATUS_INVALID_VALUE
+
+
+def test_topology_from_compute_unit_count():
+    """32 compute units per XCD: a whole MI355X is eight, its partitions four, two and one; anything that is not a
+    whole number of XCDs counts as one (the XCD-aware orders then turn into the plain order)."""
+    import ctypes
+    lib = _lib.load()
+    for cus, want in ((256, 8), (128, 4), (64, 2), (32, 1), (304, 1), (120, 1), (1, 1), (512, 1)):
+        xcds = ctypes.c_int(-1)
+        assert lib.mcsparseXtopologyOfCuCount(cus, ctypes.byref(xcds)) == 0
+        assert xcds.value == want, (cus, xcds.value)
+    assert lib.mcsparseXtopologyOfCuCount(0, ctypes.byref(xcds)) != 0
+    assert lib.mcsparseXtopologyOfCuCount(64, None) != 0
+
+
+def test_spmv_deterministic_switch_is_off_by_default_and_checked():
+    h = api.Handle()
+    assert h.spmv_deterministic() is False
+    h.set_spmv_deterministic(True)
+    assert h.spmv_deterministic() is True
+    h.set_spmv_deterministic(False)
+    assert h.spmv_deterministic() is False
+    lib = _lib.load()
+    assert lib.mcsparseSetSpMVDeterministic(None, 1) == api.STATUS_NOT_INITIALIZED
+    assert lib.mcsparseGetSpMVDeterministic(h.ptr, None) == api.STATUS_INVALID_VALUE
+    h.destroy()

@@ -202,3 +202,47 @@ def test_transposing_spmv_replays_in_a_hip_graph(torch_gpu, oracle, alg):
     del graph
     torch.cuda.synchronize()
     handle.destroy()
+
+
+def test_static_buffer_call_replays_in_a_hip_graph(torch_gpu, oracle):
+    """mcsparseSpMV_staticBuffer is for callers that cannot allocate, code under graph capture among them.  The
+    address of its scratch array is looked up at the first call on a device, which a capture cannot hold: that call
+    answers NOT_SUPPORTED under capture (and leaves the capture intact), any later one is captured and replays."""
+    torch = torch_gpu
+    rng = np.random.default_rng(33)
+    side = torch.cuda.Stream()
+    handle = api.Handle(stream=side.cuda_stream)
+    a = wl.power_law(m=5000, max_len=4000, dtype=np.float32)
+    d_ptr, d_col, d_val = dev(torch, a.ptr), dev(torch, a.col), dev(torch, a.val)
+    mat = api.SpMat(a.m, a.n, a.nnz, d_ptr, d_col, d_val, base=a.base)
+    mat.set_plan(api.FAMILY_MERGE)  # the family that uses the scratch; no analysis, which would read back
+    x = torch.zeros(a.n, dtype=torch.float32, device="cuda")
+    y = torch.zeros(a.m, dtype=torch.float32, device="cuda")
+    vx, vy = api.DnVec(x), api.DnVec(y)
+
+    first = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(first, stream=side):
+        st = api.spmv_static_buffer(handle, api.OP_N, 2.0, mat, vx, 0.0, vy, api.R_32F)
+    torch.cuda.synchronize()
+    assert st in (api.STATUS_SUCCESS, api.STATUS_NOT_SUPPORTED)  # SUCCESS when an earlier test made the first call
+    del first
+
+    with torch.cuda.stream(side):
+        assert api.spmv_static_buffer(handle, api.OP_N, 2.0, mat, vx, 0.0, vy, api.R_32F) == api.STATUS_SUCCESS
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        assert api.spmv_static_buffer(handle, api.OP_N, 2.0, mat, vx, 0.0, vy, api.R_32F) == api.STATUS_SUCCESS
+    torch.cuda.synchronize()
+    for replay in range(3):
+        hx = rng.uniform(-1, 1, a.n).astype(np.float32)
+        x.copy_(torch.from_numpy(hx))
+        y.fill_(-3)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        ref, bound = oracle.spmv(False, a.m, a.n, a.base, a.ptr, a.col, a.val, 2.0, 0.0, hx, np.zeros(a.m, np.float32))
+        assert_within(y.cpu().numpy(), ref, bound, np.float32, what="replay %d, static buffer" % replay)
+    del graph
+    torch.cuda.synchronize()
+    handle.destroy()

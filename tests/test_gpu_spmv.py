@@ -196,3 +196,20 @@ def test_same_result_on_repeat_and_y_transpose_identity(torch_gpu, handle, oracl
     lhs, rhs = np.dot(w.astype(np.longdouble), ax), np.dot(atw.astype(np.longdouble), x)
     scale = np.dot(np.abs(w), np.abs(a.to_scipy()) @ np.abs(x))
     assert abs(lhs - rhs) <= 64 * 2.0 ** -53 * scale
+
+
+def test_a_few_long_rows_among_many_short_ones(torch_gpu, handle, oracle):
+    """What a row-length-binned dispatch is for: rows of 16 with a handful of rows of 20000 among them.  The analysis
+    sends the whole matrix to the merge-path family in storage order (the long rows hold a minority of the nonzeros);
+    the result is held against the oracle, as is the vector family forced onto the same matrix."""
+    a = wl.mixed_rows(m=1 << 16, per_row=16, long_rows=8, long_len=20000, dtype=np.float32)
+    rng = np.random.default_rng(3)
+    x = rng.uniform(-1, 1, a.n).astype(np.float32)
+    y = rng.uniform(-1, 1, a.m).astype(np.float32)
+    y_ref, bound = oracle.spmv(False, a.m, a.n, a.base, a.ptr, a.col, a.val, 1.0, 0.0, x, y)
+    st, got, plan = run_spmv(torch_gpu, handle, a, x, y, 1.0, 0.0)
+    assert st == api.STATUS_SUCCESS and plan == (api.FAMILY_MERGE, 0), plan
+    assert_within(got, y_ref, bound, np.float32, what="mixed rows, analysed")
+    st, got, _ = run_spmv(torch_gpu, handle, a, x, y, 1.0, 0.0, family=api.FAMILY_VECTOR)
+    assert st == api.STATUS_SUCCESS
+    assert_within(got, y_ref, bound, np.float32, what="mixed rows, vector family")

@@ -192,3 +192,44 @@ def test_crowded_buckets_exact_on_integers(torch_gpu, handle, dtype, rows, per_r
     for base in (0, 1):
         got = run(torch_gpu, handle, a.with_base(base), x, y, 2.0, 1.0)
         assert np.array_equal(got.astype(np.float64), want), (shape, rows, base)
+
+
+@pytest.mark.parametrize("preprocess", [False, True])
+@pytest.mark.parametrize("op", [api.OP_N, api.OP_T])
+def test_deterministic_handle_repeats_its_bits_with_the_default_algorithm(torch_gpu, oracle, op, preprocess):
+    """mcsparseSetSpMVDeterministic: a caller that passes MCSPARSE_SPMV_ALG_DEFAULT, as a program written against the
+    reference does, gets the same bits from every run (the paths of MCSPARSE_SPMV_CSR_ALG2), with and without a
+    preprocess call, in both directions.  Long rows and many rows per column make differing orders show."""
+    torch = torch_gpu
+    handle = api.Handle(stream=torch.cuda.current_stream().cuda_stream)
+    handle.set_spmv_deterministic(True)
+    a = wl.power_law(m=1 << 16, n=1 << 18, max_len=30000, dtype=np.float32)
+    rng = np.random.default_rng(17)
+    xs, ys = (a.n, a.m) if op == api.OP_N else (a.m, a.n)
+    x = rng.uniform(-1, 1, xs).astype(np.float32)
+    y0 = rng.uniform(-1, 1, ys).astype(np.float32)
+    d_ptr, d_col, d_val, d_x = dev(torch, a.ptr), dev(torch, a.col), dev(torch, a.val), dev(torch, x)
+    d_y = dev(torch, y0)
+    mat = api.SpMat(a.m, a.n, a.nnz, d_ptr, d_col, d_val)
+    mat.set_band_bytes(1 << 16)
+    vx, vy = api.DnVec(d_x), api.DnVec(d_y)
+    if preprocess:
+        st, size = api.spmv_preprocess_buffer_size(handle, op, 1.25, mat, vx, 0.5, vy, api.R_32F)
+    else:
+        st, size = api.spmv_buffer_size(handle, op, 1.25, mat, vx, 0.5, vy, api.R_32F)
+    assert st == api.STATUS_SUCCESS
+    buf = torch.empty(size, dtype=torch.uint8, device="cuda")
+    if preprocess:
+        assert api.spmv_preprocess(handle, op, 1.25, mat, vx, 0.5, vy, api.R_32F, buf) == api.STATUS_SUCCESS
+        assert mat.spmv_preprocess_state()[0] in (0, 2)  # never the copy in column order
+    runs = []
+    for _ in range(3):
+        d_y.copy_(torch.from_numpy(y0))
+        assert api.spmv(handle, op, 1.25, mat, vx, 0.5, vy, api.R_32F, buf) == api.STATUS_SUCCESS
+        torch.cuda.synchronize()
+        runs.append(d_y.cpu().numpy())
+    assert np.array_equal(runs[0].view(np.uint32), runs[1].view(np.uint32))
+    assert np.array_equal(runs[0].view(np.uint32), runs[2].view(np.uint32))
+    ref, bound = oracle.spmv(op == api.OP_T, a.m, a.n, 0, a.ptr, a.col, a.val, 1.25, 0.5, x, y0)
+    assert_within(runs[0], ref, bound, np.float32, what="deterministic handle")
+    handle.destroy()
