@@ -511,11 +511,11 @@ mcsparseStatus_t mcsparseSpMatGetSpMVPreprocess(mcsparseSpMatDescr_t spMatDescr,
 mcsparseStatus_t mcsparseSpMatSetSpMVBandBytes(mcsparseSpMatDescr_t spMatDescr, size_t band_bytes);
 
 /* What the device's memory takes by itself, measured with kernels as plain as this library's can be (16-byte
- * non-temporal accesses, eight in flight per thread): mode 0 reads `bytes` of src, mode 1 writes `bytes` of dst,
- * mode 2 copies src to dst.  bytes must be a multiple of 16 and both arrays 16-byte aligned; mode 0 needs `sink`,
- * device memory of at least 2048 * (compute units of the device) uint32 (sink_words says how many it holds), where
- * every thread leaves a word so that its loads are not optimised away.  A yardstick for benchmarks: the rates the
- * kernels of the path are held against besides the published 8 TB/s. */
+ * accesses, a contiguous 16 KB per workgroup): mode 0 reads `bytes` of src, mode 1 writes `bytes` of dst, mode 2
+ * copies src to dst.  bytes must be a multiple of 16 and both arrays 16-byte aligned; mode 0 needs `sink`, device
+ * memory of sink_words >= 1 uint32 (a word of it is written only if a thread's data adds up to one particular
+ * value, which keeps the loads from being optimised away).  A yardstick for benchmarks: the rates the kernels of
+ * the path are held against besides the published 8 TB/s. */
 mcsparseStatus_t mcsparseXstreamProbe(mcsparseHandle_t handle, int mode, const void* src, void* dst, size_t bytes,
                                       uint32_t* sink, size_t sink_words);
 

@@ -974,14 +974,13 @@ mcsparseStatus_t mcsparseSpMM_preprocess(mcsparseHandle_t handle, mcsparseOperat
     s.blocks = false;
     const char* span_slot = static_cast<const char*>(externalBuffer) + l.span_sum;
 
-    // First choice, for operands of 65 to 512 bytes per row (the widths its kernel was measured faster at: 19 %,
-    // 4 % and 20 % at 32, 64 and 128 fp32 columns of a 27-point stencil; at 256 columns the merged lists below
-    // win by 7 %): diagonal blocks over groups of eight rows.  Kept when the blocks are large (a stencil's are 24
-    // nonzeros each) and each loaded row of op(B) serves about two nonzeros or more; matrices without such
-    // structure get the merged column lists.
+    // First choice, for operands of 65 to 1024 bytes per row (the widths its kernel was measured faster at: by 35 %,
+    // 16 %, 29 % and 4 % at 32, 64, 128 and 256 fp32 columns of a 27-point stencil): diagonal blocks over groups of
+    // eight rows.  Kept when the blocks are large (a stencil's are 24 nonzeros each) and each loaded row of op(B)
+    // serves about two nonzeros or more; matrices without such structure get the merged column lists.
     const size_t vb = value_size(matA->valueType);
     const int64_t row_bytes = matC->col_num * static_cast<int64_t>(vb);
-    const bool wide_enough = row_bytes > 64 && row_bytes <= 512 && matA->row_num < (int64_t(1) << 31);
+    const bool wide_enough = row_bytes > 64 && row_bytes <= 1024 && matA->row_num < (int64_t(1) << 31);
     if (wide_enough) {
         mcsp::launch_spmm_block_count(handle->stream, m, nnz, static_cast<idx_t>(matA->idxBase), ia.rows, ia.cols,
                                       externalBuffer);
@@ -1180,8 +1179,9 @@ mcsparseStatus_t mcsparseXstreamProbe(mcsparseHandle_t handle, int mode, const v
         return to_public_status(MCSP_STATUS_INVALID_POINTER);
     if (((reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst)) & 15u) != 0)
         return to_public_status(MCSP_STATUS_INVALID_VALUE);
-    if (mode == 0 && sink_words < mcsp::stream_probe_threads()) return to_public_status(MCSP_STATUS_INVALID_SIZE);
-    mcsp::launch_stream_probe(handle->stream, mode, src, dst, bytes, sink);
+    if ((mode == 0 && sink_words == 0) || bytes >= (size_t(1) << 44)) return to_public_status(MCSP_STATUS_INVALID_SIZE);
+    mcsp::launch_stream_probe(handle->stream, mode, src, dst, bytes, sink,
+                              static_cast<uint32_t>(sink_words < 0xffffffffu ? sink_words : 0xffffffffu));
     return MCSPARSE_STATUS_SUCCESS;
 }
 

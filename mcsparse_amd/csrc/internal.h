@@ -334,9 +334,9 @@ bool launch_spmv_banded(hipStream_t stream, const BandedShape& s, uint32_t grid,
                         void* region);
 
 // Streaming kernels that measure what the memory takes by itself (analysis.hip): mode 0 reads src, 1 writes dst,
-// 2 copies; bytes a multiple of 16, arrays 16-byte aligned, sink = stream_probe_threads() uint32 for mode 0.
-uint32_t stream_probe_threads();
-void launch_stream_probe(hipStream_t stream, int mode, const void* src, void* dst, uint64_t bytes, uint32_t* sink);
+// 2 copies; bytes a multiple of 16 and below 2^44, arrays 16-byte aligned, sink = at least one uint32 for mode 0.
+void launch_stream_probe(hipStream_t stream, int mode, const void* src, void* dst, uint64_t bytes, uint32_t* sink,
+                         uint32_t sink_words);
 
 // ---- SpMM (spmm.hip) ----
 struct SpmmArgs {
@@ -380,11 +380,13 @@ void launch_spmm_scheduled(hipStream_t stream, const SpmmArgs& a, const void* sc
 
 // Diagonal-block schedule of a CSR structure (spmm_blocks.hip), the second kind mcsparseSpMM_preprocess can leave in
 // the region spmm_schedule_layout describes: for every group of kSpmmBlockRows consecutive rows a list of blocks
-// {int32 c, uint32 n | lo << 8 | hi << 16}: each row r in [lo, hi) of the group holds the n <= kSpmmBlockMaxDiagonals
-// consecutive columns c + r .. c + r + n - 1 (zero-based), and the blocks of a group consume every row's nonzeros
-// in storage order.  group_ptr's place holds the groups+1 offsets into the blocks, entries' place the blocks
-// (8 bytes each: the schedule is only kept when they fit), span_sum's place three counters: the sum of the
-// groups' column spans and the number of rows of op(B) all blocks load (u64), the most nonzeros in one group (u32).
+// {int32 c, uint32 shape}.  A block holds n <= kSpmmBlockMaxDiagonals consecutive diagonals (shape bits 0-2: n); its
+// p-th diagonal is held by the rows lo_p .. hi_p - 1 of the group (shape bits 8+8p..11+8p: lo_p, 12+8p..15+8p: hi_p),
+// and row r holds it in column c + r + p (zero-based).  The blocks of a group consume every row's nonzeros in
+// storage order.  group_ptr's place holds the groups+1 offsets into the blocks, entries' place the blocks (8 bytes
+// each) and, at its end, the order in which the kernel takes the groups (the schedule is only kept when they fit),
+// span_sum's place three counters: the sum of the groups' column spans and the number of rows of op(B) all blocks
+// load (u64), the most nonzeros in one group (u32).
 constexpr int kSpmmBlockRows = 8;
 constexpr int kSpmmBlockMaxDiagonals = 3;
 constexpr uint64_t spmm_block_groups(idx_t m) { return (static_cast<uint64_t>(m) + kSpmmBlockRows - 1) / kSpmmBlockRows; }

@@ -107,20 +107,28 @@ __global__ __launch_bounds__(kWave) void block_cover_kernel(idx_t m, idx_t base,
                 int key[K];
 #pragma unroll
                 for (int r = 0; r < K; ++r) key[r] = key_of(r);
+                // the block being grown: keys start .. start + width - 1, key start + p held by rows lo[p] .. hi[p] - 1
                 int start = 0;
-                uint32_t width = 0, rows = 0;  // the block being grown: keys start .. start + width - 1, held by `rows`
-                auto flush = [&]() {
-                    // one block per contiguous stretch of rows
-                    uint32_t left = rows;
-                    while (left != 0) {
-                        const uint32_t lo = __ffs(left) - 1;
-                        const uint32_t run = __ffs(~(left >> lo)) - 1;  // set bits from lo on
-                        const uint32_t hi = lo + run;
-                        if (FILL) blocks[out + count] = make_uint2(static_cast<uint32_t>(start), width | (lo << 8) | (hi << 16));
-                        ++count;
-                        loads += run + width - 1;
-                        left &= ~(((1u << run) - 1u) << lo);
+                uint32_t width = 0;
+                uint32_t lo[D], hi[D];
+                auto emit = [&](int c, uint32_t w, const uint32_t (&l)[D], const uint32_t (&h)[D]) {
+                    uint32_t shape = w;
+                    uint32_t j_min = 0xffffffffu, j_max = 0;
+#pragma unroll
+                    for (int q = 0; q < D; ++q) {
+                        if (static_cast<uint32_t>(q) < w) {
+                            shape |= (l[q] | (h[q] << 4)) << (8 + 8 * q);
+                            j_min = min(j_min, l[q] + q);
+                            j_max = max(j_max, h[q] - 1 + q);
+                        }
                     }
+                    if (FILL) blocks[out + count] = make_uint2(static_cast<uint32_t>(c), shape);
+                    ++count;
+                    loads += j_max - j_min + 1;
+                };
+                auto flush = [&]() {
+                    if (width != 0) emit(start, width, lo, hi);
+                    width = 0;
                 };
                 while (true) {
                     int low = kNoKey;
@@ -136,17 +144,31 @@ __global__ __launch_bounds__(kWave) void block_cover_kernel(idx_t m, idx_t base,
                             key[r] = key_of(r);
                         }
                     }
-                    if (width != 0 && width < static_cast<uint32_t>(D) && low == start + static_cast<int>(width) &&
-                        holders == rows) {
-                        ++width;
-                    } else {
-                        if (width != 0) flush();
-                        start = low;
-                        width = 1;
-                        rows = holders;
+                    // the rows that hold this key, one contiguous stretch at a time
+                    while (holders != 0) {
+                        const uint32_t first = __ffs(holders) - 1;
+                        const uint32_t run = __ffs(~(holders >> first)) - 1;  // set bits from `first` on
+                        holders &= ~(((1u << run) - 1u) << first);
+                        // The last stretch may carry on the block being grown (the next diagonal of the same rows,
+                        // or of rows shifted by a grid line's end); the others are blocks of their own.
+                        if (holders == 0 && width != 0 && width < static_cast<uint32_t>(D) && low == start + static_cast<int>(width)) {
+                            lo[width] = first;
+                            hi[width] = first + run;
+                            ++width;
+                        } else if (holders == 0) {
+                            flush();
+                            start = low;
+                            lo[0] = first;
+                            hi[0] = first + run;
+                            width = 1;
+                        } else {
+                            flush();
+                            const uint32_t l1[D] = {first, 0, 0}, h1[D] = {first + run, 0, 0};
+                            emit(low, 1, l1, h1);
+                        }
                     }
                 }
-                if (width != 0) flush();
+                flush();
             };
             if (staged) cover(std::true_type{});
             else cover(std::false_type{});
@@ -271,9 +293,10 @@ __global__ __launch_bounds__(kBlock) void spmm_blocks_kernel(idx_t m, idx_t n, i
         const idx_t last_value = nnz - 1;  // nnz != 0: total_blocks != 0
         const uint32_t last_block = total_blocks - 1;
         const uint32_t my_row = lane / kLanesPerRow;
-        // where this lane's next value lies: its row's first unused nonzero plus its place among the row's lanes
+        // where the next unused value of this lane's row lies
         const uint64_t my_abs_row = r0 + my_row < last_row ? r0 + my_row : last_row;
-        idx_t pos = row_ptr[my_abs_row] - base + (lane % kLanesPerRow) * kValuesPerLane;
+        const uint32_t my_place = (lane % kLanesPerRow) * kValuesPerLane;  // the first diagonal this lane fetches for
+        idx_t pos = row_ptr[my_abs_row] - base;
 
         constexpr int kCap = stage_capacity<T, LR>();
         constexpr int E = 16 / sizeof(T);  // values per 16-byte piece
@@ -322,25 +345,51 @@ __global__ __launch_bounds__(kBlock) void spmm_blocks_kernel(idx_t m, idx_t n, i
         // op(B) one block ahead, into a second set of registers.  None of these loads sits under a test (a load
         // under a test makes the compiler wait for every load in flight at the join): a block past the end of
         // the list, or one that is not sound, turns into a block of no width whose loads go to places that exist.
+        // A block as the kernel sees it.  `mine` says which of the block's diagonals this lane's row holds (bit p:
+        // diagonal p): the row's values of the block are its next popcount(mine) ones, in the order of the bits.
         struct Shape {
             int cbase;
-            uint32_t w, lo, hi;
+            uint32_t w;
+            uint32_t lo[D], len[D];  // diagonal p is held by rows lo[p] .. lo[p] + len[p] - 1
+            uint32_t j_first, j_last;  // rows of op(B) the block needs, counted from cbase
+            uint32_t mine;
+            bool whole;  // every row of the group holds every diagonal of the block
         };
         auto decode = [&](uint2 d, bool exists) {
             Shape sh;
             sh.cbase = static_cast<int>(d.x);
             sh.w = d.y & 7u;
-            sh.lo = (d.y >> 8) & 15u;
-            sh.hi = (d.y >> 16) & 31u;
+            bool sound = exists && sh.w - 1u < static_cast<uint32_t>(D);
+            sh.whole = true;
+            sh.mine = 0;
+            sh.j_first = 0xffffu;
+            sh.j_last = 0;
+#pragma unroll
+            for (int q = 0; q < D; ++q) {
+                const uint32_t lo = (d.y >> (8 + 8 * q)) & 15u;
+                const uint32_t hi = (d.y >> (12 + 8 * q)) & 15u;
+                const bool used = static_cast<uint32_t>(q) < sh.w;
+                sound = sound && (!used || (lo < hi && hi <= static_cast<uint32_t>(K)));
+                sh.lo[q] = lo;
+                sh.len[q] = used ? hi - lo : 0u;
+                sh.whole = sh.whole && (!used || (lo == 0 && hi == static_cast<uint32_t>(K)));
+                if (used) {
+                    sh.j_first = min(sh.j_first, lo + q);
+                    sh.j_last = max(sh.j_last, hi - 1 + q);
+                    if (my_row - lo < hi - lo) sh.mine |= 1u << q;
+                }
+            }
             // (every extent is below 2^31 here, so the sums cannot wrap)
-            const bool sound = exists && sh.w - 1u < static_cast<uint32_t>(D) && sh.lo < sh.hi && sh.hi <= static_cast<uint32_t>(K) &&
-                               sh.cbase + static_cast<int>(sh.lo) >= 0 &&
-                               sh.cbase + static_cast<int>(sh.hi + sh.w) - 2 <= static_cast<int>(k) - 1;
+            sound = sound && sh.cbase + static_cast<int>(sh.j_first) >= 0 &&
+                    sh.cbase + static_cast<int>(sh.j_last) <= static_cast<int>(k) - 1;
             if (!sound) {
                 sh.cbase = 0;
                 sh.w = 0;
-                sh.lo = 0;
-                sh.hi = 1;
+                sh.j_first = sh.j_last = 0;
+                sh.mine = 0;
+                sh.whole = false;
+#pragma unroll
+                for (int q = 0; q < D; ++q) sh.len[q] = 0;
             }
             return sh;
         };
@@ -348,30 +397,28 @@ __global__ __launch_bounds__(kBlock) void spmm_blocks_kernel(idx_t m, idx_t n, i
             T v[kValuesPerLane];
             Vec<T, V> b[K + D - 1];
         };
+        // at_value: where the first unused value of this lane's row lies
         auto fetch = [&](const Shape& sh, idx_t at_value, Operands& o) {
+            // this lane fetches for the diagonals my_place .. my_place + kValuesPerLane - 1 of its row: the value of
+            // diagonal p is the row's (number of held diagonals below p)-th unused one
+            idx_t at[kValuesPerLane];
+#pragma unroll
+            for (int q = 0; q < kValuesPerLane; ++q)
+                at[q] = at_value + static_cast<idx_t>(__popc(sh.mine & ((1u << (my_place + q)) - 1u)));
             if constexpr (STAGED) {
                 // from the group's copy in LDS; a place past the copy (an overwritten schedule) is held inside it
 #pragma unroll
                 for (int q = 0; q < kValuesPerLane; ++q)
-                    o.v[q] = staged[min(at_value - stage_first + static_cast<idx_t>(q), static_cast<idx_t>(kCap - 1))];
-            } else if constexpr (kValuesPerLane == 2) {
-                // both in one load (the pair need not be aligned to its size); a pair that would begin on the
-                // last nonzero begins one earlier and hands its second value over as the first
-                typedef T Pair __attribute__((ext_vector_type(2), aligned(sizeof(T))));
-                const idx_t at = min(at_value, last_value - 1);  // a schedule of blocks exists from eight nonzeros on
-                const Pair pair = *reinterpret_cast<const Pair*>(val + at);
-                o.v[0] = at_value > at ? pair[1] : pair[0];
-                o.v[1] = pair[1];
+                    o.v[q] = staged[min(at[q] - stage_first, static_cast<idx_t>(kCap - 1))];
             } else {
 #pragma unroll
-                for (int q = 0; q < kValuesPerLane; ++q) o.v[q] = val[min(at_value + static_cast<idx_t>(q), last_value)];
+                for (int q = 0; q < kValuesPerLane; ++q) o.v[q] = val[min(at[q], last_value)];
             }
-            // rows lo .. hi + w - 2 of the block are needed; the others are asked for at the nearest needed one
+            // rows j_first .. j_last of the block are needed; the others are asked for at the nearest needed one
             const off_t roff = static_cast<off_t>(static_cast<int64_t>(sh.cbase)) * ldb_bytes + lane_off;
-            const uint32_t j_last = sh.hi + (sh.w != 0 ? sh.w : 1u) - 2;
             static_for<K + D - 1>([&](auto jc) {
                 constexpr uint32_t j = decltype(jc)::value;
-                const uint32_t jj = min(max(j, sh.lo), j_last);
+                const uint32_t jj = min(max(j, sh.j_first), sh.j_last);
                 o.b[j] = load_vec<T, V>(reinterpret_cast<const T*>(B_bytes + (roff + static_cast<off_t>(jj) * ldb_bytes)));
             });
         };
@@ -393,6 +440,8 @@ __global__ __launch_bounds__(kBlock) void spmm_blocks_kernel(idx_t m, idx_t n, i
                     });
                 });
             };
+            // Some rows lack some diagonals (a grid line begins or ends inside the group): the tests sit around
+            // the multiply-adds, so that a row only ever sees the rows of op(B) it names.
             auto partial = [&]() {
                 static_for<K + D - 1>([&](auto jc) {
                     constexpr int j = decltype(jc)::value;
@@ -400,7 +449,7 @@ __global__ __launch_bounds__(kBlock) void spmm_blocks_kernel(idx_t m, idx_t n, i
                         constexpr int p = decltype(pc)::value;
                         constexpr int r = j - p;
                         if constexpr (r >= 0 && r < K) {
-                            if (static_cast<uint32_t>(p) < sh.w && static_cast<uint32_t>(r) >= sh.lo && static_cast<uint32_t>(r) < sh.hi) {
+                            if (static_cast<uint32_t>(r) - sh.lo[p] < sh.len[p]) {
                                 const T a = group_bcast<LR, r * kLanesPerRow + p / kValuesPerLane>(o.v[p % kValuesPerLane]);
 #pragma unroll
                                 for (int c = 0; c < V; ++c) acc[r][c] += a * o.b[j].v[c];
@@ -409,7 +458,7 @@ __global__ __launch_bounds__(kBlock) void spmm_blocks_kernel(idx_t m, idx_t n, i
                     });
                 });
             };
-            if (sh.lo == 0 && sh.hi == static_cast<uint32_t>(K)) {
+            if (sh.whole) {
                 static_assert(D == 3, "one case per width");
                 switch (sh.w) {
                     case 1: whole(std::integral_constant<int, 1>{}); break;
@@ -421,7 +470,7 @@ __global__ __launch_bounds__(kBlock) void spmm_blocks_kernel(idx_t m, idx_t n, i
                 partial();
             }
         };
-        auto advance = [&](const Shape& sh) -> idx_t { return (my_row >= sh.lo && my_row < sh.hi) ? sh.w : 0u; };
+        auto advance = [&](const Shape& sh) -> idx_t { return static_cast<idx_t>(__popc(sh.mine)); };
         auto descriptor = [&](uint32_t s) { return blocks[min(s, last_block)]; };
 
         Operands even, odd;

@@ -112,8 +112,8 @@ def stencil_full():
     return a
 
 
-# preprocess = True runs the kernels that work from a schedule: diagonal blocks (state 3) for N = 64, merged column
-# lists (state 2) for N = 256; for N = 8 the lists are built but too narrow to use
+# preprocess = True runs the kernels that work from a schedule: diagonal blocks (state 3) for N = 64 and 256; for
+# N = 8 merged column lists are built (state 2) but too narrow to use
 @pytest.mark.parametrize("preprocess", [False, True])
 @pytest.mark.parametrize("n", [8, 64, 256])
 def test_config4_stencil_full_size(torch_gpu, handle, oracle, stencil_full, n, preprocess):
@@ -121,7 +121,7 @@ def test_config4_stencil_full_size(torch_gpu, handle, oracle, stencil_full, n, p
     rng = np.random.default_rng(n)
     B = rng.uniform(-1, 1, (a.n, n)).astype(np.float32)
     st, got, _ = run_spmm(torch_gpu, handle, a, B, np.zeros((a.m, n), np.float32), 1.0, 0.0, preprocess=preprocess,
-                          expect_schedule=(3 if n == 64 else 2) if preprocess else None)
+                          expect_schedule=(2 if n == 8 else 3) if preprocess else None)
     assert st == 0
     # oracle on a sample of rows: first/last planes, and random interior rows
     rows = np.unique(np.concatenate([np.arange(0, 300), np.arange(a.m - 300, a.m),

@@ -247,7 +247,7 @@ def test_overwritten_schedule_stays_in_bounds(torch_gpu, handle, grid, n):
 # ---- diagonal blocks (mcsparseSpMM_preprocess on matrices whose neighbouring rows hold the same diagonals) ----
 
 def read_blocks(torch, buf, m):
-    """The block schedule as it lies in the buffer: offsets per group of 8 rows, then (c, n | lo << 8 | hi << 16)."""
+    """The block schedule as it lies in the buffer: offsets per group of 8 rows, then (c, shape) pairs."""
     def align(x):
         return (x + 127) // 128 * 128
     raw = buf.cpu().numpy()
@@ -259,15 +259,22 @@ def read_blocks(torch, buf, m):
 
 
 def columns_from_blocks(ptr, words, m):
-    """Expands the blocks into every row's column sequence (zero-based)."""
+    """Expands the blocks into every row's column sequence (zero-based): shape bits 0-2 = number of diagonals n, and
+    for p < n bits 8+8p.. = first row, 12+8p.. = end row of diagonal p; row r holds it in column c + r + p."""
     rows = [[] for _ in range(m)]
     for g in range(len(ptr) - 1):
         for c, shape in words[ptr[g]:ptr[g + 1]]:
-            c = int(np.int32(c))
-            n, lo, hi = int(shape & 7), int((shape >> 8) & 15), int((shape >> 16) & 31)
-            assert 1 <= n <= 4 and 0 <= lo < hi <= 8
-            for r in range(lo, hi):
-                rows[8 * g + r].extend(range(c + r, c + r + n))
+            c, shape = int(np.int32(c)), int(shape)
+            n = shape & 7
+            assert 1 <= n <= 3
+            for p in range(n):
+                lo, hi = (shape >> (8 + 8 * p)) & 15, (shape >> (12 + 8 * p)) & 15
+                assert 0 <= lo < hi <= 8
+            for r in range(8):
+                for p in range(n):
+                    lo, hi = (shape >> (8 + 8 * p)) & 15, (shape >> (12 + 8 * p)) & 15
+                    if lo <= r < hi:
+                        rows[8 * g + r].append(c + r + p)
     return rows
 
 
@@ -315,7 +322,7 @@ def test_blocks_cover_every_nonzero_once_and_in_storage_order(torch_gpu, handle,
 
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
-@pytest.mark.parametrize("n", [20, 36, 64, 72, 128])
+@pytest.mark.parametrize("n", [20, 36, 64, 72, 128, 256, 264])
 def test_blocks_banded_matrix_with_broken_rows(torch_gpu, handle, oracle, dtype, n):
     """Diagonal runs of one to six, rows with holes, empty rows, unsorted rows, a group too long to cover, a row
     count that leaves the last group short; every width of lane group; both layouts of C."""
@@ -337,8 +344,8 @@ def test_blocks_banded_matrix_with_broken_rows(torch_gpu, handle, oracle, dtype,
         rows.append(c)
     ptr = np.concatenate([[0], np.cumsum([len(c) for c in rows])]).astype(np.int32)
     a = wl.Csr(m, k, ptr, np.concatenate(rows).astype(np.int32), rng.uniform(-1, 1, int(ptr[-1])).astype(dtype))
-    # blocks for operands of 65 to 512 bytes per row, merged column lists beyond
-    want = 3 if 64 < n * np.dtype(dtype).itemsize <= 512 else (1, 2)
+    # blocks for operands of 65 to 1024 bytes per row, merged column lists beyond
+    want = 3 if 64 < n * np.dtype(dtype).itemsize <= 1024 else (1, 2)
     for c_order in (api.ORDER_ROW, api.ORDER_COL):
         check(torch_gpu, handle, oracle, a, n, 1.0, 0.0, preprocess=True, expect_schedule=want, c_order=c_order)
     check(torch_gpu, handle, oracle, a.with_base(1), n, -0.5, 1.5, preprocess=True, expect_schedule=want, pad_b=4, pad_c=8)
