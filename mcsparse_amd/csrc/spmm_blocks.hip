@@ -3,13 +3,17 @@
 //
 // The reference's kernel (src/kernels/level3/spmm/csr_spmm_device.hpp:121-137) walks a row's nonzeros
 // once per output column.  Here a lane group owns kSpmmBlockRows consecutive rows of A and a few adjacent
-// columns of C.  mcsparseSpMM_preprocess has covered the nonzeros of those rows with blocks: block
-// (c, n, lo, hi) says that every row r in [lo, hi) of the group holds the n consecutive columns
-// c + r .. c + r + n - 1, so the block needs the (hi - lo) + n - 1 consecutive rows c + lo .. of op(B),
+// columns of C.  mcsparseSpMM_preprocess has covered the nonzeros of those rows with blocks of up to
+// kSpmmBlockMaxDiagonals consecutive diagonals, each with its own range of rows: block
+// (c, n, lo_0, hi_0, .., lo_{n-1}, hi_{n-1}) says that row r of the group holds column c + r + p for every
+// p < n with lo_p <= r < hi_p.  The block needs at most kSpmmBlockRows + n - 1 consecutive rows of op(B),
 // each loaded once into registers and used by up to n rows of A, and which loaded row feeds which
 // accumulator is fixed in the code: no per-nonzero flags, ballots or masks.  The values are read from the
-// CSR array on every call (a row's p-th value of a block is the next one in storage order), so the
+// CSR array on every call (a row's values inside a block are the next ones in storage order), so the
 // caller may change them freely between calls.
+//
+// A block is eight bytes: {int32 c, uint32 shape}; shape bits 0-2 hold n, bits 8+8p..11+8p hold lo_p and
+// bits 12+8p..15+8p hold hi_p.
 #include "spmm_device.h"
 
 namespace mcsp {
@@ -231,9 +235,9 @@ __global__ __launch_bounds__(kOrderChunk) void block_order_kernel(uint64_t group
 }
 
 // LR lanes (8..64) per group of K rows, V = 16 B / sizeof(T) adjacent columns per lane; blockIdx.y walks
-// panels of LR * V columns.  The lanes of a group read LR block descriptors at once, one each, and hand
-// them round through the LDS crossbar; a block's values are read by the lanes together (lane l reads for
-// row l / (LR / K)) and reach the multiply-adds as DPP or scalar broadcasts.
+// panels of LR * V columns.  Every lane of a group reads the block descriptors itself (one address for the
+// whole group: one access); a block's values are read by the lanes together (lane l reads for row
+// l / (LR / K)) and reach the multiply-adds as DPP row broadcasts.
 // STAGED: no group holds more nonzeros than stage_capacity<T, LR>() and the value array is 16-byte aligned.  A
 // group's values are then copied into LDS once, in whole 16-byte pieces, and every block reads its values from
 // there.  (Read from memory block by block, the sixteen lanes of a group ask for two values in each of eight

@@ -98,6 +98,40 @@ def test_config2_full_size_banded(torch_gpu, handle, oracle):
     assert (state, bands) == (2, 4)
 
 
+def test_config2_margin_against_the_literal_bound(torch_gpu, handle, oracle):
+    """Config 2 runs with alpha = 1.5, beta = 0.5, for which the tests accept 8u * (|alpha| (|A||x|)_i + |beta y_i|), the
+    bound the stated one turns into when the sum is scaled and added to beta * y.  Here the same results are held
+    against the literal (|A||x|)_i of the statement: the worst error, in units of u * (|A||x|)_i, of the direct kernel
+    and of both preprocessed copies is printed and stays below 8 by a wide margin."""
+    torch = torch_gpu
+    a = wl.uniform_rows(m=1 << 20, per_row=16, dtype=np.float64)
+    rng = np.random.default_rng(2)
+    x = rng.uniform(-1, 1, a.n)
+    y = rng.uniform(-1, 1, a.m)
+    y_ref, _ = oracle.spmv(False, a.m, a.n, 0, a.ptr, a.col, a.val, 1.5, 0.5, x, y)
+    _, literal = oracle.spmv(False, a.m, a.n, 0, a.ptr, a.col, a.val, 1.0, 0.0, x, None)  # (|A||x|)_i
+    u = 2.0 ** -53
+    d_ptr, d_col, d_val, d_x = dev(torch, a.ptr), dev(torch, a.col), dev(torch, a.val), dev(torch, x)
+    worst = {}
+    for name, alg, pre in (("direct", api.SPMV_ALG_DEFAULT, False), ("column order", api.SPMV_ALG_DEFAULT, True),
+                           ("banded", api.SPMV_CSR_ALG2, True)):
+        d_y = dev(torch, y)
+        mat = api.SpMat(a.m, a.n, a.nnz, d_ptr, d_col, d_val)
+        vx, vy = api.DnVec(d_x), api.DnVec(d_y)
+        size_of = api.spmv_preprocess_buffer_size if pre else api.spmv_buffer_size
+        st, size = size_of(handle, api.OP_N, 1.5, mat, vx, 0.5, vy, api.R_64F, **({"alg": alg} if pre else {}))
+        assert st == api.STATUS_SUCCESS
+        buf = torch.empty(size, dtype=torch.uint8, device="cuda")
+        if pre:
+            assert api.spmv_preprocess(handle, api.OP_N, 1.5, mat, vx, 0.5, vy, api.R_64F, buf, alg=alg) == api.STATUS_SUCCESS
+        assert api.spmv(handle, api.OP_N, 1.5, mat, vx, 0.5, vy, api.R_64F, buf, alg=alg) == api.STATUS_SUCCESS
+        torch.cuda.synchronize()
+        err = np.abs(d_y.cpu().numpy().astype(np.longdouble) - y_ref)
+        worst[name] = float((err / (u * literal)).max())
+    print("config 2, worst |y - y_ref| / (u (|A||x|)_i):", {k: round(v, 3) for k, v in worst.items()})
+    assert max(worst.values()) <= 8.0, worst
+
+
 def test_config2_full_size_column_order(torch_gpu, handle, oracle):
     a = wl.uniform_rows(m=1 << 20, per_row=16, dtype=np.float64)
     state, bands, rows = run_banded(torch_gpu, handle, oracle, a, 1.5, 0.5, calls=2, what="C2 column order",
