@@ -522,12 +522,48 @@ __global__ __launch_bounds__(kBlock) void spmm_blocks_kernel(idx_t m, idx_t n, i
             row_times_b<T, LR, V, WIDE>(i[r], e[r], lane, base, col, val, B_bytes, lane_off, ldb_bytes, acc[r]);
     }
 
-    if (!stores) return;
     // A column-major C holds the rows of the group next to each other in every column: 32 or 64 bytes per
     // column and lane, which the lane groups of a workgroup complete to whole lines.
     static_assert(K % 4 == 0, "rows of a group are written four at a time into a column-major C");
     const bool whole_columns = !c_row_major && r0 + K <= static_cast<uint64_t>(m) &&
                                ((reinterpret_cast<uintptr_t>(C) | static_cast<uintptr_t>(ldc * sizeof(T))) & 15u) == 0;
+    if constexpr (sizeof(T) == 4 && K == 8) {
+        // Written lane by lane, a wavefront's store touches 64 pieces of 16 bytes, each in a line of its own.  Two
+        // neighbouring lanes swap halves instead: of every column of the two, the even lane then writes rows 0-3 and
+        // the odd lane rows 4-7, 32 adjacent bytes per store and pair.  (Both lanes of a pair belong to one group;
+        // every lane takes part in the swap, also those that store nothing.)
+        const bool odd = (lane & 1u) != 0;
+        const uint64_t partner_c_own = odd ? c_own - V : c_own + V;
+        const bool paired = whole_columns && stores && partner_c_own < static_cast<uint64_t>(n);
+        if (__builtin_amdgcn_ballot_w64(paired) != 0) {  // same for the whole wavefront
+            T got[4][V];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+#pragma unroll
+                for (int c = 0; c < V; ++c) got[i][c] = dpp_mov<kDppQuadXor1>(odd ? acc[i][c] : acc[4 + i][c]);
+            }
+            if (paired) {
+                const uint64_t pair_c0 = odd ? c0 - V : c0;
+                T* first = C + r0 + (odd ? 4 : 0);
+#pragma unroll
+                for (int c = 0; c < V; ++c) {
+                    // a column of the even lane: its own rows 0-3, and the rows 4-7 it gave to the odd lane
+                    T* at = first + static_cast<int64_t>(pair_c0 + c) * ldc;
+                    if (odd) store_c_four_rows<T>(at, got[0][c], got[1][c], got[2][c], got[3][c], alpha, beta);
+                    else store_c_four_rows<T>(at, acc[0][c], acc[1][c], acc[2][c], acc[3][c], alpha, beta);
+                }
+#pragma unroll
+                for (int c = 0; c < V; ++c) {
+                    // a column of the odd lane: the rows 0-3 it gave to the even lane, and its own rows 4-7
+                    T* at = first + static_cast<int64_t>(pair_c0 + V + c) * ldc;
+                    if (odd) store_c_four_rows<T>(at, acc[4][c], acc[5][c], acc[6][c], acc[7][c], alpha, beta);
+                    else store_c_four_rows<T>(at, got[0][c], got[1][c], got[2][c], got[3][c], alpha, beta);
+                }
+                return;
+            }
+        }
+    }
+    if (!stores) return;
     if (whole_columns) {
 #pragma unroll
         for (int c = 0; c < V; ++c) {
