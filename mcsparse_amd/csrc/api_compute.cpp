@@ -5,6 +5,8 @@
 
 #include "internal.h"
 
+#include <algorithm>
+
 using mcsp::idx_t;
 
 namespace {
@@ -577,7 +579,10 @@ mcspStatus_t spmm_typed(mcsparseHandle_t h, const mcsparseSpMatDescr* A, mcspars
         }
         // the schedule was built from batch 0's structure
         if (scheduled_here && schedule_usable()) {
-            if (by_blocks)
+            if (by_blocks && A->schedule.stride != 0)
+                mcsp::launch_spmm_strips<T>(h->stream, a, buffer, A->schedule.stride, A->schedule.entries,
+                                            A->schedule.longest_group, A->schedule.mean_span, h_alpha, beta_inner);
+            else if (by_blocks)
                 mcsp::launch_spmm_blocks<T>(h->stream, a, buffer, A->schedule.entries, A->schedule.longest_group,
                                             A->schedule.mean_span, h_alpha,
                                             beta_inner);
@@ -941,6 +946,42 @@ mcsparseStatus_t mcsparseSpMM_bufferSize(mcsparseHandle_t handle, mcsparseOperat
 // mcsparseSpMM uses it when it is handed the same buffer and the same CSR arrays, and falls back
 // to the schedule-free kernel otherwise.  Until then the caller must leave the buffer and the
 // structure of A alone; the values of A may change freely.
+namespace {
+
+// The distance, in rows, at which the strips of a strip schedule would lie for this matrix, or 0: the smallest
+// distance between the beginnings of two runs of consecutive diagonals in the middle row that is a whole number of
+// strips and leaves the matrix at least eight such stretches (a 27-point stencil on a grid of lines of 128 points
+// has runs of three diagonals 128 apart).  Reads the row back: blocks.
+uint32_t strip_stride_of_middle_row(hipStream_t stream, idx_t m, idx_t base, const idx_t* row_ptr, const idx_t* col) {
+    constexpr idx_t kMostLooked = 256;
+    const idx_t row = m / 2;
+    idx_t ends[2] = {0, 0};
+    if (hipMemcpyAsync(ends, row_ptr + row, sizeof(ends), hipMemcpyDeviceToHost, stream) != hipSuccess ||
+        hipStreamSynchronize(stream) != hipSuccess)
+        return 0;
+    if (ends[1] < ends[0] || ends[0] < base) return 0;
+    const idx_t count = ends[1] - ends[0];
+    if (count < 2 || count > kMostLooked) return 0;
+    idx_t cols[kMostLooked];
+    if (hipMemcpyAsync(cols, col + (ends[0] - base), count * sizeof(idx_t), hipMemcpyDeviceToHost, stream) != hipSuccess ||
+        hipStreamSynchronize(stream) != hipSuccess)
+        return 0;
+    std::sort(cols, cols + count);
+    uint32_t best = 0;
+    idx_t run_start = cols[0];
+    for (idx_t i = 1; i < count; ++i) {
+        if (cols[i] <= cols[i - 1] + 1) continue;  // the run goes on (or a duplicate)
+        const uint64_t gap = static_cast<uint64_t>(cols[i]) - run_start;
+        run_start = cols[i];
+        if (gap > 0xffffffffull) continue;
+        const uint32_t stride = static_cast<uint32_t>(gap);
+        if (mcsp::spmm_strip_stride_usable(m, stride) && (best == 0 || stride < best)) best = stride;
+    }
+    return best;
+}
+
+}  // namespace
+
 mcsparseStatus_t mcsparseSpMM_preprocess(mcsparseHandle_t handle, mcsparseOperation_t opA, mcsparseOperation_t opB,
                                          const void* alpha, mcsparseSpMatDescr_t matA, mcsparseDnMatDescr_t matB,
                                          const void* beta, mcsparseDnMatDescr_t matC, macaDataType /*computeType*/,
@@ -972,6 +1013,7 @@ mcsparseStatus_t mcsparseSpMM_preprocess(mcsparseHandle_t handle, mcsparseOperat
     s.nnz = matA->nnz;
     s.base = static_cast<int>(matA->idxBase);
     s.blocks = false;
+    s.stride = 0;
     const char* span_slot = static_cast<const char*>(externalBuffer) + l.span_sum;
 
     // First choice, for operands of 65 to 1024 bytes per row (the widths its kernel was measured faster at: by 35 %,
@@ -995,6 +1037,44 @@ mcsparseStatus_t mcsparseSpMM_preprocess(mcsparseHandle_t handle, mcsparseOperat
         const uint64_t nz = static_cast<uint64_t>(matA->nnz);
         if (blocks != 0 && static_cast<uint64_t>(blocks) * 8 <= nz && counters[1] * 9 <= nz * 5 &&
             mcsp::spmm_block_schedule_fits(m, nnz, blocks)) {
+            // The matrix has diagonals.  Where rows a fixed distance apart hold the same ones (the neighbouring lines
+            // of a structured grid), groups of strips that far apart share more of the loaded rows of op(B): the
+            // distance is read off a row in the middle, the gain is measured by covering the matrix that way, and the
+            // strips are kept when they load a fifth fewer rows.
+            // (Their kernel gives sixteen lanes of 16 bytes to a group and writes a column-major C in pieces of four
+            // rows: for operands of up to 128 bytes per row, and for a column-major C, the groups of eight rows stay.)
+            const bool strips_suit = row_bytes > 128 && matC->order == MCSPARSE_ORDER_ROW;
+            const uint32_t stride = !strips_suit ? 0u
+                                                 : strip_stride_of_middle_row(handle->stream, m, static_cast<idx_t>(matA->idxBase),
+                                                                              ia.rows, ia.cols);
+            if (stride != 0) {
+                mcsp::launch_spmm_strip_count(handle->stream, m, nnz, static_cast<idx_t>(matA->idxBase), stride, ia.rows,
+                                              ia.cols, externalBuffer);
+                const uint64_t strip_groups = mcsp::spmm_strip_groups(m, stride);
+                uint32_t strip_blocks = 0;
+                unsigned long long strip_counters[3] = {0, 0, 0};  // span sum, rows of op(B) loaded, longest strip
+                const char* strip_total = static_cast<const char*>(externalBuffer) + l.group_ptr + strip_groups * sizeof(uint32_t);
+                if (hipMemcpyAsync(&strip_blocks, strip_total, sizeof(strip_blocks), hipMemcpyDeviceToHost, handle->stream) != hipSuccess ||
+                    hipMemcpyAsync(strip_counters, span_slot, sizeof(strip_counters), hipMemcpyDeviceToHost, handle->stream) != hipSuccess ||
+                    hipStreamSynchronize(handle->stream) != hipSuccess)
+                    return to_public_status(MCSP_STATUS_INTERNAL_ERROR);
+                if (strip_blocks != 0 && strip_counters[1] * 5 <= counters[1] * 4 &&
+                    mcsp::spmm_strip_schedule_fits(m, nnz, stride, strip_blocks)) {
+                    mcsp::launch_spmm_strip_fill(handle->stream, m, nnz, static_cast<idx_t>(matA->idxBase), stride, ia.rows,
+                                                 ia.cols, externalBuffer);
+                    s.entries = strip_blocks;
+                    s.mean_span = strip_groups != 0 ? strip_counters[0] / strip_groups : 0;
+                    s.blocks = true;
+                    s.stride = stride;
+                    s.longest_group = static_cast<uint32_t>(strip_counters[2] & 0xffffffffull);
+                    s.useful = true;
+                    s.valid = true;
+                    return MCSPARSE_STATUS_SUCCESS;
+                }
+                // not worth it: the offsets of the groups of eight rows are counted again (the region is shared)
+                mcsp::launch_spmm_block_count(handle->stream, m, nnz, static_cast<idx_t>(matA->idxBase), ia.rows, ia.cols,
+                                              externalBuffer);
+            }
             mcsp::launch_spmm_block_fill(handle->stream, m, nnz, static_cast<idx_t>(matA->idxBase), ia.rows, ia.cols,
                                          externalBuffer);
             s.entries = blocks;

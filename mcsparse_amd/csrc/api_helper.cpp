@@ -380,7 +380,7 @@ mcsparseStatus_t mcsparseSpMatGetSpMVPlan(mcsparseSpMatDescr_t d, int* family, i
 mcsparseStatus_t mcsparseSpMatGetSpMMSchedule(mcsparseSpMatDescr_t d, int* state, int64_t* merged_entries) {
     if (d == nullptr || state == nullptr || merged_entries == nullptr)
         return to_public_status(MCSP_STATUS_INVALID_POINTER);
-    *state = !d->schedule.valid ? 0 : (!d->schedule.useful ? 1 : (d->schedule.blocks ? 3 : 2));
+    *state = !d->schedule.valid ? 0 : (!d->schedule.useful ? 1 : (d->schedule.blocks ? (d->schedule.stride != 0 ? 4 : 3) : 2));
     *merged_entries = d->schedule.valid ? static_cast<int64_t>(d->schedule.entries) : 0;
     return MCSPARSE_STATUS_SUCCESS;
 }

@@ -94,7 +94,8 @@ struct SpmmSchedule {
     uint32_t entries = 0;  // length of all merged lists together, or the number of diagonal blocks
     uint64_t mean_span = 0;  // mean distance between the first and the last column of a group
     bool blocks = false;   // the schedule holds diagonal blocks (spmm_blocks.hip) instead of merged lists
-    uint32_t longest_group = 0;  // blocks: the most nonzeros in one group of rows
+    uint32_t longest_group = 0;  // blocks: the most nonzeros in one group of rows (strips: in one strip)
+    uint32_t stride = 0;   // blocks: != 0 says the groups are strips this many rows apart (spmm_strips.hip)
 };
 
 // Column-banded copy of a CSR matrix built by mcsparseSpMV_preprocess inside the caller's buffer
@@ -393,6 +394,28 @@ constexpr uint64_t spmm_block_groups(idx_t m) { return (static_cast<uint64_t>(m)
 // Counts the blocks of every group and scans the counts (the total lands in slot `groups` of the offsets).
 void launch_spmm_block_count(hipStream_t stream, idx_t m, idx_t nnz, idx_t base, const idx_t* row_ptr, const idx_t* col,
                              void* schedule);
+// Strip schedule of a CSR structure (spmm_strips.hip), the third kind: a group is kSpmmStrips strips of
+// kSpmmStripRows consecutive rows, strip q beginning `stride` rows behind strip q - 1; the rows are cut into stretches
+// of kSpmmStrips * stride rows, each holding stride / kSpmmStripRows groups.  Blocks are 16 bytes (see the file), the
+// region is used like the one of the block schedule, and the counters' place also holds the stride.
+constexpr int kSpmmStripRows = 4;
+constexpr int kSpmmStrips = 4;
+constexpr uint64_t spmm_strip_groups(idx_t m, uint32_t stride) {
+    return (static_cast<uint64_t>(m) + static_cast<uint64_t>(kSpmmStrips) * stride - 1) /
+           (static_cast<uint64_t>(kSpmmStrips) * stride) * (stride / kSpmmStripRows);
+}
+// stride is one the schedule can be built with for a matrix of m rows
+bool spmm_strip_stride_usable(idx_t m, uint32_t stride);
+void launch_spmm_strip_count(hipStream_t stream, idx_t m, idx_t nnz, idx_t base, uint32_t stride, const idx_t* row_ptr,
+                             const idx_t* col, void* schedule);
+void launch_spmm_strip_fill(hipStream_t stream, idx_t m, idx_t nnz, idx_t base, uint32_t stride, const idx_t* row_ptr,
+                            const idx_t* col, void* schedule);
+bool spmm_strip_schedule_fits(idx_t m, idx_t nnz, uint32_t stride, uint32_t blocks);
+// Same conditions on the operands as the block schedule (spmm_blocks_usable).
+template <typename T>
+void launch_spmm_strips(hipStream_t stream, const SpmmArgs& a, const void* schedule, uint32_t stride, uint32_t total_blocks,
+                        uint32_t longest_strip, uint64_t mean_span, T alpha, T beta);
+
 // Whether `blocks` blocks of 8 bytes and the order of the groups (4 bytes each) fit the entries' place.
 bool spmm_block_schedule_fits(idx_t m, idx_t nnz, uint32_t blocks);
 // Writes the blocks and the order in which the kernel takes the groups; only after the count, and only when

@@ -146,7 +146,7 @@ def stencil_full():
     return a
 
 
-# preprocess = True runs the kernels that work from a schedule: diagonal blocks (state 3) for N = 64 and 256; for
+# preprocess = True runs the kernels that work from a schedule: blocks over groups of strips (state 4) for N = 64 and 256; for
 # N = 8 merged column lists are built (state 2) but too narrow to use
 @pytest.mark.parametrize("preprocess", [False, True])
 @pytest.mark.parametrize("n", [8, 64, 256])
@@ -155,7 +155,7 @@ def test_config4_stencil_full_size(torch_gpu, handle, oracle, stencil_full, n, p
     rng = np.random.default_rng(n)
     B = rng.uniform(-1, 1, (a.n, n)).astype(np.float32)
     st, got, _ = run_spmm(torch_gpu, handle, a, B, np.zeros((a.m, n), np.float32), 1.0, 0.0, preprocess=preprocess,
-                          expect_schedule=(2 if n == 8 else 3) if preprocess else None)
+                          expect_schedule=(2 if n == 8 else 4) if preprocess else None)
     assert st == 0
     # oracle on a sample of rows: first/last planes, and random interior rows
     rows = np.unique(np.concatenate([np.arange(0, 300), np.arange(a.m - 300, a.m),

@@ -12,8 +12,10 @@ pytestmark = pytest.mark.gpu
 
 
 def run_spmm(torch, handle, a, B, C0, alpha, beta, op_b=api.OP_N, b_order=api.ORDER_ROW, c_order=api.ORDER_ROW,
-             pad_b=0, pad_c=0, preprocess=False, expect_schedule=None):
-    """B is the k x n operand op(B); it is stored as the call's (op_b, b_order) pair requires."""
+             pad_b=0, pad_c=0, preprocess=False, expect_schedule=None, prepare_for_row_major_c=False):
+    """B is the k x n operand op(B); it is stored as the call's (op_b, b_order) pair requires.
+    prepare_for_row_major_c: mcsparseSpMM_preprocess is given a row-major C of the same shape, whatever the call's is
+    (a schedule belongs to the structure of A; which kind is built depends on the operands of the preprocess call)."""
     k, n = B.shape
     dt = a.val.dtype
     # memory image of op(B): row-major k x n  <=>  (N, ROW) or (T, COL)
@@ -45,7 +47,11 @@ def run_spmm(torch, handle, a, B, C0, alpha, beta, op_b=api.OP_N, b_order=api.OR
     assert st == 0 and size >= 128
     buf = torch.empty(size, dtype=torch.uint8, device="cuda")
     if preprocess:
-        assert api.spmm_preprocess(handle, api.OP_N, op_b, alpha, mat, mB, beta, mC, ct, buf) == 0
+        mC_pre = mC
+        if prepare_for_row_major_c:
+            d_C_pre = torch.zeros((a.m, n), dtype=d_C.dtype, device="cuda")
+            mC_pre = api.DnMat(a.m, n, n, d_C_pre, order=api.ORDER_ROW)
+        assert api.spmm_preprocess(handle, api.OP_N, op_b, alpha, mat, mB, beta, mC_pre, ct, buf) == 0
         if expect_schedule is not None:
             wanted = expect_schedule if isinstance(expect_schedule, tuple) else (expect_schedule,)
             assert mat.spmm_schedule()[0] in wanted, mat.spmm_schedule()
@@ -133,8 +139,16 @@ def test_preprocessed_stencil_in_xcd_stretches(torch_gpu, handle, oracle):
     workgroups (the column span of a 48^3 stencil is 4,706 rows), with a last round that is only
     partly filled."""
     a = wl.stencil_27pt(48, dtype=np.float32)
+    # lines of 48 points, a whole number of strips of four rows: state 4, blocks over groups of strips a line apart
     for n in (64, 40):
-        check(torch_gpu, handle, oracle, a, n, 1.0, 0.0, preprocess=True, expect_schedule=3)
+        check(torch_gpu, handle, oracle, a, n, 1.0, 0.0, preprocess=True, expect_schedule=4)
+    # for a column-major C the groups of eight rows are built, unless the call prepared for a row-major one
+    check(torch_gpu, handle, oracle, a, 64, 0.5, -1.0, preprocess=True, expect_schedule=3, c_order=api.ORDER_COL)
+    check(torch_gpu, handle, oracle, a, 64, 0.5, -1.0, preprocess=True, expect_schedule=4, c_order=api.ORDER_COL,
+          prepare_for_row_major_c=True)
+    # lines of 46 points: no stride the strips could use, blocks over groups of eight consecutive rows (state 3)
+    a = wl.stencil_27pt(46, dtype=np.float32)
+    check(torch_gpu, handle, oracle, a, 64, 1.0, 0.0, preprocess=True, expect_schedule=3)
     check(torch_gpu, handle, oracle, a, 64, 0.5, -1.0, preprocess=True, expect_schedule=3, c_order=api.ORDER_COL)
     check(torch_gpu, handle, oracle, a, 16, 1.0, 0.0, preprocess=True, expect_schedule=2)  # too narrow for blocks
 
@@ -210,7 +224,7 @@ def test_schedule_is_dropped_with_other_buffer_or_pointers(torch_gpu, handle, or
     assert mat.spmm_schedule()[0] == 0
 
 
-@pytest.mark.parametrize("grid,n", [(10, 64), (40, 64), (40, 128), (10, 16)])
+@pytest.mark.parametrize("grid,n", [(10, 64), (40, 64), (40, 128), (41, 64), (41, 128), (10, 16)])
 def test_overwritten_schedule_stays_in_bounds(torch_gpu, handle, grid, n):
     """The reference's preprocess is a no-op, so a caller written against it may reuse the scratch
     buffer between preprocess and SpMM.  The schedule is then garbage: the product may be wrong, but
@@ -225,7 +239,7 @@ def test_overwritten_schedule_stays_in_bounds(torch_gpu, handle, grid, n):
     st, size = api.spmm_buffer_size(handle, api.OP_N, api.OP_N, 1.0, mat, mB, 0.0, mC, api.R_32F)
     buf = torch.empty(size, dtype=torch.uint8, device="cuda")
     assert api.spmm_preprocess(handle, api.OP_N, api.OP_N, 1.0, mat, mB, 0.0, mC, api.R_32F, buf) == 0
-    assert mat.spmm_schedule()[0] in (2, 3)
+    assert mat.spmm_schedule()[0] == (4 if grid == 40 else 3 if grid == 41 else 2), mat.spmm_schedule()
     gen = torch.Generator(device="cuda")
     gen.manual_seed(3)
     for fill in (0xFF, None, 0x00):
@@ -278,16 +292,59 @@ def columns_from_blocks(ptr, words, m):
     return rows
 
 
-@pytest.mark.parametrize("shape", ["stencil", "banded", "unsorted"])
+def read_strip_blocks(torch, buf, m):
+    """The strip schedule as it lies in the buffer: the stride among the counters, offsets per group, 16-byte blocks."""
+    def align(x):
+        return (x + 127) // 128 * 128
+    raw = buf.cpu().numpy()
+    counters_at = align(4 * ((m + 3) // 4 + 1))
+    stride = int(raw[counters_at + 24:counters_at + 28].view(np.uint32)[0])
+    groups = (m + 4 * stride - 1) // (4 * stride) * (stride // 4)
+    ptr = raw[:4 * (groups + 1)].view(np.uint32)
+    at = counters_at + 128
+    words = raw[at:at + 16 * int(ptr[groups])].view(np.uint32).reshape(-1, 4)
+    return stride, ptr, words
+
+
+def columns_from_strip_blocks(stride, ptr, words, m):
+    """Expands the blocks of the groups of strips into every row's column sequence (zero-based).  Group g of the
+    stretch t of 4 * stride rows holds the rows t * 4 * stride + q * stride + 4 * g + i (strip q, row i); bit
+    3 * (4 * q + i) + p of a block's 48 bits says that this row holds column c + i + p."""
+    rows = [[] for _ in range(m)]
+    per_stretch = stride // 4
+    for g in range(len(ptr) - 1):
+        g0 = g // per_stretch * 4 * stride + g % per_stretch * 4
+        for c, shape, lo, hi in words[ptr[g]:ptr[g + 1]]:
+            c, shape, held = int(np.int32(c)), int(shape), int(lo) | (int(hi) << 32)
+            n, j_first, j_last = shape & 15, (shape >> 4) & 15, (shape >> 8) & 15
+            assert 1 <= n <= 3 and held != 0 and held >> 48 == 0
+            needed = set()
+            for r in range(16):
+                for p in range(3):
+                    if (held >> (3 * r + p)) & 1:
+                        assert p < n
+                        row = g0 + (r // 4) * stride + r % 4
+                        assert row < m
+                        rows[row].append(c + r % 4 + p)
+                        needed.add(r % 4 + p)
+            assert j_first == min(needed) and j_last == max(needed)
+    return rows
+
+
+@pytest.mark.parametrize("shape", ["stencil", "stencil41", "banded", "unsorted", "banded69", "unsorted69"])
 def test_blocks_cover_every_nonzero_once_and_in_storage_order(torch_gpu, handle, shape):
     """Structural outputs are bit-exact: the blocks of a group, expanded, are the rows' column indices as stored."""
     torch = torch_gpu
     rng = np.random.default_rng(3)
     if shape == "stencil":
-        a = wl.stencil_27pt(40, dtype=np.float32).with_base(1)
+        a = wl.stencil_27pt(40, dtype=np.float32).with_base(1)   # lines of 40 points: groups of strips a line apart
+    elif shape == "stencil41":
+        a = wl.stencil_27pt(41, dtype=np.float32).with_base(1)   # no usable stride: groups of eight consecutive rows
     else:
         m = 4099
         offsets = np.array([-70, -69, -68, -2, -1, 0, 1, 2, 3, 64, 65, 66, 67, 68, 69])  # runs of 3, 6 (cut at 4) and 6
+        if shape.endswith("69"):
+            offsets[:3] -= 1   # the runs begin 69 and 66 apart: no distance the strips could use, groups of eight rows
         rows = []
         for r in range(m):
             c = r + offsets
@@ -296,7 +353,7 @@ def test_blocks_cover_every_nonzero_once_and_in_storage_order(torch_gpu, handle,
                 c = c[::2]                      # a row with holes breaks the blocks around it
             if r % 211 == 7:
                 c = np.zeros(0, np.int64)       # an empty row
-            if shape == "unsorted" and r % 120 == 0:
+            if shape.startswith("unsorted") and r % 120 == 0:
                 c = rng.permutation(c)          # consumed in storage order: single nonzeros around intact blocks
             rows.append(c)
         ptr = np.concatenate([[0], np.cumsum([len(c) for c in rows])]).astype(np.int32)
@@ -311,11 +368,17 @@ def test_blocks_cover_every_nonzero_once_and_in_storage_order(torch_gpu, handle,
     buf = torch.zeros(size, dtype=torch.uint8, device="cuda")
     assert api.spmm_preprocess(handle, api.OP_N, api.OP_N, 1.0, mat, mB, 0.0, mC, api.R_32F, buf) == 0
     state, blocks = mat.spmm_schedule()
-    assert state == 3, (state, blocks)
+    # the stencils' kind follows from the length of their lines; the banded matrices get whichever loads fewer rows
+    assert state == {"stencil": 4, "stencil41": 3, "banded69": 3, "unsorted69": 3}.get(shape, state) and state in (3, 4), (state, blocks)
     torch.cuda.synchronize()
-    ptr, words = read_blocks(torch, buf, a.m)
+    if state == 4:
+        stride, ptr, words = read_strip_blocks(torch, buf, a.m)
+        assert stride == (40 if shape == "stencil" else 68)
+        got = columns_from_strip_blocks(stride, ptr, words, a.m)
+    else:
+        ptr, words = read_blocks(torch, buf, a.m)
+        got = columns_from_blocks(ptr, words, a.m)
     assert int(ptr[-1]) == blocks and (np.diff(ptr.astype(np.int64)) >= 0).all()
-    got = columns_from_blocks(ptr, words, a.m)
     for r in range(a.m):
         want = (a.col[a.ptr[r] - a.base:a.ptr[r + 1] - a.base].astype(np.int64) - a.base).tolist()
         assert got[r] == want, (r, got[r], want)
@@ -328,7 +391,7 @@ def test_blocks_banded_matrix_with_broken_rows(torch_gpu, handle, oracle, dtype,
     count that leaves the last group short; every width of lane group; both layouts of C."""
     rng = np.random.default_rng(5)
     m, k = 3003, 3100
-    offsets = np.array([-70, -69, -68, -2, -1, 0, 1, 2, 3, 64, 65, 66, 67, 68, 69, 200])
+    offsets = np.array([-71, -70, -69, -2, -1, 0, 1, 2, 3, 64, 65, 66, 67, 68, 69, 201])  # runs 69, 66 and 137 apart
     rows = []
     for r in range(m):
         c = r + offsets
@@ -370,11 +433,75 @@ def test_blocks_row_ignores_rows_of_b_only_its_neighbours_use(torch_gpu, handle)
             assert np.all(got[r] == 3.0), r
 
 
-def test_blocks_schedule_used_with_a_wider_operand_than_it_was_built_for(torch_gpu, handle, oracle):
+def grid_9pt(line, lines, dtype, rng, broken=False):
+    """9-point stencil on `lines` grid lines of `line` points, numbered line by line; broken: rows with holes, empty
+    rows, unsorted rows, one row with 2500 nonzeros (its group is too long to cover) and a duplicate column."""
+    m = line * lines
+    rows = []
+    for r in range(m):
+        y, x = divmod(r, line)
+        c = [yy * line + xx for yy in (y - 1, y, y + 1) for xx in (x - 1, x, x + 1) if 0 <= yy < lines and 0 <= xx < line]
+        c = np.array(c, np.int64)
+        if broken:
+            if r % 97 == 5:
+                c = c[::2]
+            if r % 211 == 7:
+                c = np.zeros(0, np.int64)
+            if r % 120 == 0:
+                c = rng.permutation(c)
+            if r % 333 == 9 and len(c) > 2:
+                c = np.concatenate([c[:2], c[1:]])     # a column twice in a row
+            if r == 1000:
+                c = rng.choice(m, 2500, replace=False)
+        rows.append(c)
+    ptr = np.concatenate([[0], np.cumsum([len(c) for c in rows])]).astype(np.int32)
+    return wl.Csr(m, m, ptr, np.concatenate(rows).astype(np.int32), rng.uniform(-1, 1, int(ptr[-1])).astype(dtype))
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("n", [20, 36, 64, 72, 128, 260])
+def test_strips_grid_with_broken_rows(torch_gpu, handle, oracle, dtype, n):
+    """Groups of strips a grid line apart (lines of 20 points, 151 of them: the last stretch of four lines is short),
+    rows with holes, empty, unsorted and overlong rows, duplicates; panels of 16 lanes; both layouts of C."""
+    a = grid_9pt(20, 151, dtype, np.random.default_rng(6), broken=True)
+    row_bytes = n * np.dtype(dtype).itemsize
+    # strips for operands of 129 to 1024 bytes per row, groups of eight rows from 65 bytes, merged column lists otherwise
+    want = 4 if 128 < row_bytes <= 1024 else 3 if 64 < row_bytes <= 128 else (1, 2)
+    for c_order in (api.ORDER_ROW, api.ORDER_COL):
+        check(torch_gpu, handle, oracle, a, n, 1.0, 0.0, preprocess=True, expect_schedule=want, c_order=c_order,
+              prepare_for_row_major_c=True)
+    check(torch_gpu, handle, oracle, a.with_base(1), n, -0.5, 1.5, preprocess=True, expect_schedule=want, pad_b=4, pad_c=8)
+    check(torch_gpu, handle, oracle, a, n, 0.5, -1.0, preprocess=True, expect_schedule=want, c_order=api.ORDER_COL, pad_c=4,
+          prepare_for_row_major_c=True)
+
+
+def test_strips_row_ignores_rows_of_b_only_other_strips_use(torch_gpu, handle):
+    """A block of a group of strips loads rows of op(B) for up to sixteen rows of A; a row must only see the ones it
+    names (0 * inf = NaN)."""
+    line, lines, n = 16, 64, 64
+    a = grid_9pt(line, lines, np.float32, np.random.default_rng(1))
+    a = wl.Csr(a.m, a.n, a.ptr, a.col, np.ones(a.nnz, np.float32))
+    B = np.ones((a.n, n), np.float32)
+    hot = 20 * line + 7
+    B[hot, :] = np.inf
+    st, got, _ = run_spmm(torch_gpu, handle, a, B, np.zeros((a.m, n), np.float32), 1.0, 0.0, preprocess=True,
+                          expect_schedule=4)
+    assert st == 0
+    names = {r for r in range(a.m) if hot in a.col[a.ptr[r]:a.ptr[r + 1]]}
+    assert len(names) == 9
+    for r in range(a.m):
+        if r in names:
+            assert np.all(np.isinf(got[r])), r
+        else:
+            assert np.all(got[r] == float(a.ptr[r + 1] - a.ptr[r])), r
+
+
+@pytest.mark.parametrize("grid,state", [(40, 4), (41, 3)])
+def test_blocks_schedule_used_with_a_wider_operand_than_it_was_built_for(torch_gpu, handle, oracle, grid, state):
     """The schedule belongs to the structure of A: built with a 64-column operand it also serves 256 columns (cut into
     panels) and 8 columns (too narrow for its kernel: the schedule-free kernel runs)."""
     torch = torch_gpu
-    a = wl.stencil_27pt(40, dtype=np.float32)
+    a = wl.stencil_27pt(grid, dtype=np.float32)
     rng = np.random.default_rng(9)
     d_ptr, d_col, d_val = dev(torch, a.ptr), dev(torch, a.col), dev(torch, a.val)
     mat = api.SpMat(a.m, a.n, a.nnz, d_ptr, d_col, d_val)
@@ -389,7 +516,7 @@ def test_blocks_schedule_used_with_a_wider_operand_than_it_was_built_for(torch_g
         assert st == 0
     buf = torch.empty(max(sizes.values()), dtype=torch.uint8, device="cuda")
     assert api.spmm_preprocess(handle, api.OP_N, api.OP_N, 1.0, mat, ops[64][3], 0.0, ops[64][4], api.R_32F, buf) == 0
-    assert mat.spmm_schedule()[0] == 3
+    assert mat.spmm_schedule()[0] == state
     for n in (64, 256, 8):
         B, d_B, d_C, mB, mC = ops[n]
         assert api.spmm(handle, api.OP_N, api.OP_N, 1.0, mat, mB, 0.0, mC, api.R_32F, buf) == 0
