@@ -455,8 +455,11 @@ mcsparseStatus_t mcsparseSpMatSetSpMVPlan(mcsparseSpMatDescr_t spMatDescr, int f
 
 /* What mcsparseSpMM_preprocess left on a CSR descriptor:
  * state 0 = no schedule, 1 = built but the rows share too few columns for it to pay off
- * (SpMM ignores it), 2 = SpMM uses it when called with the same buffer and CSR arrays.
- * merged_entries = total length of the merged column lists of all row groups (compare with nnz). */
+ * (SpMM ignores it); 2, 3, 4 = SpMM uses it when called with the same buffer and CSR arrays:
+ * 2 = merged column lists of groups of four rows, 3 = diagonal blocks over groups of eight consecutive rows,
+ * 4 = diagonal blocks over groups of four strips of four rows a fixed distance (a grid line) apart.
+ * merged_entries = total length of the merged column lists of all row groups (compare with nnz), or the
+ * number of blocks. */
 mcsparseStatus_t mcsparseSpMatGetSpMMSchedule(mcsparseSpMatDescr_t spMatDescr, int* state, int64_t* merged_entries);
 
 /* Optional preparation of y = alpha*op(A)*x + beta*y for a matrix that is multiplied many times (the
