@@ -387,6 +387,7 @@ def run_workload(name, args, ctx, steps=None, warmup=None, with_cpu=True):
                                       "second pass of the same steps"},
         "spmv_plan": {"family": plan[0], "lanes_per_row": plan[1]} if plan else None,
         "spmv_preprocess": {"state": banded[0], "bands": banded[1], "rows_per_tile": banded[2]} if banded else None,
+        "spmm_schedule": mat0.spmm_schedule()[0] if mat0 is not None and kind.startswith("spmm") else None,
         "roofline": {"bound": "hbm", "achieved": round(achieved, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4),
                      "traffic": traffic[0] if traffic else None,

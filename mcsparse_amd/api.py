@@ -148,14 +148,16 @@ class SpMat:
         check(self.lib.mcsparseSpMatSetSpMVBandBytes(self._d, band_bytes), "mcsparseSpMatSetSpMVBandBytes")
 
     def spmv_preprocess_state(self):
-        """(state, bands, rows_per_tile) left by mcsparseSpMV_preprocess; state 2 = banded copy in use."""
+        """(state, bands, rows_per_tile) left by mcsparseSpMV_preprocess; state 2 = banded copy, 3 = copy in column
+        order (both in use), 0 = none."""
         state, bands, rows = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
         check(self.lib.mcsparseSpMatGetSpMVPreprocess(self._d, ctypes.byref(state), ctypes.byref(bands),
                                                       ctypes.byref(rows)))
         return state.value, bands.value, rows.value
 
     def spmm_schedule(self):
-        """(state, merged_entries) left by mcsparseSpMM_preprocess; state 2 = in use."""
+        """(state, entries) left by mcsparseSpMM_preprocess; state 2 = merged column lists, 3 = diagonal blocks over
+        groups of eight rows, 4 = diagonal blocks over groups of strips (all three in use), 1 = built and declined."""
         state, entries = ctypes.c_int(), ctypes.c_int64()
         check(self.lib.mcsparseSpMatGetSpMMSchedule(self._d, ctypes.byref(state), ctypes.byref(entries)))
         return state.value, entries.value

@@ -475,6 +475,28 @@ def test_strips_grid_with_broken_rows(torch_gpu, handle, oracle, dtype, n):
           prepare_for_row_major_c=True)
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_strips_with_more_values_per_strip_than_the_copy_in_lds_holds(torch_gpu, handle, oracle, dtype):
+    """A strip's values are copied into LDS when they are at most 512 bytes; beyond that the blocks read them where
+    they lie: a 27-point stencil in fp64 (4 rows x 27 x 8 bytes), a 7 x 7 stencil on a plane grid in fp32 (4 x 49 x 4)."""
+    if dtype == np.float64:
+        a = wl.stencil_27pt(16, dtype=dtype)
+    else:
+        line, lines = 24, 40
+        rng = np.random.default_rng(2)
+        rows = []
+        for r in range(line * lines):
+            y, x = divmod(r, line)
+            rows.append(np.array([yy * line + xx for yy in range(y - 3, y + 4) for xx in range(x - 3, x + 4)
+                                  if 0 <= yy < lines and 0 <= xx < line], np.int64))
+        ptr = np.concatenate([[0], np.cumsum([len(c) for c in rows])]).astype(np.int32)
+        a = wl.Csr(line * lines, line * lines, ptr, np.concatenate(rows).astype(np.int32),
+                   rng.uniform(-1, 1, int(ptr[-1])).astype(dtype))
+    for n in (48, 64):
+        check(torch_gpu, handle, oracle, a, n, 1.0, 0.0, preprocess=True, expect_schedule=4)
+        check(torch_gpu, handle, oracle, a.with_base(1), n, -1.5, 0.5, preprocess=True, expect_schedule=4, pad_b=4, pad_c=4)
+
+
 def test_strips_row_ignores_rows_of_b_only_other_strips_use(torch_gpu, handle):
     """A block of a group of strips loads rows of op(B) for up to sixteen rows of A; a row must only see the ones it
     names (0 * inf = NaN)."""
