@@ -222,7 +222,7 @@ constexpr int strip_room() { return strip_capacity<T>() + 2 * (16 / static_cast<
 // the four lanes of a strip then copy its values into LDS once, in whole 16-byte pieces, and the blocks read them
 // there.
 template <typename T, bool WIDE, bool STAGED>
-__global__ __launch_bounds__(kBlock) void spmm_strips_kernel(idx_t m, idx_t n, idx_t base, uint32_t stride,
+__global__ __launch_bounds__(kBlock, 3) void spmm_strips_kernel(idx_t m, idx_t n, idx_t base, uint32_t stride,
                                                              const idx_t* __restrict__ row_ptr,
                                                              const idx_t* __restrict__ col, const T* __restrict__ val,
                                                              const uint32_t* __restrict__ block_ptr,
