@@ -41,6 +41,11 @@ struct StripCounters {
     unsigned int stride;          // rows between the strips of a group
 };
 
+struct StripPartial {
+    unsigned long long span, loads;
+    unsigned int longest, unused;
+};
+
 __global__ void zero_strip_counters_kernel(StripCounters* c, uint32_t stride) {
     c->span_sum = 0;
     c->loads = 0;
@@ -54,117 +59,205 @@ __device__ __forceinline__ uint64_t first_row_of_group(uint64_t group, uint32_t 
     return group / per_tile * (static_cast<uint64_t>(Q) * stride) + group % per_tile * H;
 }
 
-// One thread covers the nonzeros of one group with blocks.  It merges the sixteen rows by the key column - (row
-// inside its strip): rows of one strip on one diagonal of the matrix share a key, and so do rows of different
-// strips that name the same rows of op(B).  A block grows while the next key follows the last one, up to D keys;
-// which rows hold a key is recorded bit by bit, so any set of rows may.  Every row's nonzeros are consumed in storage
-// order, whatever that order is: the values of a row inside a block are always the next ones it has not used yet.
+// x of the lane `xor_mask` away inside a row of 16 lanes (quad permutes and mirrors, as in group_sum).
+template <int CTRL>
+__device__ __forceinline__ int dpp_int(int v) {
+    return __builtin_amdgcn_update_dpp(0, v, CTRL, 0xF, 0xF, false);
+}
+// min / max / or over the sixteen lanes of a group; every lane ends with the result
+template <typename F>
+__device__ __forceinline__ int group16_reduce(int v, F f) {
+    v = f(v, dpp_int<kDppQuadXor1>(v));
+    v = f(v, dpp_int<kDppQuadXor2>(v));
+    v = f(v, dpp_int<kDppRowHalfMirror>(v));
+    v = f(v, dpp_int<kDppRowMirror>(v));
+    return v;
+}
+
+// Sixteen lanes cover the nonzeros of one group with blocks, lane r walking row r of the group.  The rows are merged
+// by the key column - (row inside its strip): rows of one strip on one diagonal of the matrix share a key, and so do
+// rows of different strips that name the same rows of op(B).  A step takes the lowest key among the rows' next
+// nonzeros; a block grows while that key follows the last one, up to D keys; which rows hold a key is recorded bit
+// by bit, so any set of rows may.  Every row's nonzeros are consumed in storage order, whatever that order is: the
+// values of a row inside a block are always the next ones it has not used yet.
+constexpr int kCoverGroupsPerBlock = kBlock / kLanes;
+constexpr int kColRoom = 136;  // entries of a strip's copy: 128 and the neighbours its first and last piece bring along
 template <bool FILL>
-__global__ __launch_bounds__(kWave) void strip_cover_kernel(idx_t m, idx_t base, uint32_t stride,
-                                                            const idx_t* __restrict__ row_ptr,
-                                                            const idx_t* __restrict__ col,
-                                                            uint32_t* __restrict__ block_ptr, uint4* __restrict__ blocks,
-                                                            StripCounters* __restrict__ counters) {
+__global__ __launch_bounds__(kBlock) void strip_cover_kernel(idx_t m, idx_t nnz, idx_t base, uint32_t stride,
+                                                             const idx_t* __restrict__ row_ptr,
+                                                             const idx_t* __restrict__ col,
+                                                             uint32_t* __restrict__ block_ptr, uint4* __restrict__ blocks,
+                                                             StripCounters* __restrict__ counters,
+                                                             StripPartial* __restrict__ partials) {
+    __shared__ __attribute__((aligned(16))) idx_t s_col[kCoverGroupsPerBlock * Q][kColRoom];
     const uint64_t groups = spmm_strip_groups(m, stride);
-    const uint64_t group = static_cast<uint64_t>(blockIdx.x) * kWave + threadIdx.x;
+    const uint64_t group = static_cast<uint64_t>(blockIdx.x) * kCoverGroupsPerBlock + threadIdx.x / kLanes;
+    const uint32_t lane = threadIdx.x % kLanes;
+    // (lane groups behind the last group leave a zero for the scan, or nothing, and add nothing to the counters)
+    const bool slot_exists = group <= groups;
+    auto imin = [](int a, int b) { return a < b ? a : b; };
+    auto imax = [](int a, int b) { return a > b ? a : b; };
+    auto ior = [](int a, int b) { return a | b; };
     uint32_t count = 0;
-    unsigned long long loads = 0;
-    uint32_t first_col = 0xffffffffu, last_col = 0;
-    uint32_t longest_strip = 0;
+    uint32_t loads = 0;
+    int first_col = 0x7fffffff, last_col = -1;
+    int longest_strip = 0;
     if (group < groups) {
-        idx_t i[R], e[R];
-        const uint64_t g0 = first_row_of_group(group, stride);
-        idx_t group_nnz = 0;
-#pragma unroll
-        for (int q = 0; q < Q; ++q) {
-            idx_t strip_nnz = 0;
-#pragma unroll
-            for (int h = 0; h < H; ++h) {
-                const uint64_t row = g0 + static_cast<uint64_t>(q) * stride + h;
-                const bool exists = row < static_cast<uint64_t>(m);
-                i[q * H + h] = exists ? row_ptr[row] - base : 0;
-                e[q * H + h] = exists ? row_ptr[row + 1] - base : 0;
-                strip_nnz += e[q * H + h] - i[q * H + h];
-            }
-            group_nnz += strip_nnz;
-            longest_strip = strip_nnz > longest_strip ? strip_nnz : longest_strip;
-        }
-        if (group_nnz <= kSpmmMaxMergedGroup) {
-            uint32_t out = FILL ? block_ptr[group] : 0;
-            auto key_of = [&](int r) -> int {
-                if (i[r] >= e[r]) return kNoKey;
-                const uint32_t c = static_cast<uint32_t>(col[i[r]] - base);
-                first_col = c < first_col ? c : first_col;
-                last_col = c > last_col ? c : last_col;
-                return static_cast<int>(c) - r % H;
-            };
-            int key[R];
-#pragma unroll
-            for (int r = 0; r < R; ++r) key[r] = key_of(r);
-            int start = 0;
-            uint32_t width = 0;
-            unsigned long long held = 0;
-            auto flush = [&]() {
-                if (width == 0) return;
-                uint32_t j_first = 0xffu, j_last = 0;
-#pragma unroll
-                for (int r = 0; r < R; ++r) {
-#pragma unroll
-                    for (int p = 0; p < D; ++p) {
-                        if ((held >> (3 * r + p)) & 1ull) {
-                            const uint32_t j = static_cast<uint32_t>(r % H + p);
-                            j_first = j < j_first ? j : j_first;
-                            j_last = j > j_last ? j : j_last;
-                        }
+        const uint64_t row = first_row_of_group(group, stride) + static_cast<uint64_t>(lane / H) * stride + lane % H;
+        const bool exists = row < static_cast<uint64_t>(m);
+        idx_t i = exists ? row_ptr[row] - base : 0;
+        const idx_t e = exists ? row_ptr[row + 1] - base : 0;
+        const int row_nnz = static_cast<int>(e - i);
+        int strip_nnz = row_nnz + dpp_int<kDppQuadXor1>(row_nnz);
+        strip_nnz += dpp_int<kDppQuadXor2>(strip_nnz);
+        const int group_nnz = strip_nnz + dpp_int<kDppRowHalfMirror>(strip_nnz) +
+                              dpp_int<kDppRowMirror>(strip_nnz + dpp_int<kDppRowHalfMirror>(strip_nnz));
+        if (static_cast<idx_t>(group_nnz) <= kSpmmMaxMergedGroup) {
+            longest_strip = group16_reduce(strip_nnz, imax);
+            const uint32_t out = FILL ? block_ptr[group] : 0;
+            // A strip's column indices are one contiguous stretch: its four lanes copy it into LDS in 16-byte pieces
+            // first (read entry by entry while the merge goes on, the lines would be fetched again and again: the
+            // many groups in flight push each other's out of L2).  Longer strips, or an unaligned array, are read in
+            // place.
+            const idx_t strip_begin = static_cast<idx_t>(dpp_int<0x00>(static_cast<int>(i)));   // the quad's first lane
+            const idx_t strip_end = static_cast<idx_t>(dpp_int<0xFF>(static_cast<int>(e)));     // the quad's last lane
+            const idx_t stage_first = strip_begin & ~idx_t(3);
+            const bool staged = strip_end >= strip_begin && strip_end - stage_first <= static_cast<idx_t>(kColRoom) &&
+                                reinterpret_cast<uintptr_t>(col) % 16 == 0;
+            idx_t* mine_staged = s_col[(threadIdx.x / kLanes) * Q + lane / H];
+            if (staged) {
+                typedef idx_t Piece __attribute__((ext_vector_type(4)));
+                const idx_t pieces = (strip_end - stage_first + 3) / 4;  // at most kColRoom / 4
+                const idx_t whole_pieces = nnz / 4;                      // pieces that lie inside the array altogether
+                for (idx_t piece = lane % H; piece < pieces; piece += H) {
+                    const idx_t at = stage_first / 4 + piece;
+                    if (at < whole_pieces) {
+                        reinterpret_cast<Piece*>(mine_staged)[piece] = reinterpret_cast<const Piece*>(col)[at];
+                    } else {  // the array's last entries, when they do not fill a piece
+                        for (idx_t t = at * 4; t < nnz; ++t) mine_staged[t - stage_first] = col[t];
                     }
                 }
-                if (FILL) {
-                    blocks[out + count] = make_uint4(static_cast<uint32_t>(start), width | (j_first << 4) | (j_last << 8),
-                                                     static_cast<uint32_t>(held), static_cast<uint32_t>(held >> 32));
+            }
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+            int start = 0;
+            uint32_t width = 0;
+            uint32_t mine = 0;  // bit p: this lane's row holds diagonal p of the block being grown
+            auto flush = [&]() {
+                if (width == 0) return;
+                // the rows of op(B) the held diagonals need, and the 48 bits
+                int j_lo = 0xff, j_hi = 0;
+#pragma unroll
+                for (int p = 0; p < D; ++p) {
+                    if ((mine >> p) & 1u) {
+                        j_lo = imin(j_lo, static_cast<int>(lane % H) + p);
+                        j_hi = imax(j_hi, static_cast<int>(lane % H) + p);
+                    }
                 }
+                const uint32_t j_first = static_cast<uint32_t>(group16_reduce(j_lo, imin));
+                const uint32_t j_last = static_cast<uint32_t>(group16_reduce(j_hi, imax));
+                const unsigned long long my_bits = static_cast<unsigned long long>(mine) << (3 * lane);
+                const uint32_t held_lo = static_cast<uint32_t>(group16_reduce(static_cast<int>(static_cast<uint32_t>(my_bits)), ior));
+                const uint32_t held_hi = static_cast<uint32_t>(group16_reduce(static_cast<int>(static_cast<uint32_t>(my_bits >> 32)), ior));
+                if (FILL && lane == 0)
+                    blocks[out + count] = make_uint4(static_cast<uint32_t>(start), width | (j_first << 4) | (j_last << 8), held_lo, held_hi);
                 ++count;
                 loads += j_last - j_first + 1;
                 width = 0;
-                held = 0;
+                mine = 0;
             };
             while (true) {
-                int low = kNoKey;
-#pragma unroll
-                for (int r = 0; r < R; ++r) low = key[r] < low ? key[r] : low;
-                if (low == kNoKey) break;
+                int key = kNoKey;
+                if (i < e) {
+                    const int c = static_cast<int>((staged ? mine_staged[i - stage_first] : col[i]) - base);
+                    key = c - static_cast<int>(lane % H);
+                }
+                const int low = group16_reduce(key, imin);
+                if (low == kNoKey) break;  // the whole lane group
                 if (!(width != 0 && width < static_cast<uint32_t>(D) && low == start + static_cast<int>(width))) {
                     flush();
                     start = low;
                 }
                 const uint32_t p = width++;
-#pragma unroll
-                for (int r = 0; r < R; ++r) {
-                    if (key[r] == low) {
-                        held |= 1ull << (3 * r + p);
-                        ++i[r];
-                        key[r] = key_of(r);
-                    }
+                if (key == low) {
+                    mine |= 1u << p;
+                    const int c = key + static_cast<int>(lane % H);
+                    first_col = imin(first_col, c);
+                    last_col = imax(last_col, c);
+                    ++i;
                 }
             }
             flush();
-        } else {
-            longest_strip = 0;  // row by row in the kernel: no evidence about the strips
+            first_col = group16_reduce(first_col, imin);
+            last_col = group16_reduce(last_col, imax);
         }
     }
     if (!FILL) {
-        if (group <= groups) block_ptr[group] = count;  // slot `groups` receives the total after the scan
-        unsigned long long span = count != 0 ? last_col - first_col : 0;
+        if (lane == 0 && slot_exists) block_ptr[group] = count;  // slot `groups` receives the total after the scan
+        // the four groups of a wavefront add to the counters together (every lane of a group holds the group's figures)
+        unsigned long long span = count != 0 ? static_cast<unsigned long long>(last_col - first_col) : 0ull;
+        unsigned long long all_loads = loads;
+        int longest = count != 0 ? longest_strip : 0;
 #pragma unroll
-        for (int off = kWave / 2; off > 0; off >>= 1) {
+        for (int off = kLanes; off < kWave; off <<= 1) {
             span += __shfl_xor(span, off, kWave);
-            loads += __shfl_xor(loads, off, kWave);
-            longest_strip = max(longest_strip, static_cast<uint32_t>(__shfl_xor(static_cast<int>(longest_strip), off, kWave)));
+            all_loads += __shfl_xor(all_loads, off, kWave);
+            longest = imax(longest, __shfl_xor(longest, off, kWave));
         }
-        if (lane_id() == 0) {
-            if (span != 0) atomicAdd(&counters->span_sum, span);
-            if (loads != 0) atomicAdd(&counters->loads, loads);
-            if (longest_strip != 0) atomicMax(&counters->longest_strip, longest_strip);
+        // and the wavefronts of the workgroup: adds of all workgroups to the three counters would queue on one line
+        // (a millisecond for 2 M rows), so every workgroup leaves its figures in a slot of its own where there is room
+        __shared__ StripPartial s_part[kBlock / kWave];
+        if (lane_id() == 0) s_part[threadIdx.x / kWave] = {span, all_loads, static_cast<unsigned int>(longest), 0u};
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            StripPartial sum = s_part[0];
+#pragma unroll
+            for (int w = 1; w < kBlock / kWave; ++w) {
+                sum.span += s_part[w].span;
+                sum.loads += s_part[w].loads;
+                sum.longest = sum.longest > s_part[w].longest ? sum.longest : s_part[w].longest;
+            }
+            if (partials != nullptr) {
+                partials[blockIdx.x] = sum;
+            } else {
+                if (sum.span != 0) atomicAdd(&counters->span_sum, sum.span);
+                if (sum.loads != 0) atomicAdd(&counters->loads, sum.loads);
+                if (sum.longest != 0) atomicMax(&counters->longest_strip, sum.longest);
+            }
         }
+    }
+}
+
+// The figures the workgroups of the count pass left, added up into the counters (one workgroup, no atomics).
+__global__ __launch_bounds__(kBlock) void strip_counters_sum_kernel(const StripPartial* __restrict__ partials, uint32_t count,
+                                                                    StripCounters* __restrict__ counters) {
+    __shared__ StripPartial s_part[kBlock / kWave];
+    StripPartial sum = {0ull, 0ull, 0u, 0u};
+    for (uint32_t i = threadIdx.x; i < count; i += kBlock) {
+        const StripPartial p = partials[i];
+        sum.span += p.span;
+        sum.loads += p.loads;
+        sum.longest = sum.longest > p.longest ? sum.longest : p.longest;
+    }
+#pragma unroll
+    for (int off = 1; off < kWave; off <<= 1) {
+        sum.span += __shfl_xor(sum.span, off, kWave);
+        sum.loads += __shfl_xor(sum.loads, off, kWave);
+        const unsigned int other = static_cast<unsigned int>(__shfl_xor(static_cast<int>(sum.longest), off, kWave));
+        sum.longest = sum.longest > other ? sum.longest : other;
+    }
+    if (lane_id() == 0) s_part[threadIdx.x / kWave] = sum;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int w = 1; w < kBlock / kWave; ++w) {
+            sum.span += s_part[w].span;
+            sum.loads += s_part[w].loads;
+            sum.longest = sum.longest > s_part[w].longest ? sum.longest : s_part[w].longest;
+        }
+        counters->span_sum = sum.span;
+        counters->loads = sum.loads;
+        counters->longest_strip = sum.longest;
     }
 }
 
@@ -516,10 +609,15 @@ void launch_spmm_strip_count(hipStream_t stream, idx_t m, idx_t nnz, idx_t base,
                              const idx_t* col, void* schedule) {
     const Carved c = carve(m, nnz, stride, schedule);
     const uint64_t slots = spmm_strip_groups(m, stride) + 1;
-    const dim3 grid(static_cast<uint32_t>((slots + kWave - 1) / kWave));
+    const dim3 grid(static_cast<uint32_t>((slots + kCoverGroupsPerBlock - 1) / kCoverGroupsPerBlock));
     hipLaunchKernelGGL(zero_strip_counters_kernel, dim3(1), dim3(1), 0, stream, c.counters, stride);
-    hipLaunchKernelGGL((strip_cover_kernel<false>), grid, dim3(kWave), 0, stream, m, base, stride, row_ptr, col, c.block_ptr,
-                       c.blocks, c.counters);
+    // the place of the blocks, not yet written, takes the workgroups' figures when it has room for them
+    StripPartial* partials = static_cast<uint64_t>(grid.x) * sizeof(StripPartial) <= static_cast<uint64_t>(nnz) * sizeof(uint32_t)
+                                 ? reinterpret_cast<StripPartial*>(c.blocks) : nullptr;
+    hipLaunchKernelGGL((strip_cover_kernel<false>), grid, dim3(kBlock), 0, stream, m, nnz, base, stride, row_ptr, col, c.block_ptr,
+                       c.blocks, c.counters, partials);
+    if (partials != nullptr)
+        hipLaunchKernelGGL(strip_counters_sum_kernel, dim3(1), dim3(kBlock), 0, stream, partials, grid.x, c.counters);
     launch_exclusive_scan_u32(stream, c.block_ptr, slots, c.scan_ws);
 }
 
@@ -527,9 +625,9 @@ void launch_spmm_strip_fill(hipStream_t stream, idx_t m, idx_t nnz, idx_t base, 
                             const idx_t* col, void* schedule) {
     const Carved c = carve(m, nnz, stride, schedule);
     const uint64_t groups = spmm_strip_groups(m, stride);
-    const dim3 grid(static_cast<uint32_t>((groups + 1 + kWave - 1) / kWave));
-    hipLaunchKernelGGL((strip_cover_kernel<true>), grid, dim3(kWave), 0, stream, m, base, stride, row_ptr, col, c.block_ptr,
-                       c.blocks, c.counters);
+    const dim3 grid(static_cast<uint32_t>((groups + kCoverGroupsPerBlock - 1) / kCoverGroupsPerBlock));
+    hipLaunchKernelGGL((strip_cover_kernel<true>), grid, dim3(kBlock), 0, stream, m, nnz, base, stride, row_ptr, col, c.block_ptr,
+                       c.blocks, c.counters, static_cast<StripPartial*>(nullptr));
     hipLaunchKernelGGL(strip_order_kernel, dim3(static_cast<uint32_t>((groups + kOrderChunk - 1) / kOrderChunk)),
                        dim3(kOrderChunk), 0, stream, groups, c.block_ptr, c.blocks, c.order);
 }
