@@ -103,3 +103,64 @@ def test_random_sweep(torch_gpu, handle, oracle, seed):
                 raise AssertionError(name + ": " + str(e)) from e
         else:
             conv.check_csr2csc(torch_gpu, handle, oracle, a, name)
+
+
+def draw_grid_matrix(rng, dtype, base):
+    """A matrix with diagonals: a stencil on `lines` grid lines of `line` points (sometimes in planes), with random
+    rows thinned out, emptied, shuffled or given a duplicate, so that mcsparseSpMM_preprocess builds diagonal blocks
+    over groups of eight rows or over groups of strips a line apart, whichever the matrix suits."""
+    line = int(rng.choice([8, 9, 12, 16, 20, 24, 30, 36, 64]))
+    lines = int(rng.integers(9, 80))
+    planes = int(rng.choice([1, 1, 2, 3]))
+    reach_x = int(rng.choice([1, 1, 2]))
+    reach_y = int(rng.choice([1, 1, 2]))
+    m = line * lines * planes
+    k = m + int(rng.choice([0, 0, 7]))  # sometimes more columns than rows
+    offs = [(dz, dy, dx) for dz in range(-(planes > 1), (planes > 1) + 1) for dy in range(-reach_y, reach_y + 1)
+            for dx in range(-reach_x, reach_x + 1)]
+    rows = []
+    for r in range(m):
+        z, rest = divmod(r, line * lines)
+        y, x = divmod(rest, line)
+        c = np.array([(z + dz) * line * lines + (y + dy) * line + (x + dx) for dz, dy, dx in offs
+                      if 0 <= z + dz < planes and 0 <= y + dy < lines and 0 <= x + dx < line], np.int64)
+        u = rng.random()
+        if u < 0.02:
+            c = c[rng.random(len(c)) < 0.6]
+        elif u < 0.03:
+            c = np.zeros(0, np.int64)
+        elif u < 0.05:
+            c = rng.permutation(c)
+        elif u < 0.06 and len(c) > 1:
+            c = np.concatenate([c[:1], c])
+        rows.append(c)
+    if rng.random() < 0.3:
+        rows[int(rng.integers(0, m))] = rng.choice(k, min(k, 2300), replace=False)  # a group too long to cover
+    ptr = np.concatenate([[0], np.cumsum([len(c) for c in rows])])
+    col = np.concatenate(rows) if int(ptr[-1]) else np.zeros(0, np.int64)
+    val = rng.uniform(-1, 1, int(ptr[-1])).astype(dtype)
+    return wl.Csr(m, k, ptr + base, col + base, val, base), (line, lines, planes)
+
+
+@pytest.mark.parametrize("seed", [21, 22])
+def test_random_grid_sweep(torch_gpu, handle, oracle, seed):
+    top = np.random.default_rng(seed)
+    kinds = set()
+    for case in range(40):
+        case_seed = int(top.integers(0, 1 << 30))
+        r = np.random.default_rng(case_seed)
+        dtype = [np.float32, np.float64][int(r.integers(0, 2))]
+        base = int(r.integers(0, 2))
+        a, shape = draw_grid_matrix(r, dtype, base)
+        n = int(r.choice([20, 32, 36, 48, 64, 68, 100, 128, 256, 260]))
+        alpha, beta = [(1.0, 0.0), (-1.5, 0.75), (2.0, 1.0)][int(r.integers(0, 3))]
+        c_order = [api.ORDER_ROW, api.ORDER_ROW, api.ORDER_COL][int(r.integers(0, 3))]
+        name = "seed %d case %d (%d): grid %r, %d x %d, %d nonzeros, %s, base %d, n %d" % (
+            seed, case, case_seed, shape, a.m, a.n, a.nnz, np.dtype(dtype).name, base, n)
+        try:
+            spmm.check(torch_gpu, handle, oracle, a, n, alpha, beta, seed=case_seed, c_order=c_order,
+                       pad_b=int(r.choice([0, 0, 4])), pad_c=int(r.choice([0, 0, 4])), preprocess=True,
+                       prepare_for_row_major_c=bool(r.integers(0, 2)), expect_schedule=(1, 2, 3, 4), seen=kinds)
+        except AssertionError as e:
+            raise AssertionError(name + ": " + str(e)) from e
+    assert 4 in kinds and len(kinds) >= 2, kinds  # groups of strips, and at least one other kind of schedule

@@ -12,7 +12,7 @@ pytestmark = pytest.mark.gpu
 
 
 def run_spmm(torch, handle, a, B, C0, alpha, beta, op_b=api.OP_N, b_order=api.ORDER_ROW, c_order=api.ORDER_ROW,
-             pad_b=0, pad_c=0, preprocess=False, expect_schedule=None, prepare_for_row_major_c=False):
+             pad_b=0, pad_c=0, preprocess=False, expect_schedule=None, prepare_for_row_major_c=False, seen=None):
     """B is the k x n operand op(B); it is stored as the call's (op_b, b_order) pair requires.
     prepare_for_row_major_c: mcsparseSpMM_preprocess is given a row-major C of the same shape, whatever the call's is
     (a schedule belongs to the structure of A; which kind is built depends on the operands of the preprocess call)."""
@@ -55,6 +55,8 @@ def run_spmm(torch, handle, a, B, C0, alpha, beta, op_b=api.OP_N, b_order=api.OR
         if expect_schedule is not None:
             wanted = expect_schedule if isinstance(expect_schedule, tuple) else (expect_schedule,)
             assert mat.spmm_schedule()[0] in wanted, mat.spmm_schedule()
+        if seen is not None:
+            seen.add(mat.spmm_schedule()[0])
     st = api.spmm(handle, api.OP_N, op_b, alpha, mat, mB, beta, mC, ct, buf)
     torch.cuda.synchronize()
     out = d_C.cpu().numpy()
