@@ -11,7 +11,7 @@ fp64 CSR SpMV, 1,048,576 rows x 16 nonzeros per row.  The last line of stdout is
 object (about 2 KB) with the headline figures; the default invocation also measures the other
 configurations (50 timed steps each, inside a wall-clock budget) and lists them under "others" of
 that line as workload: [ms_per_step, roofline.frac].  The full object of every workload measured
-goes to stderr, one JSON line each, and to gpurun_out/bench_details.json when that directory exists.
+goes to stderr, one JSON line each, and to bench_details.json in the results directory (see write_details).
 
 Workloads: mixed (1 M rows of 16 and 64 rows of 100000, fp32), c1 (5-pt Laplacian 256^2 fp32), c2 (default), c3 / c3t (power-law fp32, op N / T),
 c4-8 / c4-64 / c4-256 (27-pt stencil 128^3 SpMM, row-major B and C), c4-64-col (the same with
@@ -34,6 +34,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
+RESULTS_DIR = "gpurun_out"  # where the full objects of a run are kept, when it exists
 
 OTHERS = ["c4-64", "c3", "c3t", "c5", "c5-spmv", "c5-coo", "c4-8", "c4-256", "c4-64-col", "c1",
           "c2-alg2", "c3-alg2", "c3t-alg2", "c2-direct", "c3-direct", "c3t-direct", "c4-64-direct", "mixed-direct"]
@@ -489,10 +490,10 @@ def compact_line(out):
 
 def write_details(objects):
     """Every workload's full object: one JSON line each on stderr, and the list as bench_details.json in the
-    directory named by BENCH_DETAILS_DIR (default: gpurun_out beside this script, when it exists)."""
+    directory named by BENCH_DETAILS_DIR (default: RESULTS_DIR beside this script, when it exists)."""
     for o in objects:
         print(json.dumps(o), file=sys.stderr)
-    directory = os.environ.get("BENCH_DETAILS_DIR") or os.path.join(ROOT, "gpurun_out")
+    directory = os.environ.get("BENCH_DETAILS_DIR") or os.path.join(ROOT, RESULTS_DIR)
     if os.path.isdir(directory):
         try:
             with open(os.path.join(directory, "bench_details.json"), "w") as f:
