@@ -37,20 +37,20 @@ struct StripCounters {
     unsigned long long span_sum;  // sum over the groups of (last column - first column)
     unsigned long long loads;     // rows of op(B) all blocks load together
     unsigned int longest_strip;   // most nonzeros in one strip of a group that has blocks
-    unsigned int blocks_of_probe; // unused
+    unsigned int reserved;        // keeps `stride` at byte 24, where readers of the buffer look for it
     unsigned int stride;          // rows between the strips of a group
 };
 
 struct StripPartial {
     unsigned long long span, loads;
-    unsigned int longest, unused;
+    unsigned int longest, padding;
 };
 
 __global__ void zero_strip_counters_kernel(StripCounters* c, uint32_t stride) {
     c->span_sum = 0;
     c->loads = 0;
     c->longest_strip = 0;
-    c->blocks_of_probe = 0;
+    c->reserved = 0;
     c->stride = stride;
 }
 
@@ -59,7 +59,7 @@ __device__ __forceinline__ uint64_t first_row_of_group(uint64_t group, uint32_t 
     return group / per_tile * (static_cast<uint64_t>(Q) * stride) + group % per_tile * H;
 }
 
-// x of the lane `xor_mask` away inside a row of 16 lanes (quad permutes and mirrors, as in group_sum).
+// v of another lane of the same row of 16 lanes, chosen by a DPP control (quad permutes and mirrors, as in group_sum).
 template <int CTRL>
 __device__ __forceinline__ int dpp_int(int v) {
     return __builtin_amdgcn_update_dpp(0, v, CTRL, 0xF, 0xF, false);
