@@ -598,7 +598,8 @@ mcspStatus_t spmm_typed(mcsparseHandle_t h, const mcsparseSpMatDescr* A, mcspars
                                                  h_beta);
         }
     }
-    return MCSP_STATUS_SUCCESS;
+    // a launch the runtime refused (a kernel image that does not fit the device) must not pass for a product
+    return launches_taken() ? MCSP_STATUS_SUCCESS : MCSP_STATUS_INTERNAL_ERROR;
 }
 
 mcspStatus_t check_spmm_args(mcsparseHandle_t handle, const void* alpha, const mcsparseSpMatDescr* A,
