@@ -314,8 +314,11 @@ constexpr int strip_room() { return strip_capacity<T>() + 2 * (16 / static_cast<
 // broadcasts.  STAGED: no strip holds more than strip_capacity<T>() nonzeros and the value array is 16-byte aligned;
 // the four lanes of a strip then copy its values into LDS once, in whole 16-byte pieces, and the blocks read them
 // there.
+// A workgroup is one wavefront (four groups): a wavefront that is through makes room for the next at once instead of
+// waiting for the others of its workgroup (256 threads: 360 us at N = 64 on the 128^3 stencil, 128 or 64: 349 us).
+constexpr int kStripBlock = kWave;
 template <typename T, bool WIDE, bool STAGED>
-__global__ __launch_bounds__(kBlock, 3) void spmm_strips_kernel(idx_t m, idx_t n, idx_t base, uint32_t stride,
+__global__ __launch_bounds__(kStripBlock, 3) void spmm_strips_kernel(idx_t m, idx_t n, idx_t base, uint32_t stride,
                                                              const idx_t* __restrict__ row_ptr,
                                                              const idx_t* __restrict__ col, const T* __restrict__ val,
                                                              const uint32_t* __restrict__ block_ptr,
@@ -326,7 +329,7 @@ __global__ __launch_bounds__(kBlock, 3) void spmm_strips_kernel(idx_t m, idx_t n
                                                              uint32_t xcds, idx_t k, idx_t nnz, uint32_t total_blocks) {
     typedef typename ByteOffset<WIDE>::type off_t;
     constexpr int V = 16 / sizeof(T);
-    constexpr int kGroupsPerBlock = kBlock / kLanes;
+    constexpr int kGroupsPerBlock = kStripBlock / kLanes;
     const idx_t lane = threadIdx.x % kLanes;
     const uint64_t turn = xcd_position(blockIdx.x, xcd_chunk, xcds) * kGroupsPerBlock + threadIdx.x / kLanes;
     const uint64_t groups = spmm_strip_groups(m, stride);
@@ -642,7 +645,7 @@ void launch_spmm_strips(hipStream_t stream, const SpmmArgs& a, const void* sched
                         uint32_t longest_strip, uint64_t mean_span, T alpha, T beta) {
     if (a.m == 0 || a.n == 0) return;
     constexpr int V = 16 / sizeof(T);
-    constexpr int kGroupsPerBlock = kBlock / kLanes;
+    constexpr int kGroupsPerBlock = kStripBlock / kLanes;
     const Carved c = carve(a.m, a.nnz, stride, const_cast<void*>(schedule));
     const uint64_t groups = spmm_strip_groups(a.m, stride);
     const uint64_t group_blocks = (groups + kGroupsPerBlock - 1) / kGroupsPerBlock;
@@ -662,7 +665,7 @@ void launch_spmm_strips(hipStream_t stream, const SpmmArgs& a, const void* sched
     T* C = static_cast<T*>(a.C);
     const bool staged = longest_strip <= static_cast<uint32_t>(strip_capacity<T>()) && reinterpret_cast<uintptr_t>(val) % 16 == 0;
     auto launch = [&](auto wide_c, auto staged_c) {
-        hipLaunchKernelGGL((spmm_strips_kernel<T, decltype(wide_c)::value, decltype(staged_c)::value>), grid, dim3(kBlock), 0,
+        hipLaunchKernelGGL((spmm_strips_kernel<T, decltype(wide_c)::value, decltype(staged_c)::value>), grid, dim3(kStripBlock), 0,
                            stream, a.m, a.n, a.base, stride, a.row_ptr, a.col, val, c.block_ptr, c.blocks, c.order, B, a.ldb, C,
                            a.ldc, a.c_row_major, alpha, beta, xcd_chunk, xcds, a.k, a.nnz, total_blocks);
     };
