@@ -1059,7 +1059,9 @@ mcsparseStatus_t mcsparseSpMM_preprocess(mcsparseHandle_t handle, mcsparseOperat
                     hipMemcpyAsync(strip_counters, span_slot, sizeof(strip_counters), hipMemcpyDeviceToHost, handle->stream) != hipSuccess ||
                     hipStreamSynchronize(handle->stream) != hipSuccess)
                     return to_public_status(MCSP_STATUS_INTERNAL_ERROR);
+                // (and its strips' values fit the copies in LDS: read where they lie, 16 rows' values cost more than they save)
                 if (strip_blocks != 0 && strip_counters[1] * 5 <= counters[1] * 4 &&
+                    (strip_counters[2] & 0xffffffffull) <= mcsp::kSpmmStripStagedValues &&
                     mcsp::spmm_strip_schedule_fits(m, nnz, stride, strip_blocks)) {
                     mcsp::launch_spmm_strip_fill(handle->stream, m, nnz, static_cast<idx_t>(matA->idxBase), stride, ia.rows,
                                                  ia.cols, externalBuffer);

@@ -400,6 +400,8 @@ void launch_spmm_block_count(hipStream_t stream, idx_t m, idx_t nnz, idx_t base,
 // region is used like the one of the block schedule, and the counters' place also holds the stride.
 constexpr int kSpmmStripRows = 4;
 constexpr int kSpmmStrips = 4;
+// values of a strip the kernel copies into LDS; a structure with longer strips is left to the groups of eight rows
+constexpr uint32_t kSpmmStripStagedValues = 128;
 constexpr uint64_t spmm_strip_groups(idx_t m, uint32_t stride) {
     return (static_cast<uint64_t>(m) + static_cast<uint64_t>(kSpmmStrips) * stride - 1) /
            (static_cast<uint64_t>(kSpmmStrips) * stride) * (stride / kSpmmStripRows);

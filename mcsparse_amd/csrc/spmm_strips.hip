@@ -304,7 +304,7 @@ __global__ __launch_bounds__(kOrderChunk) void strip_order_kernel(uint64_t group
 // Values a strip may hold for its copy in LDS to be used, and the room of a copy (the 16-byte pieces a copy is made
 // of bring along up to a piece's worth of neighbours at either end).
 template <typename T>
-constexpr int strip_capacity() { return 512 / static_cast<int>(sizeof(T)); }
+constexpr int strip_capacity() { return static_cast<int>(kSpmmStripStagedValues); }  // 512 bytes of fp32, 1024 of fp64 (a 27-point stencil's strip: 108 values)
 template <typename T>
 constexpr int strip_room() { return strip_capacity<T>() + 2 * (16 / static_cast<int>(sizeof(T))); }
 

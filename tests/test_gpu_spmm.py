@@ -478,9 +478,9 @@ def test_strips_grid_with_broken_rows(torch_gpu, handle, oracle, dtype, n):
 
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
-def test_strips_with_more_values_per_strip_than_the_copy_in_lds_holds(torch_gpu, handle, oracle, dtype):
-    """A strip's values are copied into LDS when they are at most 512 bytes; beyond that the blocks read them where
-    they lie: a 27-point stencil in fp64 (4 rows x 27 x 8 bytes), a 7 x 7 stencil on a plane grid in fp32 (4 x 49 x 4)."""
+def test_strips_and_the_size_of_their_copy_in_lds(torch_gpu, handle, oracle, dtype):
+    """A strip's values are copied into LDS when they are at most 128: a 27-point stencil in fp64 (4 rows x 27 values)
+    gets groups of strips; a 7 x 7 stencil on a plane grid (4 x 49 values) is left to the groups of eight rows."""
     if dtype == np.float64:
         a = wl.stencil_27pt(16, dtype=dtype)
     else:
@@ -494,9 +494,39 @@ def test_strips_with_more_values_per_strip_than_the_copy_in_lds_holds(torch_gpu,
         ptr = np.concatenate([[0], np.cumsum([len(c) for c in rows])]).astype(np.int32)
         a = wl.Csr(line * lines, line * lines, ptr, np.concatenate(rows).astype(np.int32),
                    rng.uniform(-1, 1, int(ptr[-1])).astype(dtype))
+    want = 4 if dtype == np.float64 else 3
     for n in (48, 64):
-        check(torch_gpu, handle, oracle, a, n, 1.0, 0.0, preprocess=True, expect_schedule=4)
-        check(torch_gpu, handle, oracle, a.with_base(1), n, -1.5, 0.5, preprocess=True, expect_schedule=4, pad_b=4, pad_c=4)
+        check(torch_gpu, handle, oracle, a, n, 1.0, 0.0, preprocess=True, expect_schedule=want)
+        check(torch_gpu, handle, oracle, a.with_base(1), n, -1.5, 0.5, preprocess=True, expect_schedule=want, pad_b=4, pad_c=4)
+
+
+@pytest.mark.parametrize("grid,state", [(40, 4), (41, 3)])
+def test_blocks_with_a_value_array_that_is_not_16_byte_aligned(torch_gpu, handle, oracle, grid, state):
+    """The copies of the values in LDS are made of 16-byte pieces: an array that does not begin on such a boundary
+    is read where it lies (both kinds of diagonal blocks)."""
+    torch = torch_gpu
+    a = wl.stencil_27pt(grid, dtype=np.float32)
+    n = 64
+    rng = np.random.default_rng(4)
+    B = rng.uniform(-1, 1, (a.n, n)).astype(np.float32)
+    d_ptr, d_col = dev(torch, a.ptr), dev(torch, a.col)
+    d_val_room = torch.zeros(a.nnz + 1, dtype=torch.float32, device="cuda")
+    d_val = d_val_room[1:]
+    d_val.copy_(torch.from_numpy(a.val))
+    assert d_val.data_ptr() % 16 == 4
+    d_B = dev(torch, B)
+    d_C = torch.zeros((a.m, n), dtype=torch.float32, device="cuda")
+    mat = api.SpMat(a.m, a.n, a.nnz, d_ptr, d_col, d_val)
+    mB, mC = api.DnMat(a.n, n, n, d_B), api.DnMat(a.m, n, n, d_C)
+    st, size = api.spmm_buffer_size(handle, api.OP_N, api.OP_N, 1.0, mat, mB, 0.0, mC, api.R_32F)
+    buf = torch.empty(size, dtype=torch.uint8, device="cuda")
+    assert api.spmm_preprocess(handle, api.OP_N, api.OP_N, 1.0, mat, mB, 0.0, mC, api.R_32F, buf) == 0
+    assert mat.spmm_schedule()[0] == state
+    assert api.spmm(handle, api.OP_N, api.OP_N, 1.0, mat, mB, 0.0, mC, api.R_32F, buf) == 0
+    torch.cuda.synchronize()
+    c_ref, bound = oracle.spmm(a.m, n, 0, a.ptr, a.col, a.val, 1.0, 0.0, B.ravel(), n, True, np.zeros(a.m * n, np.float32),
+                               n, True)
+    assert_within(d_C.cpu().numpy(), c_ref, bound, np.float32)
 
 
 def test_strips_row_ignores_rows_of_b_only_other_strips_use(torch_gpu, handle):
