@@ -481,6 +481,13 @@ mcsparseStatus_t mcsparseSpMatGetSpMMSchedule(mcsparseSpMatDescr_t spMatDescr, i
  *     cannot help (x fits in cache as it is, a matrix too small to fill the GPU) are left to the
  *     ordinary kernels; the call still returns SUCCESS.  mcsparseSpMatGetSpMVPreprocess tells which
  *     case applies.
+ *   - For a direction that does not transpose (CSR and COO with op N, CSC with op T) the call ends with a
+ *     trial: the product is run a few times from the copy and a few times from the caller's arrays, on the
+ *     handle's stream, and the copy is kept only if it was the faster by more than a twentieth (a banded
+ *     matrix, whose rows read x line by line as it is, or long rows over an x that fits in cache, run
+ *     faster from the arrays).  The trial reads vecX, whose memory must be there but whose contents do not
+ *     matter, and writes a y of its own inside externalBuffer, never vecY.  mcsparseSetSpMVPreprocessTrial
+ *     turns it off; a descriptor whose band width or kernel family the caller has set is not tried either.
  *   - alg chooses between two layouts (the reference ignores alg; the meanings are those APIs of this
  *     family give the values).  MCSPARSE_SPMV_CSR_ALG2, the algorithm that promises the same bits on
  *     every run, builds the banded copy described above: row sums are formed in a fixed order.  Every
@@ -502,6 +509,10 @@ mcsparseStatus_t mcsparseSpMV_preprocess(mcsparseHandle_t handle, mcsparseOperat
                                          mcsparseSpMatDescr_t matA, mcsparseDnVecDescr_t vecX, const void* beta,
                                          mcsparseDnVecDescr_t vecY, macaDataType computeType, mcsparseSpMVAlg_t alg,
                                          void* externalBuffer);
+/* Whether mcsparseSpMV_preprocess ends with the trial described above (trial != 0, the default) or keeps every
+ * copy it can build.  For tests and benchmarks of the copies by themselves. */
+mcsparseStatus_t mcsparseSetSpMVPreprocessTrial(mcsparseHandle_t handle, int trial);
+mcsparseStatus_t mcsparseGetSpMVPreprocessTrial(const mcsparseHandle_t handle, int* trial);
 /* state 0 = not preprocessed, 1 = preprocessed and left to the ordinary kernels, 2 = banded copy in
  * use, 3 = the copy in column order (MCSPARSE_SPMV_CSR_ALG1) in use; bands and rows_per_tile describe
  * the copy (0 unless state is 2 or 3). */

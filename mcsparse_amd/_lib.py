@@ -58,6 +58,8 @@ PROTOTYPES = {
     "mcsparseSpMV": (c_int, [vp, c_int, vp, vp, vp, vp, vp, c_int, c_int, vp]),
     "mcsparseSetSpMVDeterministic": (c_int, [vp, c_int]),
     "mcsparseGetSpMVDeterministic": (c_int, [vp, P(c_int)]),
+    "mcsparseSetSpMVPreprocessTrial": (c_int, [vp, c_int]),
+    "mcsparseGetSpMVPreprocessTrial": (c_int, [vp, P(c_int)]),
     "mcsparseXstreamProbe": (c_int, [vp, c_int, vp, vp, ctypes.c_size_t, vp, ctypes.c_size_t]),
     "mcsparseXtopologyOfCuCount": (c_int, [c_int, P(c_int)]),
     "mcsparseSpMV_staticBuffer": (c_int, [vp, c_int, vp, vp, vp, vp, vp, c_int, c_int]),

@@ -103,6 +103,16 @@ class Handle:
         check(self.lib.mcsparseGetSpMVDeterministic(self._h, ctypes.byref(out)), "mcsparseGetSpMVDeterministic")
         return bool(out.value)
 
+    def set_spmv_preprocess_trial(self, on):
+        """mcsparseSetSpMVPreprocessTrial: whether mcsparseSpMV_preprocess times its copy against the row kernels and
+        keeps it only where it is faster (the default) or keeps every copy."""
+        check(self.lib.mcsparseSetSpMVPreprocessTrial(self._h, 1 if on else 0), "mcsparseSetSpMVPreprocessTrial")
+
+    def spmv_preprocess_trial(self):
+        out = ctypes.c_int(-1)
+        check(self.lib.mcsparseGetSpMVPreprocessTrial(self._h, ctypes.byref(out)), "mcsparseGetSpMVPreprocessTrial")
+        return bool(out.value)
+
     def destroy(self):
         if self._h:
             self.lib.mcsparseDestroy(self._h)

@@ -731,6 +731,58 @@ mcspStatus_t spmv_call(mcsparseHandle_t handle, mcsparseOperation_t opA, const v
     return spmv_typed<double>(handle, matA, opA, alpha, beta, vecX, vecY, buffer, may_read_back, alg);
 }
 
+// mcsparseSpMV_preprocess has just built a copy for a direction that does not transpose.  Whether calls run
+// faster from it than from the caller's arrays depends on what the row kernels already get from the caches (a
+// banded matrix reads x line by line as it is; an x that fits an L2 next to rows long enough to fill the lanes
+// leaves the copy's extra partial sums as pure cost), so both are run here, on the handle's stream, with the
+// caller's x and a y inside the buffer, and timed with events.  *copy_wins says whether the copy was faster by
+// more than a twentieth.
+mcspStatus_t spmv_trial(mcsparseHandle_t handle, mcsparseOperation_t opA, mcsparseSpMatDescr_t matA,
+                        mcsparseDnVecDescr_t vecX, void* trial_y, macaDataType computeType, void* buffer,
+                        mcsparseSpMVAlg_t alg, bool* copy_wins) {
+    constexpr int kRuns = 4;
+    mcsparseDnVecDescr y = {};
+    const CsrView v = make_view(matA, opA);
+    y.valueType = computeType;
+    y.size = v.transpose ? v.n : v.m;
+    y.values = trial_y;
+    const double one64 = 1.0, zero64 = 0.0;
+    const float one32 = 1.0f, zero32 = 0.0f;
+    const void* one = computeType == MACA_R_32F ? static_cast<const void*>(&one32) : &one64;
+    const void* zero = computeType == MACA_R_32F ? static_cast<const void*>(&zero32) : &zero64;
+    const mcsparsePointerMode_t callers_mode = handle->ptr_mode;
+    handle->ptr_mode = MCSPARSE_POINTER_MODE_HOST;
+    hipEvent_t marks[4] = {nullptr, nullptr, nullptr, nullptr};  // start and end of each leg's timed runs
+    mcspStatus_t st = MCSP_STATUS_SUCCESS;
+    for (hipEvent_t& e : marks)
+        if (st == MCSP_STATUS_SUCCESS && hipEventCreate(&e) != hipSuccess) st = MCSP_STATUS_INTERNAL_ERROR;
+    // leg 0 is the row kernels, leg 1 the copy; the first run of each is a warm-up
+    for (int leg = 0; leg < 2 && st == MCSP_STATUS_SUCCESS; ++leg) {
+        matA->banded.useful = leg == 1;
+        for (int run = 0; run <= kRuns && st == MCSP_STATUS_SUCCESS; ++run) {
+            if (run == 1 && hipEventRecord(marks[2 * leg], handle->stream) != hipSuccess)
+                st = MCSP_STATUS_INTERNAL_ERROR;
+            if (st == MCSP_STATUS_SUCCESS)
+                st = computeType == MACA_R_32F
+                         ? spmv_typed<float>(handle, matA, opA, one, zero, vecX, &y, buffer, true, alg)
+                         : spmv_typed<double>(handle, matA, opA, one, zero, vecX, &y, buffer, true, alg);
+        }
+        if (st == MCSP_STATUS_SUCCESS && hipEventRecord(marks[2 * leg + 1], handle->stream) != hipSuccess)
+            st = MCSP_STATUS_INTERNAL_ERROR;
+    }
+    if (st == MCSP_STATUS_SUCCESS && hipEventSynchronize(marks[3]) != hipSuccess) st = MCSP_STATUS_INTERNAL_ERROR;
+    float rows_ms = 0.0f, copy_ms = 0.0f;
+    if (st == MCSP_STATUS_SUCCESS && (hipEventElapsedTime(&rows_ms, marks[0], marks[1]) != hipSuccess ||
+                                      hipEventElapsedTime(&copy_ms, marks[2], marks[3]) != hipSuccess))
+        st = MCSP_STATUS_INTERNAL_ERROR;
+    for (hipEvent_t e : marks)
+        if (e != nullptr) (void)hipEventDestroy(e);
+    handle->ptr_mode = callers_mode;
+    matA->banded.useful = true;
+    *copy_wins = copy_ms * 20.0f < rows_ms * 19.0f;
+    return st;
+}
+
 }  // namespace mcsp
 
 extern "C" {
@@ -786,9 +838,11 @@ mcsparseStatus_t mcsparseSpMV_preprocess_bufferSize(mcsparseHandle_t handle, mcs
         const CsrView v = make_view(matA, opA);
         const idx_t rows = static_cast<idx_t>(v.transpose ? v.n : v.m);
         // the copy in column order carries its own scratch; the other builds a transpose behind itself
+        // and, for a direction that does not transpose, a y for the runs that time the copy against the row kernels
         *bufferSize = banded_region_offset(matA, opA, vb) +
                       align_up(mcsp::banded_layout(shape, rows, static_cast<idx_t>(matA->nnz), vb).total) +
-                      (v.transpose && !shape.by_column ? transpose_scratch(v, matA->nnz, vb).total : 0);
+                      (v.transpose ? (shape.by_column ? 0 : transpose_scratch(v, matA->nnz, vb).total)
+                                   : align_up(static_cast<size_t>(rows) * vb));
     }
     return MCSPARSE_STATUS_SUCCESS;
 }
@@ -920,6 +974,19 @@ mcsparseStatus_t mcsparseSpMV_preprocess(mcsparseHandle_t handle, mcsparseOperat
     for (int i = 0; i < 9; ++i) b.shape.xcd_start[i] = xcd_start[i];
     b.useful = true;
     b.valid = true;
+    // A caller who has set the band width or the kernel family is measuring one of the two by itself.  The
+    // transposing directions need no trial: without a copy each call sorts the products by column.
+    if (handle->spmv_preprocess_trial && !v.transpose && matA->banded.band_bytes == 0 &&
+        matA->plan.forced_family == kFamilyAuto) {
+        bool copy_wins = true;
+        const mcspStatus_t ts = mcsp::spmv_trial(handle, opA, matA, vecX, region + align_up(l.total), computeType,
+                                                 externalBuffer, alg, &copy_wins);
+        if (ts != MCSP_STATUS_SUCCESS) {
+            b.valid = false;
+            return to_public_status(ts);
+        }
+        b.useful = copy_wins;
+    }
     return MCSPARSE_STATUS_SUCCESS;
 }
 

@@ -186,6 +186,22 @@ mcsparseStatus_t mcsparseGetSpMVDeterministic(const mcsparseHandle_t handle, int
     return MCSPARSE_STATUS_SUCCESS;
 }
 
+// EXTENSION.  Whether mcsparseSpMV_preprocess, having built its copy for a direction that does not transpose, runs
+// the call both ways and keeps the copy only where it is the faster one (the default), or keeps every copy it
+// can build.
+mcsparseStatus_t mcsparseSetSpMVPreprocessTrial(mcsparseHandle_t handle, int trial) {
+    if (handle == nullptr) return to_public_status(MCSP_STATUS_INVALID_HANDLE);
+    handle->spmv_preprocess_trial = trial != 0;
+    return MCSPARSE_STATUS_SUCCESS;
+}
+
+mcsparseStatus_t mcsparseGetSpMVPreprocessTrial(const mcsparseHandle_t handle, int* trial) {
+    if (handle == nullptr) return to_public_status(MCSP_STATUS_INVALID_HANDLE);
+    if (trial == nullptr) return to_public_status(MCSP_STATUS_INVALID_POINTER);
+    *trial = handle->spmv_preprocess_trial ? 1 : 0;
+    return MCSPARSE_STATUS_SUCCESS;
+}
+
 // ---- dense vector: src/common/mcsp_helper.cpp:325-387 ------------------------------------
 
 mcsparseStatus_t mcsparseCreateDnVec(mcsparseDnVecDescr_t* dnVecDescr, int64_t size, void* values,

@@ -23,6 +23,9 @@ struct mcsparseContext {
     mcsparsePointerMode_t ptr_mode = MCSPARSE_POINTER_MODE_HOST;
     // mcsparseSetSpMVDeterministic: every SpMV call of this handle is treated as MCSPARSE_SPMV_CSR_ALG2
     bool spmv_deterministic = false;
+    // mcsparseSetSpMVPreprocessTrial: mcsparseSpMV_preprocess times its copy against the row kernels and keeps
+    // it only where it is faster
+    bool spmv_preprocess_trial = true;
 };
 
 // reference: src/include/mcsp_internal_types.h:86-94
@@ -122,8 +125,8 @@ struct BandedShape {
 };
 struct SpmvBanded {
     bool valid = false;
-    bool useful = false;     // false: preprocess looked at the matrix and left it to the row kernels (kept for
-                             // structures a later version may decline; every candidate is banded today)
+    bool useful = false;     // false: preprocess built the copy, timed it against the row kernels and found it
+                             // no faster; calls run the row kernels
     const void* buffer = nullptr;
     const void* rows = nullptr;
     const void* cols = nullptr;

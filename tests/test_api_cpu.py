@@ -495,3 +495,16 @@ def test_spmv_deterministic_switch_is_off_by_default_and_checked():
     assert lib.mcsparseSetSpMVDeterministic(None, 1) == api.STATUS_NOT_INITIALIZED
     assert lib.mcsparseGetSpMVDeterministic(h.ptr, None) == api.STATUS_INVALID_VALUE
     h.destroy()
+
+
+def test_spmv_preprocess_trial_switch_is_on_by_default_and_checked():
+    h = api.Handle()
+    assert h.spmv_preprocess_trial() is True
+    h.set_spmv_preprocess_trial(False)
+    assert h.spmv_preprocess_trial() is False
+    h.set_spmv_preprocess_trial(True)
+    assert h.spmv_preprocess_trial() is True
+    lib = _lib.load()
+    assert lib.mcsparseSetSpMVPreprocessTrial(None, 1) == api.STATUS_NOT_INITIALIZED
+    assert lib.mcsparseGetSpMVPreprocessTrial(h.ptr, None) == api.STATUS_INVALID_VALUE
+    h.destroy()

@@ -127,6 +127,7 @@ def test_preprocessed_spmv_replays_in_a_hip_graph(torch_gpu, oracle, alg, state,
     rng = np.random.default_rng(22)
     side = torch.cuda.Stream()
     handle = api.Handle(stream=side.cuda_stream)
+    handle.set_spmv_preprocess_trial(False)  # the copy is what is replayed, whether or not it is the faster here
     a = wl.random_ragged(600000, 100000, 4, dtype=np.float64, seed=9) if tall else \
         wl.random_ragged(20000, 40000, 10, dtype=np.float64, seed=9)
     d_ptr, d_col, d_val = dev(torch, a.ptr), dev(torch, a.col), dev(torch, a.val)

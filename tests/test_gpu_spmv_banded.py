@@ -16,6 +16,14 @@ pytestmark = pytest.mark.gpu
 GOLDEN = sorted(glob.glob(os.path.join(os.path.dirname(__file__), "golden", "csr_*.npz")))
 
 
+@pytest.fixture()
+def handle(handle):
+    """These tests are of the copies themselves: preprocess keeps every copy it builds, also where the row kernels
+    would be faster (small matrices)."""
+    handle.set_spmv_preprocess_trial(False)
+    return handle
+
+
 def run_banded(torch, handle, oracle, a, alpha, beta, band_bytes=0, seed=1, expect_state=2, what="", calls=1,
                as_csc=False, reference=None, alg=api.SPMV_CSR_ALG2):
     """as_csc: the arrays are handed over as the CSC of the n x m transpose and applied with op T.

@@ -12,6 +12,14 @@ from gpu_util import assert_within, dev
 pytestmark = pytest.mark.gpu
 
 
+@pytest.fixture()
+def handle(handle):
+    """These tests are of the copies themselves: preprocess keeps every copy it builds, also where the row kernels
+    would be faster (small matrices)."""
+    handle.set_spmv_preprocess_trial(False)
+    return handle
+
+
 def run(torch, handle, oracle, a, alpha, beta, op=api.OP_N, fmt=api.FORMAT_CSR, band_bytes=0, seed=1, expect_state=3,
         calls=2, call_alg=api.SPMV_CSR_ALG1, what="column order"):
     """a: the matrix whose arrays are handed over (m x n CSR).  fmt CSC reads the same arrays as the CSC of
