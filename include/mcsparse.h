@@ -482,7 +482,7 @@ mcsparseStatus_t mcsparseSpMatGetSpMMSchedule(mcsparseSpMatDescr_t spMatDescr, i
  *     ordinary kernels; the call still returns SUCCESS.  mcsparseSpMatGetSpMVPreprocess tells which
  *     case applies.
  *   - For a direction that does not transpose (CSR and COO with op N, CSC with op T) the call ends with a
- *     trial: the product is run a few times from the copy and a few times from the caller's arrays, on the
+ *     trial: the product is run from the caller's arrays and from the copy, one to three times each, on the
  *     handle's stream, and the copy is kept only if it was the faster by more than a twentieth (a banded
  *     matrix, whose rows read x line by line as it is, or long rows over an x that fits in cache, run
  *     faster from the arrays).  The trial reads vecX, whose memory must be there but whose contents do not

@@ -735,12 +735,12 @@ mcspStatus_t spmv_call(mcsparseHandle_t handle, mcsparseOperation_t opA, const v
 // faster from it than from the caller's arrays depends on what the row kernels already get from the caches (a
 // banded matrix reads x line by line as it is; an x that fits an L2 next to rows long enough to fill the lanes
 // leaves the copy's extra partial sums as pure cost), so both are run here, on the handle's stream, with the
-// caller's x and a y inside the buffer, and timed with events.  *copy_wins says whether the copy was faster by
-// more than a twentieth.
+// caller's x and a y inside the buffer, and timed with events: once each, which settles it where one takes more
+// than twice the other's time, else twice more.  *copy_wins says whether the copy was faster by more than a
+// twentieth.
 mcspStatus_t spmv_trial(mcsparseHandle_t handle, mcsparseOperation_t opA, mcsparseSpMatDescr_t matA,
                         mcsparseDnVecDescr_t vecX, void* trial_y, macaDataType computeType, void* buffer,
                         mcsparseSpMVAlg_t alg, bool* copy_wins) {
-    constexpr int kRuns = 4;
     mcsparseDnVecDescr y = {};
     const CsrView v = make_view(matA, opA);
     y.valueType = computeType;
@@ -752,29 +752,28 @@ mcspStatus_t spmv_trial(mcsparseHandle_t handle, mcsparseOperation_t opA, mcspar
     const void* zero = computeType == MACA_R_32F ? static_cast<const void*>(&zero32) : &zero64;
     const mcsparsePointerMode_t callers_mode = handle->ptr_mode;
     handle->ptr_mode = MCSPARSE_POINTER_MODE_HOST;
-    hipEvent_t marks[4] = {nullptr, nullptr, nullptr, nullptr};  // start and end of each leg's timed runs
+    hipEvent_t marks[3] = {nullptr, nullptr, nullptr};  // before the row kernels, between the two, after the copy
     mcspStatus_t st = MCSP_STATUS_SUCCESS;
     for (hipEvent_t& e : marks)
         if (st == MCSP_STATUS_SUCCESS && hipEventCreate(&e) != hipSuccess) st = MCSP_STATUS_INTERNAL_ERROR;
-    // leg 0 is the row kernels, leg 1 the copy; the first run of each is a warm-up
-    for (int leg = 0; leg < 2 && st == MCSP_STATUS_SUCCESS; ++leg) {
-        matA->banded.useful = leg == 1;
-        for (int run = 0; run <= kRuns && st == MCSP_STATUS_SUCCESS; ++run) {
-            if (run == 1 && hipEventRecord(marks[2 * leg], handle->stream) != hipSuccess)
-                st = MCSP_STATUS_INTERNAL_ERROR;
-            if (st == MCSP_STATUS_SUCCESS)
+    float rows_ms = 0.0f, copy_ms = 0.0f;
+    for (int runs = 1; runs <= 2 && st == MCSP_STATUS_SUCCESS; ++runs) {
+        for (int leg = 0; leg < 2 && st == MCSP_STATUS_SUCCESS; ++leg) {
+            matA->banded.useful = leg == 1;  // leg 0 runs the row kernels, leg 1 the copy
+            if (hipEventRecord(marks[leg], handle->stream) != hipSuccess) st = MCSP_STATUS_INTERNAL_ERROR;
+            for (int run = 0; run < runs && st == MCSP_STATUS_SUCCESS; ++run)
                 st = computeType == MACA_R_32F
                          ? spmv_typed<float>(handle, matA, opA, one, zero, vecX, &y, buffer, true, alg)
                          : spmv_typed<double>(handle, matA, opA, one, zero, vecX, &y, buffer, true, alg);
         }
-        if (st == MCSP_STATUS_SUCCESS && hipEventRecord(marks[2 * leg + 1], handle->stream) != hipSuccess)
+        if (st == MCSP_STATUS_SUCCESS &&
+            (hipEventRecord(marks[2], handle->stream) != hipSuccess || hipEventSynchronize(marks[2]) != hipSuccess ||
+             hipEventElapsedTime(&rows_ms, marks[0], marks[1]) != hipSuccess ||
+             hipEventElapsedTime(&copy_ms, marks[1], marks[2]) != hipSuccess))
             st = MCSP_STATUS_INTERNAL_ERROR;
+        // the first runs of the two are their slowest (cold caches): enough to tell two from one, not 20 from 19
+        if (rows_ms > 2.0f * copy_ms || copy_ms > 2.0f * rows_ms) break;
     }
-    if (st == MCSP_STATUS_SUCCESS && hipEventSynchronize(marks[3]) != hipSuccess) st = MCSP_STATUS_INTERNAL_ERROR;
-    float rows_ms = 0.0f, copy_ms = 0.0f;
-    if (st == MCSP_STATUS_SUCCESS && (hipEventElapsedTime(&rows_ms, marks[0], marks[1]) != hipSuccess ||
-                                      hipEventElapsedTime(&copy_ms, marks[2], marks[3]) != hipSuccess))
-        st = MCSP_STATUS_INTERNAL_ERROR;
     for (hipEvent_t e : marks)
         if (e != nullptr) (void)hipEventDestroy(e);
     handle->ptr_mode = callers_mode;
