@@ -148,6 +148,9 @@ def describe(name):
     if name == "mixed":
         return ("mixed", "spmv", False, 0, 1.0, 0.0,
                 "fp32 CSR SpMV, 1048576 rows x 16 nnz/row uniform + 64 rows of 100000")
+    if name.startswith("c3-spmm-"):  # not among the others of the default run
+        return ("power_law", "spmm", False, int(name.split("-")[2]), 1.0, 0.0,
+                "fp32 CSR SpMM, the power-law matrix of c3, B and C row-major N=%d" % int(name.split("-")[2]))
     if name.startswith("c4-"):
         parts = name.split("-")
         n_cols = int(parts[1])

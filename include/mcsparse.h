@@ -307,7 +307,11 @@ mcsparseStatus_t mcsparseSpMV_bufferSize(mcsparseHandle_t handle, mcsparseOperat
                                          mcsparseSpMVAlg_t alg, size_t* bufferSize);
 
 /* ---- C = alpha*A*op(B) + beta*C : include/interface/mcsp_generic.h:54-67 ---------- */
-/* opA must be NON_TRANSPOSE for CSR (src/kernels/level3/spmm/mcsp_spmm_gpu.cpp:105-108). */
+/* opA must be NON_TRANSPOSE for CSR (src/kernels/level3/spmm/mcsp_spmm_gpu.cpp:105-108).
+ * The first mcsparseSpMM on a CSR structure reads the row lengths back once (136 bytes, kept on the descriptor and
+ * shared with mcsparseSpMV; not on a stream under graph capture); later calls only enqueue kernels.  Rows of more
+ * than 1024 nonzeros are cut into pieces of 4096 that a workgroup each takes, their partial sums kept in
+ * externalBuffer and added in the order of the pieces: results repeat bit for bit from run to run. */
 mcsparseStatus_t mcsparseSpMM_bufferSize(mcsparseHandle_t handle, mcsparseOperation_t opA, mcsparseOperation_t opB,
                                          const void* alpha, mcsparseSpMatDescr_t matA, mcsparseDnMatDescr_t matB,
                                          const void* beta, mcsparseDnMatDescr_t matC, macaDataType computeType,

@@ -17,7 +17,7 @@ LIB_PATH = os.path.join(LIB_DIR, "libmcsparse.so")
 EXPORTS = os.path.join(CSRC, "exports.map")
 
 SOURCES = ["api_helper.cpp", "api_compute.cpp", "api_legacy.cpp", "api_sort.cpp", "topology.cpp", "analysis.hip", "spmv.hip",
-           "spmv_banded.hip", "spmm.hip", "spmm_blocks.hip", "spmm_strips.hip", "convert.hip", "static_scratch.hip"]
+           "spmv_banded.hip", "spmm.hip", "spmm_blocks.hip", "spmm_strips.hip", "spmm_long.hip", "convert.hip", "static_scratch.hip"]
 HEADERS = ["internal.h", "device_util.h", "spmm_device.h"]
 
 COMPILE_FLAGS = [

@@ -425,7 +425,7 @@ mcspStatus_t spmv_typed(mcsparseHandle_t h, mcsparseSpMatDescr* A, mcsparseOpera
 // CSC gets the transposed copy [row_ptr m+1 | col_ind nnz][values][csr2csc workspace]
 // (mcsp_spmm_gpu.cpp:818-849); 64-bit index arrays add their narrowed copies at the end.
 struct SpmmLayout {
-    size_t ptr, ind, vals, csr2csc_ws, bt, ct, narrow, total;
+    size_t ptr, ind, vals, csr2csc_ws, bt, ct, long_ws, narrow, total;
     int64_t n_padded;  // leading dimension of the row-major copies of op(B) and C
     bool copy_b, copy_c;
 };
@@ -477,6 +477,10 @@ SpmmLayout spmm_layout(const mcsparseSpMatDescr* A, const mcsparseDnMatDescr* B,
     if (l.copy_b) off += align_up(static_cast<size_t>(A->col_num) * l.n_padded * value_bytes);
     l.ct = off;
     if (l.copy_c) off += align_up(static_cast<size_t>(A->row_num) * l.n_padded * value_bytes);
+    // the pieces long rows are cut into, their partial sums, and the counters of the row-length analysis
+    l.long_ws = off;
+    if (A->nnz > 0 && A->row_num > 0 && n > 0)
+        off += align_up(mcsp::spmm_long_rows_bytes(static_cast<idx_t>(A->nnz), l.n_padded, value_bytes));
     l.narrow = off;
     off += narrow_bytes(A);
     l.total = off < kMinBuffer ? kMinBuffer : off;
@@ -484,7 +488,7 @@ SpmmLayout spmm_layout(const mcsparseSpMatDescr* A, const mcsparseDnMatDescr* B,
 }
 
 template <typename T>
-mcspStatus_t spmm_typed(mcsparseHandle_t h, const mcsparseSpMatDescr* A, mcsparseOperation_t opB, const void* alpha,
+mcspStatus_t spmm_typed(mcsparseHandle_t h, mcsparseSpMatDescr* A, mcsparseOperation_t opB, const void* alpha,
                         const void* beta, const mcsparseDnMatDescr* B, mcsparseDnMatDescr* C, void* buffer) {
     T h_alpha, h_beta;
     if (!scalar_to_host(h, beta, &h_beta) || !scalar_to_host(h, alpha, &h_alpha))
@@ -549,6 +553,26 @@ mcspStatus_t spmm_typed(mcsparseHandle_t h, const mcsparseSpMatDescr* A, mcspars
         a.C = c_user;
         a.ldc = C->ld;
         a.c_row_major = C->order == MCSPARSE_ORDER_ROW;
+        // Rows far longer than the rest are cut into pieces (spmm_long.hip), which costs four small launches: only
+        // where the matrix has such rows.  Whether it has is part of the row-length analysis that SpMV keeps on the
+        // descriptor (one kernel and a 136-byte read-back the first time a structure is seen); a call that cannot
+        // use it (a stream under capture, batches with offsets of their own, COO and CSC inputs, whose offsets are
+        // built in the buffer) takes the launches.
+        if (A->nnz != 0 && a.m != 0 && a.n != 0) {
+            bool may_have_long_rows = true;
+            if (A->format == MCSPARSE_FORMAT_CSR && (batches == 1 || shared_structure)) {
+                const mcspStatus_t ps = ensure_plan(h, A, ia.rows, A->rows, A->row_num, A->nnz,
+                                                    A->col_num * static_cast<int64_t>(sizeof(T)), buf + l.long_ws, true);
+                if (ps != MCSP_STATUS_SUCCESS) return ps;
+                if (A->plan.valid && A->plan.forced_family == kFamilyAuto)
+                    may_have_long_rows = A->plan.max_row_len > mcsp::kSpmmLongRow;
+            }
+            if (may_have_long_rows) {
+                a.long_row = mcsp::kSpmmLongRow;
+                a.long_ws = buf + l.long_ws;
+                a.long_n = l.n_padded;
+            }
+        }
         T beta_inner = h_beta;
         if (l.copy_b && A->nnz != 0) {  // without nonzeros op(B) is never read (and may be NULL)
             // the column-major image is a row-major n x k matrix: its transpose is op(B), row-major
@@ -1064,7 +1088,8 @@ mcsparseStatus_t mcsparseSpMM_preprocess(mcsparseHandle_t handle, mcsparseOperat
     matA->schedule.valid = false;
     // the schedule's size is read back: not possible on a stream under graph capture
     if (stream_is_capturing(handle->stream)) return to_public_status(MCSP_STATUS_NOT_IMPLEMENTED);
-    if (opA != MCSPARSE_OPERATION_NON_TRANSPOSE || !schedulable(matA) || matA->rows == nullptr || matA->cols == nullptr)
+    if (opA != MCSPARSE_OPERATION_NON_TRANSPOSE || !schedulable(matA) || matA->rows == nullptr || matA->cols == nullptr ||
+        matC->col_num <= 0)
         return MCSPARSE_STATUS_SUCCESS;  // nothing to prepare for this call
 
     const idx_t m = static_cast<idx_t>(matA->row_num);
@@ -1081,6 +1106,21 @@ mcsparseStatus_t mcsparseSpMM_preprocess(mcsparseHandle_t handle, mcsparseOperat
     s.base = static_cast<int>(matA->idxBase);
     s.blocks = false;
     s.stride = 0;
+    {
+        // The kernels that work from a schedule walk every row in one piece; a matrix with rows of thousands of
+        // nonzeros is left to the row kernels, which hand such rows to the kernels of spmm_long.hip.
+        const size_t vb0 = value_size(matA->valueType);
+        const mcspStatus_t ps =
+            ensure_plan(handle, matA, ia.rows, matA->rows, matA->row_num, matA->nnz, matA->col_num * static_cast<int64_t>(vb0),
+                        static_cast<char*>(externalBuffer) + spmm_layout(matA, matB, matC, opB, vb0).long_ws, true);
+        if (ps != MCSP_STATUS_SUCCESS) return to_public_status(ps);
+        if (matA->plan.valid && matA->plan.forced_family == kFamilyAuto && matA->plan.max_row_len > mcsp::kSpmmLongRow) {
+            s.entries = 0;
+            s.useful = false;
+            s.valid = true;
+            return MCSPARSE_STATUS_SUCCESS;
+        }
+    }
     const char* span_slot = static_cast<const char*>(externalBuffer) + l.span_sum;
 
     // First choice, for operands of 65 to 1024 bytes per row (the widths its kernel was measured faster at: by 35 %,

@@ -354,9 +354,26 @@ struct SpmmArgs {
     void* C;
     int64_t ldc;
     bool c_row_major;
+    // Rows of more than long_row nonzeros (0: none are treated apart) are left out by the row kernels and taken in
+    // pieces by the kernels of spmm_long.hip, which need spmm_long_rows_bytes(nnz, long_n, value size) bytes at
+    // long_ws; long_n is the width the area was sized for (at least n).
+    idx_t long_row = 0;
+    void* long_ws = nullptr;
+    int64_t long_n = 0;
 };
 template <typename T>
 void launch_spmm(hipStream_t stream, const SpmmArgs& a, T alpha, T beta);
+
+// Long rows (spmm_long.hip): a lane group of the row kernels walks a row by itself, so a row of tens of thousands
+// of nonzeros outlasts the rest of the launch.  Rows above kSpmmLongRow nonzeros are cut into pieces of
+// kSpmmLongChunk, a workgroup each.  The first 2 * kAlign bytes of the area are not used by these kernels (the
+// row-length analysis of the call writes its counters there).
+constexpr idx_t kSpmmLongRow = 1024;
+constexpr idx_t kSpmmLongChunk = 4096;
+size_t spmm_long_rows_bytes(idx_t nnz, int64_t n, size_t value_bytes);
+void launch_spmm_long_find(hipStream_t stream, const SpmmArgs& a, size_t value_bytes);
+template <typename T>
+void launch_spmm_long_rows(hipStream_t stream, const SpmmArgs& a, T alpha, T beta);
 
 // Row-group schedule of a CSR structure (spmm.hip): for every group of kSpmmGroupRows
 // consecutive rows the merged list of their column indices, each entry =

@@ -23,7 +23,8 @@ __global__ __launch_bounds__(kBlock) void spmm_rowb_kernel(idx_t m, idx_t n, idx
                                                            const idx_t* __restrict__ row_ptr,
                                                            const idx_t* __restrict__ col, const T* __restrict__ val,
                                                            const T* __restrict__ B, int64_t ldb, T* __restrict__ C,
-                                                           int64_t ldc, bool c_row_major, T alpha, T beta) {
+                                                           int64_t ldc, bool c_row_major, T alpha, T beta,
+                                                           idx_t long_row) {
     typedef typename ByteOffset<WIDE>::type off_t;
     constexpr int kRowsPerBlock = kBlock / LR;
     const idx_t lane = threadIdx.x % LR;
@@ -37,6 +38,8 @@ __global__ __launch_bounds__(kBlock) void spmm_rowb_kernel(idx_t m, idx_t n, idx
 
     const idx_t start = row_ptr[row] - base;
     const idx_t end = row_ptr[row + 1] - base;
+    // long_row != 0: rows with more nonzeros are the work of the kernels in spmm_long.hip, C included
+    if (long_row != 0 && end - start > long_row) return;  // whole lane groups
     T acc[V];
 #pragma unroll
     for (int i = 0; i < V; ++i) acc[i] = T(0);
@@ -65,7 +68,7 @@ __global__ __launch_bounds__(kBlock) void spmm_narrow_kernel(idx_t m, idx_t n, i
                                                              const idx_t* __restrict__ col,
                                                              const T* __restrict__ val, const T* __restrict__ B,
                                                              int64_t ldb, T* __restrict__ Cm, int64_t ldc,
-                                                             bool c_row_major, T alpha, T beta) {
+                                                             bool c_row_major, T alpha, T beta, idx_t long_row) {
     constexpr int kLanes = 16;
     constexpr int P = kLanes / C;
     constexpr int kSteps = 4;  // measured on a 27-point stencil, n = 8: 1, 2, 4, 8 steps -> 305, 280, 260, 291 us
@@ -93,16 +96,20 @@ __global__ __launch_bounds__(kBlock) void spmm_narrow_kernel(idx_t m, idx_t n, i
     // row clamped to the last one and nonzeros from an index clamped to the last nonzero, and whether
     // a row or a nonzero is really there is only asked where its product would be added.
     const idx_t last_nonzero = nnz - 1;
-    auto range_of = [&](uint64_t row, idx_t& at, idx_t& end) {
+    // left: the row is not this kernel's to write (past the end, or longer than long_row != 0: such rows are the
+    // work of the kernels in spmm_long.hip, C included)
+    auto range_of = [&](uint64_t row, idx_t& at, idx_t& end, bool& left) {
         const uint64_t r = row < last_row ? row : last_row;
         const idx_t b = row_ptr[r] - base;
         const idx_t e = row_ptr[r + 1] - base;
+        left = row >= m || (long_row != 0 && e - b > long_row);
         at = b + phase;
-        end = row < m ? e : b;  // a row past the end is empty
+        end = left ? b : e;  // and counts as empty
     };
     idx_t at, end, at_next, end_next;
-    range_of(first_row, at, end);
-    range_of(first_row + kGroups, at_next, end_next);
+    bool left, left_next;
+    range_of(first_row, at, end, left);
+    range_of(first_row + kGroups, at_next, end_next, left_next);
     idx_t cc[kSteps];
     T aa[kSteps];
 #pragma unroll
@@ -130,7 +137,8 @@ __global__ __launch_bounds__(kBlock) void spmm_narrow_kernel(idx_t m, idx_t n, i
             aa_next[u] = val[j];
         }
         idx_t at_after, end_after;
-        range_of(row + 2 * kGroups, at_after, end_after);
+        bool left_after;
+        range_of(row + 2 * kGroups, at_after, end_after, left_after);
 #pragma unroll
         for (int u = 0; u < kSteps; ++u) {
             if (at + u * P < end) {  // a lane without a nonzero stays out: 0 * inf would be NaN
@@ -174,11 +182,13 @@ __global__ __launch_bounds__(kBlock) void spmm_narrow_kernel(idx_t m, idx_t n, i
                 acc[i] += dpp_mov<kRowRor8>(acc[i]);
             }
         }
-        if (row < m && phase == 0 && in_panel) store_c<T, V>(Cm, ldc, c_row_major, row, c0, acc, alpha, beta);
+        if (!left && phase == 0 && in_panel) store_c<T, V>(Cm, ldc, c_row_major, row, c0, acc, alpha, beta);
         at = at_next;
         end = end_next;
+        left = left_next;
         at_next = at_after;
         end_next = end_after;
+        left_next = left_after;
 #pragma unroll
         for (int u = 0; u < kSteps; ++u) {
             cc[u] = cc_next[u];
@@ -193,7 +203,8 @@ void launch_narrow(hipStream_t stream, const SpmmArgs& a, T alpha, T beta) {
     const uint64_t blocks = (static_cast<uint64_t>(a.m) + kRowsPerBlock - 1) / kRowsPerBlock;
     hipLaunchKernelGGL((spmm_narrow_kernel<T, V, C>), dim3(static_cast<uint32_t>(blocks)), dim3(kBlock), 0, stream, a.m,
                        a.n, a.nnz, a.base, a.row_ptr, a.col, static_cast<const T*>(a.val),
-                       static_cast<const T*>(a.B), a.ldb, static_cast<T*>(a.C), a.ldc, a.c_row_major, alpha, beta);
+                       static_cast<const T*>(a.B), a.ldb, static_cast<T*>(a.C), a.ldc, a.c_row_major, alpha, beta,
+                       a.long_row);
 }
 
 // op(B) column-major: element (kk, j) at j*ldb + kk.  One wavefront per row of A, lanes strided
@@ -205,10 +216,12 @@ __global__ __launch_bounds__(kBlock) void spmm_colb_kernel(idx_t m, idx_t n, idx
                                                            const idx_t* __restrict__ col, const T* __restrict__ val,
                                                            const T* __restrict__ B, int64_t ldb, T* __restrict__ C,
                                                            int64_t c_row_stride, int64_t c_col_stride, T alpha,
-                                                           T beta) {
+                                                           T beta, idx_t long_row) {
     const unsigned lane = threadIdx.x % kWave;
     const uint64_t row = static_cast<uint64_t>(blockIdx.x) * (kBlock / kWave) + threadIdx.x / kWave;
-    const bool live = row < m;  // dead waves still run the reductions with zero work
+    bool live = row < m;  // dead waves still run the reductions with zero work
+    // long_row != 0: rows with more nonzeros are the work of the kernels in spmm_long.hip, C included
+    if (live && long_row != 0 && row_ptr[row + 1] - row_ptr[row] > long_row) live = false;
     const idx_t start = live ? row_ptr[row] - base : 0;
     const idx_t end = live ? row_ptr[row + 1] - base : 0;
 
@@ -657,10 +670,10 @@ void launch_rowb(hipStream_t stream, const SpmmArgs& a, T alpha, T beta) {
     T* C = static_cast<T*>(a.C);
     if (narrow_offsets(a, sizeof(T))) {
         hipLaunchKernelGGL((spmm_rowb_kernel<T, LR, V, false>), grid, dim3(kBlock), 0, stream, a.m, a.n, a.base,
-                           a.row_ptr, a.col, val, B, a.ldb, C, a.ldc, a.c_row_major, alpha, beta);
+                           a.row_ptr, a.col, val, B, a.ldb, C, a.ldc, a.c_row_major, alpha, beta, a.long_row);
     } else {
         hipLaunchKernelGGL((spmm_rowb_kernel<T, LR, V, true>), grid, dim3(kBlock), 0, stream, a.m, a.n, a.base,
-                           a.row_ptr, a.col, val, B, a.ldb, C, a.ldc, a.c_row_major, alpha, beta);
+                           a.row_ptr, a.col, val, B, a.ldb, C, a.ldc, a.c_row_major, alpha, beta, a.long_row);
     }
 }
 
@@ -699,11 +712,17 @@ void launch_spmm(hipStream_t stream, const SpmmArgs& a, T alpha, T beta) {
         T* C = static_cast<T*>(a.C);
         if (beta == T(0)) {
             hipLaunchKernelGGL((spmm_colb_kernel<T, kJB, true>), dim3(static_cast<uint32_t>(blocks)), dim3(kBlock), 0,
-                               stream, a.m, a.n, a.base, a.row_ptr, a.col, val, B, a.ldb, C, rs, cs, alpha, beta);
+                               stream, a.m, a.n, a.base, a.row_ptr, a.col, val, B, a.ldb, C, rs, cs, alpha, beta,
+                               a.long_row);
         } else {
             hipLaunchKernelGGL((spmm_colb_kernel<T, kJB, false>), dim3(static_cast<uint32_t>(blocks)), dim3(kBlock), 0,
-                               stream, a.m, a.n, a.base, a.row_ptr, a.col, val, B, a.ldb, C, rs, cs, alpha, beta);
+                               stream, a.m, a.n, a.base, a.row_ptr, a.col, val, B, a.ldb, C, rs, cs, alpha, beta,
+                               a.long_row);
         }
+    }
+    if (a.long_row != 0) {
+        launch_spmm_long_find(stream, a, sizeof(T));
+        launch_spmm_long_rows<T>(stream, a, alpha, beta);
     }
 }
 

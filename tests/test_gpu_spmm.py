@@ -163,8 +163,10 @@ def test_preprocessed_ragged_rows_with_overlap(torch_gpu, handle, oracle):
     for r in range(m):
         if r % 7 == 3:
             cols = np.zeros(0, np.int64)
-        elif r in (100, 101):
-            cols = rng.choice(k, 1100, replace=False)           # 2200 nonzeros in their group: not merged
+        elif r in (100, 101, 102):
+            # 2700 nonzeros in their group: not merged (each row short of the 1024 above which rows are cut into
+            # pieces and preprocess builds no schedule at all)
+            cols = rng.choice(k, 900, replace=False)
         else:
             prev = rows[-1] if rows and len(rows[-1]) else rng.choice(k, 12, replace=False)
             keep = prev[rng.random(len(prev)) < 0.8]
@@ -402,8 +404,8 @@ def test_blocks_banded_matrix_with_broken_rows(torch_gpu, handle, oracle, dtype,
             c = c[::2]
         if r % 211 == 7:
             c = np.zeros(0, np.int64)
-        if r in (1000, 1001):
-            c = rng.choice(k, 1500, replace=False)   # 3000 nonzeros in their group: not covered, row by row
+        if r in (1000, 1001, 1002):
+            c = rng.choice(k, 900, replace=False)   # 2700 nonzeros in their group: not covered, row by row
         if r % 120 == 0:
             c = rng.permutation(c)
         rows.append(c)
@@ -437,7 +439,7 @@ def test_blocks_row_ignores_rows_of_b_only_its_neighbours_use(torch_gpu, handle)
 
 def grid_9pt(line, lines, dtype, rng, broken=False):
     """9-point stencil on `lines` grid lines of `line` points, numbered line by line; broken: rows with holes, empty
-    rows, unsorted rows, one row with 2500 nonzeros (its group is too long to cover) and a duplicate column."""
+    rows, unsorted rows, three rows with 800 nonzeros each (their group is too long to cover) and a duplicate column."""
     m = line * lines
     rows = []
     for r in range(m):
@@ -453,8 +455,8 @@ def grid_9pt(line, lines, dtype, rng, broken=False):
                 c = rng.permutation(c)
             if r % 333 == 9 and len(c) > 2:
                 c = np.concatenate([c[:2], c[1:]])     # a column twice in a row
-            if r == 1000:
-                c = rng.choice(m, 2500, replace=False)
+            if r in (1000, 1001, 1002):
+                c = rng.choice(m, 800, replace=False)
         rows.append(c)
     ptr = np.concatenate([[0], np.cumsum([len(c) for c in rows])]).astype(np.int32)
     return wl.Csr(m, m, ptr, np.concatenate(rows).astype(np.int32), rng.uniform(-1, 1, int(ptr[-1])).astype(dtype))
