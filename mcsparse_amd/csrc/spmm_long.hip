@@ -30,29 +30,90 @@ __global__ void spmm_long_zero_kernel(LongCounters* c) {
 }
 
 // item: {row, piece, pieces of the row, first row of partial sums of the row (unused for one piece)}
+//
+// The places in the three lists come off three counters, and atomic adds to one address take their turns (3.4 ns
+// each: 12,000 long rows among 4 M, found by a thread each, 195 us).  So a workgroup looks at kFindRows rows,
+// collects its long ones in LDS with places relative to the workgroup, and takes its share of the lists with one
+// add per counter (the same matrix: 36 us).
+constexpr uint32_t kFindRows = 8192;   // rows a workgroup looks at
+constexpr uint32_t kFindList = 2048;   // long rows it can collect; further ones take their places one by one
+
+__device__ __forceinline__ void write_long_row(uint32_t row, uint32_t pieces, uint32_t first, uint32_t slot, uint32_t at,
+                                               uint4* __restrict__ items, uint4* __restrict__ rows, uint32_t cap_items,
+                                               uint32_t cap_rows, uint32_t cap_slots) {
+    // (the capacities hold for every structure whose offsets add up to nnz; for one that does not, nothing is
+    // written out of bounds, and the rows that found no room are missing from the product)
+    bool fits = first + pieces <= cap_items && first + pieces >= first;
+    if (pieces > 1) {
+        fits = fits && slot + pieces <= cap_slots && slot + pieces >= slot && at < cap_rows;
+        if (at < cap_rows) rows[at] = fits ? make_uint4(row, slot, pieces, 0u) : make_uint4(row, 0u, 0u, 0u);
+    }
+    for (uint32_t j = 0; j < pieces && first + j < cap_items; ++j)
+        items[first + j] = make_uint4(row, j, fits ? pieces : 0u, slot);
+}
+
 __global__ __launch_bounds__(kBlock) void spmm_long_find_kernel(idx_t m, const idx_t* __restrict__ row_ptr,
                                                                 LongCounters* __restrict__ c, uint4* __restrict__ items,
                                                                 uint4* __restrict__ rows, uint32_t cap_items,
                                                                 uint32_t cap_rows, uint32_t cap_slots) {
-    const uint64_t row = static_cast<uint64_t>(blockIdx.x) * kBlock + threadIdx.x;
-    if (row >= m) return;
-    const idx_t len = row_ptr[row + 1] - row_ptr[row];
-    if (len <= kSpmmLongRow) return;
-    const uint32_t pieces = (len + kSpmmLongChunk - 1) / kSpmmLongChunk;
-    const uint32_t first = atomicAdd(&c->items, pieces);
-    uint32_t slot = 0;
-    bool fits = first + pieces <= cap_items && first + pieces >= first;
-    if (pieces > 1) {
-        slot = atomicAdd(&c->slots, pieces);
-        const uint32_t at = atomicAdd(&c->rows, 1u);
-        fits = fits && slot + pieces <= cap_slots && at < cap_rows;
-        // (the capacities hold for every structure whose offsets add up to nnz; for one that does not, nothing is
-        // written out of bounds, and the rows that found no room are missing from the product)
-        if (fits) rows[at] = make_uint4(static_cast<uint32_t>(row), slot, pieces, 0u);
-        else if (at < cap_rows) rows[at] = make_uint4(static_cast<uint32_t>(row), 0u, 0u, 0u);
+    __shared__ uint4 s_list[kFindList];      // {row, pieces, first item, first slot}, relative to the workgroup
+    __shared__ uint32_t s_list_row[kFindList];  // place in the list of rows of several pieces
+    __shared__ uint32_t s_count, s_items, s_slots, s_rows;
+    __shared__ uint32_t s_base[3];
+    const uint32_t tid = threadIdx.x;
+    if (tid == 0) {
+        s_count = 0;
+        s_items = 0;
+        s_slots = 0;
+        s_rows = 0;
     }
-    for (uint32_t j = 0; j < pieces && first + j < cap_items; ++j)
-        items[first + j] = make_uint4(static_cast<uint32_t>(row), j, fits ? pieces : 0u, slot);
+    __syncthreads();
+    const uint64_t row0 = static_cast<uint64_t>(blockIdx.x) * kFindRows;
+    constexpr uint32_t kAtOnce = 8;  // rows a thread asks for before it looks at any: one trip to memory for the lot
+    static_assert(kFindRows % (kBlock * kAtOnce) == 0, "whole rounds");
+    for (uint32_t k0 = tid; k0 < kFindRows; k0 += kBlock * kAtOnce) {
+        idx_t lens[kAtOnce];
+#pragma unroll
+        for (uint32_t u = 0; u < kAtOnce; ++u) {
+            const uint64_t row = row0 + k0 + u * kBlock;
+            const uint64_t r = row < m ? row : m - 1;  // m != 0 here
+            lens[u] = row < m ? row_ptr[r + 1] - row_ptr[r] : 0;
+        }
+#pragma unroll
+        for (uint32_t u = 0; u < kAtOnce; ++u) {
+            const uint64_t row = row0 + k0 + u * kBlock;
+            const idx_t len = lens[u];
+            if (len <= kSpmmLongRow) continue;
+            const uint32_t pieces = (len + kSpmmLongChunk - 1) / kSpmmLongChunk;
+            const uint32_t at = atomicAdd(&s_count, 1u);
+            if (at < kFindList) {
+                const uint32_t first = atomicAdd(&s_items, pieces);
+                const uint32_t slot = pieces > 1 ? atomicAdd(&s_slots, pieces) : 0u;
+                s_list_row[at] = pieces > 1 ? atomicAdd(&s_rows, 1u) : 0u;
+                s_list[at] = make_uint4(static_cast<uint32_t>(row), pieces, first, slot);
+            } else {  // no room in the workgroup's list: places straight off the counters
+                const uint32_t first = atomicAdd(&c->items, pieces);
+                const uint32_t slot = pieces > 1 ? atomicAdd(&c->slots, pieces) : 0u;
+                const uint32_t place = pieces > 1 ? atomicAdd(&c->rows, 1u) : 0u;
+                write_long_row(static_cast<uint32_t>(row), pieces, first, slot, place, items, rows, cap_items, cap_rows,
+                               cap_slots);
+            }
+        }
+    }
+    __syncthreads();
+    const uint32_t listed = min(s_count, kFindList);
+    if (listed == 0) return;  // whole workgroup
+    if (tid == 0) {
+        s_base[0] = atomicAdd(&c->items, s_items);
+        s_base[1] = s_slots != 0 ? atomicAdd(&c->slots, s_slots) : 0u;
+        s_base[2] = s_rows != 0 ? atomicAdd(&c->rows, s_rows) : 0u;
+    }
+    __syncthreads();
+    for (uint32_t k = tid; k < listed; k += kBlock) {
+        const uint4 e = s_list[k];
+        write_long_row(e.x, e.y, s_base[0] + e.z, s_base[1] + e.w, s_base[2] + s_list_row[k], items, rows, cap_items,
+                       cap_rows, cap_slots);
+    }
 }
 
 // lanes: lane groups of `lanes` threads (a power of two up to 64) hold the columns of a panel of lanes * V columns
@@ -197,7 +258,7 @@ void launch_spmm_long_find(hipStream_t stream, const SpmmArgs& a, size_t value_b
     char* w = static_cast<char*>(a.long_ws);
     LongCounters* c = reinterpret_cast<LongCounters*>(w + l.counters);
     hipLaunchKernelGGL(spmm_long_zero_kernel, dim3(1), dim3(1), 0, stream, c);
-    hipLaunchKernelGGL(spmm_long_find_kernel, dim3((a.m + kBlock - 1) / kBlock), dim3(kBlock), 0, stream, a.m, a.row_ptr,
+    hipLaunchKernelGGL(spmm_long_find_kernel, dim3((a.m + kFindRows - 1) / kFindRows), dim3(kBlock), 0, stream, a.m, a.row_ptr,
                        c, reinterpret_cast<uint4*>(w + l.items), reinterpret_cast<uint4*>(w + l.rows), l.cap_items,
                        l.cap_rows, l.cap_slots);
 }
