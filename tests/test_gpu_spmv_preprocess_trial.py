@@ -79,8 +79,9 @@ def test_a_prepared_call_is_not_slower_than_one_that_was_not(torch_gpu, handle, 
     mat, buf, y, vx2, vy, state = prepared(torch, handle, a, d, x, alg, trial=True)
     assert state in states, (name, state)
     t_prepared = timed_us(torch, handle, mat, vx2, vy, ct, buf, alg)
-    # the trial keeps a copy that is faster by a twentieth; the slack here is for the noise of two timings
-    assert t_prepared <= 1.15 * t_plain, (name, state, t_plain, t_prepared)
+    # the trial keeps a copy that is faster by a twentieth; the slack here is for the noise of two timings (the copies
+    # that were turned down took 1.5 to 3.6 times as long as the row kernels)
+    assert t_prepared <= 1.25 * t_plain, (name, state, t_plain, t_prepared)
 
     y_ref, bound = oracle.spmv(False, a.m, a.n, a.base, a.ptr, a.col, a.val, 1.0, 0.0, x_host, np.zeros(a.m, dt))
     assert api.spmv(handle, api.OP_N, 1.0, mat, vx2, 0.0, vy, ct, buf, alg=alg) == api.STATUS_SUCCESS
