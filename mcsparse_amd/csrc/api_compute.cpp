@@ -1123,13 +1123,15 @@ mcsparseStatus_t mcsparseSpMM_preprocess(mcsparseHandle_t handle, mcsparseOperat
     }
     const char* span_slot = static_cast<const char*>(externalBuffer) + l.span_sum;
 
-    // First choice, for operands of 65 to 1024 bytes per row (the widths its kernel was measured faster at: by 35 %,
+    // First choice, for operands of 65 (fp64: 129) to 1024 bytes per row (the widths its kernel was measured faster at: by 35 %,
     // 16 %, 29 % and 4 % at 32, 64, 128 and 256 fp32 columns of a 27-point stencil): diagonal blocks over groups of
     // eight rows.  Kept when the blocks are large (a stencil's are 24 nonzeros each) and each loaded row of op(B)
     // serves about two nonzeros or more; matrices without such structure get the merged column lists.
     const size_t vb = value_size(matA->valueType);
     const int64_t row_bytes = matC->col_num * static_cast<int64_t>(vb);
-    const bool wide_enough = row_bytes > 64 && row_bytes <= 1024 && matA->row_num < (int64_t(1) << 31);
+    // (in fp64 from 129 bytes: at 12 and 16 columns of a 27-point stencil the kernel without a schedule is 2 and 5 %
+    // faster)
+    const bool wide_enough = row_bytes > (vb == 8 ? 128 : 64) && row_bytes <= 1024 && matA->row_num < (int64_t(1) << 31);
     if (wide_enough) {
         mcsp::launch_spmm_block_count(handle->stream, m, nnz, static_cast<idx_t>(matA->idxBase), ia.rows, ia.cols,
                                       externalBuffer);

@@ -758,9 +758,13 @@ void launch_spmm_schedule(hipStream_t stream, idx_t m, idx_t nnz, idx_t base, co
 
 bool spmm_schedule_usable(const SpmmArgs& a, size_t value_bytes) {
     const int64_t wide = static_cast<int64_t>(16 / value_bytes);
-    // up to four 128-bit vectors per row: too few lanes per group to share the fetching (four lanes: 27-point
-    // stencil, 16 fp32 columns 0.62 ms against 0.32 ms without the schedule; 8 fp64 columns 0.87 against 0.39 ms)
-    return a.b_row_major && a.n >= 4 * wide + 1 && a.k <= kSpmmMaxScheduledColumns &&
+    // Few 128-bit vectors per row are too few lanes per group to share the fetching.  Against the kernel without a
+    // schedule, on a 27-point stencil, rows of three degrees of freedom per node and a 5-point Laplacian: four lanes
+    // (16 fp32 columns) half as fast; five and eight lanes (20 and 32 fp32 columns) 8 to 25 % slower or level; nine
+    // and more lanes of fp32 6 to 28 % faster; ten to sixteen lanes of fp64 between 9 % slower and 13 % faster, more
+    // lanes level or faster (up to 56 %).
+    const int64_t lanes_at_least = value_bytes == 4 ? 9 : 17;
+    return a.b_row_major && a.n > (lanes_at_least - 1) * wide && a.k <= kSpmmMaxScheduledColumns &&
            reinterpret_cast<uintptr_t>(a.B) % 16 == 0 &&
            a.ldb % wide == 0 && a.n % wide == 0 &&
            (!a.c_row_major || (reinterpret_cast<uintptr_t>(a.C) % 16 == 0 && a.ldc % wide == 0));

@@ -411,8 +411,9 @@ def test_blocks_banded_matrix_with_broken_rows(torch_gpu, handle, oracle, dtype,
         rows.append(c)
     ptr = np.concatenate([[0], np.cumsum([len(c) for c in rows])]).astype(np.int32)
     a = wl.Csr(m, k, ptr, np.concatenate(rows).astype(np.int32), rng.uniform(-1, 1, int(ptr[-1])).astype(dtype))
-    # blocks for operands of 65 to 1024 bytes per row, merged column lists beyond
-    want = 3 if 64 < n * np.dtype(dtype).itemsize <= 1024 else (1, 2)
+    # blocks for operands of 65 (fp64: 129) to 1024 bytes per row, merged column lists beyond
+    least = 128 if dtype == np.float64 else 64
+    want = 3 if least < n * np.dtype(dtype).itemsize <= 1024 else (1, 2)
     for c_order in (api.ORDER_ROW, api.ORDER_COL):
         check(torch_gpu, handle, oracle, a, n, 1.0, 0.0, preprocess=True, expect_schedule=want, c_order=c_order)
     check(torch_gpu, handle, oracle, a.with_base(1), n, -0.5, 1.5, preprocess=True, expect_schedule=want, pad_b=4, pad_c=8)
@@ -470,7 +471,7 @@ def test_strips_grid_with_broken_rows(torch_gpu, handle, oracle, dtype, n):
     a = grid_9pt(20, 151, dtype, np.random.default_rng(6), broken=True)
     row_bytes = n * np.dtype(dtype).itemsize
     # strips for operands of 129 to 1024 bytes per row, groups of eight rows from 65 bytes, merged column lists otherwise
-    want = 4 if 128 < row_bytes <= 1024 else 3 if 64 < row_bytes <= 128 else (1, 2)
+    want = 4 if 128 < row_bytes <= 1024 else 3 if 64 < row_bytes <= 128 and dtype == np.float32 else (1, 2)
     for c_order in (api.ORDER_ROW, api.ORDER_COL):
         check(torch_gpu, handle, oracle, a, n, 1.0, 0.0, preprocess=True, expect_schedule=want, c_order=c_order,
               prepare_for_row_major_c=True)
