@@ -138,3 +138,28 @@ def test_the_trial_leaves_the_pointer_mode_and_takes_any_x(torch_gpu, handle, or
     handle.set_pointer_mode(api.PTR_HOST)
     y_ref, bound = oracle.spmv(False, a.m, a.n, a.base, a.ptr, a.col, a.val, 1.5, -0.5, x_host, y_host)
     assert_within(y.cpu().numpy(), y_ref, bound, np.float64, what="device scalars after the trial (state %d)" % state)
+
+
+def test_a_band_width_set_by_the_caller_is_not_tried(torch_gpu, handle, oracle):
+    """mcsparseSpMatSetSpMVBandBytes says that the caller is measuring the copy by itself: it is kept, also on the
+    Laplacian, where the trial turns it down."""
+    torch = torch_gpu
+    a = wl.laplacian_5pt(2048, dtype=np.float32)
+    rng = np.random.default_rng(8)
+    x_host = rng.uniform(-1, 1, a.n).astype(np.float32)
+    d = [dev(torch, v) for v in (a.ptr, a.col, a.val)]
+    x = dev(torch, x_host)
+    y = torch.zeros(a.m, dtype=torch.float32, device="cuda")
+    mat = api.SpMat(a.m, a.n, a.nnz, d[0], d[1], d[2], base=a.base)
+    mat.set_band_bytes(1 << 21)
+    vx, vy = api.DnVec(x), api.DnVec(y)
+    assert handle.spmv_preprocess_trial() is True
+    st, size = api.spmv_preprocess_buffer_size(handle, api.OP_N, 1.0, mat, vx, 0.0, vy, api.R_32F)
+    assert st == api.STATUS_SUCCESS
+    buf = torch.empty(size, dtype=torch.uint8, device="cuda")
+    assert api.spmv_preprocess(handle, api.OP_N, 1.0, mat, vx, 0.0, vy, api.R_32F, buf) == api.STATUS_SUCCESS
+    assert mat.spmv_preprocess_state()[0] == 3
+    assert api.spmv(handle, api.OP_N, 1.0, mat, vx, 0.0, vy, api.R_32F, buf) == api.STATUS_SUCCESS
+    torch.cuda.synchronize()
+    y_ref, bound = oracle.spmv(False, a.m, a.n, a.base, a.ptr, a.col, a.val, 1.0, 0.0, x_host, np.zeros(a.m, np.float32))
+    assert_within(y.cpu().numpy(), y_ref, bound, np.float32, what="copy of a caller who set the band width")
