@@ -760,7 +760,7 @@ mcspStatus_t spmv_call(mcsparseHandle_t handle, mcsparseOperation_t opA, const v
 // banded matrix reads x line by line as it is; an x that fits an L2 next to rows long enough to fill the lanes
 // leaves the copy's extra partial sums as pure cost), so both are run here, on the handle's stream, with the
 // caller's x and a y inside the buffer, and timed with events: once each, which settles it where one takes more
-// than twice the other's time, else twice more.  *copy_wins says whether the copy was faster by more than a
+// than twice the other's time (or, for long runs, a quarter more), else twice more.  *copy_wins says whether the copy was faster by more than a
 // twentieth.
 mcspStatus_t spmv_trial(mcsparseHandle_t handle, mcsparseOperation_t opA, mcsparseSpMatDescr_t matA,
                         mcsparseDnVecDescr_t vecX, void* trial_y, macaDataType computeType, void* buffer,
@@ -795,8 +795,10 @@ mcspStatus_t spmv_trial(mcsparseHandle_t handle, mcsparseOperation_t opA, mcspar
              hipEventElapsedTime(&rows_ms, marks[0], marks[1]) != hipSuccess ||
              hipEventElapsedTime(&copy_ms, marks[1], marks[2]) != hipSuccess))
             st = MCSP_STATUS_INTERNAL_ERROR;
-        // the first runs of the two are their slowest (cold caches): enough to tell two from one, not 20 from 19
-        if (rows_ms > 2.0f * copy_ms || copy_ms > 2.0f * rows_ms) break;
+        // the first runs of the two are their slowest (cold caches, by some tens of microseconds): enough to tell two
+        // from one, or five from four where a run takes a third of a millisecond and more, not 20 from 19
+        const float slower = rows_ms > copy_ms ? rows_ms : copy_ms, faster = rows_ms > copy_ms ? copy_ms : rows_ms;
+        if (slower > 2.0f * faster || (faster > 0.3f && slower > 1.25f * faster)) break;
     }
     for (hipEvent_t e : marks)
         if (e != nullptr) (void)hipEventDestroy(e);
