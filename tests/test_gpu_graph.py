@@ -205,6 +205,49 @@ def test_transposing_spmv_replays_in_a_hip_graph(torch_gpu, oracle, alg):
     handle.destroy()
 
 
+@pytest.mark.parametrize("analysed", [True, False])
+def test_spmm_with_long_rows_replays_in_a_hip_graph(torch_gpu, oracle, analysed):
+    """Rows of thousands of nonzeros: the list of their pieces is rebuilt by every call (a kernel clears its counters,
+    not a memset), the pieces and the sums of the partial sums are kernels.  analysed: an eager call has left the
+    row lengths on the descriptor; else the captured call is the first on the structure, cannot read them back and
+    takes the launches for long rows without knowing whether there are any."""
+    torch = torch_gpu
+    rng = np.random.default_rng(24)
+    side = torch.cuda.Stream()
+    handle = api.Handle(stream=side.cuda_stream)
+    a = wl.mixed_rows(m=6000, per_row=9, long_rows=5, long_len=9000, dtype=np.float64)
+    n = 24
+    d_ptr, d_col, d_val = dev(torch, a.ptr), dev(torch, a.col), dev(torch, a.val)
+    A = api.SpMat(a.m, a.n, a.nnz, d_ptr, d_col, d_val, base=a.base)
+    B = torch.zeros((a.n, n), dtype=torch.float64, device="cuda")
+    C = torch.zeros((a.m, n), dtype=torch.float64, device="cuda")
+    mB, mC = api.DnMat(a.n, n, n, B), api.DnMat(a.m, n, n, C)
+    st, size = api.spmm_buffer_size(handle, api.OP_N, api.OP_N, 1.5, A, mB, -0.25, mC, api.R_64F)
+    assert st == 0
+    buf = torch.empty(size, dtype=torch.uint8, device="cuda")
+    if analysed:
+        with torch.cuda.stream(side):
+            assert api.spmm(handle, api.OP_N, api.OP_N, 1.5, A, mB, -0.25, mC, api.R_64F, buf) == 0
+        torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        assert api.spmm(handle, api.OP_N, api.OP_N, 1.5, A, mB, -0.25, mC, api.R_64F, buf) == 0
+    torch.cuda.synchronize()
+    for replay in range(3):
+        hB = rng.uniform(-1, 1, (a.n, n))
+        hC = rng.uniform(-1, 1, (a.m, n))
+        B.copy_(torch.from_numpy(hB))
+        C.copy_(torch.from_numpy(hC))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        ref, bound = oracle.spmm(a.m, n, a.base, a.ptr, a.col, a.val, 1.5, -0.25, hB.ravel(), n, True, hC.ravel(), n, True)
+        assert_within(C.cpu().numpy(), ref, bound, np.float64, what="replay %d, analysed %r" % (replay, analysed))
+    del graph
+    torch.cuda.synchronize()
+    handle.destroy()
+
+
 def test_static_buffer_call_replays_in_a_hip_graph(torch_gpu, oracle):
     """mcsparseSpMV_staticBuffer is for callers that cannot allocate, code under graph capture among them.  The
     address of its scratch array is looked up at the first call on a device, which a capture cannot hold: that call
