@@ -306,6 +306,28 @@ def test_spmm_argument_checks(lib):
     assert size.value == 128
 
 
+def test_spmm_buffer_size_has_room_for_the_pieces_of_long_rows(lib):
+    """Rows of more than 1024 nonzeros are cut into pieces of 4096; a row of several pieces needs a row of partial
+    sums per piece, at most 2 * nnz / 4096 of them whatever the row lengths are (the size cannot depend on them: it
+    is asked for before the matrix is looked at)."""
+    m, k, nnz = 1 << 16, 1 << 16, 1 << 22
+    o = Objs(lib, m=m, n=k, nnz=nnz)
+    sizes = {}
+    for n in (16, 64, 250):
+        B, C = ctypes.c_void_p(), ctypes.c_void_p()
+        lib.mcsparseCreateDnMat(ctypes.byref(B), k, n, n, FAKE, api.R_32F, api.ORDER_ROW)
+        lib.mcsparseCreateDnMat(ctypes.byref(C), m, n, n, FAKE, api.R_32F, api.ORDER_ROW)
+        size = ctypes.c_size_t()
+        assert lib.mcsparseSpMM_bufferSize(o.h, 0, 0, o.pa, o.A, B, o.pa, C, api.R_32F, 0, ctypes.byref(size)) == 0
+        sizes[n] = size.value
+    padded = {16: 16, 64: 64, 250: 252}
+    rows_of_sums = 2 * (nnz // 4096)
+    for n in sizes:
+        assert sizes[n] >= 4 * nnz + rows_of_sums * padded[n] * 4, (n, sizes[n])     # the schedule and the partial sums
+        assert sizes[n] <= 4 * nnz + 4 * m + (rows_of_sums + 2) * padded[n] * 4 + (1 << 18), (n, sizes[n])
+    assert sizes[16] < sizes[64] < sizes[250]
+
+
 def test_conversion_argument_checks(lib):
     # conversion/mcsp_coo2csr.cpp:7-59, mcsp_csr2csc.cpp:9-63, :293-310
     h = ctypes.c_void_p()
